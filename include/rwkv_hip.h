@@ -1,0 +1,227 @@
+/*
+ * C ABI of the MI355X (gfx950) RWKV-7 inference kernels.
+ *
+ * Plain pointers and sizes only: no HIP, CUDA or torch types.  Every `void*` tensor argument
+ * is a device address unless the name ends in `_host`.  fp16 tensors are IEEE binary16.
+ * `rwkv_stream_t` is an opaque stream handle (NULL = the default stream).
+ *
+ * Every function returns 0 on success or a negative RWKV_E_* code and never terminates the
+ * process; rwkv_hip_last_error() returns the calling thread's last message.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * reference repository root).  The reference's kernel ABI is the C++-linkage launcher list in
+ * cuda/rwkv7_fast_v4_kernels.cuh:8-211 plus src/utils/sampling.h:10-46.
+ */
+#ifndef RWKV_HIP_H
+#define RWKV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* rwkv_stream_t;
+
+enum {
+  RWKV_OK = 0,
+  RWKV_E_INVALID = -1,     /* bad argument / shape the kernels do not support */
+  RWKV_E_RUNTIME = -2,     /* HIP runtime error */
+  RWKV_E_NOMEM = -3,       /* device or host allocation failed */
+  RWKV_E_STATE = -4,       /* object used before it was fully set up */
+};
+
+enum { RWKV_FMT_F16 = 0, RWKV_FMT_W8 = 1, RWKV_FMT_W4 = 2 };
+enum { RWKV_W_RAW_LOGIT = 0, RWKV_W_DECAY = 1 };
+enum { RWKV_IO_F16 = 0, RWKV_IO_F32 = 1 };
+enum { RWKV_ACT_NONE = 0, RWKV_ACT_TANH = 1, RWKV_ACT_SIGMOID = 2 };
+enum { RWKV_EPI_NONE = 0, RWKV_EPI_RELU_SQUARE = 1 };
+
+const char* rwkv_hip_last_error(void);
+
+/* ---- runtime plumbing.  Replaces the cudaMalloc/cudaMemcpy/cudaMemset/cudaStream* calls
+ * inside DeviceBuffer<T> (include/rwkv7_fast_v4_common.hpp:64-110), run_backend_forward
+ * (src/rwkv7_fast_v4.cu:1087-1096,1343-1344) and StateCacheManager
+ * (src/rwkv_state_cache.cpp:132-223). ---- */
+int rwkv_hip_device_count(int* count);
+int rwkv_hip_device_name(char* buf, size_t buf_len);
+int rwkv_hip_malloc(void** ptr, size_t bytes);
+int rwkv_hip_free(void* ptr);
+int rwkv_hip_host_alloc(void** ptr_host, size_t bytes); /* pinned */
+int rwkv_hip_host_free(void* ptr_host);
+int rwkv_hip_memcpy_h2d(void* dst, const void* src_host, size_t bytes);
+int rwkv_hip_memcpy_d2h(void* dst_host, const void* src, size_t bytes);
+int rwkv_hip_memcpy_d2d(void* dst, const void* src, size_t bytes);
+int rwkv_hip_memcpy_h2d_async(rwkv_stream_t s, void* dst, const void* src_host, size_t bytes);
+int rwkv_hip_memcpy_d2h_async(rwkv_stream_t s, void* dst_host, const void* src, size_t bytes);
+int rwkv_hip_memcpy_d2d_async(rwkv_stream_t s, void* dst, const void* src, size_t bytes);
+int rwkv_hip_memset(void* ptr, int value, size_t bytes);
+int rwkv_hip_mem_info(size_t* free_bytes, size_t* total_bytes);
+int rwkv_hip_stream_create(rwkv_stream_t* s);
+int rwkv_hip_stream_destroy(rwkv_stream_t s);
+int rwkv_hip_stream_sync(rwkv_stream_t s);
+int rwkv_hip_device_sync(void);
+/* event timing on a stream: ms between two recorded points, for benchmarks */
+int rwkv_hip_event_create(void** ev);
+int rwkv_hip_event_destroy(void* ev);
+int rwkv_hip_event_record(void* ev, rwkv_stream_t s);
+int rwkv_hip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms);
+
+/* ---- WKV7 time-mix recurrence.  Replaces rwkv7_wkv_fp32io16_launch
+ * (cuda/rwkv7_fast_v4_kernels.cuh:49-52, cuda/rwkv7_wkv_fp32_v2.cu:237-294).
+ * state f32 [B,H,64,64] in/out; r,w,k,v,a,b,y [B,T,C], C == H*64.
+ * w_mode RWKV_W_RAW_LOGIT: decay = exp(-e^-1/2 * sigmoid(w)) (the reference's only mode);
+ * RWKV_W_DECAY: w is the decay itself.  io RWKV_IO_F16 / RWKV_IO_F32 selects the element type of
+ * r..y (the reference builds one or the other with _IO_FP16_, rwkv7_wkv_fp32_v2.cu:16-24).
+ * Running T1+T2 tokens in one call or in two consecutive calls gives bitwise the same result. */
+int rwkv_hip_wkv7(rwkv_stream_t s, int B, int T, int C, int H, int w_mode, int io, void* state,
+                  const void* r, const void* w, const void* k, const void* v, const void* a, const void* b,
+                  void* y);
+
+/* ---- weight formats (no counterpart in the reference, whose weights are fp16 only).
+ * W8: int8 [N,K] + f16 scale [N].  W4: packed u8 [N,K/2] (element k even -> low nibble of byte
+ * k/2) + f16 scale [N,K/128] + u8 zero point [N,K/128]; K % 128 == 0. ---- */
+int rwkv_hip_quantize_w8(rwkv_stream_t s, int N, int K, const void* w_f16, void* q, void* scale);
+int rwkv_hip_dequant_w8(rwkv_stream_t s, int N, int K, const void* q, const void* scale, void* w_f16);
+int rwkv_hip_quantize_w4(rwkv_stream_t s, int N, int K, const void* w_f16, void* q, void* scale, void* zp);
+int rwkv_hip_dequant_w4(rwkv_stream_t s, int N, int K, const void* q, const void* scale, const void* zp,
+                        void* w_f16);
+
+/* Synthetic fp16 weights ~ mean + std*N(0,1) from a counter-based hash of (seed, index): random-init
+ * models for benchmarks without a checkpoint (no counterpart in the reference, which loads .pth files). */
+int rwkv_hip_fill_normal_f16(rwkv_stream_t s, int64_t n, uint64_t seed, float mean, float stdv, void* out);
+
+/* ---- linear layers, y[M,N] = x[M,K] . W[N,K]^T, fp32 accumulate.
+ * Replaces rwkv7_v3a_linear_orig_rows_exact_f16_launch / _orig_rows_f16_launch / _f16_orig_launch /
+ * _f16_orig_lt_cfg_launch (cuda/rwkv7_fast_v4_kernels.cuh:155-177) and the dispatch in
+ * linear_orig_layout_launch (src/rwkv7_fast_v4.cu:709-959).  Any M: small M streams the weights
+ * once through a GEMV kernel, M >= 16 uses MFMA tiles.
+ * out_f32 == 0: y is f16 [M,N].  out_f32 == 1: y is f32 [M,N] holding the f16-rounded value
+ * (the lm_head path, src/rwkv7_fast_v4.cu:1325-1341 + rwkv7_v4_f16_to_f32_launch).
+ * epilogue RWKV_EPI_RELU_SQUARE applies relu(.)^2 to the f16-rounded result and rounds again
+ * (rwkv7_relu_square_launch, cuda/rwkv7_fast_v4_kernels.cuh:83). */
+int rwkv_hip_linear(rwkv_stream_t s, int fmt, int M, int N, int K, const void* x, const void* w,
+                    const void* scale, const void* zp, int epilogue, int out_f32, void* y);
+
+/* ---- LoRA pairs.  Replaces rwkv7_v3a_linear_wag(v)_rank_in_f16_launch,
+ * rwkv7_v3a_linear_wag(v)_rank_out_f16_launch, rwkv7_v3a_linear_t_f16_launch,
+ * rwkv7_v3a_linear_t_act_f16_launch, rwkv7_v3a_linear_t_vres_f16_launch
+ * (cuda/rwkv7_fast_v4_kernels.cuh:147-211).
+ * lora_in:  h[M,R] = f16(x[M,C] . W1[R,C]^T).
+ * lora_out: o[M,C] = act(h[M,R]) . W2[C,R]^T in fp32; then
+ *   vres == 0: out = f16(o + bias[c])              (bias may be NULL: w0 folded for the decay logit)
+ *   vres == 1: out = f16(v + (v_first - v) * sigmoid(bias[c] + o))   (the v-residual gate). */
+int rwkv_hip_lora_in(rwkv_stream_t s, int M, int C, int R, const void* x, const void* w1, void* h);
+int rwkv_hip_lora_out(rwkv_stream_t s, int M, int C, int R, int act, const void* h, const void* w2,
+                      const void* bias, int vres, const void* v, const void* v_first, void* out);
+
+/* ---- fused element-wise ops ---- */
+/* rwkv7_v3a_layer_norm_f16_launch (cuda/rwkv7_fast_v4_kernels.cuh:118-120) */
+int rwkv_hip_layer_norm(rwkv_stream_t s, int rows, int C, const void* x, const void* w, const void* b,
+                        void* y, float eps);
+/* rwkv7_v3a_add_layer_norm_f16_launch (:122-125) */
+int rwkv_hip_add_layer_norm(rwkv_stream_t s, int rows, int C, const void* x, const void* res, const void* w,
+                            const void* b, void* x_out, void* y, float eps);
+/* rwkv7_v3a_add_last_layer_norm_f16_launch (:127-130): y [B,C] from the last token of each row */
+int rwkv_hip_add_last_layer_norm(rwkv_stream_t s, int B, int T, int C, const void* x, const void* res,
+                                 const void* w, const void* b, void* y, float eps);
+/* rwkv7_tmix_mix6_launch (:54-60) and rwkv7_cmix_mix_launch (:79-81), including the shift-state
+ * update.  n_mix in {1,6}; mu and out are host arrays of n_mix device pointers. */
+int rwkv_hip_token_shift_mix(rwkv_stream_t s, int B, int T, int C, int n_mix, const void* x, void* shift,
+                             const void* const* mu_host, void* const* out_host);
+/* rwkv7_v3a_add_layer_norm_cmix_mix_f16_launch (:132-136); rows = B, T == 1 */
+int rwkv_hip_add_layer_norm_cmix_mix(rwkv_stream_t s, int rows, int C, const void* x, const void* res,
+                                     void* shift, const void* w, const void* b, const void* mu_k,
+                                     void* x_out, void* mixed, float eps);
+/* rwkv7_v3a_add_layer_norm_tmix_mix6_f16_launch (:138-145); rows = B, T == 1 */
+int rwkv_hip_add_layer_norm_tmix_mix6(rwkv_stream_t s, int rows, int C, const void* x, const void* res,
+                                      void* shift, const void* w, const void* b, const void* const* mu6_host,
+                                      void* x_out, void* const* out6_host, float eps);
+/* rwkv7_tmix_kk_a_gate_launch (:62-66) */
+int rwkv_hip_kk_a_gate(rwkv_stream_t s, int rows, int C, int H, const void* k, const void* k_k, const void* a0,
+                       const void* a12, const void* k_a, void* new_k, void* neg_kk, void* kka);
+/* rwkv7_tmix_lnx_rkvres_xg_launch (:68-72) */
+int rwkv_hip_lnx_rkvres_xg(rwkv_stream_t s, int rows, int C, int H, const void* y, const void* r, const void* k,
+                           const void* v, const void* r_k, const void* lnw, const void* lnb, const void* g,
+                           void* out);
+/* rwkv7_relu_square_launch (:83), rwkv7_add_vec_launch (:87-88), rwkv7_v4_f16_to_f32_launch (:31-32),
+ * rwkv7_v3a_advance_i32_launch (:116) */
+int rwkv_hip_relu_square(rwkv_stream_t s, int64_t n, const void* x, void* out);
+int rwkv_hip_add_vec(rwkv_stream_t s, int rows, int C, const void* x, const void* vec, void* out);
+int rwkv_hip_f16_to_f32(rwkv_stream_t s, int64_t n, const void* src, void* dst);
+int rwkv_hip_advance_i32(rwkv_stream_t s, int n, int amount, void* x);
+
+/* ---- sampler.  Replaces rwkv_sampling::setup_rand_raw / batch_sampling_repetition_temperature_topk_topp_raw
+ * / batch_sampling_temperature_topk_topp_raw (src/utils/sampling.h:14-46).
+ * logits f32 [B,V]; penalties f32 [B,V] in/out (NULL = no penalty, as the no-penalty reference entry);
+ * probs f32 [B,V] scratch; out i32 [B].  The random stream is a counter-based Philox4x32-10 keyed by
+ * (seed, row, step): same arguments give the same tokens.  V % 4 == 0, V <= 1048576,
+ * temperature in [0.001, 1000], as the reference checks (src/utils/sampling.cu:492-512). */
+int rwkv_hip_sample(rwkv_stream_t s, int B, int V, const void* logits, void* penalties, void* probs, void* out,
+                    double presence, double frequency, double decay, double temperature, int top_k,
+                    double top_p, uint64_t seed, uint64_t step);
+/* lm_head -> argmax without the sampler: out i32 [B] = lowest index of the row maximum */
+int rwkv_hip_argmax(rwkv_stream_t s, int B, int V, const void* logits, void* out);
+
+/* ---- model graph.  Replaces CudaWeights + run_backend_forward (src/rwkv7_fast_v4.cu:1046-1345) and
+ * ModelBackend::{create_state,forward_prefill,forward_decode} (:1373-1419) below IModelBackend. ---- */
+/* global tensors use layer = -1 */
+enum {
+  RWKV_T_EMB_LN0 = 0, /* f16 [V,C]: embedding with ln0 applied (build_cpu_emb_ln0_f16, src/rwkv7_fast_v4.cu:450-572) */
+  RWKV_T_LN_OUT_W = 1,
+  RWKV_T_LN_OUT_B = 2,
+  /* per-layer f16 vectors [C] (LayerWeights, include/rwkv7_fast_v4_common.hpp:146-190) */
+  RWKV_T_LN1_W = 10, RWKV_T_LN1_B, RWKV_T_LN2_W, RWKV_T_LN2_B,
+  RWKV_T_X_R, RWKV_T_X_W, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_A, RWKV_T_X_G,
+  RWKV_T_W0, RWKV_T_A0, RWKV_T_V0, RWKV_T_K_K, RWKV_T_K_A, RWKV_T_R_K, RWKV_T_LNX_W, RWKV_T_LNX_B,
+  RWKV_T_FFN_X_K,
+  /* per-layer LoRA matrices in "out,in" layout: *1 is [R,C] (the reference's w1_t), *2 is [C,R] (w2_t) */
+  RWKV_T_W1 = 40, RWKV_T_W2, RWKV_T_A1, RWKV_T_A2, RWKV_T_G1, RWKV_T_G2, RWKV_T_V1, RWKV_T_V2,
+};
+/* big matrices, all [N_out,K_in] row-major (ffn.value as [C,F], the checkpoint's own layout) */
+enum {
+  RWKV_M_ATT_R = 0, RWKV_M_ATT_K, RWKV_M_ATT_V, RWKV_M_ATT_O, RWKV_M_FFN_KEY, RWKV_M_FFN_VALUE, RWKV_M_HEAD,
+};
+
+typedef struct rwkv_hip_model rwkv_hip_model;
+typedef struct rwkv_hip_session rwkv_hip_session;
+
+int rwkv_hip_model_create(rwkv_hip_model** out, int L, int C, int H, int F, int V, int Rw, int Ra, int Rg,
+                          int Rv);
+int rwkv_hip_model_destroy(rwkv_hip_model* m);
+/* Device pointers are borrowed: the caller owns the weights and keeps them alive. */
+int rwkv_hip_model_set_tensor(rwkv_hip_model* m, int layer, int id, const void* data);
+int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, const void* data,
+                              const void* scale, const void* zp);
+/* bytes of weights one decode step streams (for roofline accounting) */
+int rwkv_hip_model_weight_bytes(const rwkv_hip_model* m, uint64_t* bytes);
+
+/* A session owns a stream, the activation arena and captured decode graphs.  One session serves
+ * one caller at a time; several sessions may run concurrently against one model (the reference
+ * instead allocates a stream + arena per call, src/rwkv7_fast_v4.cu:1087-1096). */
+int rwkv_hip_session_create(rwkv_hip_session** out, const rwkv_hip_model* m);
+int rwkv_hip_session_destroy(rwkv_hip_session* s);
+int rwkv_hip_session_stream(rwkv_hip_session* s, rwkv_stream_t* stream);
+/* use_graph != 0: T == 1 steps replay a captured HIP graph (default on) */
+int rwkv_hip_session_set_graph(rwkv_hip_session* s, int use_graph);
+
+/* tokens_host [B,T] int64 (host); shift f16 [L,2,B,C]; wkv f32 [L,B,H,64,64]; elapsed i32 [B];
+ * logits f32 [B,V] for the last token of each row.  All state tensors are updated in place.
+ * Returns after the work is enqueued AND complete (the reference synchronises too,
+ * src/rwkv7_fast_v4.cu:1343) unless sync == 0. */
+int rwkv_hip_forward(rwkv_hip_session* s, const int64_t* tokens_host, int B, int T, void* shift, void* wkv,
+                     void* elapsed, void* logits, int sync);
+/* Greedy decode loop kept on the device: runs `steps` decode steps at batch B, feeding each row's
+ * argmax back as its next token without a host round trip; out_tokens_host [steps,B] int32.
+ * first_tokens_host [B] are the tokens of step 0. */
+int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host, int B, int steps, void* shift,
+                           void* wkv, void* elapsed, void* logits, int32_t* out_tokens_host);
+/* debugging/parity tap: residual stream after every layer of the last rwkv_hip_forward call,
+ * f16 [L, B*T, C], valid only if enabled before the call */
+int rwkv_hip_session_set_trace(rwkv_hip_session* s, void* trace);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

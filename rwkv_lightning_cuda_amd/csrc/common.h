@@ -1,0 +1,103 @@
+// Shared helpers for the gfx950 kernels: error plumbing for the C ABI, fp16 vector types,
+// wave64 reductions.  Internal to the library; nothing here is exported.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdio>
+#include <string>
+
+#include "../../include/rwkv_hip.h"
+
+namespace rwkv {
+
+void set_error(const char* fmt, ...);
+
+inline hipStream_t as_stream(rwkv_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+#define RWKV_HIP_TRY(expr)                                                              \
+  do {                                                                                  \
+    hipError_t err__ = (expr);                                                          \
+    if (err__ != hipSuccess) {                                                          \
+      ::rwkv::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(err__), __FILE__, __LINE__); \
+      return err__ == hipErrorOutOfMemory ? RWKV_E_NOMEM : RWKV_E_RUNTIME;              \
+    }                                                                                   \
+  } while (0)
+
+#define RWKV_REQUIRE(cond, ...)          \
+  do {                                   \
+    if (!(cond)) {                       \
+      ::rwkv::set_error(__VA_ARGS__);    \
+      return RWKV_E_INVALID;             \
+    }                                    \
+  } while (0)
+
+#define RWKV_LAUNCH_CHECK()                                                             \
+  do {                                                                                  \
+    hipError_t err__ = hipGetLastError();                                               \
+    if (err__ != hipSuccess) {                                                          \
+      ::rwkv::set_error("kernel launch failed: %s (%s:%d)", hipGetErrorString(err__), __FILE__, __LINE__); \
+      return RWKV_E_RUNTIME;                                                            \
+    }                                                                                   \
+  } while (0)
+
+// ---- device-side types -----------------------------------------------------------------
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kHead = 64;
+constexpr float kLnEps = 1e-5f;        // include/rwkv7_fast_v4_common.hpp:24
+constexpr float kLnxEps = 64.0e-5f;    // cuda/rwkv7_fast_ops_fp16.cu:17
+constexpr float kKkEps = 1.0e-12f;     // cuda/rwkv7_fast_ops_fp16.cu:16
+
+__device__ __forceinline__ float h2f(half_t h) { return static_cast<float>(h); }
+__device__ __forceinline__ half_t f2h(float f) { return static_cast<half_t>(f); }  // v_cvt_f16_f32, RNE
+// value after a round trip through fp16: the rounding point where the reference stores fp16
+__device__ __forceinline__ float round_h(float f) { return static_cast<float>(static_cast<half_t>(f)); }
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// Sum over the 64 lanes of a wave, result in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+// Sum over aligned groups of `Width` lanes (Width a power of two <= 64).
+template <int Width>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int off = Width / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Block-wide sum for blocks of NW waves; `scratch` holds NW floats of LDS.  All threads get the sum.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  if constexpr (NW == 1) return v;
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();  // scratch may still be read from a previous call
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) t += scratch[i];
+  return t;
+}
+
+inline int ceil_div(int64_t a, int64_t b) { return static_cast<int>((a + b - 1) / b); }
+
+}  // namespace rwkv

@@ -1,0 +1,430 @@
+// Fused element-wise / normalisation kernels of the RWKV-7 layer graph.
+//
+// Reference kernels restated here (same arithmetic and fp16 rounding points, re-tiled for wave64):
+//   LayerNorm family ........ cuda/rwkv7_v3a_ops.cu:1272-1351 (LN, add+LN), :1800-1931 (add + last-token LN),
+//                             :1933-1985 (add+LN+cmix lerp), :1987-2060 (add+LN+6 lerps)
+//   token shift ............. cuda/rwkv7_fast_ops_fp16.cu:53-127 (mix6 + shift update), :393-419 (cmix mix)
+//   kk / a-gate ............. cuda/rwkv7_fast_ops_fp16.cu:129-172
+//   GroupNorm+rkv-res+gate .. cuda/rwkv7_fast_ops_fp16.cu:174-237
+//   relu^2, add_vec, f16->f32 cuda/rwkv7_fast_ops_fp16.cu:421-485;  advance_i32 cuda/rwkv7_v3a_ops.cu:202-207
+//
+// The LN kernels keep the whole row in registers (one 256-thread block per row, 16-byte loads), so a
+// row is read from HBM once for the two-pass mean/variance and the normalise+lerp epilogue.
+#include "ops.h"
+
+namespace rwkv {
+
+constexpr int kLnThreads = 256;
+constexpr int kLnMaxVec = 4;  // 8-element vectors per thread -> C <= 8192
+
+
+
+template <int MODE>
+__global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
+  __shared__ float red[4];
+  const int row = blockIdx.x;
+  const int C = a.C;
+  int64_t src = static_cast<int64_t>(row) * C;
+  if constexpr (MODE == kAddLastLn) src = (static_cast<int64_t>(row) * a.T + (a.T - 1)) * C;
+  int64_t xsrc = src;
+  if constexpr (MODE == kLnMix) {
+    if (a.tokens) xsrc = a.tokens[row] * static_cast<int64_t>(C);
+  }
+  const int64_t dst = static_cast<int64_t>(row) * C;
+
+  float v[kLnMaxVec][8];
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kLnMaxVec; ++i) {
+    const int c = (i * kLnThreads + threadIdx.x) * 8;
+    if (c < C) {
+      const half8_t xv = *reinterpret_cast<const half8_t*>(a.x + xsrc + c);
+      if constexpr (MODE == kLn || MODE == kLnMix) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = h2f(xv[e]);
+      } else {
+        const half8_t rv = *reinterpret_cast<const half8_t*>(a.res + src + c);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = h2f(xv[e]) + h2f(rv[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += v[i][e];
+    }
+  }
+  sum = block_sum<4>(sum, red);
+  const float mean = sum / static_cast<float>(C);
+  float sv = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kLnMaxVec; ++i) {
+    const int c = (i * kLnThreads + threadIdx.x) * 8;
+    if (c < C) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = v[i][e] - mean;
+        sv += d * d;
+      }
+    }
+  }
+  sv = block_sum<4>(sv, red);
+  const float rstd = rsqrtf(sv / static_cast<float>(C) + a.eps);
+
+#pragma unroll
+  for (int i = 0; i < kLnMaxVec; ++i) {
+    const int c = (i * kLnThreads + threadIdx.x) * 8;
+    if (c < C) {
+      const half8_t wv = *reinterpret_cast<const half8_t*>(a.w + c);
+      const half8_t bv = *reinterpret_cast<const half8_t*>(a.b + c);
+      half8_t yv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) yv[e] = f2h((v[i][e] - mean) * rstd * h2f(wv[e]) + h2f(bv[e]));
+      if constexpr (MODE == kAddLn || MODE == kAddLnMix) {
+        half8_t xo;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xo[e] = f2h(v[i][e]);
+        *reinterpret_cast<half8_t*>(a.x_out + dst + c) = xo;
+      }
+      if constexpr (MODE == kLnMix) {
+        if (a.x_out) {  // the residual stream starts as the (already fp16) embedding row
+          half8_t xo;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) xo[e] = f2h(v[i][e]);
+          *reinterpret_cast<half8_t*>(a.x_out + dst + c) = xo;
+        }
+      }
+      if constexpr (MODE == kAddLnMix || MODE == kLnMix) {
+        // lerps read the fp16-rounded LN output (rwkv7_v3a_ops.cu:1978-1983)
+        const half8_t pv = *reinterpret_cast<const half8_t*>(a.shift + dst + c);
+        for (int s = 0; s < a.n_mix; ++s) {
+          const half8_t mv = *reinterpret_cast<const half8_t*>(a.mu[s] + c);
+          half8_t ov;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float yf = h2f(yv[e]);
+            ov[e] = f2h(yf + (h2f(pv[e]) - yf) * h2f(mv[e]));
+          }
+          *reinterpret_cast<half8_t*>(a.out[s] + dst + c) = ov;
+        }
+        *reinterpret_cast<half8_t*>(a.shift + dst + c) = yv;
+        if (a.y) *reinterpret_cast<half8_t*>(a.y + dst + c) = yv;
+      } else {
+        *reinterpret_cast<half8_t*>(a.y + dst + c) = yv;
+      }
+    }
+  }
+}
+
+static int check_ln_shape(int rows, int C) {
+  RWKV_REQUIRE(rows > 0, "layer norm: rows must be positive");
+  RWKV_REQUIRE(C > 0 && C % 8 == 0 && C <= kLnThreads * 8 * kLnMaxVec,
+               "layer norm: C (%d) must be a multiple of 8 and at most %d", C, kLnThreads * 8 * kLnMaxVec);
+  return RWKV_OK;
+}
+
+int ln_launch(hipStream_t st, int mode, int rows, const LnArgs& a) {
+  if (int rc = check_ln_shape(rows, a.C)) return rc;
+  switch (mode) {
+    case kLn: hipLaunchKernelGGL(ln_fused_kernel<kLn>, dim3(rows), dim3(kLnThreads), 0, st, a); break;
+    case kAddLn: hipLaunchKernelGGL(ln_fused_kernel<kAddLn>, dim3(rows), dim3(kLnThreads), 0, st, a); break;
+    case kAddLastLn: hipLaunchKernelGGL(ln_fused_kernel<kAddLastLn>, dim3(rows), dim3(kLnThreads), 0, st, a); break;
+    case kAddLnMix: hipLaunchKernelGGL(ln_fused_kernel<kAddLnMix>, dim3(rows), dim3(kLnThreads), 0, st, a); break;
+    case kLnMix: hipLaunchKernelGGL(ln_fused_kernel<kLnMix>, dim3(rows), dim3(kLnThreads), 0, st, a); break;
+    default: set_error("bad layer-norm mode %d", mode); return RWKV_E_INVALID;
+  }
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+// ---- token shift: out_s = x + (prev - x) * mu_s with prev = shift[b] at t == 0, else x[b,t-1];
+// then shift[b] = x[b,T-1].  One thread per (row, 8 channels).  For T == 1 the same thread reads and
+// then overwrites its shift slice; for T > 1 the shift rows are rewritten by a second launch so no
+// thread can overwrite a slice another one still has to read. ----------------------------------
+
+__global__ __launch_bounds__(256) void token_shift_mix_kernel(MixArgs a) {
+  const int cvecs = a.C / 8;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= static_cast<int64_t>(a.B) * a.T * cvecs) return;
+  const int64_t row = idx / cvecs;
+  const int c = static_cast<int>(idx - row * cvecs) * 8;
+  const int b = static_cast<int>(row / a.T);
+  const int t = static_cast<int>(row - static_cast<int64_t>(b) * a.T);
+  const int64_t o = row * a.C + c;
+  const half8_t cur = *reinterpret_cast<const half8_t*>(a.x + o);
+  const half8_t prev = (t == 0) ? *reinterpret_cast<const half8_t*>(a.shift + static_cast<int64_t>(b) * a.C + c)
+                                : *reinterpret_cast<const half8_t*>(a.x + o - a.C);
+  for (int s = 0; s < a.n_mix; ++s) {
+    const half8_t mu = *reinterpret_cast<const half8_t*>(a.mu[s] + c);
+    half8_t ov;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float cf = h2f(cur[e]);
+      ov[e] = f2h(cf + (h2f(prev[e]) - cf) * h2f(mu[e]));
+    }
+    *reinterpret_cast<half8_t*>(a.out[s] + o) = ov;
+  }
+  if (a.T == 1) *reinterpret_cast<half8_t*>(a.shift + static_cast<int64_t>(b) * a.C + c) = cur;
+}
+
+__global__ __launch_bounds__(256) void shift_update_kernel(int B, int T, int C, const half_t* __restrict__ x,
+                                                           half_t* __restrict__ shift) {
+  const int cvecs = C / 8;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= B * cvecs) return;
+  const int b = idx / cvecs;
+  const int c = (idx - b * cvecs) * 8;
+  *reinterpret_cast<half8_t*>(shift + static_cast<int64_t>(b) * C + c) =
+      *reinterpret_cast<const half8_t*>(x + (static_cast<int64_t>(b) * T + (T - 1)) * C + c);
+}
+
+int token_shift_mix_launch(hipStream_t st, const MixArgs& a) {
+  RWKV_REQUIRE(a.B > 0 && a.T > 0 && a.C > 0 && a.C % 8 == 0, "token shift: bad shape B=%d T=%d C=%d", a.B, a.T, a.C);
+  RWKV_REQUIRE(a.n_mix >= 1 && a.n_mix <= 6, "token shift: n_mix %d out of range", a.n_mix);
+  const int64_t n = static_cast<int64_t>(a.B) * a.T * (a.C / 8);
+  hipLaunchKernelGGL(token_shift_mix_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, st, a);
+  if (a.T > 1) {
+    hipLaunchKernelGGL(shift_update_kernel, dim3(ceil_div(a.B * (a.C / 8), 256)), dim3(256), 0, st, a.B, a.T, a.C,
+                       a.x, a.shift);
+  }
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+// ---- kk normalise + a-gate: one wave per (row, head), lane = channel --------------------------------
+// Optional fp32 outputs feed the WKV sequence kernel directly (values are the fp16-rounded ones).
+
+__global__ __launch_bounds__(256) void kk_a_gate_kernel(KkArgs p) {
+  const int64_t rh = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (rh >= p.rows_heads) return;
+  const int lane = threadIdx.x & 63;
+  const int h = static_cast<int>(rh % p.H);
+  const int64_t idx = rh * kHead + lane;
+  const int c = h * kHead + lane;
+  const float kv = h2f(p.k[idx]);
+  const float u = kv * h2f(p.k_k[c]);
+  const float total = wave_sum(u * u);
+  const float inv = 1.0f / fmaxf(sqrtf(total), kKkEps);
+  const float kk = u * inv;
+  const float av = sigmoid_f(h2f(p.a0[c]) + h2f(p.a12[idx]));
+  const float ka = h2f(p.k_a[c]);
+  const half_t nk = f2h(kv * fmaf(av, ka, 1.0f - ka));
+  const half_t nkk = f2h(-kk);
+  const half_t kka = f2h(kk * av);
+  if (p.new_k) p.new_k[idx] = nk;
+  if (p.neg_kk) p.neg_kk[idx] = nkk;
+  if (p.kka) p.kka[idx] = kka;
+  if (p.k32) {
+    p.k32[idx] = h2f(nk);
+    p.a32[idx] = h2f(nkk);
+    p.b32[idx] = h2f(kka);
+    const float wraw = round_h(h2f(p.w12[idx]) + h2f(p.w0[c]));  // rwkv7_add_vec_launch rounding point
+    p.d32[idx] = exp2f(-0.8750387749145276f / (1.0f + exp2f(-1.4426950408889634f * wraw)));
+    p.r32[idx] = h2f(p.r[idx]);
+  }
+}
+
+int kk_a_gate_launch(hipStream_t st, const KkArgs& p) {
+  RWKV_REQUIRE(p.rows_heads > 0 && p.H > 0, "kk_a_gate: bad shape");
+  hipLaunchKernelGGL(kk_a_gate_kernel, dim3(ceil_div(p.rows_heads, 4)), dim3(256), 0, st, p);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+// ---- per-head GroupNorm + rkv residual + gate: one wave per (row, head) --------------------------------
+__global__ __launch_bounds__(256) void lnx_rkvres_xg_kernel(int64_t rows_heads, int H, const half_t* __restrict__ y,
+                                                            const half_t* __restrict__ r, const half_t* __restrict__ k,
+                                                            const half_t* __restrict__ v, const half_t* __restrict__ r_k,
+                                                            const half_t* __restrict__ lnw, const half_t* __restrict__ lnb,
+                                                            const half_t* __restrict__ g, half_t* __restrict__ out) {
+  const int64_t rh = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (rh >= rows_heads) return;
+  const int lane = threadIdx.x & 63;
+  const int h = static_cast<int>(rh % H);
+  const int64_t idx = rh * kHead + lane;
+  const int c = h * kHead + lane;
+  const float yv = h2f(y[idx]);
+  const float mean = wave_sum(yv) * (1.0f / 64.0f);
+  const float d = yv - mean;
+  const float var = wave_sum(d * d) * (1.0f / 64.0f);
+  const float rstd = rsqrtf(var + kLnxEps);
+  const float rkv = wave_sum(h2f(r[idx]) * h2f(k[idx]) * h2f(r_k[c]));
+  const float o = (d * rstd * h2f(lnw[c]) + h2f(lnb[c]) + rkv * h2f(v[idx])) * h2f(g[idx]);
+  out[idx] = f2h(o);
+}
+
+// ---- small element-wise kernels ---------------------------------------------------------------------
+__global__ __launch_bounds__(256) void relu_square_kernel(int64_t n, const half_t* __restrict__ x, half_t* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float v = fmaxf(h2f(x[i]), 0.0f);
+  out[i] = f2h(v * v);
+}
+
+__global__ __launch_bounds__(256) void add_vec_kernel(int64_t n, int C, const half_t* __restrict__ x,
+                                                      const half_t* __restrict__ vec, half_t* __restrict__ out) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  out[i] = f2h(h2f(x[i]) + h2f(vec[i % C]));
+}
+
+__global__ __launch_bounds__(256) void f16_to_f32_kernel(int64_t n, const half_t* __restrict__ src, float* __restrict__ dst) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= n) return;
+  dst[i] = h2f(src[i]);
+}
+
+__global__ __launch_bounds__(256) void advance_i32_kernel(int n, int amount, int* __restrict__ x) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] += amount;
+}
+
+// gather embedding rows for T > 1: out[row] = table[tokens[row]]
+__global__ __launch_bounds__(256) void embed_gather_kernel(int C, const int64_t* __restrict__ tokens,
+                                                           const half_t* __restrict__ table, half_t* __restrict__ out) {
+  const int row = blockIdx.x;
+  const int64_t src = tokens[row] * static_cast<int64_t>(C);
+  for (int c = threadIdx.x * 8; c < C; c += 256 * 8)
+    *reinterpret_cast<half8_t*>(out + static_cast<int64_t>(row) * C + c) = *reinterpret_cast<const half8_t*>(table + src + c);
+}
+
+int embed_gather_launch(hipStream_t st, int rows, int C, const int64_t* tokens, const half_t* table, half_t* out) {
+  hipLaunchKernelGGL(embed_gather_kernel, dim3(rows), dim3(256), 0, st, C, tokens, table, out);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+int lnx_launch(hipStream_t st, int64_t rows_heads, int H, const half_t* y, const half_t* r, const half_t* k,
+               const half_t* v, const half_t* r_k, const half_t* lnw, const half_t* lnb, const half_t* g, half_t* out) {
+  hipLaunchKernelGGL(lnx_rkvres_xg_kernel, dim3(ceil_div(rows_heads, 4)), dim3(256), 0, st, rows_heads, H, y, r, k, v,
+                     r_k, lnw, lnb, g, out);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+int advance_launch(hipStream_t st, int n, int amount, int* x) {
+  hipLaunchKernelGGL(advance_i32_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, st, n, amount, x);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+}  // namespace rwkv
+
+using namespace rwkv;
+
+#define H16(p) static_cast<const half_t*>(p)
+#define H16M(p) static_cast<half_t*>(p)
+
+extern "C" {
+
+int rwkv_hip_layer_norm(rwkv_stream_t s, int rows, int C, const void* x, const void* w, const void* b, void* y,
+                        float eps) {
+  RWKV_REQUIRE(x && w && b && y, "layer_norm: NULL tensor");
+  LnArgs a = {};
+  a.x = H16(x); a.w = H16(w); a.b = H16(b); a.y = H16M(y); a.C = C; a.T = 1; a.eps = eps;
+  return ln_launch(as_stream(s), kLn, rows, a);
+}
+
+int rwkv_hip_add_layer_norm(rwkv_stream_t s, int rows, int C, const void* x, const void* res, const void* w,
+                            const void* b, void* x_out, void* y, float eps) {
+  RWKV_REQUIRE(x && res && w && b && x_out && y, "add_layer_norm: NULL tensor");
+  LnArgs a = {};
+  a.x = H16(x); a.res = H16(res); a.w = H16(w); a.b = H16(b); a.x_out = H16M(x_out); a.y = H16M(y);
+  a.C = C; a.T = 1; a.eps = eps;
+  return ln_launch(as_stream(s), kAddLn, rows, a);
+}
+
+int rwkv_hip_add_last_layer_norm(rwkv_stream_t s, int B, int T, int C, const void* x, const void* res, const void* w,
+                                 const void* b, void* y, float eps) {
+  RWKV_REQUIRE(x && res && w && b && y && T > 0, "add_last_layer_norm: bad arguments");
+  LnArgs a = {};
+  a.x = H16(x); a.res = H16(res); a.w = H16(w); a.b = H16(b); a.y = H16M(y); a.C = C; a.T = T; a.eps = eps;
+  return ln_launch(as_stream(s), kAddLastLn, B, a);
+}
+
+int rwkv_hip_token_shift_mix(rwkv_stream_t s, int B, int T, int C, int n_mix, const void* x, void* shift,
+                             const void* const* mu_host, void* const* out_host) {
+  RWKV_REQUIRE(x && shift && mu_host && out_host, "token_shift_mix: NULL tensor");
+  RWKV_REQUIRE(n_mix >= 1 && n_mix <= 6, "token_shift_mix: n_mix %d out of range", n_mix);
+  MixArgs a = {};
+  a.x = H16(x); a.shift = H16M(shift); a.B = B; a.T = T; a.C = C; a.n_mix = n_mix;
+  for (int i = 0; i < n_mix; ++i) {
+    RWKV_REQUIRE(mu_host[i] && out_host[i], "token_shift_mix: NULL tensor");
+    a.mu[i] = H16(mu_host[i]);
+    a.out[i] = H16M(out_host[i]);
+  }
+  return token_shift_mix_launch(as_stream(s), a);
+}
+
+int rwkv_hip_add_layer_norm_cmix_mix(rwkv_stream_t s, int rows, int C, const void* x, const void* res, void* shift,
+                                     const void* w, const void* b, const void* mu_k, void* x_out, void* mixed,
+                                     float eps) {
+  RWKV_REQUIRE(x && res && shift && w && b && mu_k && x_out && mixed, "add_layer_norm_cmix_mix: NULL tensor");
+  LnArgs a = {};
+  a.x = H16(x); a.res = H16(res); a.w = H16(w); a.b = H16(b); a.x_out = H16M(x_out); a.shift = H16M(shift);
+  a.mu[0] = H16(mu_k); a.out[0] = H16M(mixed); a.n_mix = 1; a.C = C; a.T = 1; a.eps = eps;
+  return ln_launch(as_stream(s), kAddLnMix, rows, a);
+}
+
+int rwkv_hip_add_layer_norm_tmix_mix6(rwkv_stream_t s, int rows, int C, const void* x, const void* res, void* shift,
+                                      const void* w, const void* b, const void* const* mu6_host, void* x_out,
+                                      void* const* out6_host, float eps) {
+  RWKV_REQUIRE(x && res && shift && w && b && mu6_host && x_out && out6_host, "add_layer_norm_tmix_mix6: NULL tensor");
+  LnArgs a = {};
+  a.x = H16(x); a.res = H16(res); a.w = H16(w); a.b = H16(b); a.x_out = H16M(x_out); a.shift = H16M(shift);
+  for (int i = 0; i < 6; ++i) {
+    RWKV_REQUIRE(mu6_host[i] && out6_host[i], "add_layer_norm_tmix_mix6: NULL tensor");
+    a.mu[i] = H16(mu6_host[i]);
+    a.out[i] = H16M(out6_host[i]);
+  }
+  a.n_mix = 6; a.C = C; a.T = 1; a.eps = eps;
+  return ln_launch(as_stream(s), kAddLnMix, rows, a);
+}
+
+int rwkv_hip_kk_a_gate(rwkv_stream_t s, int rows, int C, int H, const void* k, const void* k_k, const void* a0,
+                       const void* a12, const void* k_a, void* new_k, void* neg_kk, void* kka) {
+  RWKV_REQUIRE(rows > 0 && H > 0 && C == H * kHead, "kk_a_gate: C (%d) must equal H*64", C);
+  RWKV_REQUIRE(k && k_k && a0 && a12 && k_a && new_k && neg_kk && kka, "kk_a_gate: NULL tensor");
+  KkArgs p = {};
+  p.k = H16(k); p.k_k = H16(k_k); p.a0 = H16(a0); p.a12 = H16(a12); p.k_a = H16(k_a);
+  p.new_k = H16M(new_k); p.neg_kk = H16M(neg_kk); p.kka = H16M(kka);
+  p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
+  return kk_a_gate_launch(as_stream(s), p);
+}
+
+int rwkv_hip_lnx_rkvres_xg(rwkv_stream_t s, int rows, int C, int H, const void* y, const void* r, const void* k,
+                           const void* v, const void* r_k, const void* lnw, const void* lnb, const void* g,
+                           void* out) {
+  RWKV_REQUIRE(rows > 0 && H > 0 && C == H * kHead, "lnx_rkvres_xg: C (%d) must equal H*64", C);
+  RWKV_REQUIRE(y && r && k && v && r_k && lnw && lnb && g && out, "lnx_rkvres_xg: NULL tensor");
+  return lnx_launch(as_stream(s), static_cast<int64_t>(rows) * H, H, H16(y), H16(r), H16(k), H16(v), H16(r_k),
+                    H16(lnw), H16(lnb), H16(g), H16M(out));
+}
+
+int rwkv_hip_relu_square(rwkv_stream_t s, int64_t n, const void* x, void* out) {
+  RWKV_REQUIRE(n > 0 && x && out, "relu_square: bad arguments");
+  hipLaunchKernelGGL(relu_square_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, as_stream(s), n, H16(x), H16M(out));
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+int rwkv_hip_add_vec(rwkv_stream_t s, int rows, int C, const void* x, const void* vec, void* out) {
+  RWKV_REQUIRE(rows > 0 && C > 0 && x && vec && out, "add_vec: bad arguments");
+  const int64_t n = static_cast<int64_t>(rows) * C;
+  hipLaunchKernelGGL(add_vec_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, as_stream(s), n, C, H16(x), H16(vec),
+                     H16M(out));
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+int rwkv_hip_f16_to_f32(rwkv_stream_t s, int64_t n, const void* src, void* dst) {
+  RWKV_REQUIRE(n > 0 && src && dst, "f16_to_f32: bad arguments");
+  hipLaunchKernelGGL(f16_to_f32_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, as_stream(s), n, H16(src),
+                     static_cast<float*>(dst));
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+int rwkv_hip_advance_i32(rwkv_stream_t s, int n, int amount, void* x) {
+  RWKV_REQUIRE(n > 0 && x, "advance_i32: bad arguments");
+  return advance_launch(as_stream(s), n, amount, static_cast<int*>(x));
+}
+
+}  // extern "C"

@@ -1,0 +1,670 @@
+// RWKV-7 layer graph on one GPU: model handle (borrowed weight pointers), session (stream, activation
+// arena, captured decode graphs) and the forward pass for prefill chunks (T > 1) and decode steps (T == 1).
+//
+// Reference: run_backend_forward, src/rwkv7_fast_v4.cu:1046-1345 -- same op order, same layer-0 special
+// cases (no v LoRA, v_first = v: :1171,1246-1247), same state slices (:1177-1185), logits for the last
+// token of each row only (:1314-1342), elapsed += T (:1320).  Differences by design:
+//   * the arena and stream live in the session instead of being allocated on every call (:1087-1096);
+//   * the embedding+ln0 table stays in HBM and rows are gathered on the device (the reference gathers on
+//     the host and copies, :1103-1116,1155);
+//   * T == 1 steps are captured once into a HIP graph per (batch, state, logits) tuple and replayed;
+//   * LN1 + the six token-shift lerps are fused for every batch size (the reference does it for B == 1).
+#include <algorithm>
+#include <mutex>
+#include <vector>
+
+#include "ops.h"
+
+using namespace rwkv;
+
+struct Matrix {
+  int fmt = RWKV_FMT_F16;
+  const void* data = nullptr;
+  const half_t* scale = nullptr;
+  const uint8_t* zp = nullptr;
+};
+
+struct Layer {
+  const half_t* t[64] = {nullptr};
+  Matrix m[6];
+};
+
+struct rwkv_hip_model {
+  int L = 0, C = 0, H = 0, F = 0, V = 0, Rw = 0, Ra = 0, Rg = 0, Rv = 0;
+  const half_t* emb_ln0 = nullptr;
+  const half_t* ln_out_w = nullptr;
+  const half_t* ln_out_b = nullptr;
+  Matrix head;
+  std::vector<Layer> layers;
+};
+
+namespace {
+
+struct GraphEntry {
+  int B = 0;
+  void* shift = nullptr;
+  void* wkv = nullptr;
+  void* elapsed = nullptr;
+  void* logits = nullptr;
+  hipGraphExec_t exec = nullptr;
+  hipGraph_t graph = nullptr;
+  uint64_t last_use = 0;
+};
+
+constexpr size_t kMaxGraphs = 8;
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct Arena {
+  unsigned char* base = nullptr;
+  size_t cap = 0;
+  size_t off = 0;
+  template <typename T>
+  T* take(size_t n) {
+    const size_t bytes = align_up(n * sizeof(T), 256);
+    T* p = reinterpret_cast<T*>(base + off);
+    off += bytes;
+    return p;
+  }
+};
+
+struct Buffers {
+  half_t *x, *xx, *xr, *xw, *xk, *xv, *xa, *xg, *r, *k, *v, *v_first, *w12, *a12, *g, *hw, *ha, *hg, *hv, *k2, *nkk,
+      *kka, *y, *y2, *att, *x1, *ln2, *mixed, *act, *cm, *xf, *scratch;
+  float *r32, *d32, *k32, *a32, *b32;
+};
+
+}  // namespace
+
+struct rwkv_hip_session {
+  const rwkv_hip_model* model = nullptr;
+  hipStream_t stream = nullptr;
+  Arena arena;
+  int arena_B = 0, arena_T = 0;
+  Buffers buf = {};
+  int64_t* tokens_dev = nullptr;
+  int64_t* tokens_pinned = nullptr;
+  int tokens_cap = 0;
+  int* argmax_dev = nullptr;
+  int* history_dev = nullptr;
+  size_t history_cap = 0;
+  int argmax_cap = 0;
+  bool use_graph = true;
+  half_t* trace = nullptr;
+  std::vector<GraphEntry> graphs;
+  uint64_t tick = 0;
+};
+
+namespace {
+
+int model_ready(const rwkv_hip_model* m) {
+  RWKV_REQUIRE(m != nullptr, "model is NULL");
+  if (!m->emb_ln0 || !m->ln_out_w || !m->ln_out_b || !m->head.data) {
+    set_error("model: global tensors (emb_ln0, ln_out, head) are not all set");
+    return RWKV_E_STATE;
+  }
+  static const int vec_ids[] = {RWKV_T_LN1_W, RWKV_T_LN1_B, RWKV_T_LN2_W, RWKV_T_LN2_B, RWKV_T_X_R, RWKV_T_X_W,
+                                RWKV_T_X_K,   RWKV_T_X_V,   RWKV_T_X_A,   RWKV_T_X_G,   RWKV_T_W0,  RWKV_T_A0,
+                                RWKV_T_K_K,   RWKV_T_K_A,   RWKV_T_R_K,   RWKV_T_LNX_W, RWKV_T_LNX_B, RWKV_T_FFN_X_K,
+                                RWKV_T_W1,    RWKV_T_W2,    RWKV_T_A1,    RWKV_T_A2,    RWKV_T_G1,  RWKV_T_G2};
+  for (int l = 0; l < m->L; ++l) {
+    for (int id : vec_ids) {
+      if (!m->layers[l].t[id]) {
+        set_error("model: layer %d tensor %d is not set", l, id);
+        return RWKV_E_STATE;
+      }
+    }
+    if (l > 0 && (!m->layers[l].t[RWKV_T_V0] || !m->layers[l].t[RWKV_T_V1] || !m->layers[l].t[RWKV_T_V2])) {
+      set_error("model: layer %d value-residual tensors are not set", l);
+      return RWKV_E_STATE;
+    }
+    for (int i = 0; i < 6; ++i) {
+      if (!m->layers[l].m[i].data) {
+        set_error("model: layer %d matrix %d is not set", l, i);
+        return RWKV_E_STATE;
+      }
+    }
+  }
+  return RWKV_OK;
+}
+
+int ensure_arena(rwkv_hip_session* s, int B, int T) {
+  const rwkv_hip_model* m = s->model;
+  const size_t rows = static_cast<size_t>(B) * T;
+  if (s->arena.base && B <= s->arena_B && T <= s->arena_T && B * T <= s->arena_B * s->arena_T) {
+    // shapes are laid out per call below, so only capacity matters
+  }
+  const size_t RC = rows * m->C;
+  const size_t rank_max = static_cast<size_t>(std::max(std::max(m->Rw, m->Ra), std::max(m->Rg, m->Rv)));
+  size_t need = 0;
+  auto add = [&](size_t n, size_t elt) { need += align_up(n * elt, 256); };
+  for (int i = 0; i < 27; ++i) add(RC, 2);           // f16 [rows,C] buffers
+  for (int i = 0; i < 4; ++i) add(rows * rank_max, 2);  // LoRA hidden
+  add(rows * m->F, 2);                                // act
+  add(static_cast<size_t>(B) * m->C, 2);              // xf
+  add(RC, 2);                                         // scratch
+  for (int i = 0; i < 5; ++i) add(RC, 4);             // fp32 WKV operands
+  if (need > s->arena.cap) {
+    // a larger shape invalidates captured graphs (they hold arena addresses)
+    for (auto& g : s->graphs) {
+      if (g.exec) (void)hipGraphExecDestroy(g.exec);
+      if (g.graph) (void)hipGraphDestroy(g.graph);
+    }
+    s->graphs.clear();
+    RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+    if (s->arena.base) RWKV_HIP_TRY(hipFree(s->arena.base));
+    s->arena.base = nullptr;
+    s->arena.cap = 0;
+    RWKV_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->arena.base), need));
+    s->arena.cap = need;
+    s->arena_B = 0;
+    s->arena_T = 0;
+  }
+  if (B != s->arena_B || T != s->arena_T) {
+    // new layout: graphs captured for another (B,T) layout of the same arena stay valid only if the
+    // layout for that B is unchanged; decode graphs are keyed by B and T == 1, and the layout below
+    // depends on (B,T) only, so a (B,1) layout is always the same addresses.
+    Arena& a = s->arena;
+    a.off = 0;
+    Buffers& b = s->buf;
+    half_t** f16s[] = {&b.x, &b.xx, &b.xr, &b.xw, &b.xk, &b.xv, &b.xa, &b.xg, &b.r, &b.k, &b.v, &b.v_first, &b.w12,
+                       &b.a12, &b.g, &b.k2, &b.nkk, &b.kka, &b.y, &b.y2, &b.att, &b.x1, &b.ln2, &b.mixed, &b.cm,
+                       &b.scratch};
+    for (half_t** p : f16s) *p = a.take<half_t>(RC);
+    b.hw = a.take<half_t>(rows * rank_max);
+    b.ha = a.take<half_t>(rows * rank_max);
+    b.hg = a.take<half_t>(rows * rank_max);
+    b.hv = a.take<half_t>(rows * rank_max);
+    b.act = a.take<half_t>(rows * m->F);
+    b.xf = a.take<half_t>(static_cast<size_t>(B) * m->C);
+    b.r32 = a.take<float>(RC);
+    b.d32 = a.take<float>(RC);
+    b.k32 = a.take<float>(RC);
+    b.a32 = a.take<float>(RC);
+    b.b32 = a.take<float>(RC);
+    s->arena_B = B;
+    s->arena_T = T;
+  }
+  if (static_cast<int>(rows) > s->tokens_cap) {
+    RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+    if (s->tokens_dev) RWKV_HIP_TRY(hipFree(s->tokens_dev));
+    if (s->tokens_pinned) RWKV_HIP_TRY(hipHostFree(s->tokens_pinned));
+    s->tokens_dev = nullptr;
+    s->tokens_pinned = nullptr;
+    s->tokens_cap = 0;
+    RWKV_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->tokens_dev), rows * sizeof(int64_t)));
+    RWKV_HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&s->tokens_pinned), rows * sizeof(int64_t), hipHostMallocDefault));
+    s->tokens_cap = static_cast<int>(rows);
+  }
+  return RWKV_OK;
+}
+
+int apply_matrix(hipStream_t st, const Matrix& mat, int M, int N, int K, const half_t* x, int epilogue, int out_f32,
+                 void* y) {
+  return linear_any_m(st, mat.fmt, M, N, K, x, mat.data, mat.scale, mat.zp, epilogue, out_f32, y);
+}
+
+#define TRY(expr)                  \
+  do {                             \
+    const int rc__ = (expr);       \
+    if (rc__ != RWKV_OK) return rc__; \
+  } while (0)
+
+// Enqueues the whole forward pass on the session stream.  tokens are already in s->tokens_dev.
+int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv, int* elapsed, float* logits) {
+  const rwkv_hip_model* m = s->model;
+  hipStream_t st = s->stream;
+  Buffers& b = s->buf;
+  const int C = m->C, H = m->H, F = m->F, V = m->V, L = m->L;
+  const int rows = B * T;
+  const int64_t RC = static_cast<int64_t>(rows) * C;
+  const bool step = (T == 1);
+  const bool small = rows <= 8;
+
+  auto mix6_args = [&](const Layer& w, LnArgs& a) {
+    const int ids[6] = {RWKV_T_X_R, RWKV_T_X_W, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_A, RWKV_T_X_G};
+    half_t* outs[6] = {b.xr, b.xw, b.xk, b.xv, b.xa, b.xg};
+    for (int i = 0; i < 6; ++i) {
+      a.mu[i] = w.t[ids[i]];
+      a.out[i] = outs[i];
+    }
+    a.n_mix = 6;
+  };
+
+  if (step) {
+    // embedding gather + LN1(layer 0) + six lerps + shift0 write in one kernel
+    LnArgs a = {};
+    a.x = m->emb_ln0; a.tokens = s->tokens_dev; a.x_out = b.x;
+    a.w = m->layers[0].t[RWKV_T_LN1_W]; a.b = m->layers[0].t[RWKV_T_LN1_B];
+    a.shift = shift; a.C = C; a.T = 1; a.eps = kLnEps;
+    mix6_args(m->layers[0], a);
+    TRY(ln_launch(st, kLnMix, rows, a));
+  } else {
+    TRY(embed_gather_launch(st, rows, C, s->tokens_dev, m->emb_ln0, b.x));
+    LnArgs a = {};
+    a.x = b.x; a.w = m->layers[0].t[RWKV_T_LN1_W]; a.b = m->layers[0].t[RWKV_T_LN1_B]; a.y = b.xx;
+    a.C = C; a.T = 1; a.eps = kLnEps;
+    TRY(ln_launch(st, kLn, rows, a));
+  }
+
+  for (int l = 0; l < L; ++l) {
+    const Layer& w = m->layers[l];
+    half_t* shift0 = shift + static_cast<int64_t>(l) * 2 * B * C;
+    half_t* shift1 = shift0 + static_cast<int64_t>(B) * C;
+    float* S = wkv + static_cast<int64_t>(l) * B * H * kHead * kHead;
+    half_t* v_cur = (l == 0) ? b.v_first : b.v;  // layer 0 writes v straight into v_first
+
+    if (!step) {
+      MixArgs a = {};
+      a.x = b.xx; a.shift = shift0; a.B = B; a.T = T; a.C = C; a.n_mix = 6;
+      const int ids[6] = {RWKV_T_X_R, RWKV_T_X_W, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_A, RWKV_T_X_G};
+      half_t* outs[6] = {b.xr, b.xw, b.xk, b.xv, b.xa, b.xg};
+      for (int i = 0; i < 6; ++i) {
+        a.mu[i] = w.t[ids[i]];
+        a.out[i] = outs[i];
+      }
+      TRY(token_shift_mix_launch(st, a));
+    }
+
+    // r, k, v projections
+    const bool same_fmt = w.m[RWKV_M_ATT_R].fmt == w.m[RWKV_M_ATT_K].fmt && w.m[RWKV_M_ATT_R].fmt == w.m[RWKV_M_ATT_V].fmt;
+    if (small && same_fmt) {
+      LinearProblem p[3];
+      const int mids[3] = {RWKV_M_ATT_R, RWKV_M_ATT_K, RWKV_M_ATT_V};
+      const half_t* xs[3] = {b.xr, b.xk, b.xv};
+      half_t* ys[3] = {b.r, b.k, v_cur};
+      for (int i = 0; i < 3; ++i) {
+        p[i].w = w.m[mids[i]].data; p[i].scale = w.m[mids[i]].scale; p[i].zp = w.m[mids[i]].zp;
+        p[i].x = xs[i]; p[i].y = ys[i]; p[i].N = C;
+      }
+      TRY(linear_small_m(st, w.m[RWKV_M_ATT_R].fmt, rows, C, 3, p, RWKV_EPI_NONE, 0));
+    } else {
+      TRY(apply_matrix(st, w.m[RWKV_M_ATT_R], rows, C, C, b.xr, RWKV_EPI_NONE, 0, b.r));
+      TRY(apply_matrix(st, w.m[RWKV_M_ATT_K], rows, C, C, b.xk, RWKV_EPI_NONE, 0, b.k));
+      TRY(apply_matrix(st, w.m[RWKV_M_ATT_V], rows, C, C, b.xv, RWKV_EPI_NONE, 0, v_cur));
+    }
+
+    // LoRA rank-in (w, a, g and, past layer 0, v)
+    {
+      const int n_lora = (l == 0) ? 3 : 4;
+      const int w1_ids[4] = {RWKV_T_W1, RWKV_T_A1, RWKV_T_G1, RWKV_T_V1};
+      const int ranks[4] = {m->Rw, m->Ra, m->Rg, m->Rv};
+      const half_t* xs[4] = {b.xw, b.xa, b.xg, b.xv};
+      half_t* hs[4] = {b.hw, b.ha, b.hg, b.hv};
+      if (small) {
+        LinearProblem p[4];
+        for (int i = 0; i < n_lora; ++i) {
+          p[i].w = w.t[w1_ids[i]]; p[i].scale = nullptr; p[i].zp = nullptr;
+          p[i].x = xs[i]; p[i].y = hs[i]; p[i].N = ranks[i];
+        }
+        TRY(linear_small_m(st, RWKV_FMT_F16, rows, C, n_lora, p, RWKV_EPI_NONE, 0));
+      } else {
+        for (int i = 0; i < n_lora; ++i)
+          TRY(linear_any_m(st, RWKV_FMT_F16, rows, ranks[i], C, xs[i], w.t[w1_ids[i]], nullptr, nullptr, RWKV_EPI_NONE,
+                           0, hs[i]));
+      }
+    }
+    // LoRA rank-out (+ activation, + v-residual gate)
+    {
+      LoraOutArgs a = {};
+      a.M = rows; a.C = C;
+      a.h = b.hw; a.w2 = w.t[RWKV_T_W2]; a.R = m->Rw; a.act = RWKV_ACT_TANH; a.out = b.w12;
+      TRY(lora_out_launch(st, a));
+      a.h = b.ha; a.w2 = w.t[RWKV_T_A2]; a.R = m->Ra; a.act = RWKV_ACT_NONE; a.out = b.a12;
+      TRY(lora_out_launch(st, a));
+      a.h = b.hg; a.w2 = w.t[RWKV_T_G2]; a.R = m->Rg; a.act = RWKV_ACT_SIGMOID; a.out = b.g;
+      TRY(lora_out_launch(st, a));
+      if (l > 0) {
+        a.h = b.hv; a.w2 = w.t[RWKV_T_V2]; a.R = m->Rv; a.act = RWKV_ACT_NONE; a.bias = w.t[RWKV_T_V0];
+        a.vres = 1; a.v = b.v; a.v_first = b.v_first; a.out = b.xv;  // xv is free after the projections
+        TRY(lora_out_launch(st, a));
+        v_cur = b.xv;
+      }
+    }
+
+    // kk normalise, a-gate, decay; operands widened to fp32 for the scalar-fed WKV kernel
+    {
+      KkArgs p = {};
+      p.k = b.k; p.k_k = w.t[RWKV_T_K_K]; p.a0 = w.t[RWKV_T_A0]; p.a12 = b.a12; p.k_a = w.t[RWKV_T_K_A];
+      p.new_k = b.k2; p.neg_kk = nullptr; p.kka = nullptr;
+      p.w12 = b.w12; p.w0 = w.t[RWKV_T_W0]; p.r = b.r;
+      p.k32 = b.k32; p.a32 = b.a32; p.b32 = b.b32; p.d32 = b.d32; p.r32 = b.r32;
+      p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
+      TRY(kk_a_gate_launch(st, p));
+    }
+    TRY(wkv7_seq_f16_launch(st, B, T, C, H, S, b.r32, b.d32, b.k32, b.a32, b.b32, static_cast<int64_t>(T) * C, v_cur,
+                            b.y, static_cast<int64_t>(T) * C));
+    TRY(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
+                   w.t[RWKV_T_LNX_B], b.g, b.y2));
+    TRY(apply_matrix(st, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
+
+    // residual add + LN2 + channel-mix token shift
+    if (step) {
+      LnArgs a = {};
+      a.x = b.x; a.res = b.att; a.w = w.t[RWKV_T_LN2_W]; a.b = w.t[RWKV_T_LN2_B]; a.x_out = b.x1; a.shift = shift1;
+      a.mu[0] = w.t[RWKV_T_FFN_X_K]; a.out[0] = b.mixed; a.n_mix = 1; a.C = C; a.T = 1; a.eps = kLnEps;
+      TRY(ln_launch(st, kAddLnMix, rows, a));
+    } else {
+      LnArgs a = {};
+      a.x = b.x; a.res = b.att; a.w = w.t[RWKV_T_LN2_W]; a.b = w.t[RWKV_T_LN2_B]; a.x_out = b.x1; a.y = b.ln2;
+      a.C = C; a.T = 1; a.eps = kLnEps;
+      TRY(ln_launch(st, kAddLn, rows, a));
+      MixArgs mx = {};
+      mx.x = b.ln2; mx.shift = shift1; mx.B = B; mx.T = T; mx.C = C; mx.n_mix = 1;
+      mx.mu[0] = w.t[RWKV_T_FFN_X_K]; mx.out[0] = b.mixed;
+      TRY(token_shift_mix_launch(st, mx));
+    }
+
+    // channel mix
+    TRY(apply_matrix(st, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
+    TRY(apply_matrix(st, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+
+    // residual add + next layer's LN1 (+ lerps), or the final LN on the last token of each row
+    if (l + 1 < L) {
+      const Layer& nx = m->layers[l + 1];
+      LnArgs a = {};
+      a.x = b.x1; a.res = b.cm; a.w = nx.t[RWKV_T_LN1_W]; a.b = nx.t[RWKV_T_LN1_B]; a.x_out = b.x;
+      a.C = C; a.T = 1; a.eps = kLnEps;
+      if (step) {
+        a.shift = shift + static_cast<int64_t>(l + 1) * 2 * B * C;
+        mix6_args(nx, a);
+        TRY(ln_launch(st, kAddLnMix, rows, a));
+      } else {
+        a.y = b.xx;
+        TRY(ln_launch(st, kAddLn, rows, a));
+      }
+    } else {
+      LnArgs a = {};
+      a.x = b.x1; a.res = b.cm; a.w = m->ln_out_w; a.b = m->ln_out_b; a.y = b.xf; a.C = C; a.T = T; a.eps = kLnEps;
+      TRY(ln_launch(st, kAddLastLn, B, a));
+      if (s->trace) {
+        LnArgs t = {};
+        t.x = b.x1; t.res = b.cm; t.w = m->ln_out_w; t.b = m->ln_out_b; t.x_out = b.x; t.y = b.scratch;
+        t.C = C; t.T = 1; t.eps = kLnEps;
+        TRY(ln_launch(st, kAddLn, rows, t));
+      }
+    }
+    if (s->trace) {
+      RWKV_HIP_TRY(hipMemcpyAsync(s->trace + static_cast<int64_t>(l) * RC, b.x, sizeof(half_t) * RC,
+                                  hipMemcpyDeviceToDevice, st));
+    }
+  }
+
+  TRY(advance_launch(st, B, T, elapsed));
+  TRY(apply_matrix(st, m->head, B, V, C, b.xf, RWKV_EPI_NONE, 1, logits));
+  return RWKV_OK;
+}
+
+GraphEntry* find_graph(rwkv_hip_session* s, int B, void* shift, void* wkv, void* elapsed, void* logits) {
+  for (auto& g : s->graphs) {
+    if (g.B == B && g.shift == shift && g.wkv == wkv && g.elapsed == elapsed && g.logits == logits) return &g;
+  }
+  return nullptr;
+}
+
+// T == 1 step through a captured graph (captures on first use of this (B, state, logits) tuple).
+int run_step(rwkv_hip_session* s, int B, half_t* shift, float* wkv, int* elapsed, float* logits) {
+  if (!s->use_graph || s->trace) return enqueue_forward(s, B, 1, shift, wkv, elapsed, logits);
+  GraphEntry* g = find_graph(s, B, shift, wkv, elapsed, logits);
+  if (!g) {
+    if (s->graphs.size() >= kMaxGraphs) {
+      auto victim = std::min_element(s->graphs.begin(), s->graphs.end(),
+                                     [](const GraphEntry& x, const GraphEntry& y) { return x.last_use < y.last_use; });
+      RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+      if (victim->exec) (void)hipGraphExecDestroy(victim->exec);
+      if (victim->graph) (void)hipGraphDestroy(victim->graph);
+      s->graphs.erase(victim);
+    }
+    GraphEntry e;
+    e.B = B; e.shift = shift; e.wkv = wkv; e.elapsed = elapsed; e.logits = logits;
+    RWKV_HIP_TRY(hipStreamBeginCapture(s->stream, hipStreamCaptureModeThreadLocal));
+    const int rc = enqueue_forward(s, B, 1, shift, wkv, elapsed, logits);
+    hipGraph_t graph = nullptr;
+    const hipError_t end = hipStreamEndCapture(s->stream, &graph);
+    if (rc != RWKV_OK) {
+      if (graph) (void)hipGraphDestroy(graph);
+      return rc;
+    }
+    if (end != hipSuccess) {
+      set_error("hipStreamEndCapture failed: %s", hipGetErrorString(end));
+      return RWKV_E_RUNTIME;
+    }
+    e.graph = graph;
+    RWKV_HIP_TRY(hipGraphInstantiate(&e.exec, graph, nullptr, nullptr, 0));
+    s->graphs.push_back(e);
+    g = &s->graphs.back();
+  }
+  g->last_use = ++s->tick;
+  RWKV_HIP_TRY(hipGraphLaunch(g->exec, s->stream));
+  return RWKV_OK;
+}
+
+int check_forward_args(const rwkv_hip_session* s, int B, int T, const void* shift, const void* wkv, const void* elapsed,
+                       const void* logits) {
+  RWKV_REQUIRE(s != nullptr, "session is NULL");
+  RWKV_REQUIRE(B > 0, "token_batches must not be empty");         // src/rwkv7_fast_v4.cu:1054-1056
+  RWKV_REQUIRE(T > 0, "token batch length must be positive");     // :1065-1067
+  RWKV_REQUIRE(shift && wkv && elapsed && logits, "forward: NULL state or logits tensor");
+  return model_ready(s->model);
+}
+
+__global__ void feed_tokens_kernel(int B, const int* __restrict__ picked, int64_t* __restrict__ tokens,
+                                   int* __restrict__ history) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < B) {
+    tokens[i] = picked[i];
+    history[i] = picked[i];
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int rwkv_hip_model_create(rwkv_hip_model** out, int L, int C, int H, int F, int V, int Rw, int Ra, int Rg, int Rv) {
+  RWKV_REQUIRE(out != nullptr, "model out is NULL");
+  *out = nullptr;
+  RWKV_REQUIRE(L > 0 && H > 0 && F > 0 && V > 0, "model: L, H, F, V must be positive");
+  RWKV_REQUIRE(C == H * kHead, "C must equal H*N with head size 64 (C=%d, H=%d)", C, H);  // rwkv7_fast_v4_common.hpp:285-286
+  RWKV_REQUIRE(C % 32 == 0 && F % 32 == 0 && V % 4 == 0, "model: C, F must be multiples of 32 and V of 4");
+  const int ranks[4] = {Rw, Ra, Rg, Rv};
+  for (int r : ranks)
+    RWKV_REQUIRE(r > 0 && r % 8 == 0 && r <= 512, "lowrank exceeds arena max or is not a multiple of 8 (%d)", r);  // :1172-1175
+  rwkv_hip_model* m = new (std::nothrow) rwkv_hip_model();
+  if (!m) {
+    set_error("model: out of host memory");
+    return RWKV_E_NOMEM;
+  }
+  m->L = L; m->C = C; m->H = H; m->F = F; m->V = V; m->Rw = Rw; m->Ra = Ra; m->Rg = Rg; m->Rv = Rv;
+  m->layers.resize(L);
+  *out = m;
+  return RWKV_OK;
+}
+
+int rwkv_hip_model_destroy(rwkv_hip_model* m) {
+  delete m;
+  return RWKV_OK;
+}
+
+int rwkv_hip_model_set_tensor(rwkv_hip_model* m, int layer, int id, const void* data) {
+  RWKV_REQUIRE(m && data, "set_tensor: NULL argument");
+  const half_t* p = static_cast<const half_t*>(data);
+  if (layer < 0) {
+    switch (id) {
+      case RWKV_T_EMB_LN0: m->emb_ln0 = p; return RWKV_OK;
+      case RWKV_T_LN_OUT_W: m->ln_out_w = p; return RWKV_OK;
+      case RWKV_T_LN_OUT_B: m->ln_out_b = p; return RWKV_OK;
+      default: break;
+    }
+    set_error("set_tensor: unknown global tensor id %d", id);
+    return RWKV_E_INVALID;
+  }
+  RWKV_REQUIRE(layer < m->L, "set_tensor: layer %d out of range", layer);
+  RWKV_REQUIRE((id >= RWKV_T_LN1_W && id <= RWKV_T_FFN_X_K) || (id >= RWKV_T_W1 && id <= RWKV_T_V2),
+               "set_tensor: unknown tensor id %d", id);
+  m->layers[layer].t[id] = p;
+  return RWKV_OK;
+}
+
+int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, const void* data, const void* scale,
+                              const void* zp) {
+  RWKV_REQUIRE(m && data, "set_matrix: NULL argument");
+  RWKV_REQUIRE(fmt == RWKV_FMT_F16 || fmt == RWKV_FMT_W8 || fmt == RWKV_FMT_W4, "set_matrix: bad format %d", fmt);
+  RWKV_REQUIRE(fmt == RWKV_FMT_F16 || scale, "set_matrix: quantised matrix needs a scale tensor");
+  RWKV_REQUIRE(fmt != RWKV_FMT_W4 || zp, "set_matrix: W4 matrix needs a zero-point tensor");
+  Matrix mat;
+  mat.fmt = fmt; mat.data = data; mat.scale = static_cast<const half_t*>(scale); mat.zp = static_cast<const uint8_t*>(zp);
+  if (id == RWKV_M_HEAD) {
+    m->head = mat;
+    return RWKV_OK;
+  }
+  RWKV_REQUIRE(layer >= 0 && layer < m->L, "set_matrix: layer %d out of range", layer);
+  RWKV_REQUIRE(id >= 0 && id < 6, "set_matrix: unknown matrix id %d", id);
+  if (fmt == RWKV_FMT_W4) {
+    const int K = (id == RWKV_M_FFN_VALUE) ? m->F : m->C;
+    RWKV_REQUIRE(K % 128 == 0, "set_matrix: W4 needs the input width (%d) to be a multiple of 128", K);
+  }
+  m->layers[layer].m[id] = mat;
+  return RWKV_OK;
+}
+
+int rwkv_hip_model_weight_bytes(const rwkv_hip_model* m, uint64_t* bytes) {
+  RWKV_REQUIRE(m && bytes, "weight_bytes: NULL argument");
+  auto mat_bytes = [](const Matrix& mat, uint64_t N, uint64_t K) -> uint64_t {
+    switch (mat.fmt) {
+      case RWKV_FMT_W8: return N * K + N * 2;
+      case RWKV_FMT_W4: return N * K / 2 + N * (K / 128) * 3;
+      default: return N * K * 2;
+    }
+  };
+  const uint64_t C = m->C, F = m->F, V = m->V;
+  uint64_t total = mat_bytes(m->head, V, C) + 2 * C * 2;  // head + ln_out
+  for (int l = 0; l < m->L; ++l) {
+    const Layer& w = m->layers[l];
+    total += mat_bytes(w.m[RWKV_M_ATT_R], C, C) + mat_bytes(w.m[RWKV_M_ATT_K], C, C) + mat_bytes(w.m[RWKV_M_ATT_V], C, C) +
+             mat_bytes(w.m[RWKV_M_ATT_O], C, C) + mat_bytes(w.m[RWKV_M_FFN_KEY], F, C) + mat_bytes(w.m[RWKV_M_FFN_VALUE], C, F);
+    total += 19 * C * 2;  // per-layer vectors
+    const uint64_t ranks = static_cast<uint64_t>(m->Rw) + m->Ra + m->Rg + (l > 0 ? m->Rv : 0);
+    total += 2 * ranks * C * 2;  // LoRA pairs, fp16
+  }
+  *bytes = total;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_create(rwkv_hip_session** out, const rwkv_hip_model* m) {
+  RWKV_REQUIRE(out && m, "session_create: NULL argument");
+  *out = nullptr;
+  rwkv_hip_session* s = new (std::nothrow) rwkv_hip_session();
+  if (!s) {
+    set_error("session: out of host memory");
+    return RWKV_E_NOMEM;
+  }
+  s->model = m;
+  const hipError_t err = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
+  if (err != hipSuccess) {
+    set_error("hipStreamCreateWithFlags failed: %s", hipGetErrorString(err));
+    delete s;
+    return RWKV_E_RUNTIME;
+  }
+  *out = s;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_destroy(rwkv_hip_session* s) {
+  if (!s) return RWKV_OK;
+  (void)hipStreamSynchronize(s->stream);
+  for (auto& g : s->graphs) {
+    if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    if (g.graph) (void)hipGraphDestroy(g.graph);
+  }
+  if (s->arena.base) (void)hipFree(s->arena.base);
+  if (s->tokens_dev) (void)hipFree(s->tokens_dev);
+  if (s->tokens_pinned) (void)hipHostFree(s->tokens_pinned);
+  if (s->argmax_dev) (void)hipFree(s->argmax_dev);
+  if (s->history_dev) (void)hipFree(s->history_dev);
+  (void)hipStreamDestroy(s->stream);
+  delete s;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_stream(rwkv_hip_session* s, rwkv_stream_t* stream) {
+  RWKV_REQUIRE(s && stream, "session_stream: NULL argument");
+  *stream = s->stream;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_set_graph(rwkv_hip_session* s, int use_graph) {
+  RWKV_REQUIRE(s, "session is NULL");
+  s->use_graph = use_graph != 0;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_set_trace(rwkv_hip_session* s, void* trace) {
+  RWKV_REQUIRE(s, "session is NULL");
+  s->trace = static_cast<half_t*>(trace);
+  return RWKV_OK;
+}
+
+int rwkv_hip_forward(rwkv_hip_session* s, const int64_t* tokens_host, int B, int T, void* shift, void* wkv,
+                     void* elapsed, void* logits, int sync) {
+  TRY(check_forward_args(s, B, T, shift, wkv, elapsed, logits));
+  RWKV_REQUIRE(tokens_host != nullptr, "forward: tokens is NULL");
+  const int rows = B * T;
+  for (int i = 0; i < rows; ++i) {
+    RWKV_REQUIRE(tokens_host[i] >= 0 && tokens_host[i] < s->model->V, "token id out of range");  // :1107-1110
+  }
+  TRY(ensure_arena(s, B, T));
+  // the pinned staging buffer may still be in flight from the previous call
+  RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+  std::copy(tokens_host, tokens_host + rows, s->tokens_pinned);
+  RWKV_HIP_TRY(hipMemcpyAsync(s->tokens_dev, s->tokens_pinned, sizeof(int64_t) * rows, hipMemcpyHostToDevice, s->stream));
+  if (T == 1) {
+    TRY(run_step(s, B, static_cast<half_t*>(shift), static_cast<float*>(wkv), static_cast<int*>(elapsed),
+                 static_cast<float*>(logits)));
+  } else {
+    TRY(enqueue_forward(s, B, T, static_cast<half_t*>(shift), static_cast<float*>(wkv), static_cast<int*>(elapsed),
+                        static_cast<float*>(logits)));
+  }
+  if (sync) RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+  return RWKV_OK;
+}
+
+int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host, int B, int steps, void* shift,
+                           void* wkv, void* elapsed, void* logits, int32_t* out_tokens_host) {
+  TRY(check_forward_args(s, B, 1, shift, wkv, elapsed, logits));
+  RWKV_REQUIRE(first_tokens_host && out_tokens_host && steps > 0, "decode_greedy: bad arguments");
+  for (int i = 0; i < B; ++i)
+    RWKV_REQUIRE(first_tokens_host[i] >= 0 && first_tokens_host[i] < s->model->V, "token id out of range");
+  TRY(ensure_arena(s, B, 1));
+  RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+  if (B > s->argmax_cap) {
+    if (s->argmax_dev) RWKV_HIP_TRY(hipFree(s->argmax_dev));
+    s->argmax_dev = nullptr;
+    s->argmax_cap = 0;
+    RWKV_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->argmax_dev), sizeof(int) * B));
+    s->argmax_cap = B;
+  }
+  const size_t hist = static_cast<size_t>(steps) * B;
+  if (hist > s->history_cap) {
+    if (s->history_dev) RWKV_HIP_TRY(hipFree(s->history_dev));
+    s->history_dev = nullptr;
+    s->history_cap = 0;
+    RWKV_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&s->history_dev), sizeof(int) * hist));
+    s->history_cap = hist;
+  }
+  std::copy(first_tokens_host, first_tokens_host + B, s->tokens_pinned);
+  RWKV_HIP_TRY(hipMemcpyAsync(s->tokens_dev, s->tokens_pinned, sizeof(int64_t) * B, hipMemcpyHostToDevice, s->stream));
+  for (int i = 0; i < steps; ++i) {
+    TRY(run_step(s, B, static_cast<half_t*>(shift), static_cast<float*>(wkv), static_cast<int*>(elapsed),
+                 static_cast<float*>(logits)));
+    TRY(argmax_launch(s->stream, B, s->model->V, static_cast<float*>(logits), s->argmax_dev));
+    hipLaunchKernelGGL(feed_tokens_kernel, dim3(ceil_div(B, 64)), dim3(64), 0, s->stream, B, s->argmax_dev,
+                       s->tokens_dev, s->history_dev + static_cast<size_t>(i) * B);
+    RWKV_LAUNCH_CHECK();
+  }
+  RWKV_HIP_TRY(hipMemcpyAsync(out_tokens_host, s->history_dev, sizeof(int) * hist, hipMemcpyDeviceToHost, s->stream));
+  RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+  return RWKV_OK;
+}
+
+}  // extern "C"

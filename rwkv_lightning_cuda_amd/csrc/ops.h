@@ -1,0 +1,118 @@
+// Internal launcher interface shared by the op files and the model graph (not exported).
+#pragma once
+
+#include "common.h"
+
+namespace rwkv {
+
+// ---- linear.hip / gemm_mfma.hip ------------------------------------------------------------------
+constexpr int kMaxProblems = 4;
+
+struct LinearProblem {
+  const void* w;
+  const half_t* scale;
+  const uint8_t* zp;
+  const half_t* x;
+  void* y;
+  int N;
+};
+
+// Batched small-M (<= 8) linear through the weight-streaming GEMV kernel.
+int linear_small_m(hipStream_t st, int fmt, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
+                   int out_f32);
+// Any M: MFMA tiles for M >= 16 where supported, else row tiles through the GEMV kernel.
+int linear_any_m(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* w, const half_t* scale,
+                 const uint8_t* zp, int epilogue, int out_f32, void* y);
+int linear_mfma(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* w, const half_t* scale,
+                const uint8_t* zp, int epilogue, int out_f32, void* y);
+bool linear_mfma_supported(int fmt, int M, int N, int K);
+
+// ---- fused_ops.hip ------------------------------------------------------------------------------
+enum LnMode {
+  kLn = 0,          // y = LN(x)
+  kAddLn = 1,       // s = x + res; x_out = s; y = LN(s)
+  kAddLastLn = 2,   // rows = B, reads row b*T + T-1; y only
+  kAddLnMix = 3,    // kAddLn + n_mix lerps against shift, shift <- LN output (T == 1)
+  kLnMix = 4,       // y = LN(x) without residual, then lerps + shift write (embedding row of layer 0)
+};
+
+struct LnArgs {
+  const half_t* x;
+  const half_t* res;
+  const half_t* w;
+  const half_t* b;
+  half_t* x_out;
+  half_t* y;
+  half_t* shift;
+  const half_t* mu[6];
+  half_t* out[6];
+  const int64_t* tokens;  // kLnMix: if not NULL, x is a [V,C] table indexed by tokens[row]
+  int C;
+  int T;
+  int n_mix;
+  float eps;
+};
+
+int ln_launch(hipStream_t st, int mode, int rows, const LnArgs& a);
+
+struct MixArgs {
+  const half_t* x;
+  half_t* shift;
+  const half_t* mu[6];
+  half_t* out[6];
+  int B, T, C, n_mix;
+};
+
+int token_shift_mix_launch(hipStream_t st, const MixArgs& a);
+
+struct KkArgs {
+  const half_t* k;
+  const half_t* k_k;
+  const half_t* a0;
+  const half_t* a12;
+  const half_t* k_a;
+  half_t* new_k;
+  half_t* neg_kk;
+  half_t* kka;
+  // optional extras (all may be NULL): decay logits w12 (+ w0) and r, widened for the WKV kernel
+  const half_t* w12;
+  const half_t* w0;
+  const half_t* r;
+  float* k32;
+  float* a32;
+  float* b32;
+  float* d32;
+  float* r32;
+  int64_t rows_heads;
+  int H;
+};
+
+int kk_a_gate_launch(hipStream_t st, const KkArgs& p);
+int lnx_launch(hipStream_t st, int64_t rows_heads, int H, const half_t* y, const half_t* r, const half_t* k,
+               const half_t* v, const half_t* r_k, const half_t* lnw, const half_t* lnb, const half_t* g, half_t* out);
+int advance_launch(hipStream_t st, int n, int amount, int* x);
+int embed_gather_launch(hipStream_t st, int rows, int C, const int64_t* tokens, const half_t* table, half_t* out);
+
+// ---- lora.hip -----------------------------------------------------------------------------------
+struct LoraOutArgs {
+  const half_t* h;        // [M,R]
+  const half_t* w2;       // [C,R]
+  const half_t* bias;     // [C] or NULL
+  const half_t* v;        // [M,C] (vres)
+  const half_t* v_first;  // [M,C] (vres)
+  half_t* out;            // [M,C]
+  int M, C, R, act, vres;
+};
+int lora_out_launch(hipStream_t st, const LoraOutArgs& a);
+
+// ---- sampler.hip --------------------------------------------------------------------------------
+int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out);
+
+// ---- wkv7.hip -----------------------------------------------------------------------------------
+// T tokens of the recurrence from fp32 operands (decay applied); v, y fp16.  op_bs / io_bs: elements
+// between batch rows of the operand / io tensors.
+int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
+                        const float* k, const float* a, const float* b, int64_t op_bs, const half_t* v, half_t* y,
+                        int64_t io_bs);
+
+}  // namespace rwkv

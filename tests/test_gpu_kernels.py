@@ -1,0 +1,334 @@
+"""GPU parity tests of the individual C-ABI ops against the CPU oracle (same seeded inputs).
+
+Bars: integer / byte work bit-exact; WKV fp32 state max-rel <= 1e-4; fp16 paths <= 2e-3.
+"""
+import numpy as np
+import pytest
+
+from conftest import elem_err, rel_err
+from inputs import pattern_value, wkv_inputs
+
+pytestmark = pytest.mark.gpu
+
+WKV_TOL = 1e-4
+F16_TOL = 2e-3
+
+
+def dev(hip, a):
+    return hip.DeviceArray.from_numpy(a)
+
+
+# ---------------------------------------------------------------------------------------------- WKV7
+@pytest.mark.parametrize("B,T,H", [(1, 64, 12), (2, 7, 3), (3, 1, 2)])
+@pytest.mark.parametrize("mode", ["decay", "raw"])
+def test_wkv7_f32_matches_oracle(gpu, orc, B, T, H, mode):
+    hip = gpu
+    C = H * 64
+    inp = wkv_inputs(B, T, H, seed=100 + B + T)
+    w = inp["decay"] if mode == "decay" else inp["w_raw"]
+    w_mode = hip.W_DECAY if mode == "decay" else hip.W_RAW_LOGIT
+    s_ref = np.zeros((B, H, 64, 64), np.float32)
+    y_ref = orc.wkv7(s_ref, inp["r"], w, inp["k"], inp["v"], inp["a"], inp["b"], H, w_mode)
+    state = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y = hip.DeviceArray((B, T, C), np.float32)
+    hip.wkv7(B, T, C, H, w_mode, hip.IO_F32, state, dev(hip, inp["r"]), dev(hip, w), dev(hip, inp["k"]),
+             dev(hip, inp["v"]), dev(hip, inp["a"]), dev(hip, inp["b"]), y)
+    hip.device_sync()
+    assert rel_err(y.numpy(), y_ref) <= WKV_TOL
+    assert rel_err(state.numpy(), s_ref) <= WKV_TOL
+    assert elem_err(state.numpy(), s_ref) <= WKV_TOL
+
+
+def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):
+    hip = gpu
+    B, T, H = 2, 40, 4
+    C = H * 64
+    inp = wkv_inputs(B, T, H, seed=7, dtype=np.float16)
+    names = ["r", "w_raw", "k", "v", "a", "b"]
+    s_ref = np.zeros((B, H, 64, 64), np.float32)
+    y_ref = orc.wkv7(s_ref, *[inp[n] for n in names], H, 0)
+    d = {n: dev(hip, inp[n]) for n in names}
+    state = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y = hip.DeviceArray((B, T, C), np.float16)
+    hip.wkv7(B, T, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state, *[d[n] for n in names], y)
+    hip.device_sync()
+    assert rel_err(y.numpy().astype(np.float32), y_ref.astype(np.float32)) <= F16_TOL
+    assert rel_err(state.numpy(), s_ref) <= WKV_TOL
+
+    # the same tokens in two calls (T1 + T2): bitwise identical state and outputs
+    T1 = 13
+    state2 = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y2 = np.zeros((B, T, C), np.float16)
+    for t0, tn in ((0, T1), (T1, T - T1)):
+        part = {n: dev(hip, np.ascontiguousarray(inp[n][:, t0:t0 + tn])) for n in names}
+        yp = hip.DeviceArray((B, tn, C), np.float16)
+        hip.wkv7(B, tn, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state2, *[part[n] for n in names], yp)
+        hip.device_sync()
+        y2[:, t0:t0 + tn] = yp.numpy()
+    assert np.array_equal(state2.numpy().view(np.uint32), state.numpy().view(np.uint32))
+    assert np.array_equal(y2.view(np.uint16), y.numpy().view(np.uint16))
+
+
+# ------------------------------------------------------------------------------------------- formats
+def test_quantize_dequant_bit_exact(gpu, orc):
+    hip = gpu
+    rng = np.random.default_rng(3)
+    N, K = 96, 1024
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    w[5] = 0  # an all-zero row exercises scale == 0
+    w[6, :128] = 0
+    wd = dev(hip, w)
+    q_ref, s_ref = orc.quantize_w8(w)
+    q = hip.DeviceArray((N, K), np.int8)
+    s = hip.DeviceArray((N,), np.float16)
+    hip.quantize_w8(N, K, wd, q, s)
+    out = hip.DeviceArray((N, K), np.float16)
+    hip.dequant_w8(N, K, q, s, out)
+    hip.device_sync()
+    assert np.array_equal(q.numpy(), q_ref)
+    assert np.array_equal(s.numpy().view(np.uint16), s_ref.view(np.uint16))
+    assert np.array_equal(out.numpy().view(np.uint16), orc.dequant_w8(q_ref, s_ref).view(np.uint16))
+
+    q4_ref, s4_ref, z4_ref = orc.quantize_w4(w)
+    q4 = hip.DeviceArray((N, K // 2), np.uint8)
+    s4 = hip.DeviceArray((N, K // 128), np.float16)
+    z4 = hip.DeviceArray((N, K // 128), np.uint8)
+    hip.quantize_w4(N, K, wd, q4, s4, z4)
+    out4 = hip.DeviceArray((N, K), np.float16)
+    hip.dequant_w4(N, K, q4, s4, z4, out4)
+    hip.device_sync()
+    assert np.array_equal(q4.numpy(), q4_ref)
+    assert np.array_equal(s4.numpy().view(np.uint16), s4_ref.view(np.uint16))
+    assert np.array_equal(z4.numpy(), z4_ref)
+    assert np.array_equal(out4.numpy().view(np.uint16), orc.dequant_w4(q4_ref, s4_ref, z4_ref).view(np.uint16))
+
+
+def test_dequant_all_codes_bit_exact(gpu, orc):
+    """Every int8 code and every (int4 code, zero point) pair against a spread of scales."""
+    hip = gpu
+    scales = np.array([6.1e-5, 1e-3, 0.0137, 0.5, 1.0, 3.3, 6.0e-8, 100.0], np.float16)
+    q = np.tile(np.arange(-128, 128, dtype=np.int8), (len(scales), 1))
+    out = hip.DeviceArray(q.shape, np.float16)
+    hip.dequant_w8(q.shape[0], q.shape[1], dev(hip, q), dev(hip, scales), out)
+    hip.device_sync()
+    assert np.array_equal(out.numpy().view(np.uint16), orc.dequant_w8(q, scales).view(np.uint16))
+
+    rows = []
+    zps = []
+    for zp in range(16):
+        codes = np.tile(np.arange(16, dtype=np.uint8), 8)  # 128 codes: every nibble value at even and odd k
+        codes = np.roll(codes, zp)  # shift parity so each code lands in both nibble positions
+        rows.append((codes[0::2] | (codes[1::2] << 4)).astype(np.uint8))
+        zps.append(zp)
+    q4 = np.stack(rows)
+    z4 = np.array(zps, np.uint8).reshape(16, 1)
+    s4 = np.linspace(0.001, 2.0, 16).astype(np.float16).reshape(16, 1)
+    out4 = hip.DeviceArray((16, 128), np.float16)
+    hip.dequant_w4(16, 128, dev(hip, q4), dev(hip, s4), dev(hip, z4), out4)
+    hip.device_sync()
+    assert np.array_equal(out4.numpy().view(np.uint16), orc.dequant_w4(q4, s4, z4).view(np.uint16))
+
+
+# -------------------------------------------------------------------------------------------- linear
+@pytest.mark.parametrize("fmt_name", ["f16", "w8", "w4"])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 11])
+def test_linear_small_m(gpu, orc, fmt_name, M):
+    hip = gpu
+    rng = np.random.default_rng(11 + M)
+    N, K = 264, 768
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    fmt = {"f16": hip.FMT_F16, "w8": hip.FMT_W8, "w4": hip.FMT_W4}[fmt_name]
+    if fmt == hip.FMT_F16:
+        parts = (w, None, None)
+    elif fmt == hip.FMT_W8:
+        parts = orc.quantize_w8(w) + (None,)
+    else:
+        parts = orc.quantize_w4(w)
+    y_ref = orc.gemv(fmt, x, parts[0], parts[1], parts[2])
+    y = hip.DeviceArray((M, N), np.float16)
+    dparts = [dev(hip, p) if p is not None else None for p in parts]
+    hip.linear(fmt, M, N, K, dev(hip, x), dparts[0], dparts[1], dparts[2], y)
+    hip.device_sync()
+    assert rel_err(y.numpy().astype(np.float32), y_ref.astype(np.float32)) <= F16_TOL
+
+
+@pytest.mark.parametrize("K", [1024, 2560, 4096, 16384])
+def test_linear_w8_relu_square_and_f32_out(gpu, orc, K):
+    hip = gpu
+    rng = np.random.default_rng(K)
+    N, M = 128, 2
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    q, s = orc.quantize_w8(w)
+    hid = orc.gemv(orc.FMT_W8, x, q, s)
+    act_ref = orc.relu_square(hid)
+    y = hip.DeviceArray((M, N), np.float16)
+    hip.linear(hip.FMT_W8, M, N, K, dev(hip, x), dev(hip, q), dev(hip, s), None, y, epilogue=hip.EPI_RELU_SQUARE)
+    y32 = hip.DeviceArray((M, N), np.float32)
+    hip.linear(hip.FMT_W8, M, N, K, dev(hip, x), dev(hip, q), dev(hip, s), None, y32, out_f32=1)
+    hip.device_sync()
+    assert rel_err(y.numpy().astype(np.float32), act_ref.astype(np.float32)) <= 2 * F16_TOL
+    got32 = y32.numpy()
+    assert rel_err(got32, hid.astype(np.float32)) <= F16_TOL
+    # fp32 logits hold fp16-representable values
+    assert np.array_equal(got32, got32.astype(np.float16).astype(np.float32))
+
+
+def test_linear_rejects_bad_shapes(gpu):
+    hip = gpu
+    x = hip.DeviceArray((1, 100), np.float16)
+    with pytest.raises(hip.RwkvHipError):
+        hip.linear(hip.FMT_W8, 1, 8, 100, x, x, x, None, x)  # K not a multiple of 16
+    with pytest.raises(hip.RwkvHipError):
+        hip.linear(hip.FMT_W8, 1, 8, 128, x, x, None, None, x)  # missing scale
+
+
+# ----------------------------------------------------------------------------------------- fused ops
+def _ref_test_inputs(rows, C, offs):
+    i = np.arange(rows * C)
+    x = pattern_value(i + offs[0], 0.2, -0.05).reshape(rows, C)
+    res = pattern_value(i + offs[1], 0.15, 0.03).reshape(rows, C)
+    sh = pattern_value(i + offs[2], 0.25, -0.02).reshape(rows, C)
+    c = np.arange(C)
+    w = pattern_value(c + 5, 0.08, 1.0)
+    b = pattern_value(c + 9, 0.03, 0.01)
+    return [t.astype(np.float16) for t in (x, res, sh, w, b)]
+
+
+@pytest.mark.parametrize("C", [768, 2560, 4096])
+def test_layer_norm_family(gpu, orc, C):
+    hip = gpu
+    rows = 3
+    x, res, sh, w, b = _ref_test_inputs(rows, C, (0, 17, 33))
+    y = hip.DeviceArray((rows, C), np.float16)
+    hip.layer_norm(rows, C, dev(hip, x), dev(hip, w), dev(hip, b), y)
+    xo = hip.DeviceArray((rows, C), np.float16)
+    y2 = hip.DeviceArray((rows, C), np.float16)
+    hip.add_layer_norm(rows, C, dev(hip, x), dev(hip, res), dev(hip, w), dev(hip, b), xo, y2)
+    hip.device_sync()
+    assert rel_err(y.numpy().astype(np.float32), orc.layer_norm(x, w, b).astype(np.float32)) <= F16_TOL
+    xo_ref, y2_ref = orc.add_layer_norm(x, res, w, b)
+    assert np.array_equal(xo.numpy().view(np.uint16), xo_ref.view(np.uint16))
+    assert rel_err(y2.numpy().astype(np.float32), y2_ref.astype(np.float32)) <= F16_TOL
+
+    # add + last-token LN (B=1, T=rows)
+    yl = hip.DeviceArray((1, C), np.float16)
+    hip.add_last_layer_norm(1, rows, C, dev(hip, x), dev(hip, res), dev(hip, w), dev(hip, b), yl)
+    hip.device_sync()
+    assert rel_err(yl.numpy().astype(np.float32), orc.add_last_layer_norm(x, res, w, b, 1, rows).astype(np.float32)) <= F16_TOL
+
+    # add + LN + cmix lerp + shift write (T == 1 fusion)
+    c = np.arange(C)
+    mu = (0.5 + 0.4 * np.sin(c.astype(np.float32) * 0.007)).astype(np.float16)
+    sh_ref = sh.copy()
+    xo_r, mixed_r = orc.add_layer_norm_cmix_mix(x, res, sh_ref, w, b, mu)
+    shd = dev(hip, sh)
+    xo3 = hip.DeviceArray((rows, C), np.float16)
+    mixed = hip.DeviceArray((rows, C), np.float16)
+    hip.add_layer_norm_cmix_mix(rows, C, dev(hip, x), dev(hip, res), shd, dev(hip, w), dev(hip, b), dev(hip, mu), xo3, mixed)
+    hip.device_sync()
+    assert np.array_equal(xo3.numpy().view(np.uint16), xo_r.view(np.uint16))
+    assert rel_err(mixed.numpy().astype(np.float32), mixed_r.astype(np.float32)) <= F16_TOL
+    assert rel_err(shd.numpy().astype(np.float32), sh_ref.astype(np.float32)) <= F16_TOL
+
+    # add + LN + six lerps
+    mus = [pattern_value(c + o, s, bb).astype(np.float16) for o, s, bb in
+           ((23, 0.09, 0.5), (29, 0.07, 0.4), (31, 0.05, 0.3), (37, 0.08, 0.2), (41, 0.06, 0.1), (43, 0.04, 0.6))]
+    sh_ref = sh.copy()
+    xo_r, outs_r = orc.add_layer_norm_tmix_mix6(x, res, sh_ref, w, b, mus)
+    shd = dev(hip, sh)
+    outs = [hip.DeviceArray((rows, C), np.float16) for _ in range(6)]
+    hip.add_layer_norm_tmix_mix6(rows, C, dev(hip, x), dev(hip, res), shd, dev(hip, w), dev(hip, b),
+                                 [dev(hip, m) for m in mus], xo3, outs)
+    hip.device_sync()
+    for o, o_r in zip(outs, outs_r):
+        assert rel_err(o.numpy().astype(np.float32), o_r.astype(np.float32)) <= F16_TOL
+    assert rel_err(shd.numpy().astype(np.float32), sh_ref.astype(np.float32)) <= F16_TOL
+
+
+@pytest.mark.parametrize("B,T", [(1, 1), (2, 5), (3, 1)])
+def test_token_shift_mix(gpu, orc, B, T):
+    hip = gpu
+    C = 256
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((B * T, C)).astype(np.float16)
+    sh = rng.standard_normal((B, C)).astype(np.float16)
+    mus = [rng.uniform(0, 1, C).astype(np.float16) for _ in range(6)]
+    sh_ref = sh.copy()
+    outs_r = orc.token_shift_mix(x, sh_ref, mus, B, T)
+    shd = dev(hip, sh)
+    outs = [hip.DeviceArray((B * T, C), np.float16) for _ in range(6)]
+    hip.token_shift_mix(B, T, C, dev(hip, x), shd, [dev(hip, m) for m in mus], outs)
+    hip.device_sync()
+    for o, o_r in zip(outs, outs_r):
+        assert rel_err(o.numpy().astype(np.float32), o_r.astype(np.float32)) <= F16_TOL
+    assert np.array_equal(shd.numpy().view(np.uint16), sh_ref.view(np.uint16))
+
+
+def test_kk_gate_groupnorm_lora(gpu, orc):
+    hip = gpu
+    rng = np.random.default_rng(9)
+    rows, H = 5, 6
+    C = H * 64
+
+    def rnd(*shape, s=1.0):
+        return (rng.standard_normal(shape) * s).astype(np.float16)
+
+    k, a12 = rnd(rows, C), rnd(rows, C, s=0.5)
+    k_k, a0, k_a = rnd(C, s=0.3) + np.float16(1), rnd(C, s=0.2), rnd(C, s=0.3) + np.float16(1)
+    nk_r, nkk_r, kka_r = orc.kk_a_gate(k, k_k, a0, a12, k_a, H)
+    nk, nkk, kka = (hip.DeviceArray((rows, C), np.float16) for _ in range(3))
+    hip.kk_a_gate(rows, C, H, dev(hip, k), dev(hip, k_k), dev(hip, a0), dev(hip, a12), dev(hip, k_a), nk, nkk, kka)
+    hip.device_sync()
+    for got, ref in ((nk, nk_r), (nkk, nkk_r), (kka, kka_r)):
+        assert rel_err(got.numpy().astype(np.float32), ref.astype(np.float32)) <= F16_TOL
+
+    y, r, v, g = rnd(rows, C), rnd(rows, C), rnd(rows, C), rnd(rows, C)
+    r_k, lnw, lnb = rnd(C, s=0.1), rnd(C, s=0.1) + np.float16(1), rnd(C, s=0.1)
+    out_r = orc.lnx_rkvres_xg(y, r, k, v, r_k, lnw, lnb, g, H)
+    out = hip.DeviceArray((rows, C), np.float16)
+    hip.lnx_rkvres_xg(rows, C, H, dev(hip, y), dev(hip, r), dev(hip, k), dev(hip, v), dev(hip, r_k), dev(hip, lnw),
+                      dev(hip, lnb), dev(hip, g), out)
+    hip.device_sync()
+    assert rel_err(out.numpy().astype(np.float32), out_r.astype(np.float32)) <= F16_TOL
+
+    # LoRA pair, each activation, and the v-residual epilogue
+    for R, act in ((64, hip.ACT_TANH), (32, hip.ACT_NONE), (136, hip.ACT_SIGMOID)):
+        x = rnd(rows, C)
+        w1, w2 = rnd(R, C, s=0.05), rnd(C, R, s=0.05)
+        o32 = orc.lora(x, w1, w2, act)
+        h = hip.DeviceArray((rows, R), np.float16)
+        hip.lora_in(rows, C, R, dev(hip, x), dev(hip, w1), h)
+        o = hip.DeviceArray((rows, C), np.float16)
+        hip.lora_out(rows, C, R, act, h, dev(hip, w2), o)
+        hip.device_sync()
+        assert rel_err(o.numpy().astype(np.float32), o32) <= F16_TOL
+        if act == hip.ACT_NONE:
+            v_first, v0 = rnd(rows, C), rnd(C, s=0.3)
+            ref = orc.vres_gate(v, v_first, v0, o32)
+            og = hip.DeviceArray((rows, C), np.float16)
+            hip.lora_out(rows, C, R, act, h, dev(hip, w2), og, bias=dev(hip, v0), vres=1, v=dev(hip, v), v_first=dev(hip, v_first))
+            hip.device_sync()
+            assert rel_err(og.numpy().astype(np.float32), ref.astype(np.float32)) <= F16_TOL
+
+
+def test_small_elementwise(gpu, orc):
+    hip = gpu
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((4, 512)).astype(np.float16)
+    vec = rng.standard_normal(512).astype(np.float16)
+    out = hip.DeviceArray(x.shape, np.float16)
+    hip.relu_square(x.size, dev(hip, x), out)
+    hip.device_sync()
+    assert np.array_equal(out.numpy().view(np.uint16), orc.relu_square(x).view(np.uint16))
+    hip.add_vec(4, 512, dev(hip, x), dev(hip, vec), out)
+    hip.device_sync()
+    assert np.array_equal(out.numpy().view(np.uint16), orc.add_vec(x, vec).view(np.uint16))
+    o32 = hip.DeviceArray(x.shape, np.float32)
+    hip.f16_to_f32(x.size, dev(hip, x), o32)
+    e = dev(hip, np.array([3, 9], np.int32))
+    hip.advance_i32(2, 128, e)
+    hip.device_sync()
+    assert np.array_equal(o32.numpy(), x.astype(np.float32))
+    assert e.numpy().tolist() == [131, 137]
