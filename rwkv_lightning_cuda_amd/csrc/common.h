@@ -62,6 +62,11 @@ __device__ __forceinline__ half_t f2h(float f) { return static_cast<half_t>(f); 
 // value after a round trip through fp16: the rounding point where the reference stores fp16
 __device__ __forceinline__ float round_h(float f) { return static_cast<float>(static_cast<half_t>(f)); }
 
+// Reinterpret a dword as two fp16 values.  Always go through this by-value helper: applying
+// __builtin_bit_cast directly to a vector element (`bit_cast<half2>(vec[i])`) makes this compiler read
+// element 0 for every i.
+__device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
+
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + __expf(-x)); }
 
 // Sum over the 64 lanes of a wave, result in every lane.

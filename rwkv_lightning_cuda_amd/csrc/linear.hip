@@ -31,8 +31,8 @@ __device__ __forceinline__ void cvt_i8x4(uint32_t d, half2_t& lo, half2_t& hi) {
   const uint32_t l = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
   const uint32_t h = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
   const half2_t bias = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
-  lo = __builtin_bit_cast(half2_t, l) - bias;
-  hi = __builtin_bit_cast(half2_t, h) - bias;
+  lo = as_half2(l) - bias;
+  hi = as_half2(h) - bias;
 }
 
 __device__ __forceinline__ float dot2(half2_t a, half2_t b, float c) {
@@ -63,7 +63,7 @@ struct WeightVec<RWKV_FMT_F16> {
   static constexpr int kElems = 8;
   __device__ static __forceinline__ float dot(const uint4_t& wv, const half2_t* x, float acc) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc = dot2(__builtin_bit_cast(half2_t, wv[i]), x[i], acc);
+    for (int i = 0; i < 4; ++i) acc = dot2(as_half2(wv[i]), x[i], acc);
     return acc;
   }
 };
@@ -84,7 +84,7 @@ struct WeightVec<RWKV_FMT_W4> {
         // half2 (element 2j, element 2j+1) = bytes j of `even` and `odd`, each OR 0x6400
         const uint32_t sel = 0x0c040c00u + j * 0x00010001u;
         const uint32_t pk = __builtin_amdgcn_perm(odd, even, sel) | 0x64006400u;
-        acc = dot2(__builtin_bit_cast(half2_t, pk) - bias, x[4 * i + j], acc);
+        acc = dot2(as_half2(pk) - bias, x[4 * i + j], acc);
       }
     }
     return acc;
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
             for (int q = 0; q < 4; ++q) {
               const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KT + k0 + q * 8);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) xv[q * 4 + e] = __builtin_bit_cast(half2_t, t[e]);
+              for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
             }
             float xsum = 0.0f;
             const half2_t ones = {static_cast<half_t>(1.0f), static_cast<half_t>(1.0f)};
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
             for (int q = 0; q < XV / 4; ++q) {
               const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KT + k0 + q * 8);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) xv[q * 4 + e] = __builtin_bit_cast(half2_t, t[e]);
+              for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(wv[r], xv, acc[r][m]);

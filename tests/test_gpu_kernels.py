@@ -34,9 +34,12 @@ def test_wkv7_f32_matches_oracle(gpu, orc, B, T, H, mode):
     hip.wkv7(B, T, C, H, w_mode, hip.IO_F32, state, dev(hip, inp["r"]), dev(hip, w), dev(hip, inp["k"]),
              dev(hip, inp["v"]), dev(hip, inp["a"]), dev(hip, inp["b"]), y)
     hip.device_sync()
-    assert rel_err(y.numpy(), y_ref) <= WKV_TOL
-    assert rel_err(state.numpy(), s_ref) <= WKV_TOL
-    assert elem_err(state.numpy(), s_ref) <= WKV_TOL
+    err = rel_err(y.numpy(), y_ref)
+    assert err <= WKV_TOL
+    err = rel_err(state.numpy(), s_ref)
+    assert err <= WKV_TOL
+    err = elem_err(state.numpy(), s_ref)
+    assert err <= WKV_TOL
 
 
 def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):
@@ -52,8 +55,10 @@ def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):
     y = hip.DeviceArray((B, T, C), np.float16)
     hip.wkv7(B, T, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state, *[d[n] for n in names], y)
     hip.device_sync()
-    assert rel_err(y.numpy().astype(np.float32), y_ref.astype(np.float32)) <= F16_TOL
-    assert rel_err(state.numpy(), s_ref) <= WKV_TOL
+    err = rel_err(y.numpy().astype(np.float32), y_ref.astype(np.float32))
+    assert err <= F16_TOL
+    err = rel_err(state.numpy(), s_ref)
+    assert err <= WKV_TOL
 
     # the same tokens in two calls (T1 + T2): bitwise identical state and outputs
     T1 = 13
@@ -65,8 +70,10 @@ def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):
         hip.wkv7(B, tn, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state2, *[part[n] for n in names], yp)
         hip.device_sync()
         y2[:, t0:t0 + tn] = yp.numpy()
-    assert np.array_equal(state2.numpy().view(np.uint32), state.numpy().view(np.uint32))
-    assert np.array_equal(y2.view(np.uint16), y.numpy().view(np.uint16))
+    same = np.array_equal(state2.numpy().view(np.uint32), state.numpy().view(np.uint32))
+    assert same
+    same = np.array_equal(y2.view(np.uint16), y.numpy().view(np.uint16))
+    assert same
 
 
 # ------------------------------------------------------------------------------------------- formats
@@ -85,9 +92,12 @@ def test_quantize_dequant_bit_exact(gpu, orc):
     out = hip.DeviceArray((N, K), np.float16)
     hip.dequant_w8(N, K, q, s, out)
     hip.device_sync()
-    assert np.array_equal(q.numpy(), q_ref)
-    assert np.array_equal(s.numpy().view(np.uint16), s_ref.view(np.uint16))
-    assert np.array_equal(out.numpy().view(np.uint16), orc.dequant_w8(q_ref, s_ref).view(np.uint16))
+    same = np.array_equal(q.numpy(), q_ref)
+    assert same
+    same = np.array_equal(s.numpy().view(np.uint16), s_ref.view(np.uint16))
+    assert same
+    same = np.array_equal(out.numpy().view(np.uint16), orc.dequant_w8(q_ref, s_ref).view(np.uint16))
+    assert same
 
     q4_ref, s4_ref, z4_ref = orc.quantize_w4(w)
     q4 = hip.DeviceArray((N, K // 2), np.uint8)
@@ -97,10 +107,14 @@ def test_quantize_dequant_bit_exact(gpu, orc):
     out4 = hip.DeviceArray((N, K), np.float16)
     hip.dequant_w4(N, K, q4, s4, z4, out4)
     hip.device_sync()
-    assert np.array_equal(q4.numpy(), q4_ref)
-    assert np.array_equal(s4.numpy().view(np.uint16), s4_ref.view(np.uint16))
-    assert np.array_equal(z4.numpy(), z4_ref)
-    assert np.array_equal(out4.numpy().view(np.uint16), orc.dequant_w4(q4_ref, s4_ref, z4_ref).view(np.uint16))
+    same = np.array_equal(q4.numpy(), q4_ref)
+    assert same
+    same = np.array_equal(s4.numpy().view(np.uint16), s4_ref.view(np.uint16))
+    assert same
+    same = np.array_equal(z4.numpy(), z4_ref)
+    assert same
+    same = np.array_equal(out4.numpy().view(np.uint16), orc.dequant_w4(q4_ref, s4_ref, z4_ref).view(np.uint16))
+    assert same
 
 
 def test_dequant_all_codes_bit_exact(gpu, orc):
@@ -111,7 +125,8 @@ def test_dequant_all_codes_bit_exact(gpu, orc):
     out = hip.DeviceArray(q.shape, np.float16)
     hip.dequant_w8(q.shape[0], q.shape[1], dev(hip, q), dev(hip, scales), out)
     hip.device_sync()
-    assert np.array_equal(out.numpy().view(np.uint16), orc.dequant_w8(q, scales).view(np.uint16))
+    same = np.array_equal(out.numpy().view(np.uint16), orc.dequant_w8(q, scales).view(np.uint16))
+    assert same
 
     rows = []
     zps = []
@@ -126,7 +141,8 @@ def test_dequant_all_codes_bit_exact(gpu, orc):
     out4 = hip.DeviceArray((16, 128), np.float16)
     hip.dequant_w4(16, 128, dev(hip, q4), dev(hip, s4), dev(hip, z4), out4)
     hip.device_sync()
-    assert np.array_equal(out4.numpy().view(np.uint16), orc.dequant_w4(q4, s4, z4).view(np.uint16))
+    same = np.array_equal(out4.numpy().view(np.uint16), orc.dequant_w4(q4, s4, z4).view(np.uint16))
+    assert same
 
 
 # -------------------------------------------------------------------------------------------- linear
@@ -150,7 +166,8 @@ def test_linear_small_m(gpu, orc, fmt_name, M):
     dparts = [dev(hip, p) if p is not None else None for p in parts]
     hip.linear(fmt, M, N, K, dev(hip, x), dparts[0], dparts[1], dparts[2], y)
     hip.device_sync()
-    assert rel_err(y.numpy().astype(np.float32), y_ref.astype(np.float32)) <= F16_TOL
+    err = rel_err(y.numpy().astype(np.float32), y_ref.astype(np.float32))
+    assert err <= F16_TOL
 
 
 @pytest.mark.parametrize("K", [1024, 2560, 4096, 16384])
@@ -168,11 +185,14 @@ def test_linear_w8_relu_square_and_f32_out(gpu, orc, K):
     y32 = hip.DeviceArray((M, N), np.float32)
     hip.linear(hip.FMT_W8, M, N, K, dev(hip, x), dev(hip, q), dev(hip, s), None, y32, out_f32=1)
     hip.device_sync()
-    assert rel_err(y.numpy().astype(np.float32), act_ref.astype(np.float32)) <= 2 * F16_TOL
+    err = rel_err(y.numpy().astype(np.float32), act_ref.astype(np.float32))
+    assert err <= 2 * F16_TOL
     got32 = y32.numpy()
-    assert rel_err(got32, hid.astype(np.float32)) <= F16_TOL
+    err = rel_err(got32, hid.astype(np.float32))
+    assert err <= F16_TOL
     # fp32 logits hold fp16-representable values
-    assert np.array_equal(got32, got32.astype(np.float16).astype(np.float32))
+    same = np.array_equal(got32, got32.astype(np.float16).astype(np.float32))
+    assert same
 
 
 def test_linear_rejects_bad_shapes(gpu):
@@ -207,16 +227,20 @@ def test_layer_norm_family(gpu, orc, C):
     y2 = hip.DeviceArray((rows, C), np.float16)
     hip.add_layer_norm(rows, C, dev(hip, x), dev(hip, res), dev(hip, w), dev(hip, b), xo, y2)
     hip.device_sync()
-    assert rel_err(y.numpy().astype(np.float32), orc.layer_norm(x, w, b).astype(np.float32)) <= F16_TOL
+    err = rel_err(y.numpy().astype(np.float32), orc.layer_norm(x, w, b).astype(np.float32))
+    assert err <= F16_TOL
     xo_ref, y2_ref = orc.add_layer_norm(x, res, w, b)
-    assert np.array_equal(xo.numpy().view(np.uint16), xo_ref.view(np.uint16))
-    assert rel_err(y2.numpy().astype(np.float32), y2_ref.astype(np.float32)) <= F16_TOL
+    same = np.array_equal(xo.numpy().view(np.uint16), xo_ref.view(np.uint16))
+    assert same
+    err = rel_err(y2.numpy().astype(np.float32), y2_ref.astype(np.float32))
+    assert err <= F16_TOL
 
     # add + last-token LN (B=1, T=rows)
     yl = hip.DeviceArray((1, C), np.float16)
     hip.add_last_layer_norm(1, rows, C, dev(hip, x), dev(hip, res), dev(hip, w), dev(hip, b), yl)
     hip.device_sync()
-    assert rel_err(yl.numpy().astype(np.float32), orc.add_last_layer_norm(x, res, w, b, 1, rows).astype(np.float32)) <= F16_TOL
+    err = rel_err(yl.numpy().astype(np.float32), orc.add_last_layer_norm(x, res, w, b, 1, rows).astype(np.float32))
+    assert err <= F16_TOL
 
     # add + LN + cmix lerp + shift write (T == 1 fusion)
     c = np.arange(C)
@@ -228,9 +252,12 @@ def test_layer_norm_family(gpu, orc, C):
     mixed = hip.DeviceArray((rows, C), np.float16)
     hip.add_layer_norm_cmix_mix(rows, C, dev(hip, x), dev(hip, res), shd, dev(hip, w), dev(hip, b), dev(hip, mu), xo3, mixed)
     hip.device_sync()
-    assert np.array_equal(xo3.numpy().view(np.uint16), xo_r.view(np.uint16))
-    assert rel_err(mixed.numpy().astype(np.float32), mixed_r.astype(np.float32)) <= F16_TOL
-    assert rel_err(shd.numpy().astype(np.float32), sh_ref.astype(np.float32)) <= F16_TOL
+    same = np.array_equal(xo3.numpy().view(np.uint16), xo_r.view(np.uint16))
+    assert same
+    err = rel_err(mixed.numpy().astype(np.float32), mixed_r.astype(np.float32))
+    assert err <= F16_TOL
+    err = rel_err(shd.numpy().astype(np.float32), sh_ref.astype(np.float32))
+    assert err <= F16_TOL
 
     # add + LN + six lerps
     mus = [pattern_value(c + o, s, bb).astype(np.float16) for o, s, bb in
@@ -243,8 +270,10 @@ def test_layer_norm_family(gpu, orc, C):
                                  [dev(hip, m) for m in mus], xo3, outs)
     hip.device_sync()
     for o, o_r in zip(outs, outs_r):
-        assert rel_err(o.numpy().astype(np.float32), o_r.astype(np.float32)) <= F16_TOL
-    assert rel_err(shd.numpy().astype(np.float32), sh_ref.astype(np.float32)) <= F16_TOL
+        err = rel_err(o.numpy().astype(np.float32), o_r.astype(np.float32))
+        assert err <= F16_TOL
+    err = rel_err(shd.numpy().astype(np.float32), sh_ref.astype(np.float32))
+    assert err <= F16_TOL
 
 
 @pytest.mark.parametrize("B,T", [(1, 1), (2, 5), (3, 1)])
@@ -262,8 +291,10 @@ def test_token_shift_mix(gpu, orc, B, T):
     hip.token_shift_mix(B, T, C, dev(hip, x), shd, [dev(hip, m) for m in mus], outs)
     hip.device_sync()
     for o, o_r in zip(outs, outs_r):
-        assert rel_err(o.numpy().astype(np.float32), o_r.astype(np.float32)) <= F16_TOL
-    assert np.array_equal(shd.numpy().view(np.uint16), sh_ref.view(np.uint16))
+        err = rel_err(o.numpy().astype(np.float32), o_r.astype(np.float32))
+        assert err <= F16_TOL
+    same = np.array_equal(shd.numpy().view(np.uint16), sh_ref.view(np.uint16))
+    assert same
 
 
 def test_kk_gate_groupnorm_lora(gpu, orc):
@@ -282,7 +313,8 @@ def test_kk_gate_groupnorm_lora(gpu, orc):
     hip.kk_a_gate(rows, C, H, dev(hip, k), dev(hip, k_k), dev(hip, a0), dev(hip, a12), dev(hip, k_a), nk, nkk, kka)
     hip.device_sync()
     for got, ref in ((nk, nk_r), (nkk, nkk_r), (kka, kka_r)):
-        assert rel_err(got.numpy().astype(np.float32), ref.astype(np.float32)) <= F16_TOL
+        err = rel_err(got.numpy().astype(np.float32), ref.astype(np.float32))
+        assert err <= F16_TOL
 
     y, r, v, g = rnd(rows, C), rnd(rows, C), rnd(rows, C), rnd(rows, C)
     r_k, lnw, lnb = rnd(C, s=0.1), rnd(C, s=0.1) + np.float16(1), rnd(C, s=0.1)
@@ -291,7 +323,8 @@ def test_kk_gate_groupnorm_lora(gpu, orc):
     hip.lnx_rkvres_xg(rows, C, H, dev(hip, y), dev(hip, r), dev(hip, k), dev(hip, v), dev(hip, r_k), dev(hip, lnw),
                       dev(hip, lnb), dev(hip, g), out)
     hip.device_sync()
-    assert rel_err(out.numpy().astype(np.float32), out_r.astype(np.float32)) <= F16_TOL
+    err = rel_err(out.numpy().astype(np.float32), out_r.astype(np.float32))
+    assert err <= F16_TOL
 
     # LoRA pair, each activation, and the v-residual epilogue
     for R, act in ((64, hip.ACT_TANH), (32, hip.ACT_NONE), (136, hip.ACT_SIGMOID)):
@@ -303,14 +336,16 @@ def test_kk_gate_groupnorm_lora(gpu, orc):
         o = hip.DeviceArray((rows, C), np.float16)
         hip.lora_out(rows, C, R, act, h, dev(hip, w2), o)
         hip.device_sync()
-        assert rel_err(o.numpy().astype(np.float32), o32) <= F16_TOL
+        err = rel_err(o.numpy().astype(np.float32), o32)
+        assert err <= F16_TOL
         if act == hip.ACT_NONE:
             v_first, v0 = rnd(rows, C), rnd(C, s=0.3)
             ref = orc.vres_gate(v, v_first, v0, o32)
             og = hip.DeviceArray((rows, C), np.float16)
             hip.lora_out(rows, C, R, act, h, dev(hip, w2), og, bias=dev(hip, v0), vres=1, v=dev(hip, v), v_first=dev(hip, v_first))
             hip.device_sync()
-            assert rel_err(og.numpy().astype(np.float32), ref.astype(np.float32)) <= F16_TOL
+            err = rel_err(og.numpy().astype(np.float32), ref.astype(np.float32))
+            assert err <= F16_TOL
 
 
 def test_small_elementwise(gpu, orc):
@@ -321,14 +356,17 @@ def test_small_elementwise(gpu, orc):
     out = hip.DeviceArray(x.shape, np.float16)
     hip.relu_square(x.size, dev(hip, x), out)
     hip.device_sync()
-    assert np.array_equal(out.numpy().view(np.uint16), orc.relu_square(x).view(np.uint16))
+    same = np.array_equal(out.numpy().view(np.uint16), orc.relu_square(x).view(np.uint16))
+    assert same
     hip.add_vec(4, 512, dev(hip, x), dev(hip, vec), out)
     hip.device_sync()
-    assert np.array_equal(out.numpy().view(np.uint16), orc.add_vec(x, vec).view(np.uint16))
+    same = np.array_equal(out.numpy().view(np.uint16), orc.add_vec(x, vec).view(np.uint16))
+    assert same
     o32 = hip.DeviceArray(x.shape, np.float32)
     hip.f16_to_f32(x.size, dev(hip, x), o32)
     e = dev(hip, np.array([3, 9], np.int32))
     hip.advance_i32(2, 128, e)
     hip.device_sync()
-    assert np.array_equal(o32.numpy(), x.astype(np.float32))
+    same = np.array_equal(o32.numpy(), x.astype(np.float32))
+    assert same
     assert e.numpy().tolist() == [131, 137]
