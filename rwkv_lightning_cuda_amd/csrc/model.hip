@@ -93,6 +93,8 @@ struct rwkv_hip_session {
   half_t* trace = nullptr;
   std::vector<GraphEntry> graphs;
   uint64_t tick = 0;
+  bool profile = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;
 };
 
 namespace {
@@ -210,6 +212,23 @@ int apply_matrix(hipStream_t st, const Matrix& mat, int M, int N, int K, const h
     if (rc__ != RWKV_OK) return rc__; \
   } while (0)
 
+// Profiling mode: bracket a weight-streaming linear launch with a pair of events on the session stream.
+#define TRY_PROF(expr)                                              \
+  do {                                                              \
+    hipEvent_t e0__ = nullptr, e1__ = nullptr;                      \
+    if (s->profile) {                                               \
+      RWKV_HIP_TRY(hipEventCreate(&e0__));                          \
+      RWKV_HIP_TRY(hipEventCreate(&e1__));                          \
+      RWKV_HIP_TRY(hipEventRecord(e0__, st));                       \
+    }                                                               \
+    const int rc__ = (expr);                                        \
+    if (s->profile) {                                               \
+      RWKV_HIP_TRY(hipEventRecord(e1__, st));                       \
+      s->prof_events.push_back(std::make_pair(e0__, e1__));         \
+    }                                                               \
+    if (rc__ != RWKV_OK) return rc__;                               \
+  } while (0)
+
 // Enqueues the whole forward pass on the session stream.  tokens are already in s->tokens_dev.
 int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv, int* elapsed, float* logits) {
   const rwkv_hip_model* m = s->model;
@@ -277,11 +296,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         p[i].w = w.m[mids[i]].data; p[i].scale = w.m[mids[i]].scale; p[i].zp = w.m[mids[i]].zp;
         p[i].x = xs[i]; p[i].y = ys[i]; p[i].N = C;
       }
-      TRY(linear_small_m(st, w.m[RWKV_M_ATT_R].fmt, rows, C, 3, p, RWKV_EPI_NONE, 0));
+      TRY_PROF(linear_small_m(st, w.m[RWKV_M_ATT_R].fmt, rows, C, 3, p, RWKV_EPI_NONE, 0));
     } else {
-      TRY(apply_matrix(st, w.m[RWKV_M_ATT_R], rows, C, C, b.xr, RWKV_EPI_NONE, 0, b.r));
-      TRY(apply_matrix(st, w.m[RWKV_M_ATT_K], rows, C, C, b.xk, RWKV_EPI_NONE, 0, b.k));
-      TRY(apply_matrix(st, w.m[RWKV_M_ATT_V], rows, C, C, b.xv, RWKV_EPI_NONE, 0, v_cur));
+      TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_R], rows, C, C, b.xr, RWKV_EPI_NONE, 0, b.r));
+      TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_K], rows, C, C, b.xk, RWKV_EPI_NONE, 0, b.k));
+      TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_V], rows, C, C, b.xv, RWKV_EPI_NONE, 0, v_cur));
     }
 
     // LoRA rank-in (w, a, g and, past layer 0, v)
@@ -336,7 +355,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
                             b.y, static_cast<int64_t>(T) * C));
     TRY(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
                    w.t[RWKV_T_LNX_B], b.g, b.y2));
-    TRY(apply_matrix(st, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
+    TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
 
     // residual add + LN2 + channel-mix token shift
     if (step) {
@@ -356,8 +375,8 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     }
 
     // channel mix
-    TRY(apply_matrix(st, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
-    TRY(apply_matrix(st, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+    TRY_PROF(apply_matrix(st, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
+    TRY_PROF(apply_matrix(st, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
 
     // residual add + next layer's LN1 (+ lerps), or the final LN on the last token of each row
     if (l + 1 < L) {
@@ -391,7 +410,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   }
 
   TRY(advance_launch(st, B, T, elapsed));
-  TRY(apply_matrix(st, m->head, B, V, C, b.xf, RWKV_EPI_NONE, 1, logits));
+  TRY_PROF(apply_matrix(st, m->head, B, V, C, b.xf, RWKV_EPI_NONE, 1, logits));
   return RWKV_OK;
 }
 
@@ -404,7 +423,7 @@ GraphEntry* find_graph(rwkv_hip_session* s, int B, void* shift, void* wkv, void*
 
 // T == 1 step through a captured graph (captures on first use of this (B, state, logits) tuple).
 int run_step(rwkv_hip_session* s, int B, half_t* shift, float* wkv, int* elapsed, float* logits) {
-  if (!s->use_graph || s->trace) return enqueue_forward(s, B, 1, shift, wkv, elapsed, logits);
+  if (!s->use_graph || s->trace || s->profile) return enqueue_forward(s, B, 1, shift, wkv, elapsed, logits);
   GraphEntry* g = find_graph(s, B, shift, wkv, elapsed, logits);
   if (!g) {
     if (s->graphs.size() >= kMaxGraphs) {
@@ -596,6 +615,29 @@ int rwkv_hip_session_stream(rwkv_hip_session* s, rwkv_stream_t* stream) {
 int rwkv_hip_session_set_graph(rwkv_hip_session* s, int use_graph) {
   RWKV_REQUIRE(s, "session is NULL");
   s->use_graph = use_graph != 0;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_set_profile(rwkv_hip_session* s, int on) {
+  RWKV_REQUIRE(s, "session is NULL");
+  s->profile = on != 0;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double* total_ms) {
+  RWKV_REQUIRE(s && launches && total_ms, "read_profile: NULL argument");
+  RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+  double ms = 0.0;
+  for (auto& pr : s->prof_events) {
+    float t = 0.0f;
+    RWKV_HIP_TRY(hipEventElapsedTime(&t, pr.first, pr.second));
+    ms += t;
+    (void)hipEventDestroy(pr.first);
+    (void)hipEventDestroy(pr.second);
+  }
+  *launches = static_cast<int64_t>(s->prof_events.size());
+  *total_ms = ms;
+  s->prof_events.clear();
   return RWKV_OK;
 }
 

@@ -250,6 +250,15 @@ class Session:
         self._trace = dev
         hip.check(hip.load().rwkv_hip_session_set_trace(self.handle, hip._p(dev)))
 
+    def set_profile(self, on):
+        hip.check(hip.load().rwkv_hip_session_set_profile(self.handle, ctypes.c_int(1 if on else 0)))
+
+    def read_profile(self):
+        """(launches, total_ms) of the event-bracketed linear launches since the last read."""
+        n, ms = ctypes.c_int64(0), ctypes.c_double(0)
+        hip.check(hip.load().rwkv_hip_session_read_profile(self.handle, ctypes.byref(n), ctypes.byref(ms)))
+        return n.value, ms.value
+
     def forward(self, tokens, state, logits, sync=True):
         """tokens: int array [B,T].  Updates state in place, writes logits f32 [B,V] (last token per row)."""
         tokens = np.ascontiguousarray(tokens, dtype=np.int64)
