@@ -34,6 +34,7 @@ def parse_args():
     ap.add_argument("--fmt", default="w8", choices=["f16", "w8", "w4"])
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--prefill", type=int, default=64, help="tokens prefilled (chunk 128) before the decode loop")
+    ap.add_argument("--no-graph", action="store_true", help="launch decode steps eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     return ap.parse_args()
@@ -114,6 +115,8 @@ def main():
 
     model = HipModel.random_on_device(dims, fmt, seed=1)
     sess = Session(model)
+    if args.no_graph:
+        sess.set_graph(False)
     state = State(dims, B)
     logits = hip.DeviceArray((B, dims.V), np.float32)
     rng = np.random.default_rng(0)
@@ -151,7 +154,7 @@ def main():
         "config": {"workload": "RWKV-7 %s-shape greedy decode, batch %d, %d-token prefill, lm_head+argmax on device"
                                % (args.preset, B, args.prefill),
                    "L": dims.L, "C": dims.C, "H": dims.H, "F": dims.F, "V": dims.V,
-                   "weight_format": args.fmt, "weight_bytes_per_step": weight_bytes,
+                   "weight_format": args.fmt, "hip_graph": not args.no_graph, "weight_bytes_per_step": weight_bytes,
                    "state_bytes_per_step": state_bytes,
                    "step_hbm_fraction": (weight_bytes + state_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                    "distinct_tokens": int(len(np.unique(toks)))},
