@@ -323,38 +323,51 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
                            0, hs[i]));
       }
     }
-    // LoRA rank-out (+ activation, + v-residual gate)
-    {
-      LoraOutArgs a = {};
-      a.M = rows; a.C = C;
-      a.h = b.hw; a.w2 = w.t[RWKV_T_W2]; a.R = m->Rw; a.act = RWKV_ACT_TANH; a.out = b.w12;
-      TRY(lora_out_launch(st, a));
-      a.h = b.ha; a.w2 = w.t[RWKV_T_A2]; a.R = m->Ra; a.act = RWKV_ACT_NONE; a.out = b.a12;
-      TRY(lora_out_launch(st, a));
-      a.h = b.hg; a.w2 = w.t[RWKV_T_G2]; a.R = m->Rg; a.act = RWKV_ACT_SIGMOID; a.out = b.g;
-      TRY(lora_out_launch(st, a));
-      if (l > 0) {
-        a.h = b.hv; a.w2 = w.t[RWKV_T_V2]; a.R = m->Rv; a.act = RWKV_ACT_NONE; a.bias = w.t[RWKV_T_V0];
-        a.vres = 1; a.v = b.v; a.v_first = b.v_first; a.out = b.xv;  // xv is free after the projections
+    if (step) {
+      // the whole time-mix core of a decode step in one launch per layer
+      TmixStepArgs p = {};
+      p.B = B; p.H = H; p.C = C; p.Rw = m->Rw; p.Ra = m->Ra; p.Rg = m->Rg; p.Rv = m->Rv;
+      p.hw = b.hw; p.ha = b.ha; p.hg = b.hg; p.hv = (l > 0) ? b.hv : nullptr;
+      p.w2 = w.t[RWKV_T_W2]; p.a2 = w.t[RWKV_T_A2]; p.g2 = w.t[RWKV_T_G2]; p.v2 = w.t[RWKV_T_V2];
+      p.w0 = w.t[RWKV_T_W0]; p.a0 = w.t[RWKV_T_A0]; p.v0 = w.t[RWKV_T_V0]; p.k_k = w.t[RWKV_T_K_K];
+      p.k_a = w.t[RWKV_T_K_A]; p.r_k = w.t[RWKV_T_R_K]; p.lnx_w = w.t[RWKV_T_LNX_W]; p.lnx_b = w.t[RWKV_T_LNX_B];
+      p.r = b.r; p.k = b.k; p.v = v_cur; p.v_first = b.v_first; p.v_first_out = nullptr;
+      p.state = S; p.y2 = b.y2;
+      TRY(tmix_step_launch(st, p));
+    } else {
+      // LoRA rank-out (+ activation, + v-residual gate)
+      {
+        LoraOutArgs a = {};
+        a.M = rows; a.C = C;
+        a.h = b.hw; a.w2 = w.t[RWKV_T_W2]; a.R = m->Rw; a.act = RWKV_ACT_TANH; a.out = b.w12;
         TRY(lora_out_launch(st, a));
-        v_cur = b.xv;
+        a.h = b.ha; a.w2 = w.t[RWKV_T_A2]; a.R = m->Ra; a.act = RWKV_ACT_NONE; a.out = b.a12;
+        TRY(lora_out_launch(st, a));
+        a.h = b.hg; a.w2 = w.t[RWKV_T_G2]; a.R = m->Rg; a.act = RWKV_ACT_SIGMOID; a.out = b.g;
+        TRY(lora_out_launch(st, a));
+        if (l > 0) {
+          a.h = b.hv; a.w2 = w.t[RWKV_T_V2]; a.R = m->Rv; a.act = RWKV_ACT_NONE; a.bias = w.t[RWKV_T_V0];
+          a.vres = 1; a.v = b.v; a.v_first = b.v_first; a.out = b.xv;  // xv is free after the projections
+          TRY(lora_out_launch(st, a));
+          v_cur = b.xv;
+        }
       }
-    }
 
-    // kk normalise, a-gate, decay; operands widened to fp32 for the scalar-fed WKV kernel
-    {
-      KkArgs p = {};
-      p.k = b.k; p.k_k = w.t[RWKV_T_K_K]; p.a0 = w.t[RWKV_T_A0]; p.a12 = b.a12; p.k_a = w.t[RWKV_T_K_A];
-      p.new_k = b.k2; p.neg_kk = nullptr; p.kka = nullptr;
-      p.w12 = b.w12; p.w0 = w.t[RWKV_T_W0]; p.r = b.r;
-      p.k32 = b.k32; p.a32 = b.a32; p.b32 = b.b32; p.d32 = b.d32; p.r32 = b.r32;
-      p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
-      TRY(kk_a_gate_launch(st, p));
+      // kk normalise, a-gate, decay; operands widened to fp32 for the scalar-fed WKV kernel
+      {
+        KkArgs p = {};
+        p.k = b.k; p.k_k = w.t[RWKV_T_K_K]; p.a0 = w.t[RWKV_T_A0]; p.a12 = b.a12; p.k_a = w.t[RWKV_T_K_A];
+        p.new_k = b.k2; p.neg_kk = nullptr; p.kka = nullptr;
+        p.w12 = b.w12; p.w0 = w.t[RWKV_T_W0]; p.r = b.r;
+        p.k32 = b.k32; p.a32 = b.a32; p.b32 = b.b32; p.d32 = b.d32; p.r32 = b.r32;
+        p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
+        TRY(kk_a_gate_launch(st, p));
+      }
+      TRY(wkv7_seq_f16_launch(st, B, T, C, H, S, b.r32, b.d32, b.k32, b.a32, b.b32, static_cast<int64_t>(T) * C, v_cur,
+                              b.y, static_cast<int64_t>(T) * C));
+      TRY(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
+                     w.t[RWKV_T_LNX_B], b.g, b.y2));
     }
-    TRY(wkv7_seq_f16_launch(st, B, T, C, H, S, b.r32, b.d32, b.k32, b.a32, b.b32, static_cast<int64_t>(T) * C, v_cur,
-                            b.y, static_cast<int64_t>(T) * C));
-    TRY(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
-                   w.t[RWKV_T_LNX_B], b.g, b.y2));
     TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
 
     // residual add + LN2 + channel-mix token shift

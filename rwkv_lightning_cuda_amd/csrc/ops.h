@@ -116,3 +116,21 @@ int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state
                         int64_t io_bs);
 
 }  // namespace rwkv
+
+namespace rwkv {
+
+// ---- tmix_step.hip: the whole time-mix core of a decode step, one workgroup per (batch row, head) ----
+struct TmixStepArgs {
+  int B, H, C, Rw, Ra, Rg, Rv;
+  const half_t *hw, *ha, *hg, *hv;          // LoRA hidden vectors [B,R]; hv == NULL on layer 0
+  const half_t *w2, *a2, *g2, *v2;          // LoRA rank-out matrices [C,R]
+  const half_t *w0, *a0, *v0, *k_k, *k_a, *r_k, *lnx_w, *lnx_b;
+  const half_t *r, *k, *v;                  // projections [B,C]
+  const half_t* v_first;                    // [B,C], read when hv != NULL
+  half_t* v_first_out;                      // [B,C], written when hv == NULL (layer 0), may be NULL
+  float* state;                             // [B,H,64,64], updated in place
+  half_t* y2;                               // [B,C] input of the output projection
+};
+int tmix_step_launch(hipStream_t st, const TmixStepArgs& p);
+
+}  // namespace rwkv
