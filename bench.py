@@ -42,7 +42,8 @@ def parse_args():
 
 def gemv_bytes_per_step(dims, fmt):
     """Algorithmic bytes the weight-streaming linear launches move per decode step: every code of the seven
-    big matrices once + their scales (+ zero points), + x in and y out (fp16).  Returns (bytes, launches)."""
+    big matrices once + their scales (+ zero points), the fp16 LoRA rank-in matrices that share the r/k/v launch,
+    + x in and y out (fp16).  Returns (bytes, launches)."""
     C, F, V, L = dims.C, dims.F, dims.V, dims.L
 
     def mat(N, K):
@@ -54,9 +55,16 @@ def gemv_bytes_per_step(dims, fmt):
             w = 2 * N * K
         return w + 2 * K + 2 * N
 
-    per_layer = 3 * mat(C, C) + mat(C, C) + mat(F, C) + mat(C, F)   # fused r/k/v launch, output, ffn.key, ffn.value
+    def lora_in(l):
+        ranks = dims.Rw + dims.Ra + dims.Rg + (dims.Rv if l > 0 else 0)
+        return 2 * C * ranks + 2 * ranks + (3 if l > 0 else 3) * 2 * C  # fp16 [R,C] rows, hidden out, x_w/x_a/x_g in
+
+    total = mat(V, C)
+    for l in range(L):
+        # launch 1: r/k/v + the LoRA rank-ins (one launch); 2: output; 3: ffn.key; 4: ffn.value
+        total += 3 * mat(C, C) + lora_in(l) + mat(C, C) + mat(F, C) + mat(C, F)
     launches = 4 * L + 1
-    return L * per_layer + mat(V, C), launches
+    return total, launches
 
 
 def cpu_baseline(dims, fmt_name):

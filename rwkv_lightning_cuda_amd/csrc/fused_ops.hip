@@ -32,18 +32,31 @@ __global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
   }
   const int64_t dst = static_cast<int64_t>(row) * C;
 
+  // every global load of the kernel is issued here, before the first reduction, so the block pays one
+  // memory round trip instead of three
   float v[kLnMaxVec][8];
+  half8_t wv[kLnMaxVec], bv[kLnMaxVec], pv[kLnMaxVec], mv[kLnMaxVec][6];
+  constexpr bool kMix = (MODE == kAddLnMix || MODE == kLnMix);
   float sum = 0.0f;
 #pragma unroll
   for (int i = 0; i < kLnMaxVec; ++i) {
     const int c = (i * kLnThreads + threadIdx.x) * 8;
     if (c < C) {
       const half8_t xv = *reinterpret_cast<const half8_t*>(a.x + xsrc + c);
+      half8_t rv = {};
+      if constexpr (MODE != kLn && MODE != kLnMix) rv = *reinterpret_cast<const half8_t*>(a.res + src + c);
+      wv[i] = *reinterpret_cast<const half8_t*>(a.w + c);
+      bv[i] = *reinterpret_cast<const half8_t*>(a.b + c);
+      if constexpr (kMix) {
+        pv[i] = *reinterpret_cast<const half8_t*>(a.shift + dst + c);
+#pragma unroll
+        for (int s = 0; s < 6; ++s)
+          if (s < a.n_mix) mv[i][s] = *reinterpret_cast<const half8_t*>(a.mu[s] + c);
+      }
       if constexpr (MODE == kLn || MODE == kLnMix) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[i][e] = h2f(xv[e]);
       } else {
-        const half8_t rv = *reinterpret_cast<const half8_t*>(a.res + src + c);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[i][e] = h2f(xv[e]) + h2f(rv[e]);
       }
@@ -72,11 +85,9 @@ __global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
   for (int i = 0; i < kLnMaxVec; ++i) {
     const int c = (i * kLnThreads + threadIdx.x) * 8;
     if (c < C) {
-      const half8_t wv = *reinterpret_cast<const half8_t*>(a.w + c);
-      const half8_t bv = *reinterpret_cast<const half8_t*>(a.b + c);
       half8_t yv;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) yv[e] = f2h((v[i][e] - mean) * rstd * h2f(wv[e]) + h2f(bv[e]));
+      for (int e = 0; e < 8; ++e) yv[e] = f2h((v[i][e] - mean) * rstd * h2f(wv[i][e]) + h2f(bv[i][e]));
       if constexpr (MODE == kAddLn || MODE == kAddLnMix) {
         half8_t xo;
 #pragma unroll
@@ -91,18 +102,19 @@ __global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
           *reinterpret_cast<half8_t*>(a.x_out + dst + c) = xo;
         }
       }
-      if constexpr (MODE == kAddLnMix || MODE == kLnMix) {
+      if constexpr (kMix) {
         // lerps read the fp16-rounded LN output (rwkv7_v3a_ops.cu:1978-1983)
-        const half8_t pv = *reinterpret_cast<const half8_t*>(a.shift + dst + c);
-        for (int s = 0; s < a.n_mix; ++s) {
-          const half8_t mv = *reinterpret_cast<const half8_t*>(a.mu[s] + c);
-          half8_t ov;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float yf = h2f(yv[e]);
-            ov[e] = f2h(yf + (h2f(pv[e]) - yf) * h2f(mv[e]));
+        for (int s = 0; s < 6; ++s) {
+          if (s < a.n_mix) {
+            half8_t ov;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float yf = h2f(yv[e]);
+              ov[e] = f2h(yf + (h2f(pv[i][e]) - yf) * h2f(mv[i][s][e]));
+            }
+            *reinterpret_cast<half8_t*>(a.out[s] + dst + c) = ov;
           }
-          *reinterpret_cast<half8_t*>(a.out[s] + dst + c) = ov;
         }
         *reinterpret_cast<half8_t*>(a.shift + dst + c) = yv;
         if (a.y) *reinterpret_cast<half8_t*>(a.y + dst + c) = yv;

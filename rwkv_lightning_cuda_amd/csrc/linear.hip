@@ -3,23 +3,28 @@
 //
 // Reference: cuda/rwkv7_v3a_ops.cu:464-560 (linear_orig_row1_exact_f16_kernel: one block per two
 // output rows, half2 loads, fp32 accumulate) and the rows 2-4 family :369-462,562-683; dispatch in
-// src/rwkv7_fast_v4.cu:709-959.
+// src/rwkv7_fast_v4.cu:709-959; the fused LoRA rank-in launches :813-940.
 //
 // gfx950 design: the work is HBM-bound, so each lane streams 16-byte weight vectors (global_load_dwordx4)
-// with many loads in flight, x is staged once per block in LDS (re-read by every row), integer codes
-// are expanded to fp16 in registers (v_perm_b32 + one packed fp16 add, exact) and accumulated against
-// x with v_dot2_f32_f16 in fp32.  The per-row (W8) or per-128-group (W4) scale is applied to the fp32
-// partial sums, so no dequantised weight is ever rounded to fp16.  One wavefront owns R output rows
-// over the whole K range: no atomics, no cross-wave reduction, deterministic summation order.
+// and a wavefront keeps R*U of them in flight per lane (R output rows x U steps along K), double-buffered
+// in registers so the next batch is requested before the current one is consumed.  The first batch is
+// requested before x is staged in LDS, so the two latencies overlap.  Integer codes are expanded to fp16
+// in registers (v_perm_b32 + one packed fp16 subtract, exact) and accumulated against x with
+// v_dot2_f32_f16 in fp32.  The per-row (W8) or per-128-group (W4) scale is applied to the fp32 partial
+// sums, so no dequantised weight is ever rounded to fp16.  One wavefront owns R output rows over the whole
+// K range: no atomics, no cross-wave reduction, deterministic summation order.  Up to eight problems
+// that share x-length K (r/k/v and the four LoRA rank-ins of a layer, in different weight formats) go out
+// as one launch over a flattened block range.
 #include "ops.h"
 
 namespace rwkv {
 
-
 struct LinearArgs {
   LinearProblem p[kMaxProblems];
+  int block_end[kMaxProblems];  // exclusive prefix of blocks per problem
+  int n_problems;
   int K;
-  int KT;        // K tile staged in LDS (multiple of the per-wave K step)
+  int KT;  // K tile staged in LDS (>= K when the whole x fits)
   int epilogue;
   int out_f32;
 };
@@ -76,8 +81,8 @@ struct WeightVec<RWKV_FMT_W4> {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t d = wv[i];
-      const uint32_t even = d & 0x0f0f0f0fu;          // elements 0,2,4,6 of this dword
-      const uint32_t odd = (d >> 4) & 0x0f0f0f0fu;    // elements 1,3,5,7
+      const uint32_t even = d & 0x0f0f0f0fu;        // elements 0,2,4,6 of this dword
+      const uint32_t odd = (d >> 4) & 0x0f0f0f0fu;  // elements 1,3,5,7
       const half2_t bias = {static_cast<half_t>(1024.0f), static_cast<half_t>(1024.0f)};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -91,26 +96,92 @@ struct WeightVec<RWKV_FMT_W4> {
   }
 };
 
-// grid = (ceil(maxN / (4*R)), n_problems); block = 256 (4 waves); dynamic LDS = M*KT*2 bytes.
-template <int FMT, int M, int R>
-__global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
-  extern __shared__ __align__(16) unsigned char lds_raw[];
-  half_t* xs = reinterpret_cast<half_t*>(lds_raw);
+template <int FMT>
+struct FmtTraits {
+  static constexpr int kElems = WeightVec<FMT>::kElems;
+  static constexpr int kStep = 64 * kElems;  // K covered by one wave-wide load
+  // byte offset of element k within a row
+  __device__ static __forceinline__ int64_t byte_off(int64_t k) {
+    return FMT == RWKV_FMT_F16 ? k * 2 : (FMT == RWKV_FMT_W8 ? k : k / 2);
+  }
+};
 
-  constexpr int E = WeightVec<FMT>::kElems;      // weights per lane per load
-  constexpr int kStep = 64 * E;                  // K covered by one wave-wide load
-  constexpr int kBytesPerRowNum = (FMT == RWKV_FMT_F16) ? 4 : (FMT == RWKV_FMT_W8 ? 2 : 1);  // bytes*2 per weight
+// One wave: R rows of `prob`, K range [k_lo, k_lo + kn) whose x lives in LDS at xs[m*KT + k - k_lo].
+template <int FMT, int M, int R, int U>
+struct WaveGemv {
+  using T = FmtTraits<FMT>;
 
-  const LinearProblem prob = args.p[blockIdx.y];
+  __device__ static __forceinline__ void load_batch(uint4_t (&w)[U][R], const unsigned char* wbase, int64_t row_bytes,
+                                                    int k_lo, int kn, int step0, int lane) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k0 = (step0 + u) * T::kStep + lane * T::kElems;
+      if (k0 < kn) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          w[u][r] = *reinterpret_cast<const uint4_t*>(wbase + r * row_bytes + T::byte_off(k_lo + k0));
+      }
+    }
+  }
+
+  __device__ static __forceinline__ void compute_batch(float (&acc)[R][M], const uint4_t (&w)[U][R], const half_t* xs,
+                                                       int KT, int k_lo, int kn, int step0, int lane,
+                                                       const LinearProblem& prob, int row0, int K) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k0 = (step0 + u) * T::kStep + lane * T::kElems;
+      if (k0 < kn) {
+        constexpr int XV = T::kElems / 2;  // half2 per lane per m
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          half2_t xv[XV];
+#pragma unroll
+          for (int q = 0; q < XV / 4; ++q) {
+            const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KT + k0 + q * 8);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
+          }
+          if constexpr (FMT == RWKV_FMT_W4) {
+            // 32 codes per lane all lie in one 128-group: scale and zero point are per (row, group)
+            const int g = (k_lo + k0) >> 7;
+            const int G = K >> 7;
+            float xsum = 0.0f;
+            const half2_t ones = {static_cast<half_t>(1.0f), static_cast<half_t>(1.0f)};
+#pragma unroll
+            for (int e = 0; e < XV; ++e) xsum = dot2(xv[e], ones, xsum);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const int64_t gi = static_cast<int64_t>(row0 + r) * G + g;
+              const float sc = h2f(prob.scale[gi]);
+              const float z = static_cast<float>(prob.zp[gi]);
+              const float part = WeightVec<FMT>::dot(w[u][r], xv, 0.0f) - z * xsum;
+              acc[r][m] = fmaf(part, sc, acc[r][m]);
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(w[u][r], xv, acc[r][m]);
+          }
+        }
+      }
+    }
+  }
+};
+
+template <int FMT, int M, int R, int U>
+__device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearProblem& prob, int block_in_problem,
+                                           half_t* xs) {
+  using T = FmtTraits<FMT>;
+  using W = WaveGemv<FMT, M, R, U>;
   const int K = args.K;
   const int KT = args.KT;
   const int N = prob.N;
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-  const int row0 = (blockIdx.x * 4 + wave) * R;
+  const int row0 = (block_in_problem * 4 + wave) * R;
   const bool active = row0 < N;
-  const int64_t row_bytes = static_cast<int64_t>(K) * kBytesPerRowNum / 2;
-  const unsigned char* wbase = static_cast<const unsigned char*>(prob.w) + static_cast<int64_t>(row0) * row_bytes;
+  const int64_t row_bytes = T::byte_off(K);
+  const unsigned char* wbase =
+      static_cast<const unsigned char*>(prob.w) + static_cast<int64_t>(active ? row0 : 0) * row_bytes;
 
   float acc[R][M];
 #pragma unroll
@@ -118,8 +189,12 @@ __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
 
+  uint4_t wa[U][R], wb[U][R];
   for (int kt = 0; kt < K; kt += KT) {
     const int kn = min(KT, K - kt);
+    const int nsteps = (kn + T::kStep - 1) / T::kStep;
+    // request the first batch of weights, then stage x: the two latencies overlap
+    if (active) W::load_batch(wa, wbase, row_bytes, kt, kn, 0, lane);
     if (kt > 0) __syncthreads();
     for (int i = threadIdx.x * 8; i < M * kn; i += 256 * 8) {
       const int m = i / kn;
@@ -129,53 +204,13 @@ __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
     }
     __syncthreads();
     if (active) {
-      for (int k0 = lane * E; k0 < kn; k0 += kStep) {
-        uint4_t wv[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          wv[r] = *reinterpret_cast<const uint4_t*>(wbase + r * row_bytes +
-                                                    static_cast<int64_t>(kt + k0) * kBytesPerRowNum / 2);
-        }
-        if constexpr (FMT == RWKV_FMT_W4) {
-          // 32 codes per lane all lie in one 128-group: scale and zero point are per (row, group)
-          const int g = (kt + k0) >> 7;
-          const int G = K >> 7;
-#pragma unroll
-          for (int m = 0; m < M; ++m) {
-            half2_t xv[16];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KT + k0 + q * 8);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
-            }
-            float xsum = 0.0f;
-            const half2_t ones = {static_cast<half_t>(1.0f), static_cast<half_t>(1.0f)};
-#pragma unroll
-            for (int e = 0; e < 16; ++e) xsum = dot2(xv[e], ones, xsum);
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-              const int64_t gi = static_cast<int64_t>(row0 + r) * G + g;
-              const float sc = h2f(prob.scale[gi]);
-              const float z = static_cast<float>(prob.zp[gi]);
-              const float part = WeightVec<FMT>::dot(wv[r], xv, 0.0f) - z * xsum;
-              acc[r][m] = fmaf(part, sc, acc[r][m]);
-            }
-          }
-        } else {
-          constexpr int XV = E / 2;  // half2 per lane per m
-#pragma unroll
-          for (int m = 0; m < M; ++m) {
-            half2_t xv[XV];
-#pragma unroll
-            for (int q = 0; q < XV / 4; ++q) {
-              const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KT + k0 + q * 8);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(wv[r], xv, acc[r][m]);
-          }
+      // ping-pong over batches of U steps
+      for (int s0 = 0; s0 < nsteps; s0 += 2 * U) {
+        if (s0 + U < nsteps) W::load_batch(wb, wbase, row_bytes, kt, kn, s0 + U, lane);
+        W::compute_batch(acc, wa, xs, KT, kt, kn, s0, lane, prob, row0, K);
+        if (s0 + U < nsteps) {
+          if (s0 + 2 * U < nsteps) W::load_batch(wa, wbase, row_bytes, kt, kn, s0 + 2 * U, lane);
+          W::compute_batch(acc, wb, xs, KT, kt, kn, s0 + U, lane, prob, row0, K);
         }
       }
     }
@@ -211,69 +246,82 @@ __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
   }
 }
 
-template <int FMT, int M, int R>
-static int launch_one(hipStream_t st, const LinearArgs& args, int n_problems, int max_n) {
+// grid = total blocks over all problems (each block: 4 waves x R rows); dynamic LDS = M*KT*2 bytes.
+template <int M, int R, int U>
+__global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  half_t* xs = reinterpret_cast<half_t*>(lds_raw);
+  int pi = 0;
+  int first = 0;
+  for (int i = 0; i < args.n_problems - 1; ++i) {
+    if (static_cast<int>(blockIdx.x) >= args.block_end[i]) {
+      pi = i + 1;
+      first = args.block_end[i];
+    }
+  }
+  const LinearProblem prob = args.p[pi];
+  const int blk = blockIdx.x - first;
+  switch (prob.fmt) {  // uniform per block
+    case RWKV_FMT_W8: gemv_block<RWKV_FMT_W8, M, R, U>(args, prob, blk, xs); break;
+    case RWKV_FMT_W4: gemv_block<RWKV_FMT_W4, M, R, U>(args, prob, blk, xs); break;
+    default: gemv_block<RWKV_FMT_F16, M, R, U>(args, prob, blk, xs); break;
+  }
+}
+
+template <int M, int R, int U>
+static int launch_one(hipStream_t st, LinearArgs& args) {
+  int total = 0;
+  for (int i = 0; i < args.n_problems; ++i) {
+    total += ceil_div(args.p[i].N, 4 * R);
+    args.block_end[i] = total;
+  }
   const size_t lds = static_cast<size_t>(M) * args.KT * sizeof(half_t);
-  const dim3 grid(ceil_div(max_n, 4 * R), n_problems);
-  hipLaunchKernelGGL((linear_gemv_kernel<FMT, M, R>), grid, dim3(256), lds, st, args);
+  hipLaunchKernelGGL((linear_gemv_kernel<M, R, U>), dim3(total), dim3(256), lds, st, args);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
-template <int FMT>
-static int launch_fmt(hipStream_t st, const LinearArgs& args, int n_problems, int max_n, int M) {
-  switch (M) {
-    case 1: return launch_one<FMT, 1, 2>(st, args, n_problems, max_n);
-    case 2: return launch_one<FMT, 2, 2>(st, args, n_problems, max_n);
-    case 3: return launch_one<FMT, 3, 2>(st, args, n_problems, max_n);
-    case 4: return launch_one<FMT, 4, 2>(st, args, n_problems, max_n);
-    case 5: return launch_one<FMT, 5, 4>(st, args, n_problems, max_n);
-    case 6: return launch_one<FMT, 6, 4>(st, args, n_problems, max_n);
-    case 7: return launch_one<FMT, 7, 4>(st, args, n_problems, max_n);
-    case 8: return launch_one<FMT, 8, 4>(st, args, n_problems, max_n);
-    default: break;
-  }
-  set_error("linear: bad row tile %d", M);
-  return RWKV_E_INVALID;
-}
-
-// Batched small-M linear: n_problems problems sharing fmt, M (<= 8), K, epilogue and output type.
-int linear_small_m(hipStream_t st, int fmt, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
+// Batched small-M linear: n_problems problems sharing M (<= 8), K, epilogue and output type.
+int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
                    int out_f32) {
   RWKV_REQUIRE(M >= 1 && M <= 8, "linear_small_m: M %d out of range", M);
   RWKV_REQUIRE(n_problems >= 1 && n_problems <= kMaxProblems, "linear_small_m: %d problems", n_problems);
-  const int elems = fmt == RWKV_FMT_F16 ? 8 : (fmt == RWKV_FMT_W8 ? 16 : 32);
-  RWKV_REQUIRE(K > 0 && K % elems == 0, "linear: K (%d) must be a multiple of %d for this weight format", K, elems);
-  if (fmt == RWKV_FMT_W4) RWKV_REQUIRE(K % 128 == 0, "linear: W4 needs K %% 128 == 0 (K = %d)", K);
-  LinearArgs args;
-  int max_n = 0;
+  LinearArgs args = {};
+  int max_elems = 8;
   for (int i = 0; i < n_problems; ++i) {
-    RWKV_REQUIRE(problems[i].N > 0 && problems[i].N % 4 == 0, "linear: N (%d) must be a positive multiple of 4",
-                 problems[i].N);
-    RWKV_REQUIRE(problems[i].w && problems[i].x && problems[i].y, "linear: NULL tensor");
-    RWKV_REQUIRE(fmt == RWKV_FMT_F16 || problems[i].scale, "linear: quantised weights need a scale tensor");
-    RWKV_REQUIRE(fmt != RWKV_FMT_W4 || problems[i].zp, "linear: W4 weights need a zero-point tensor");
-    args.p[i] = problems[i];
-    max_n = std::max(max_n, problems[i].N);
+    const LinearProblem& p = problems[i];
+    RWKV_REQUIRE(p.fmt == RWKV_FMT_F16 || p.fmt == RWKV_FMT_W8 || p.fmt == RWKV_FMT_W4,
+                 "linear: unknown weight format %d", p.fmt);
+    const int elems = p.fmt == RWKV_FMT_F16 ? 8 : (p.fmt == RWKV_FMT_W8 ? 16 : 32);
+    max_elems = std::max(max_elems, elems);
+    RWKV_REQUIRE(K > 0 && K % elems == 0, "linear: K (%d) must be a multiple of %d for this weight format", K, elems);
+    if (p.fmt == RWKV_FMT_W4) RWKV_REQUIRE(K % 128 == 0, "linear: W4 needs K %% 128 == 0 (K = %d)", K);
+    RWKV_REQUIRE(p.N > 0 && p.N % 4 == 0, "linear: N (%d) must be a positive multiple of 4", p.N);
+    RWKV_REQUIRE(p.w && p.x && p.y, "linear: NULL tensor");
+    RWKV_REQUIRE(p.fmt == RWKV_FMT_F16 || p.scale, "linear: quantised weights need a scale tensor");
+    RWKV_REQUIRE(p.fmt != RWKV_FMT_W4 || p.zp, "linear: W4 weights need a zero-point tensor");
+    args.p[i] = p;
   }
-  for (int i = n_problems; i < kMaxProblems; ++i) args.p[i] = problems[0];
+  args.n_problems = n_problems;
   args.K = K;
   args.epilogue = epilogue;
   args.out_f32 = out_f32;
-  // LDS tile of x: at most 32 KiB per block, a whole number of wave steps
-  const int step = 64 * elems;
-  int kt = (32768 / (2 * M)) / step * step;
-  if (kt < step) kt = step;
+  // LDS tile of x: the whole K when M*K*2 bytes <= 64 KiB, else a whole number of the widest wave step
+  const int step = 64 * max_elems;
   const int k_round = (K + step - 1) / step * step;
+  int kt = (65536 / (2 * M)) / step * step;
+  if (kt < step) kt = step;
   args.KT = std::min(kt, k_round);
-  switch (fmt) {
-    case RWKV_FMT_F16: return launch_fmt<RWKV_FMT_F16>(st, args, n_problems, max_n, M);
-    case RWKV_FMT_W8: return launch_fmt<RWKV_FMT_W8>(st, args, n_problems, max_n, M);
-    case RWKV_FMT_W4: return launch_fmt<RWKV_FMT_W4>(st, args, n_problems, max_n, M);
-    default: break;
+  switch (M) {
+    case 1: return launch_one<1, 2, 4>(st, args);
+    case 2: return launch_one<2, 2, 4>(st, args);
+    case 3: return launch_one<3, 2, 2>(st, args);
+    case 4: return launch_one<4, 2, 2>(st, args);
+    case 5: return launch_one<5, 4, 1>(st, args);
+    case 6: return launch_one<6, 4, 1>(st, args);
+    case 7: return launch_one<7, 4, 1>(st, args);
+    default: return launch_one<8, 4, 1>(st, args);
   }
-  set_error("linear: unknown weight format %d", fmt);
-  return RWKV_E_INVALID;
 }
 
 // Any M: MFMA tiles when the shape allows it and M >= 16, else row tiles of <= 8 through the GEMV kernel.
@@ -293,7 +341,8 @@ int linear_any_m(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, 
     p.y = out_f32 ? static_cast<void*>(static_cast<float*>(y) + static_cast<int64_t>(m0) * N)
                   : static_cast<void*>(static_cast<half_t*>(y) + static_cast<int64_t>(m0) * N);
     p.N = N;
-    const int rc = linear_small_m(st, fmt, mt, K, 1, &p, epilogue, out_f32);
+    p.fmt = fmt;
+    const int rc = linear_small_m(st, mt, K, 1, &p, epilogue, out_f32);
     if (rc != RWKV_OK) return rc;
   }
   return RWKV_OK;

@@ -285,44 +285,36 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       TRY(token_shift_mix_launch(st, a));
     }
 
-    // r, k, v projections
-    const bool same_fmt = w.m[RWKV_M_ATT_R].fmt == w.m[RWKV_M_ATT_K].fmt && w.m[RWKV_M_ATT_R].fmt == w.m[RWKV_M_ATT_V].fmt;
-    if (small && same_fmt) {
-      LinearProblem p[3];
-      const int mids[3] = {RWKV_M_ATT_R, RWKV_M_ATT_K, RWKV_M_ATT_V};
-      const half_t* xs[3] = {b.xr, b.xk, b.xv};
-      half_t* ys[3] = {b.r, b.k, v_cur};
-      for (int i = 0; i < 3; ++i) {
-        p[i].w = w.m[mids[i]].data; p[i].scale = w.m[mids[i]].scale; p[i].zp = w.m[mids[i]].zp;
-        p[i].x = xs[i]; p[i].y = ys[i]; p[i].N = C;
-      }
-      TRY_PROF(linear_small_m(st, w.m[RWKV_M_ATT_R].fmt, rows, C, 3, p, RWKV_EPI_NONE, 0));
-    } else {
-      TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_R], rows, C, C, b.xr, RWKV_EPI_NONE, 0, b.r));
-      TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_K], rows, C, C, b.xk, RWKV_EPI_NONE, 0, b.k));
-      TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_V], rows, C, C, b.xv, RWKV_EPI_NONE, 0, v_cur));
-    }
-
-    // LoRA rank-in (w, a, g and, past layer 0, v)
+    // r, k, v projections and the LoRA rank-ins (w, a, g and, past layer 0, v)
     {
       const int n_lora = (l == 0) ? 3 : 4;
       const int w1_ids[4] = {RWKV_T_W1, RWKV_T_A1, RWKV_T_G1, RWKV_T_V1};
       const int ranks[4] = {m->Rw, m->Ra, m->Rg, m->Rv};
-      const half_t* xs[4] = {b.xw, b.xa, b.xg, b.xv};
-      half_t* hs[4] = {b.hw, b.ha, b.hg, b.hv};
+      const half_t* lx[4] = {b.xw, b.xa, b.xg, b.xv};
+      half_t* lh[4] = {b.hw, b.ha, b.hg, b.hv};
+      const int mids[3] = {RWKV_M_ATT_R, RWKV_M_ATT_K, RWKV_M_ATT_V};
+      const half_t* xs[3] = {b.xr, b.xk, b.xv};
+      half_t* ys[3] = {b.r, b.k, v_cur};
       if (small) {
-        LinearProblem p[4];
-        for (int i = 0; i < n_lora; ++i) {
-          p[i].w = w.t[w1_ids[i]]; p[i].scale = nullptr; p[i].zp = nullptr;
-          p[i].x = xs[i]; p[i].y = hs[i]; p[i].N = ranks[i];
+        // one launch: three big matrices (any format) + the rank-in matrices (fp16), all with K = C
+        LinearProblem p[7];
+        for (int i = 0; i < 3; ++i) {
+          p[i].w = w.m[mids[i]].data; p[i].scale = w.m[mids[i]].scale; p[i].zp = w.m[mids[i]].zp;
+          p[i].x = xs[i]; p[i].y = ys[i]; p[i].N = C; p[i].fmt = w.m[mids[i]].fmt;
         }
-        TRY(linear_small_m(st, RWKV_FMT_F16, rows, C, n_lora, p, RWKV_EPI_NONE, 0));
+        for (int i = 0; i < n_lora; ++i) {
+          p[3 + i].w = w.t[w1_ids[i]]; p[3 + i].scale = nullptr; p[3 + i].zp = nullptr;
+          p[3 + i].x = lx[i]; p[3 + i].y = lh[i]; p[3 + i].N = ranks[i]; p[3 + i].fmt = RWKV_FMT_F16;
+        }
+        TRY_PROF(linear_small_m(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0));
       } else {
+        for (int i = 0; i < 3; ++i) TRY_PROF(apply_matrix(st, w.m[mids[i]], rows, C, C, xs[i], RWKV_EPI_NONE, 0, ys[i]));
         for (int i = 0; i < n_lora; ++i)
-          TRY(linear_any_m(st, RWKV_FMT_F16, rows, ranks[i], C, xs[i], w.t[w1_ids[i]], nullptr, nullptr, RWKV_EPI_NONE,
-                           0, hs[i]));
+          TRY(linear_any_m(st, RWKV_FMT_F16, rows, ranks[i], C, lx[i], w.t[w1_ids[i]], nullptr, nullptr, RWKV_EPI_NONE,
+                           0, lh[i]));
       }
     }
+
     if (step) {
       // the whole time-mix core of a decode step in one launch per layer
       TmixStepArgs p = {};

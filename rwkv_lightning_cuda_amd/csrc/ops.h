@@ -6,7 +6,7 @@
 namespace rwkv {
 
 // ---- linear.hip / gemm_mfma.hip ------------------------------------------------------------------
-constexpr int kMaxProblems = 4;
+constexpr int kMaxProblems = 8;
 
 struct LinearProblem {
   const void* w;
@@ -15,10 +15,12 @@ struct LinearProblem {
   const half_t* x;
   void* y;
   int N;
+  int fmt;  // RWKV_FMT_*
 };
 
-// Batched small-M (<= 8) linear through the weight-streaming GEMV kernel.
-int linear_small_m(hipStream_t st, int fmt, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
+// Batched small-M (<= 8) linear through the weight-streaming GEMV kernel: up to kMaxProblems problems that
+// share M and K (each with its own weight format, x and y) in one launch.
+int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
                    int out_f32);
 // Any M: MFMA tiles for M >= 16 where supported, else row tiles through the GEMV kernel.
 int linear_any_m(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* w, const half_t* scale,
