@@ -15,6 +15,8 @@
 // K range: no atomics, no cross-wave reduction, deterministic summation order.  Up to eight problems
 // that share x-length K (r/k/v and the four LoRA rank-ins of a layer, in different weight formats) go out
 // as one launch over a flattened block range.
+#include <cstdlib>
+
 #include "ops.h"
 
 namespace rwkv {
@@ -312,9 +314,25 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
   int kt = (65536 / (2 * M)) / step * step;
   if (kt < step) kt = step;
   args.KT = std::min(kt, k_round);
+  if (M == 1) {
+    // RWKV_GEMV_RU=<R><U> picks the rows-per-wave / steps-in-flight variant for M == 1 (tuning aid)
+    static const int ru = [] { const char* e = getenv("RWKV_GEMV_RU"); return e ? atoi(e) : 0; }();
+    switch (ru) {
+      case 11: return launch_one<1, 1, 1>(st, args);
+      case 12: return launch_one<1, 1, 2>(st, args);
+      case 14: return launch_one<1, 1, 4>(st, args);
+      case 24: return launch_one<1, 2, 4>(st, args);
+      case 22: return launch_one<1, 2, 2>(st, args);
+      case 41: return launch_one<1, 4, 1>(st, args);
+      case 42: return launch_one<1, 4, 2>(st, args);
+      case 44: return launch_one<1, 4, 4>(st, args);
+      case 81: return launch_one<1, 8, 1>(st, args);
+      default: break;
+    }
+  }
   switch (M) {
-    case 1: return launch_one<1, 2, 4>(st, args);
-    case 2: return launch_one<2, 2, 4>(st, args);
+    case 1: return launch_one<1, 2, 1>(st, args);
+    case 2: return launch_one<2, 2, 1>(st, args);
     case 3: return launch_one<3, 2, 2>(st, args);
     case 4: return launch_one<4, 2, 2>(st, args);
     case 5: return launch_one<5, 4, 1>(st, args);
