@@ -147,7 +147,7 @@ def test_dequant_all_codes_bit_exact(gpu, orc):
 
 # -------------------------------------------------------------------------------------------- linear
 @pytest.mark.parametrize("fmt_name", ["f16", "w8", "w4"])
-@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 11])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 11, 16, 37, 128, 200])
 def test_linear_small_m(gpu, orc, fmt_name, M):
     hip = gpu
     rng = np.random.default_rng(11 + M)
