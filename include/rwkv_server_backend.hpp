@@ -1,0 +1,123 @@
+// Host-side backend API, signature-compatible with the reference's include/rwkv_server_backend.hpp:15-147,
+// implemented over librwkv_hip.so.  Only the fp32 WKV state mode is provided.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "rwkv7_fast_v4_common.hpp"
+
+namespace rwkv7_server {
+
+struct PrefillCapacity {
+  std::size_t free_vram_bytes = 0;
+  std::size_t total_vram_bytes = 0;
+  std::size_t reserve_vram_bytes = 0;
+  std::size_t bytes_per_batch = 0;
+  int max_batch_size = 0;
+};
+
+enum class ThinkType { Fast, Free, PreferChinese, En, EnShort, EnLong };
+
+struct GenerateOptions {
+  int max_tokens = 8192;
+  std::vector<int64_t> stop_tokens{0, 261, 24281};
+  double temperature = 1.0;
+  int top_k = 20;
+  double top_p = 0.3;
+  double alpha_presence = 2.0;
+  double alpha_frequency = 0.2;
+  double alpha_decay = 0.996;
+  bool force_reasoning = false;
+  int force_reasoning_token_offset = 0;
+};
+
+// shift f16 [L,2,B,C]; wkv_state32 f32 [L,B,H,64,64]; elapsed i32 [B].  wkv_state (fp16 state) is kept as
+// a member for layout compatibility and is never allocated by this backend.
+struct GenerationState {
+  int batch_size = 0;
+  bool wkv32 = false;
+  rwkv7_fast_v4::DeviceBuffer<half> shift;
+  rwkv7_fast_v4::DeviceBuffer<half> wkv_state;
+  rwkv7_fast_v4::DeviceBuffer<float> wkv_state32;
+  rwkv7_fast_v4::DeviceBuffer<int> elapsed;
+
+  GenerationState() = default;
+  GenerationState(const GenerationState&) = delete;
+  GenerationState& operator=(const GenerationState&) = delete;
+  GenerationState(GenerationState&&) noexcept = default;
+  GenerationState& operator=(GenerationState&&) noexcept = default;
+};
+
+struct DeviceLogits {
+  int rows = 0;
+  int vocab_size = 0;
+  rwkv7_fast_v4::DeviceBuffer<float> values;
+
+  DeviceLogits() = default;
+  DeviceLogits(const DeviceLogits&) = delete;
+  DeviceLogits& operator=(const DeviceLogits&) = delete;
+  DeviceLogits(DeviceLogits&&) noexcept = default;
+  DeviceLogits& operator=(DeviceLogits&&) noexcept = default;
+};
+
+class IModelBackend {
+ public:
+  virtual ~IModelBackend() = default;
+
+  virtual GenerationState create_state(int batch_size) const = 0;
+  virtual void forward_prefill(const std::vector<std::vector<int64_t>>& token_batches, GenerationState& state,
+                               DeviceLogits& logits) const = 0;
+  virtual void forward_decode(const std::vector<int64_t>& token_batch, GenerationState& state,
+                              DeviceLogits& logits) const = 0;
+  virtual void copy_state_slice(const GenerationState& src, int src_offset, GenerationState& dst, int dst_offset,
+                                int count) const = 0;
+  virtual void copy_logits_slice(const DeviceLogits& src, int src_offset, DeviceLogits& dst, int dst_offset,
+                                 int count) const = 0;
+  virtual PrefillCapacity query_prefill_capacity(int prefill_chunk_size) const = 0;
+
+  virtual int vocab_size() const = 0;
+  virtual const std::string& model_path() const = 0;
+  virtual const std::string& model_name() const = 0;
+};
+
+// model_path selects the weights.  The reference reads a .pth checkpoint here; that reader is not part of
+// this build, so the path names a synthetic random-init model instead:
+//   "synthetic:<0.1B|1.5B|7.2B|tiny>[:f16|w8|w4][:seed=<n>]"
+// use_wkv32 must be true (fp32 state only); chunk_load is accepted and ignored.
+class ModelBackend final : public IModelBackend {
+ public:
+  explicit ModelBackend(std::string model_path, bool use_wkv32 = false, bool chunk_load = false);
+  ~ModelBackend() override;
+
+  ModelBackend(const ModelBackend&) = delete;
+  ModelBackend& operator=(const ModelBackend&) = delete;
+  ModelBackend(ModelBackend&&) noexcept;
+  ModelBackend& operator=(ModelBackend&&) noexcept;
+
+  GenerationState create_state(int batch_size) const override;
+  void forward_prefill(const std::vector<std::vector<int64_t>>& token_batches, GenerationState& state,
+                       DeviceLogits& logits) const override;
+  void forward_decode(const std::vector<int64_t>& token_batch, GenerationState& state,
+                      DeviceLogits& logits) const override;
+  void copy_state_slice(const GenerationState& src, int src_offset, GenerationState& dst, int dst_offset,
+                        int count) const override;
+  void copy_logits_slice(const DeviceLogits& src, int src_offset, DeviceLogits& dst, int dst_offset,
+                         int count) const override;
+  PrefillCapacity query_prefill_capacity(int prefill_chunk_size) const override;
+
+  int vocab_size() const override;
+  const std::string& model_path() const override;
+  const std::string& model_name() const override;
+
+  const rwkv7_fast_v4::ModelDims& dims() const;
+
+ private:
+  struct Impl;
+  std::unique_ptr<Impl> impl_;
+};
+
+}  // namespace rwkv7_server

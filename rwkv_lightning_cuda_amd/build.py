@@ -1,9 +1,11 @@
-"""Builds the gfx950 kernel library (csrc/*.hip -> librwkv_hip.so) in-tree with hipcc.
+"""Builds the native code in-tree.
 
     python -m rwkv_lightning_cuda_amd.build [--force]
 
-hipcc cross-compiles for gfx950 without a GPU present.  The shared library has no Python or torch
-dependency: it exports only the C ABI declared in include/rwkv_hip.h.
+  csrc/*.hip -> librwkv_hip.so    gfx950 kernels behind the C ABI of include/rwkv_hip.h (hipcc; it
+                                  cross-compiles without a GPU present).  No Python or torch dependency.
+  host/*.cpp -> librwkv_host.so   the C++ host API of include/*.hpp (g++), linked against librwkv_hip.so.
+  tests/cpp/*_test.cpp -> tests/cpp/bin/*   test executables of the host API.
 """
 import concurrent.futures
 import os
@@ -15,6 +17,12 @@ REPO_DIR = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 LIB_PATH = os.path.join(PKG_DIR, "librwkv_hip.so")
+HOST_SRC = os.path.join(PKG_DIR, "host")
+HOST_LIB_PATH = os.path.join(PKG_DIR, "librwkv_host.so")
+TEST_SRC = os.path.join(REPO_DIR, "tests", "cpp")
+TEST_BIN = os.path.join(TEST_SRC, "bin")
+CXX = os.environ.get("CXX", "g++")
+CXX_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-I" + os.path.join(REPO_DIR, "include")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 VALU ops are disabled for every device translation unit (see csrc/common.h users)
@@ -67,5 +75,44 @@ def build_all(force=False, verbose=True):
     return LIB_PATH
 
 
+def _run(cmd, what):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("%s failed:\n%s" % (what, proc.stderr))
+
+
+def build_host(verbose=True):
+    """Compiles host/*.cpp into librwkv_host.so (needs librwkv_hip.so to be built).  Returns its path."""
+    srcs = sorted(os.path.join(HOST_SRC, f) for f in os.listdir(HOST_SRC) if f.endswith(".cpp"))
+    cmd = ([CXX] + CXX_FLAGS + ["-shared", "-o", HOST_LIB_PATH] + srcs
+           + ["-L" + PKG_DIR, "-lrwkv_hip", "-ldl", "-pthread", "-Wl,-rpath,$ORIGIN"])
+    _run(cmd, "host library build")
+    if verbose:
+        print("built", HOST_LIB_PATH)
+    return HOST_LIB_PATH
+
+
+def host_test_names():
+    return sorted(f[:-4] for f in os.listdir(TEST_SRC) if f.endswith("_test.cpp"))
+
+
+def build_host_tests(verbose=True):
+    """Compiles every tests/cpp/*_test.cpp into tests/cpp/bin/ (needs both libraries)."""
+    os.makedirs(TEST_BIN, exist_ok=True)
+    rpath = "-Wl,-rpath," + PKG_DIR + ":$ORIGIN/../../../rwkv_lightning_cuda_amd"
+    outs = []
+    for name in host_test_names():
+        out = os.path.join(TEST_BIN, name)
+        cmd = ([CXX] + CXX_FLAGS + ["-I" + TEST_SRC, os.path.join(TEST_SRC, name + ".cpp"), "-o", out,
+                                   "-L" + PKG_DIR, "-lrwkv_host", "-lrwkv_hip", "-pthread", rpath])
+        _run(cmd, "test build " + name)
+        outs.append(out)
+    if verbose:
+        print("built", len(outs), "host test executables")
+    return outs
+
+
 if __name__ == "__main__":
     build_all(force="--force" in sys.argv)
+    build_host()
+    build_host_tests()
