@@ -104,6 +104,21 @@ int rwkv_hip_fill_normal_f16(rwkv_stream_t s, int64_t n, uint64_t seed, float me
 int rwkv_hip_linear(rwkv_stream_t s, int fmt, int M, int N, int K, const void* x, const void* w,
                     const void* scale, const void* zp, int epilogue, int out_f32, void* y);
 
+/* The same product over weights in the MFMA-native packed order: the path for M >= 16 (prefill chunks
+ * and batched decode; the reference sends these to cuBLAS / cuBLASLt,
+ * cuda/rwkv7_v3a_ops.cu:2235-2368, with per-shape algorithm ids at src/rwkv7_fast_v4.cu:753-958).
+ * rwkv_hip_pack_weights permutes the 16-byte pieces of row-major codes w [N,K] (fp16, int8 or int4 as
+ * for rwkv_hip_linear) into `packed` (same byte count, must not alias w); scale and zp keep their
+ * row-major layout.  Requires N % 32 == 0 and K % 256 == 0.  The workspace holds fp32 split-K
+ * partial sums; rwkv_hip_linear_packed_workspace gives the size for a shape (0 when the shape is not
+ * split; workspace may then be NULL).  Calls sharing one workspace must not overlap.  Results do not
+ * depend on scheduling (partials are summed in a fixed order). */
+int rwkv_hip_pack_weights(rwkv_stream_t s, int fmt, int N, int K, const void* w, void* packed);
+int rwkv_hip_linear_packed_workspace(int M, int N, int K, size_t* bytes);
+int rwkv_hip_linear_packed(rwkv_stream_t s, int fmt, int M, int N, int K, const void* x, const void* packed,
+                           const void* scale, const void* zp, int epilogue, int out_f32, void* y,
+                           void* workspace, size_t workspace_bytes);
+
 /* ---- LoRA pairs.  Replaces rwkv7_v3a_linear_wag(v)_rank_in_f16_launch,
  * rwkv7_v3a_linear_wag(v)_rank_out_f16_launch, rwkv7_v3a_linear_t_f16_launch,
  * rwkv7_v3a_linear_t_act_f16_launch, rwkv7_v3a_linear_t_vres_f16_launch

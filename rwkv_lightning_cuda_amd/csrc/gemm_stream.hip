@@ -1,0 +1,536 @@
+// Weight-streaming MFMA GEMM Y[M,N] = X[M,K] . W[N,K]^T over weights stored in an MFMA-native packed order.
+// This is the M >= 16 path of the model: batched decode (M = batch) and prefill chunks (M = batch * 128).
+//
+// Reference: the cuBLAS / cuBLASLt calls behind rwkv7_v3a_linear_f16_orig_launch and
+// rwkv7_v3a_linear_f16_orig_lt_cfg_launch (cuda/rwkv7_v3a_ops.cu:2235-2368): fp16 in, fp32 accumulate, fp16
+// (or fp32) out.  The arithmetic there lives in a closed library; the contract is the textbook GEMM.
+//
+// Packed order.  v_mfma_f32_32x32x16_f16 takes, from lane l = j + 32h, 8 fp16 values of row j of each
+// operand for 8 of the 16 k of the step; any assignment of k to (h, step) is valid as long as both operands
+// use the same one.  A packed matrix is cut into tiles of 32 rows x G k (G = 32 for fp16 and int8 codes, 64
+// for int4 codes); inside a tile lane (j, h) owns the KR = G/2 consecutive k [h*KR, h*KR + KR) of row j, and
+// the tile is stored as 64 lanes x 16 bytes (x 2 pieces for fp16), tiles of one 32-row band consecutive
+// along k.  A wavefront therefore streams one band with 1 KiB fully coalesced loads and feeds the pieces
+// to the matrix core after an exact in-register expansion of the codes, without any transpose or LDS
+// traffic for the weights; every weight byte leaves HBM once per 32*MT rows of X.
+//
+// Work split.  Block = 4 wavefronts = 4 adjacent bands (128 output columns) x one K slice; the X rows of
+// the slice are staged in LDS in chunks of KC (128 or 256) and shared by the four wavefronts.  Chunks are
+// software-pipelined: while the matrix core works on chunk c out of one LDS tile and one register set, the
+// loads of chunk c+1 (first this thread's share of X, then the wavefront's weight pieces, so that waiting for
+// X does not wait for the weights) are in flight into the other set; one barrier per chunk.
+// grid = (row tiles, column blocks, K splits).  With more than one split each block writes an fp32 partial
+// tile and a second small kernel sums the partials in split order (a fixed order: results do not depend on
+// scheduling) and applies scale and epilogue.
+#include <algorithm>
+#include <cstdlib>
+
+#include "ops.h"
+
+namespace rwkv {
+
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+template <int FMT>
+struct PackTraits;
+template <>
+struct PackTraits<RWKV_FMT_F16> {
+  static constexpr int KR = 16, PIECES = 2;
+};
+template <>
+struct PackTraits<RWKV_FMT_W8> {
+  static constexpr int KR = 16, PIECES = 1;
+};
+template <>
+struct PackTraits<RWKV_FMT_W4> {
+  static constexpr int KR = 32, PIECES = 1;
+};
+
+bool linear_packed_supported(int fmt, int M, int N, int K) {
+  if (fmt != RWKV_FMT_F16 && fmt != RWKV_FMT_W8 && fmt != RWKV_FMT_W4) return false;
+  return M >= 1 && N >= 32 && N % 32 == 0 && K >= 256 && K % 256 == 0;
+}
+
+// ---- packing: a permutation of the 16-byte pieces of the row-major codes ---------------------------------------------
+__global__ __launch_bounds__(256) void pack_weights_kernel(int fmt, int N, int K, const uint4_t* __restrict__ src,
+                                                           uint4_t* __restrict__ dst, int64_t n_pieces) {
+  const int64_t p = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (p >= n_pieces) return;
+  const int G = fmt == RWKV_FMT_W4 ? 64 : 32;
+  const int KR = G / 2;
+  const int pieces = fmt == RWKV_FMT_F16 ? 2 : 1;
+  const int lane = static_cast<int>(p & 63);
+  int64_t q = p >> 6;
+  const int i = static_cast<int>(q % pieces);
+  q /= pieces;
+  const int KG = K / G;
+  const int kg = static_cast<int>(q % KG);
+  const int nt = static_cast<int>(q / KG);
+  const int row = nt * 32 + (lane & 31);
+  const int k = kg * G + (lane >> 5) * KR + i * 8;
+  // elements per 16-byte piece: 8 (fp16), 16 (int8), 32 (int4)
+  const int per = fmt == RWKV_FMT_F16 ? 8 : (fmt == RWKV_FMT_W8 ? 16 : 32);
+  dst[p] = src[(static_cast<int64_t>(row) * K + k) / per];
+}
+
+int pack_weights_launch(hipStream_t st, int fmt, int N, int K, const void* w, void* packed) {
+  RWKV_REQUIRE(linear_packed_supported(fmt, 16, N, K), "pack_weights: unsupported shape N=%d K=%d fmt=%d", N, K, fmt);
+  RWKV_REQUIRE(w && packed && w != packed, "pack_weights: bad pointers");
+  const int per = fmt == RWKV_FMT_F16 ? 8 : (fmt == RWKV_FMT_W8 ? 16 : 32);
+  const int64_t n_pieces = static_cast<int64_t>(N) * K / per;
+  hipLaunchKernelGGL(pack_weights_kernel, dim3(static_cast<unsigned>((n_pieces + 255) / 256)), dim3(256), 0, st, fmt,
+                     N, K, static_cast<const uint4_t*>(w), static_cast<uint4_t*>(packed), n_pieces);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+// ---- the GEMM ---------------------------------------------------------------------------------------------------------
+
+struct StreamProblem {
+  const half_t* x;
+  const uint4_t* wp;
+  const half_t* scale;
+  const uint8_t* zp;
+  void* y;
+  float* partial;  // [splits][M][N] fp32, only with splits > 1
+  int N;
+  int fmt;
+};
+
+// Up to kMaxProblems products that share M, K and the split (each with its own weights, format, x and y) in one
+// launch: grid.y runs over the column blocks of all problems, block_end[] are the prefix sums.
+struct StreamArgs {
+  StreamProblem p[kMaxProblems];
+  int block_end[kMaxProblems];
+  int n_problems;
+  int M, K;
+  int splits, k_per_split;
+  int epilogue, out_f32;
+};
+
+__device__ __forceinline__ half8_t make_half8(half2_t a, half2_t b, half2_t c, half2_t d) {
+  half8_t r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = b[0]; r[3] = b[1];
+  r[4] = c[0]; r[5] = c[1]; r[6] = d[0]; r[7] = d[1];
+  return r;
+}
+
+// 8 int8 codes (two dwords) -> 8 fp16, exact: byte^0x80 under exponent 0x64 is 1024 + (code + 128).
+__device__ __forceinline__ half8_t expand_w8(uint32_t d0, uint32_t d1) {
+  const half2_t bias = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
+  d0 ^= 0x80808080u;
+  d1 ^= 0x80808080u;
+  return make_half8(as_half2(__builtin_amdgcn_perm(0x64646464u, d0, 0x04010400u)) - bias,
+                    as_half2(__builtin_amdgcn_perm(0x64646464u, d0, 0x04030402u)) - bias,
+                    as_half2(__builtin_amdgcn_perm(0x64646464u, d1, 0x04010400u)) - bias,
+                    as_half2(__builtin_amdgcn_perm(0x64646464u, d1, 0x04030402u)) - bias);
+}
+
+// 8 int4 codes (one dword, element 2i in the low nibble of byte i) minus the zero point -> 8 fp16, exact.
+__device__ __forceinline__ half8_t expand_w4(uint32_t d, half2_t bias) {
+  const uint32_t even = d & 0x0f0f0f0fu;
+  const uint32_t odd = (d >> 4) & 0x0f0f0f0fu;
+  return make_half8(as_half2(__builtin_amdgcn_perm(odd, even, 0x0c040c00u) | 0x64006400u) - bias,
+                    as_half2(__builtin_amdgcn_perm(odd, even, 0x0c050c01u) | 0x64006400u) - bias,
+                    as_half2(__builtin_amdgcn_perm(odd, even, 0x0c060c02u) | 0x64006400u) - bias,
+                    as_half2(__builtin_amdgcn_perm(odd, even, 0x0c070c03u) | 0x64006400u) - bias);
+}
+
+template <int FMT, int MT, int KC>
+struct Tile {
+  using P = PackTraits<FMT>;
+  static constexpr int BM = 32 * MT;
+  static constexpr int G = 2 * P::KR;
+  static constexpr int GROUPS = KC / G;
+  static constexpr int NW = GROUPS * P::PIECES;     // weight pieces per lane per chunk
+  static constexpr int STEPS = P::KR / 8;
+  static constexpr int XSTRIDE = KC + 8;            // fp16 per staged row: 16-byte pad keeps b128 reads conflict-free
+  static constexpr int XV = BM * (KC / 8) / 256;    // 16-byte vectors of X per thread per chunk
+  static constexpr int QG = KC / 128;               // int4 scale groups per chunk
+  static constexpr int NACC = MT == 1 ? 2 : 1;      // independent accumulation chains per row tile
+  static constexpr int kTileHalfs = BM * XSTRIDE;   // one staged X tile
+  static_assert(KC % 128 == 0 && XV >= 1, "chunk must hold whole int4 groups and at least one vector per thread");
+};
+
+__device__ __forceinline__ float finish_value(float v, int epilogue) {
+  v = round_h(v);
+  if (epilogue == RWKV_EPI_RELU_SQUARE) {
+    v = fmaxf(v, 0.0f);
+    v = round_h(v * v);
+  }
+  return v;
+}
+
+// One chunk's operands held by a lane between request and use.
+template <int FMT, int MT, int KC>
+struct ChunkRegs {
+  using T = Tile<FMT, MT, KC>;
+  uint4_t xv[T::XV];
+  uint4_t w[T::NW];
+  float sc[T::QG], zb[T::QG];
+
+  // X first, then the weights: waiting for X (to store it to LDS) does not wait for the weight pieces.
+  __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int m0, int kc, bool active,
+                                          const uint4_t* wband, int n) {
+    using P = typename T::P;
+#pragma unroll
+    for (int i = 0; i < T::XV; ++i) {
+      const int idx = threadIdx.x + i * 256;
+      const int r = idx / (KC / 8);
+      const int c = (idx % (KC / 8)) * 8;
+      xv[i] = uint4_t{0u, 0u, 0u, 0u};
+      if (m0 + r < g.M) xv[i] = *reinterpret_cast<const uint4_t*>(pr.x + static_cast<int64_t>(m0 + r) * g.K + kc + c);
+    }
+    if (active) {
+      const uint4_t* wp = wband + static_cast<int64_t>(kc / T::G) * (P::PIECES * 64);
+#pragma unroll
+      for (int i = 0; i < T::NW; ++i) w[i] = wp[i * 64];
+      if constexpr (FMT == RWKV_FMT_W4) {
+        const int64_t q0 = static_cast<int64_t>(n) * (g.K >> 7) + (kc >> 7);
+#pragma unroll
+        for (int q = 0; q < T::QG; ++q) {
+          sc[q] = h2f(pr.scale[q0 + q]);
+          zb[q] = 1024.0f + static_cast<float>(pr.zp[q0 + q]);
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store_x(half_t* xs) const {
+#pragma unroll
+    for (int i = 0; i < T::XV; ++i) {
+      const int idx = threadIdx.x + i * 256;
+      const int r = idx / (KC / 8);
+      const int c = (idx % (KC / 8)) * 8;
+      *reinterpret_cast<uint4_t*>(xs + r * T::XSTRIDE + c) = xv[i];
+    }
+  }
+
+  __device__ __forceinline__ void multiply(const half_t* xs, int j, int h, float16_t (&acc)[MT][T::NACC],
+                                           float16_t (&part)[MT][T::NACC]) const {
+    using P = typename T::P;
+#pragma unroll
+    for (int gi = 0; gi < T::GROUPS; ++gi) {
+#pragma unroll
+      for (int s = 0; s < T::STEPS; ++s) {
+        half8_t b;
+        if constexpr (FMT == RWKV_FMT_F16) {
+          const uint4_t piece = w[gi * 2 + s];
+          b = __builtin_bit_cast(half8_t, piece);
+        } else if constexpr (FMT == RWKV_FMT_W8) {
+          const uint4_t piece = w[gi];
+          b = s == 0 ? expand_w8(piece[0], piece[1]) : expand_w8(piece[2], piece[3]);
+        } else {
+          const uint4_t piece = w[gi];
+          const half_t zf = static_cast<half_t>(zb[(gi * T::G) >> 7]);
+          const half2_t bias = {zf, zf};
+          b = expand_w4(piece[s], bias);
+        }
+        constexpr int kChainMask = T::NACC - 1;
+        const int chain = (gi * T::STEPS + s) & kChainMask;
+        const half_t* xa = xs + j * T::XSTRIDE + gi * T::G + h * P::KR + 8 * s;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const half8_t a = *reinterpret_cast<const half8_t*>(xa + mt * 32 * T::XSTRIDE);
+          if constexpr (FMT == RWKV_FMT_W4) {
+            part[mt][chain] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, part[mt][chain], 0, 0, 0);
+          } else {
+            acc[mt][chain] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[mt][chain], 0, 0, 0);
+          }
+        }
+      }
+      if constexpr (FMT == RWKV_FMT_W4) {
+        if (((gi + 1) * T::G) % 128 == 0) {  // end of a 128-group: fold with its scale
+          const float s128 = sc[(gi * T::G) >> 7];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int c = 0; c < T::NACC; ++c)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) {
+                acc[mt][c][v] = fmaf(part[mt][c][v], s128, acc[mt][c][v]);
+                part[mt][c][v] = 0.0f;
+              }
+        }
+      }
+    }
+  }
+};
+
+// One block of one problem: 128 columns x the block's K slice, which is a whole number of chunks.  Two X tiles
+// in LDS and two register sets alternate, so one barrier per chunk suffices and the next chunk's loads are in
+// flight while the matrix core works on the current one.
+template <int FMT, int MT, int KC>
+__device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamProblem& pr, int col_block, half_t* xs) {
+  using T = Tile<FMT, MT, KC>;
+  using P = typename T::P;
+  constexpr int BM = T::BM;
+
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int j = lane & 31;
+  const int h = lane >> 5;
+  const int m0 = blockIdx.x * BM;
+  const int band = col_block * 4 + wave;  // 32-row band of W = 32 output columns
+  const bool active = band * 32 < pr.N;
+  const int n = band * 32 + j;
+  const int kbeg = blockIdx.z * g.k_per_split;
+  const int nchunks = g.k_per_split / KC;
+
+  float16_t acc[MT][T::NACC], part[MT][T::NACC];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int c = 0; c < T::NACC; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        acc[mt][c][v] = 0.0f;
+        part[mt][c][v] = 0.0f;
+      }
+
+  // this lane's first piece of the band; consecutive pieces are 64 uint4 apart
+  const uint4_t* wband = pr.wp + (static_cast<int64_t>(active ? band : 0) * (g.K / T::G)) * (P::PIECES * 64) + lane;
+
+  ChunkRegs<FMT, MT, KC> r0, r1;
+  r0.request(g, pr, m0, kbeg, active, wband, n);
+  r0.store_x(xs);
+  __syncthreads();
+  for (int c = 0; c < nchunks; c += 2) {
+    // even chunk: operands in r0 / tile 0
+    if (c + 1 < nchunks) r1.request(g, pr, m0, kbeg + (c + 1) * KC, active, wband, n);
+    if (active) r0.multiply(xs, j, h, acc, part);
+    if (c + 1 >= nchunks) break;
+    r1.store_x(xs + T::kTileHalfs);
+    __syncthreads();
+    // odd chunk: operands in r1 / tile 1
+    if (c + 2 < nchunks) r0.request(g, pr, m0, kbeg + (c + 2) * KC, active, wband, n);
+    if (active) r1.multiply(xs + T::kTileHalfs, j, h, acc, part);
+    if (c + 2 < nchunks) {
+      r0.store_x(xs);
+      __syncthreads();
+    }
+  }
+  if (!active) return;
+
+  float scl = 1.0f;
+  if constexpr (FMT == RWKV_FMT_W8) {
+    if (g.splits == 1) scl = h2f(pr.scale[n]);
+  }
+  float* part_out = g.splits > 1 ? pr.partial + static_cast<int64_t>(blockIdx.z) * g.M * pr.N : nullptr;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = m0 + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+      if (row >= g.M) continue;
+      float sum = acc[mt][0][v];
+      if constexpr (T::NACC == 2) sum += acc[mt][1][v];
+      const int64_t o = static_cast<int64_t>(row) * pr.N + n;
+      if (part_out) {
+        part_out[o] = sum;
+      } else {
+        const float val = finish_value(sum * scl, g.epilogue);
+        if (g.out_f32) {
+          static_cast<float*>(pr.y)[o] = val;
+        } else {
+          static_cast<half_t*>(pr.y)[o] = f2h(val);
+        }
+      }
+    }
+}
+
+// grid = (row tiles of 32*MT, column blocks of 128 over all problems, splits); block = 256.
+template <int MT, int KC>
+__global__ __launch_bounds__(256) void gemm_stream_kernel(StreamArgs g) {
+  __shared__ __align__(16) half_t xs[2 * 32 * MT * (KC + 8)];
+  int pi = 0;
+  while (pi + 1 < g.n_problems && static_cast<int>(blockIdx.y) >= g.block_end[pi]) ++pi;
+  const int col_block = blockIdx.y - (pi > 0 ? g.block_end[pi - 1] : 0);
+  const StreamProblem& pr = g.p[pi];
+  switch (pr.fmt) {
+    case RWKV_FMT_W8: stream_block<RWKV_FMT_W8, MT, KC>(g, pr, col_block, xs); break;
+    case RWKV_FMT_W4: stream_block<RWKV_FMT_W4, MT, KC>(g, pr, col_block, xs); break;
+    default: stream_block<RWKV_FMT_F16, MT, KC>(g, pr, col_block, xs); break;
+  }
+}
+
+struct ReduceProblem {
+  const float4_t* partial;
+  const half_t* scale;  // NULL unless the problem's weights are int8 codes
+  void* y;
+  int N4;
+};
+struct ReduceArgs {
+  ReduceProblem p[kMaxProblems];
+  int block_end[kMaxProblems];
+  int n_problems;
+  int M, splits, epilogue, out_f32;
+};
+
+// y = finish(scale * sum over splits of partial), four columns per thread; blocks run over all problems.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs g) {
+  int pi = 0;
+  while (pi + 1 < g.n_problems && static_cast<int>(blockIdx.x) >= g.block_end[pi]) ++pi;
+  const ReduceProblem& pr = g.p[pi];
+  const int64_t plane4 = static_cast<int64_t>(g.M) * pr.N4;
+  const int64_t i = static_cast<int64_t>(blockIdx.x - (pi > 0 ? g.block_end[pi - 1] : 0)) * 256 + threadIdx.x;
+  if (i >= plane4) return;
+  const float4_t* partial = pr.partial;
+  float4_t sum = partial[i];
+  int s = 1;
+  for (; s + 4 <= g.splits; s += 4) {
+    const float4_t p0 = partial[(s + 0) * plane4 + i];
+    const float4_t p1 = partial[(s + 1) * plane4 + i];
+    const float4_t p2 = partial[(s + 2) * plane4 + i];
+    const float4_t p3 = partial[(s + 3) * plane4 + i];
+    sum = (((sum + p0) + p1) + p2) + p3;
+  }
+  for (; s < g.splits; ++s) sum = sum + partial[s * plane4 + i];
+  float4_t scl = {1.0f, 1.0f, 1.0f, 1.0f};
+  if (pr.scale) {
+    const half4_t sv = *reinterpret_cast<const half4_t*>(pr.scale + (i % pr.N4) * 4);
+    scl = float4_t{h2f(sv[0]), h2f(sv[1]), h2f(sv[2]), h2f(sv[3])};
+  }
+  float4_t val;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) val[c] = finish_value(sum[c] * scl[c], g.epilogue);
+  if (g.out_f32) {
+    static_cast<float4_t*>(pr.y)[i] = val;
+  } else {
+    half4_t o;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) o[c] = f2h(val[c]);
+    static_cast<half4_t*>(pr.y)[i] = o;
+  }
+}
+
+static int row_tiles(int M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
+
+// Tuning hooks: RWKV_GEMM_BLOCKS = blocks wanted per launch, RWKV_GEMM_KC = 128 or 256 (chunk of K).
+static int env_int(const char* name, int fallback) {
+  const char* e = getenv(name);
+  const int v = e ? atoi(e) : 0;
+  return v > 0 ? v : fallback;
+}
+static int target_blocks() {
+  static const int v = env_int("RWKV_GEMM_BLOCKS", 512);
+  return v;
+}
+static int chunk_k(int mt) {
+  static const int v = env_int("RWKV_GEMM_KC", 0);
+  if (v == 128 || (v == 256 && mt < 4)) return v;
+  return mt >= 4 ? 128 : 256;  // two X tiles stay within 36-70 KiB of LDS
+}
+
+// Split count: a power of two that gives enough blocks to occupy the CUs, K slices whole chunks.
+static int choose_splits(int M, int col_blocks, int K) {
+  const int mt = row_tiles(M);
+  const int kc = chunk_k(mt);
+  const int tiles = ceil_div(M, 32 * mt) * col_blocks;
+  int splits = 1;
+  while (tiles * splits < target_blocks() && K % (splits * 2 * kc) == 0 && splits < 32) splits *= 2;
+  return splits;
+}
+
+size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const int* Ns) {
+  int col_blocks = 0;
+  int64_t n_total = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    col_blocks += ceil_div(Ns[i], 128);
+    n_total += Ns[i];
+  }
+  const int splits = choose_splits(M, col_blocks, K);
+  return splits > 1 ? static_cast<size_t>(splits) * M * n_total * sizeof(float) : 0;
+}
+
+size_t linear_packed_workspace_bytes(int M, int N, int K) { return linear_packed_multi_workspace_bytes(M, K, 1, &N); }
+
+int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const PackedProblem* problems, int epilogue,
+                        int out_f32, void* workspace, size_t workspace_bytes) {
+  RWKV_REQUIRE(n_problems >= 1 && n_problems <= kMaxProblems, "linear_packed: %d problems (1..%d allowed)", n_problems,
+               kMaxProblems);
+  StreamArgs g;
+  ReduceArgs r;
+  g.n_problems = r.n_problems = n_problems;
+  g.M = r.M = M;
+  g.K = K;
+  g.epilogue = r.epilogue = epilogue;
+  g.out_f32 = r.out_f32 = out_f32;
+  int col_blocks = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    const PackedProblem& q = problems[i];
+    RWKV_REQUIRE(linear_packed_supported(q.fmt, M, q.N, K), "linear_packed: unsupported shape M=%d N=%d K=%d fmt=%d", M,
+                 q.N, K, q.fmt);
+    RWKV_REQUIRE(q.x && q.packed && q.y, "linear_packed: NULL tensor");
+    RWKV_REQUIRE(q.fmt == RWKV_FMT_F16 || q.scale, "linear_packed: quantised weights need a scale tensor");
+    RWKV_REQUIRE(q.fmt != RWKV_FMT_W4 || q.zp, "linear_packed: W4 weights need a zero-point tensor");
+    col_blocks += ceil_div(q.N, 128);
+    g.block_end[i] = col_blocks;
+    g.p[i] = StreamProblem{q.x, static_cast<const uint4_t*>(q.packed), q.scale, q.zp, q.y, nullptr, q.N, q.fmt};
+  }
+  const int mt = row_tiles(M);
+  const int kc = chunk_k(mt);
+  g.splits = r.splits = choose_splits(M, col_blocks, K);
+  g.k_per_split = K / g.splits;
+  if (g.splits > 1) {
+    size_t need = 0;
+    for (int i = 0; i < n_problems; ++i) need += static_cast<size_t>(g.splits) * M * problems[i].N * sizeof(float);
+    RWKV_REQUIRE(workspace && workspace_bytes >= need, "linear_packed: workspace of %zu bytes needed, got %zu", need,
+                 workspace_bytes);
+    float* at = static_cast<float*>(workspace);
+    int red_blocks = 0;
+    for (int i = 0; i < n_problems; ++i) {
+      g.p[i].partial = at;
+      const int64_t plane4 = static_cast<int64_t>(M) * problems[i].N / 4;
+      red_blocks += static_cast<int>((plane4 + 255) / 256);
+      r.block_end[i] = red_blocks;
+      r.p[i] = ReduceProblem{reinterpret_cast<const float4_t*>(at),
+                             problems[i].fmt == RWKV_FMT_W8 ? problems[i].scale : nullptr, problems[i].y, problems[i].N / 4};
+      at += static_cast<size_t>(g.splits) * M * problems[i].N;
+    }
+  }
+  const dim3 grid(ceil_div(M, 32 * mt), col_blocks, g.splits);
+  if (mt == 1 && kc == 128) hipLaunchKernelGGL((gemm_stream_kernel<1, 128>), grid, dim3(256), 0, st, g);
+  else if (mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 256>), grid, dim3(256), 0, st, g);
+  else if (mt == 2 && kc == 128) hipLaunchKernelGGL((gemm_stream_kernel<2, 128>), grid, dim3(256), 0, st, g);
+  else if (mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 256>), grid, dim3(256), 0, st, g);
+  else hipLaunchKernelGGL((gemm_stream_kernel<4, 128>), grid, dim3(256), 0, st, g);
+  RWKV_LAUNCH_CHECK();
+  if (g.splits == 1) return RWKV_OK;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3(r.block_end[n_problems - 1]), dim3(256), 0, st, r);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+int linear_packed(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* packed, const half_t* scale,
+                  const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes) {
+  const PackedProblem q = {packed, scale, zp, x, y, N, fmt};
+  return linear_packed_multi(st, M, K, 1, &q, epilogue, out_f32, workspace, workspace_bytes);
+}
+
+}  // namespace rwkv
+
+using namespace rwkv;
+
+extern "C" {
+
+int rwkv_hip_pack_weights(rwkv_stream_t s, int fmt, int N, int K, const void* w, void* packed) {
+  return pack_weights_launch(as_stream(s), fmt, N, K, w, packed);
+}
+
+int rwkv_hip_linear_packed_workspace(int M, int N, int K, size_t* bytes) {
+  RWKV_REQUIRE(bytes && M > 0 && N > 0 && K > 0, "linear_packed_workspace: bad arguments");
+  *bytes = linear_packed_workspace_bytes(M, N, K);
+  return RWKV_OK;
+}
+
+int rwkv_hip_linear_packed(rwkv_stream_t s, int fmt, int M, int N, int K, const void* x, const void* packed,
+                           const void* scale, const void* zp, int epilogue, int out_f32, void* y, void* workspace,
+                           size_t workspace_bytes) {
+  RWKV_REQUIRE(epilogue == RWKV_EPI_NONE || epilogue == RWKV_EPI_RELU_SQUARE, "linear_packed: bad epilogue %d", epilogue);
+  return linear_packed(as_stream(s), fmt, M, N, K, static_cast<const half_t*>(x), packed,
+                       static_cast<const half_t*>(scale), static_cast<const uint8_t*>(zp), epilogue, out_f32, y, workspace,
+                       workspace_bytes);
+}
+
+}  // extern "C"

@@ -22,11 +22,13 @@ struct Matrix {
   const void* data = nullptr;
   const half_t* scale = nullptr;
   const uint8_t* zp = nullptr;
+  void* packed = nullptr;  // owned: the same codes in the MFMA-native order, for calls with >= 16 rows
 };
 
 struct Layer {
   const half_t* t[64] = {nullptr};
   Matrix m[6];
+  void* lora_in_packed[4] = {nullptr, nullptr, nullptr, nullptr};  // owned: W1, A1, G1, V1 in the MFMA-native order
 };
 
 struct rwkv_hip_model {
@@ -36,6 +38,16 @@ struct rwkv_hip_model {
   const half_t* ln_out_b = nullptr;
   Matrix head;
   std::vector<Layer> layers;
+
+  ~rwkv_hip_model() {
+    if (head.packed) (void)hipFree(head.packed);
+    for (Layer& l : layers) {
+      for (Matrix& mat : l.m)
+        if (mat.packed) (void)hipFree(mat.packed);
+      for (void* q : l.lora_in_packed)
+        if (q) (void)hipFree(q);
+    }
+  }
 };
 
 namespace {
@@ -52,6 +64,7 @@ struct GraphEntry {
 };
 
 constexpr size_t kMaxGraphs = 8;
+constexpr size_t kPackedMinRows = 16;  // calls with at least this many rows stream the packed copy through MFMA
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -95,6 +108,8 @@ struct rwkv_hip_session {
   uint64_t tick = 0;
   bool profile = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;
+  void* gemm_ws = nullptr;  // split-K partials of the packed GEMM
+  size_t gemm_ws_bytes = 0;
 };
 
 namespace {
@@ -187,6 +202,29 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
     s->arena_B = B;
     s->arena_T = T;
   }
+  if (rows >= kPackedMinRows) {
+    const int R = static_cast<int>(rows);
+    const int qkv_ns[7] = {m->C, m->C, m->C, m->Rw, m->Ra, m->Rg, m->Rv};
+    size_t ws = std::max(linear_packed_multi_workspace_bytes(R, m->C, 7, qkv_ns),
+                         linear_packed_multi_workspace_bytes(R, m->C, 6, qkv_ns));  // layer 0 has no v rank-in
+    ws = std::max(ws, linear_packed_workspace_bytes(R, m->C, m->C));
+    ws = std::max(ws, linear_packed_workspace_bytes(R, m->F, m->C));
+    ws = std::max(ws, linear_packed_workspace_bytes(R, m->C, m->F));
+    ws = std::max(ws, linear_packed_workspace_bytes(B, m->V, m->C));
+    if (ws > s->gemm_ws_bytes) {
+      for (auto& g : s->graphs) {
+        if (g.exec) (void)hipGraphExecDestroy(g.exec);
+        if (g.graph) (void)hipGraphDestroy(g.graph);
+      }
+      s->graphs.clear();
+      RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+      if (s->gemm_ws) RWKV_HIP_TRY(hipFree(s->gemm_ws));
+      s->gemm_ws = nullptr;
+      s->gemm_ws_bytes = 0;
+      RWKV_HIP_TRY(hipMalloc(&s->gemm_ws, ws));
+      s->gemm_ws_bytes = ws;
+    }
+  }
   if (static_cast<int>(rows) > s->tokens_cap) {
     RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
     if (s->tokens_dev) RWKV_HIP_TRY(hipFree(s->tokens_dev));
@@ -201,9 +239,13 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
   return RWKV_OK;
 }
 
-int apply_matrix(hipStream_t st, const Matrix& mat, int M, int N, int K, const half_t* x, int epilogue, int out_f32,
-                 void* y) {
-  return linear_any_m(st, mat.fmt, M, N, K, x, mat.data, mat.scale, mat.zp, epilogue, out_f32, y);
+int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int K, const half_t* x, int epilogue,
+                 int out_f32, void* y) {
+  if (M >= kPackedMinRows && mat.packed) {
+    return linear_packed(s->stream, mat.fmt, M, N, K, x, mat.packed, mat.scale, mat.zp, epilogue, out_f32, y, s->gemm_ws,
+                         s->gemm_ws_bytes);
+  }
+  return linear_any_m(s->stream, mat.fmt, M, N, K, x, mat.data, mat.scale, mat.zp, epilogue, out_f32, y);
 }
 
 #define TRY(expr)                  \
@@ -308,10 +350,23 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         }
         TRY_PROF(linear_small_m(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0));
       } else {
-        for (int i = 0; i < 3; ++i) TRY_PROF(apply_matrix(st, w.m[mids[i]], rows, C, C, xs[i], RWKV_EPI_NONE, 0, ys[i]));
-        for (int i = 0; i < n_lora; ++i)
-          TRY(linear_any_m(st, RWKV_FMT_F16, rows, ranks[i], C, lx[i], w.t[w1_ids[i]], nullptr, nullptr, RWKV_EPI_NONE,
-                           0, lh[i]));
+        bool all_packed = rows >= static_cast<int>(kPackedMinRows);
+        for (int i = 0; i < 3; ++i) all_packed = all_packed && w.m[mids[i]].packed != nullptr;
+        for (int i = 0; i < n_lora; ++i) all_packed = all_packed && w.lora_in_packed[i] != nullptr;
+        if (all_packed) {
+          // one streaming-GEMM launch (+ one split-K reduce) for the three projections and the rank-ins
+          PackedProblem p[7];
+          for (int i = 0; i < 3; ++i)
+            p[i] = PackedProblem{w.m[mids[i]].packed, w.m[mids[i]].scale, w.m[mids[i]].zp, xs[i], ys[i], C, w.m[mids[i]].fmt};
+          for (int i = 0; i < n_lora; ++i)
+            p[3 + i] = PackedProblem{w.lora_in_packed[i], nullptr, nullptr, lx[i], lh[i], ranks[i], RWKV_FMT_F16};
+          TRY_PROF(linear_packed_multi(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0, s->gemm_ws, s->gemm_ws_bytes));
+        } else {
+          for (int i = 0; i < 3; ++i) TRY_PROF(apply_matrix(s, w.m[mids[i]], rows, C, C, xs[i], RWKV_EPI_NONE, 0, ys[i]));
+          for (int i = 0; i < n_lora; ++i)
+            TRY(linear_any_m(st, RWKV_FMT_F16, rows, ranks[i], C, lx[i], w.t[w1_ids[i]], nullptr, nullptr, RWKV_EPI_NONE,
+                             0, lh[i]));
+        }
       }
     }
 
@@ -360,7 +415,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       TRY(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
                      w.t[RWKV_T_LNX_B], b.g, b.y2));
     }
-    TRY_PROF(apply_matrix(st, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
+    TRY_PROF(apply_matrix(s, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
 
     // residual add + LN2 + channel-mix token shift
     if (step) {
@@ -380,8 +435,8 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     }
 
     // channel mix
-    TRY_PROF(apply_matrix(st, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
-    TRY_PROF(apply_matrix(st, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+    TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
+    TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
 
     // residual add + next layer's LN1 (+ lerps), or the final LN on the last token of each row
     if (l + 1 < L) {
@@ -415,7 +470,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   }
 
   TRY(advance_launch(st, B, T, elapsed));
-  TRY_PROF(apply_matrix(st, m->head, B, V, C, b.xf, RWKV_EPI_NONE, 1, logits));
+  TRY_PROF(apply_matrix(s, m->head, B, V, C, b.xf, RWKV_EPI_NONE, 1, logits));
   return RWKV_OK;
 }
 
@@ -527,6 +582,24 @@ int rwkv_hip_model_set_tensor(rwkv_hip_model* m, int layer, int id, const void* 
   RWKV_REQUIRE((id >= RWKV_T_LN1_W && id <= RWKV_T_FFN_X_K) || (id >= RWKV_T_W1 && id <= RWKV_T_V2),
                "set_tensor: unknown tensor id %d", id);
   m->layers[layer].t[id] = p;
+  // rank-in matrices [R, C] also get a copy in the MFMA-native order for calls with many rows
+  const int w1_ids[4] = {RWKV_T_W1, RWKV_T_A1, RWKV_T_G1, RWKV_T_V1};
+  const int ranks[4] = {m->Rw, m->Ra, m->Rg, m->Rv};
+  for (int i = 0; i < 4; ++i) {
+    if (id != w1_ids[i]) continue;
+    void*& slot = m->layers[layer].lora_in_packed[i];
+    if (slot) {
+      RWKV_HIP_TRY(hipDeviceSynchronize());
+      RWKV_HIP_TRY(hipFree(slot));
+      slot = nullptr;
+    }
+    if (linear_packed_supported(RWKV_FMT_F16, static_cast<int>(kPackedMinRows), ranks[i], m->C)) {
+      RWKV_HIP_TRY(hipMalloc(&slot, static_cast<size_t>(ranks[i]) * m->C * 2));
+      const int rc = pack_weights_launch(nullptr, RWKV_FMT_F16, ranks[i], m->C, data, slot);
+      if (rc != RWKV_OK) return rc;
+      RWKV_HIP_TRY(hipStreamSynchronize(nullptr));
+    }
+  }
   return RWKV_OK;
 }
 
@@ -538,17 +611,34 @@ int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, con
   RWKV_REQUIRE(fmt != RWKV_FMT_W4 || zp, "set_matrix: W4 matrix needs a zero-point tensor");
   Matrix mat;
   mat.fmt = fmt; mat.data = data; mat.scale = static_cast<const half_t*>(scale); mat.zp = static_cast<const uint8_t*>(zp);
-  if (id == RWKV_M_HEAD) {
-    m->head = mat;
-    return RWKV_OK;
+  if (id != RWKV_M_HEAD) {
+    RWKV_REQUIRE(layer >= 0 && layer < m->L, "set_matrix: layer %d out of range", layer);
+    RWKV_REQUIRE(id >= 0 && id < 6, "set_matrix: unknown matrix id %d", id);
   }
-  RWKV_REQUIRE(layer >= 0 && layer < m->L, "set_matrix: layer %d out of range", layer);
-  RWKV_REQUIRE(id >= 0 && id < 6, "set_matrix: unknown matrix id %d", id);
+  const int N = id == RWKV_M_HEAD ? m->V : (id == RWKV_M_FFN_KEY ? m->F : m->C);
+  const int K = id == RWKV_M_FFN_VALUE ? m->F : m->C;
   if (fmt == RWKV_FMT_W4) {
-    const int K = (id == RWKV_M_FFN_VALUE) ? m->F : m->C;
     RWKV_REQUIRE(K % 128 == 0, "set_matrix: W4 needs the input width (%d) to be a multiple of 128", K);
   }
-  m->layers[layer].m[id] = mat;
+  Matrix& slot = id == RWKV_M_HEAD ? m->head : m->layers[layer].m[id];
+  if (slot.packed) {
+    RWKV_HIP_TRY(hipDeviceSynchronize());
+    RWKV_HIP_TRY(hipFree(slot.packed));
+    slot.packed = nullptr;
+  }
+  if (linear_packed_supported(fmt, static_cast<int>(kPackedMinRows), N, K)) {
+    // second copy of the codes in the order the MFMA path streams (batched decode and prefill)
+    const size_t bytes = fmt == RWKV_FMT_F16 ? static_cast<size_t>(N) * K * 2
+                                             : (fmt == RWKV_FMT_W8 ? static_cast<size_t>(N) * K : static_cast<size_t>(N) * K / 2);
+    RWKV_HIP_TRY(hipMalloc(&mat.packed, bytes));
+    const int rc = pack_weights_launch(nullptr, fmt, N, K, data, mat.packed);
+    if (rc != RWKV_OK) {
+      (void)hipFree(mat.packed);
+      return rc;
+    }
+    RWKV_HIP_TRY(hipStreamSynchronize(nullptr));
+  }
+  slot = mat;
   return RWKV_OK;
 }
 
@@ -602,6 +692,7 @@ int rwkv_hip_session_destroy(rwkv_hip_session* s) {
     if (g.graph) (void)hipGraphDestroy(g.graph);
   }
   if (s->arena.base) (void)hipFree(s->arena.base);
+  if (s->gemm_ws) (void)hipFree(s->gemm_ws);
   if (s->tokens_dev) (void)hipFree(s->tokens_dev);
   if (s->tokens_pinned) (void)hipHostFree(s->tokens_pinned);
   if (s->argmax_dev) (void)hipFree(s->argmax_dev);

@@ -29,6 +29,27 @@ int linear_mfma(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, c
                 const uint8_t* zp, int epilogue, int out_f32, void* y);
 bool linear_mfma_supported(int fmt, int M, int N, int K);
 
+// ---- gemm_stream.hip: weights in the MFMA-native packed order ------------------------------------------------
+bool linear_packed_supported(int fmt, int M, int N, int K);
+int pack_weights_launch(hipStream_t st, int fmt, int N, int K, const void* w, void* packed);
+// Workspace for one call: fp32 split-K partials (0 when the shape needs no split).
+size_t linear_packed_workspace_bytes(int M, int N, int K);
+int linear_packed(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* packed, const half_t* scale,
+                  const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes);
+// Up to kMaxProblems products sharing M and K (own weights, format, x, y each) in one launch (+ one reduce launch).
+struct PackedProblem {
+  const void* packed;
+  const half_t* scale;
+  const uint8_t* zp;
+  const half_t* x;
+  void* y;
+  int N;
+  int fmt;
+};
+size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const int* Ns);
+int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const PackedProblem* problems, int epilogue,
+                        int out_f32, void* workspace, size_t workspace_bytes);
+
 // ---- fused_ops.hip ------------------------------------------------------------------------------
 enum LnMode {
   kLn = 0,          // y = LN(x)

@@ -33,7 +33,8 @@ EXPORTS = [
     "rwkv_hip_mem_info", "rwkv_hip_stream_create", "rwkv_hip_stream_destroy", "rwkv_hip_stream_sync",
     "rwkv_hip_device_sync", "rwkv_hip_event_create", "rwkv_hip_event_destroy", "rwkv_hip_event_record",
     "rwkv_hip_event_elapsed_ms", "rwkv_hip_wkv7", "rwkv_hip_quantize_w8", "rwkv_hip_dequant_w8",
-    "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
+    "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",
+    "rwkv_hip_pack_weights", "rwkv_hip_linear_packed_workspace", "rwkv_hip_linear_packed", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
     "rwkv_hip_layer_norm", "rwkv_hip_add_layer_norm", "rwkv_hip_add_last_layer_norm", "rwkv_hip_token_shift_mix",
     "rwkv_hip_add_layer_norm_cmix_mix", "rwkv_hip_add_layer_norm_tmix_mix6", "rwkv_hip_kk_a_gate",
     "rwkv_hip_lnx_rkvres_xg", "rwkv_hip_relu_square", "rwkv_hip_add_vec", "rwkv_hip_f16_to_f32",
@@ -213,6 +214,22 @@ def fill_normal_f16(n, seed, mean, std, out, stream=None):
 def linear(fmt, M, N, K, x, w, scale, zp, y, epilogue=EPI_NONE, out_f32=0, stream=None):
     check(load().rwkv_hip_linear(_p(stream), _i(fmt), _i(M), _i(N), _i(K), _p(x), _p(w), _p(scale), _p(zp),
                                  _i(epilogue), _i(out_f32), _p(y)))
+
+
+def pack_weights(fmt, N, K, w, packed, stream=None):
+    check(load().rwkv_hip_pack_weights(_p(stream), _i(fmt), _i(N), _i(K), _p(w), _p(packed)))
+
+
+def linear_packed_workspace(M, N, K):
+    n = ctypes.c_size_t(0)
+    check(load().rwkv_hip_linear_packed_workspace(_i(M), _i(N), _i(K), ctypes.byref(n)))
+    return n.value
+
+
+def linear_packed(fmt, M, N, K, x, packed, scale, zp, y, workspace, epilogue=EPI_NONE, out_f32=0, stream=None):
+    check(load().rwkv_hip_linear_packed(_p(stream), _i(fmt), _i(M), _i(N), _i(K), _p(x), _p(packed), _p(scale), _p(zp),
+                                        _i(epilogue), _i(out_f32), _p(y), _p(workspace),
+                                        ctypes.c_size_t(workspace.nbytes if workspace is not None else 0)))
 
 
 def lora_in(M, C, R, x, w1, h, stream=None):

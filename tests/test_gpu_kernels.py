@@ -370,3 +370,105 @@ def test_small_elementwise(gpu, orc):
     same = np.array_equal(o32.numpy(), x.astype(np.float32))
     assert same
     assert e.numpy().tolist() == [131, 137]
+
+
+# ----------------------------------------------------------------------------- packed-weight MFMA GEMM
+def _quant_parts(orc, hip, fmt, w):
+    if fmt == hip.FMT_F16:
+        return (w, None, None)
+    if fmt == hip.FMT_W8:
+        return orc.quantize_w8(w) + (None,)
+    return orc.quantize_w4(w)
+
+
+@pytest.mark.parametrize("fmt_name", ["f16", "w8", "w4"])
+@pytest.mark.parametrize("M,N,K", [(16, 128, 512), (33, 96, 256), (64, 256, 1024), (128, 160, 2048), (200, 64, 768),
+                                   (17, 4096, 256)])
+def test_linear_packed_matches_oracle(gpu, orc, fmt_name, M, N, K):
+    """Every row-tile variant (M <= 32, <= 64, > 64, several row tiles), with and without K splits, ragged M and
+    a column count that is not a multiple of the 128-column block."""
+    hip = gpu
+    if fmt_name == "w4" and K % 128:
+        pytest.skip("W4 groups are 128 wide")
+    rng = np.random.default_rng(M * 7 + N + K)
+    fmt = {"f16": hip.FMT_F16, "w8": hip.FMT_W8, "w4": hip.FMT_W4}[fmt_name]
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    parts = _quant_parts(orc, hip, fmt, w)
+    y_ref = orc.gemv(fmt, x, parts[0], parts[1], parts[2])
+    dparts = [dev(hip, p) if p is not None else None for p in parts]
+    packed = hip.DeviceArray(parts[0].shape, parts[0].dtype)
+    hip.pack_weights(fmt, N, K, dparts[0], packed)
+    ws = hip.DeviceArray((max(hip.linear_packed_workspace(M, N, K), 16),), np.uint8)
+    y = hip.DeviceArray((M, N), np.float16)
+    first = None
+    for _ in range(2):
+        y.fill0()
+        hip.linear_packed(fmt, M, N, K, dev(hip, x), packed, dparts[1], dparts[2], y, ws)
+        hip.device_sync()
+        got = y.numpy()
+        err = rel_err(got.astype(np.float32), y_ref.astype(np.float32))
+        assert err <= F16_TOL
+        if first is not None:   # split partials are summed in a fixed order: repeat calls agree bitwise
+            same = np.array_equal(first.view(np.uint16), got.view(np.uint16))
+            assert same
+        first = got
+    # relu^2 epilogue and fp32 output
+    y32 = hip.DeviceArray((M, N), np.float32)
+    hip.linear_packed(fmt, M, N, K, dev(hip, x), packed, dparts[1], dparts[2], y32, ws, out_f32=1)
+    hip.linear_packed(fmt, M, N, K, dev(hip, x), packed, dparts[1], dparts[2], y, ws, epilogue=hip.EPI_RELU_SQUARE)
+    hip.device_sync()
+    got32 = y32.numpy()
+    err = rel_err(got32, y_ref.astype(np.float32))
+    assert err <= F16_TOL
+    same = np.array_equal(got32, got32.astype(np.float16).astype(np.float32))
+    assert same
+    err = rel_err(y.numpy().astype(np.float32), orc.relu_square(y_ref).astype(np.float32))
+    assert err <= 2 * F16_TOL
+
+
+def test_pack_weights_is_the_documented_permutation(gpu):
+    """Tile (band nt, k group kg) holds, for lane j + 32h, the KR consecutive k of row 32 nt + j starting at
+    kg*G + h*KR, as 64 x 16-byte pieces (two pieces for fp16)."""
+    hip = gpu
+    rng = np.random.default_rng(4)
+    N, K = 64, 512
+    for fmt, dtype, per, G, pieces in ((hip.FMT_F16, np.float16, 8, 32, 2), (hip.FMT_W8, np.int8, 16, 32, 1),
+                                       (hip.FMT_W4, np.uint8, 32, 64, 1)):
+        cols = K if fmt != hip.FMT_W4 else K // 2
+        if dtype == np.float16:
+            src = rng.standard_normal((N, cols)).astype(dtype)
+        else:
+            src = rng.integers(-128 if dtype == np.int8 else 0, 127, (N, cols)).astype(dtype)
+        packed = hip.DeviceArray(src.shape, src.dtype)
+        hip.pack_weights(fmt, N, K, dev(hip, src), packed)
+        hip.device_sync()
+        got = packed.numpy().view(np.uint8).reshape(-1, 16)
+        src_pieces = src.view(np.uint8).reshape(-1, 16)        # row-major 16-byte pieces
+        KR = G // 2
+        want = np.empty_like(got)
+        p = 0
+        for nt in range(N // 32):
+            for kg in range(K // G):
+                for i in range(pieces):
+                    for lane in range(64):
+                        row, h = nt * 32 + lane % 32, lane // 32
+                        k = kg * G + h * KR + i * 8
+                        want[p] = src_pieces[(row * K + k) // per]
+                        p += 1
+        same = np.array_equal(got, want)
+        assert same
+
+
+def test_linear_packed_rejects_bad_arguments(gpu):
+    hip = gpu
+    x = hip.DeviceArray((16, 256), np.float16)
+    ws = hip.DeviceArray((8192,), np.uint8)
+    with pytest.raises(hip.RwkvHipError, match="unsupported shape"):
+        hip.linear_packed(hip.FMT_W8, 16, 48, 256, x, x, x, None, x, ws)      # N not a multiple of 32
+    with pytest.raises(hip.RwkvHipError, match="unsupported shape"):
+        hip.linear_packed(hip.FMT_W8, 16, 64, 320, x, x, x, None, x, ws)      # K not a multiple of 256
+    with pytest.raises(hip.RwkvHipError, match="scale"):
+        hip.linear_packed(hip.FMT_W8, 16, 64, 256, x, x, None, None, x, ws)
+    with pytest.raises(hip.RwkvHipError, match="workspace"):
+        hip.linear_packed(hip.FMT_F16, 16, 64, 4096, x, x, None, None, x, None)  # split K without a workspace
