@@ -281,6 +281,10 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   const int64_t RC = static_cast<int64_t>(rows) * C;
   const bool step = (T == 1);
   const bool small = rows <= 8;
+  // The single-launch time-mix core re-reads a head's LoRA rows for every batch row; with many rows the
+  // row-tiled kernels of the prefill path (LoRA rows shared by 16 rows) move less data; measured crossover
+  // between 32 and 64 rows.
+  const bool fused_tmix = step && rows <= 32;
 
   auto mix6_args = [&](const Layer& w, LnArgs& a) {
     const int ids[6] = {RWKV_T_X_R, RWKV_T_X_W, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_A, RWKV_T_X_G};
@@ -370,7 +374,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       }
     }
 
-    if (step) {
+    if (fused_tmix) {
       // the whole time-mix core of a decode step in one launch per layer
       TmixStepArgs p = {};
       p.B = B; p.H = H; p.C = C; p.Rw = m->Rw; p.Ra = m->Ra; p.Rg = m->Rg; p.Rv = m->Rv;
