@@ -44,14 +44,25 @@ __global__ __launch_bounds__(256) void wkv7_prepare_kernel(int64_t n, int64_t sl
 }
 
 // ---- sequence kernel -------------------------------------------------------------------------
-// grid = B*H, block = 64.  r,d,k,a,b: fp32, `op_bs` elements between batch rows, read with
-// wave-uniform addresses; v,y: IO, `io_bs` elements between batch rows.  Runs T tokens.
+// grid = B*H, block = 64 (one wavefront per head): lane i owns row i of the 64x64 state in 64 VGPRs for the
+// whole call.  r,d,k,a,b are fp32 with `op_bs` elements between batch rows; v,y are IO with `io_bs` elements
+// between batch rows.  The five operand vectors of a token are the same for every lane, so they go through
+// LDS: the wavefront stages them kSeqChunk tokens at a time with coalesced 16-byte loads (4 tokens x 256 bytes
+// per load instruction), double-buffered, and each step reads them back as broadcast 16-byte LDS reads that
+// the scheduler overlaps with the 256 FMAs of the step.  The loads of chunk c+1 are in flight while chunk c
+// computes.  Each lane keeps its own v values of the chunk in registers.  The arithmetic of a step does not
+// depend on the chunking, so splitting T over several calls is bitwise neutral.
+constexpr int kSeqChunk = 8;
+
 template <typename IO>
-__global__ __launch_bounds__(64) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void wkv7_seq_kernel(
+    int T, int C, int H, float* __restrict__ state,
                                                       const float* __restrict__ r, const float* __restrict__ d,
                                                       const float* __restrict__ k, const float* __restrict__ a,
                                                       const float* __restrict__ b, int64_t op_bs,
                                                       const IO* __restrict__ v, IO* __restrict__ y, int64_t io_bs) {
+  __shared__ __align__(16) float ops[2][5][kSeqChunk][kHead];  // [buffer][a,b,d,k,r][token][column]
+
   const int bh = blockIdx.x;
   const int bi = bh / H;
   const int h = bh - bi * H;
@@ -65,34 +76,109 @@ __global__ __launch_bounds__(64) void wkv7_seq_kernel(int T, int C, int H, float
     S[j] = q.x; S[j + 1] = q.y; S[j + 2] = q.z; S[j + 3] = q.w;
   }
 
-  int64_t base = static_cast<int64_t>(bi) * op_bs + h * kHead;  // wave-uniform
-  int64_t iob = static_cast<int64_t>(bi) * io_bs + h * kHead + lane;
-  float vi = static_cast<float>(v[iob]);
-  for (int t = 0; t < T; ++t) {
-    const float* __restrict__ ap = a + base;
-    const float* __restrict__ bp = b + base;
-    const float* __restrict__ dp = d + base;
-    const float* __restrict__ kp = k + base;
-    const float* __restrict__ rp = r + base;
-    // prefetch the next token's v (per-lane) while this token computes
-    float v_next = 0.0f;
-    if (t + 1 < T) v_next = static_cast<float>(v[iob + C]);
+  const int64_t base = static_cast<int64_t>(bi) * op_bs + h * kHead;
+  const float* src[5] = {a + base, b + base, d + base, k + base, r + base};
+  const int64_t iob = static_cast<int64_t>(bi) * io_bs + h * kHead + lane;
+  const int st_tok = lane >> 4;        // staging: this lane's token within a group of 4 ...
+  const int st_col = (lane & 15) * 4;  // ... and its 4 columns
 
-    float sa = 0.0f;
+  float4_t stage[5][kSeqChunk / 4];
+  float v_next[kSeqChunk], v_cur[kSeqChunk];
+
+  auto request = [&](int t0) {
 #pragma unroll
-    for (int j = 0; j < kHead; ++j) sa = fmaf(S[j], ap[j], sa);
-    float yy = 0.0f;
+    for (int o = 0; o < 5; ++o)
 #pragma unroll
-    for (int j = 0; j < kHead; ++j) {
-      float s = S[j];
-      s = fmaf(s, dp[j], fmaf(sa, bp[j], kp[j] * vi));
-      yy = fmaf(s, rp[j], yy);
-      S[j] = s;
+      for (int i = 0; i < kSeqChunk / 4; ++i) {
+        const int t = t0 + st_tok + 4 * i;
+        stage[o][i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (t < T) stage[o][i] = *reinterpret_cast<const float4_t*>(src[o] + static_cast<int64_t>(t) * C + st_col);
+      }
+#pragma unroll
+    for (int tt = 0; tt < kSeqChunk; ++tt) {
+      v_next[tt] = 0.0f;
+      if (t0 + tt < T) v_next[tt] = static_cast<float>(v[iob + static_cast<int64_t>(t0 + tt) * C]);
     }
-    y[iob] = static_cast<IO>(yy);
-    vi = v_next;
-    base += C;
-    iob += C;
+  };
+  auto commit = [&](int buf) {
+#pragma unroll
+    for (int o = 0; o < 5; ++o)
+#pragma unroll
+      for (int i = 0; i < kSeqChunk / 4; ++i)
+        *reinterpret_cast<float4_t*>(&ops[buf][o][st_tok + 4 * i][st_col]) = stage[o][i];
+#pragma unroll
+    for (int tt = 0; tt < kSeqChunk; ++tt) v_cur[tt] = v_next[tt];
+  };
+
+  request(0);
+  commit(0);
+  __syncthreads();
+  for (int t0 = 0; t0 < T; t0 += kSeqChunk) {
+    const int buf = (t0 / kSeqChunk) & 1;
+    const bool more = t0 + kSeqChunk < T;
+    if (more) request(t0 + kSeqChunk);
+    const int n = min(kSeqChunk, T - t0);
+    // Operand reads are software-pipelined by hand (the compiler otherwise issues each LDS read right before
+    // its use and stalls on every one): the a vector of a step and its first column group are requested during
+    // the previous step; inside a step the reads of column group g+1 are issued before group g computes.
+    // __builtin_amdgcn_sched_barrier(0) keeps the scheduler from sinking the reads back down.
+    float4_t A[kHead / 4];
+    float4_t G[2][8];  // per group of 8 columns: b, d, k, r as two float4 each
+    auto load_a = [&](int tt, int lo, int hi) {
+#pragma unroll
+      for (int j4 = lo; j4 < hi; ++j4) A[j4] = *reinterpret_cast<const float4_t*>(&ops[buf][0][tt][4 * j4]);
+    };
+    auto load_group = [&](int tt, int g, float4_t (&dst)[8]) {
+#pragma unroll
+      for (int o = 0; o < 4; ++o) {
+        dst[2 * o] = *reinterpret_cast<const float4_t*>(&ops[buf][1 + o][tt][8 * g]);
+        dst[2 * o + 1] = *reinterpret_cast<const float4_t*>(&ops[buf][1 + o][tt][8 * g + 4]);
+      }
+    };
+    load_a(0, 0, kHead / 4);
+    load_group(0, 0, G[0]);
+#pragma unroll
+    for (int tt = 0; tt < kSeqChunk; ++tt) {
+      if (tt < n) {
+        const float vi = v_cur[tt];
+        float sa = 0.0f;
+#pragma unroll
+        for (int j4 = 0; j4 < kHead / 4; ++j4) {
+          sa = fmaf(S[4 * j4 + 0], A[j4].x, sa);
+          sa = fmaf(S[4 * j4 + 1], A[j4].y, sa);
+          sa = fmaf(S[4 * j4 + 2], A[j4].z, sa);
+          sa = fmaf(S[4 * j4 + 3], A[j4].w, sa);
+        }
+        float yy = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+          // requests for later use: next column group (or the next step's first one), a slice of the next a vector
+          if (g + 1 < 8) {
+            load_group(tt, g + 1, G[(g + 1) & 1]);
+          } else if (tt + 1 < kSeqChunk) {
+            load_group(tt + 1, 0, G[0]);
+          }
+          if (tt + 1 < kSeqChunk) load_a(tt + 1, 2 * g, 2 * g + 2);
+          __builtin_amdgcn_sched_barrier(0);
+          const float4_t(&q)[8] = G[g & 1];
+          const float bb[8] = {q[0].x, q[0].y, q[0].z, q[0].w, q[1].x, q[1].y, q[1].z, q[1].w};
+          const float dd[8] = {q[2].x, q[2].y, q[2].z, q[2].w, q[3].x, q[3].y, q[3].z, q[3].w};
+          const float kk[8] = {q[4].x, q[4].y, q[4].z, q[4].w, q[5].x, q[5].y, q[5].z, q[5].w};
+          const float rr[8] = {q[6].x, q[6].y, q[6].z, q[6].w, q[7].x, q[7].y, q[7].z, q[7].w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float sv = S[8 * g + e];
+            sv = fmaf(sv, dd[e], fmaf(sa, bb[e], kk[e] * vi));
+            yy = fmaf(sv, rr[e], yy);
+            S[8 * g + e] = sv;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        y[iob + static_cast<int64_t>(t0 + tt) * C] = static_cast<IO>(yy);
+      }
+    }
+    if (more) commit(buf ^ 1);
+    __syncthreads();
   }
 
 #pragma unroll
