@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
-"""Headline benchmark: RWKV-7 7.2B-shape W8A16 greedy decode at batch 1 on one MI355X.
+"""Headline benchmark: RWKV-7 7.2B-shape W8A16 greedy decode at batch 1 on one MI355X, after a 4096-token
+prefill in chunks of 128.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--preset 7.2B] [--fmt w8] [--batch 1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--preset 7.2B] [--fmt w8] [--batch 1] [--prefill 4096]
 
 One "step" is one decode step of the whole model: embedding row -> 32 layers -> lm_head -> argmax, with the
 argmax fed back on the device (no host round trip).  Weights are random-init N(0, 0.02) generated and
@@ -9,7 +10,10 @@ quantised on the GPU; inputs are resident in HBM before the timed region.  Print
 whole-job tokens/s plus
   roofline     -- the weight-streaming GEMV kernel against the 8 TB/s HBM peak: algorithmic bytes per
                   launch / average launch duration from HIP events on the session stream
-  cpu_baseline -- the scalar C++ oracle timed on the host cores on a bounded slice of the same workload.
+  cpu_baseline -- the scalar C++ oracle timed on the host cores on a bounded slice of the same workload
+  also         -- the other figures the metric names, measured in the same run: prefill tokens/s of the
+                  4096-token prompt (and the MFMA fraction of its GEMM launches), batch-64 decode tokens/s,
+                  and the WKV7 op alone on a long sequence.
 """
 import argparse
 import json
@@ -22,19 +26,29 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak, published
+# HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled
+# by what the same counter reads for a 1 GiB device-to-device copy (FETCH_SIZE reads half the bytes copied,
+# WRITE_SIZE all of them); the summary of those runs is kept under profiles/.  Keyed by (preset, format, batch).
+MEASURED_TRAFFIC = {("7.2B", "w8", 1): 2.0 * 26445.1 * 1024 + 1.0 * 38.5 * 1024}
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--preset", default="7.2B")
     ap.add_argument("--fmt", default="w8", choices=["f16", "w8", "w4"])
     ap.add_argument("--batch", type=int, default=1)
-    ap.add_argument("--prefill", type=int, default=64, help="tokens prefilled (chunk 128) before the decode loop")
+    ap.add_argument("--prefill", type=int, default=4096, help="tokens prefilled (chunk 128) before the decode loop")
+    ap.add_argument("--no-also", action="store_true", help="skip the secondary measurements (prefill MFMA fraction, "
+                    "batch-64 decode, WKV7 op)")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps eagerly instead of replaying a HIP graph")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
+                    help="only run a device-to-device copy of BYTES (twice) and exit: the known-size kernel that "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     return ap.parse_args()
@@ -104,6 +118,56 @@ def cpu_baseline(dims, fmt_name):
     }
 
 
+def secondary_measurements(hip, model, dims, rng):
+    """Batch-64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7 op alone."""
+    from rwkv_lightning_cuda_amd.model import Session, State
+    res = {}
+    B = 64
+    sess = Session(model)
+    state = State(dims, B)
+    logits = hip.DeviceArray((B, dims.V), np.float32)
+    sess.forward(rng.integers(0, dims.V, (B, 128)), state, logits)
+    first = rng.integers(0, dims.V, (B,))
+    sess.decode_greedy(first, 8, state, logits)
+    hip.device_sync()
+    t0 = time.perf_counter()
+    steps = 64
+    sess.decode_greedy(first, steps, state, logits)
+    hip.device_sync()
+    dt = time.perf_counter() - t0
+    state_bytes = B * (2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2)
+    res["decode_bs64_tok_s"] = steps * B / dt
+    res["decode_bs64_ms_per_step"] = dt * 1e3 / steps
+    res["decode_bs64_hbm_fraction"] = (model.weight_bytes() + state_bytes) / (dt / steps) / 1e9 / HBM_PEAK_GBPS
+    sess.close()
+    del state, logits
+
+    # WKV7 op alone: fp16 r,w,k,v,a,b [B,T,C], fp32 state, raw-logit decay, one call
+    Bw, Tw, H = 16, 2048, dims.H
+    C = H * 64
+    n = Bw * Tw * C
+    bufs = []
+    for i in range(7):
+        d = hip.DeviceArray((Bw, Tw, C), np.float16)
+        hip.fill_normal_f16(n, 100 + i, 0.0, 0.5, d)
+        bufs.append(d)
+    wstate = hip.DeviceArray.zeros((Bw, H, 64, 64), np.float32)
+    r, w, k, v, a, b, y = bufs
+    hip.wkv7(Bw, Tw, C, H, hip.W_RAW_LOGIT, hip.IO_F16, wstate, r, w, k, v, a, b, y)
+    hip.device_sync()
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record()
+    hip.wkv7(Bw, Tw, C, H, hip.W_RAW_LOGIT, hip.IO_F16, wstate, r, w, k, v, a, b, y)
+    e1.record()
+    hip.device_sync()
+    ms = e0.elapsed_ms(e1)
+    res["wkv7_op"] = {"workload": "B=%d T=%d H=%d N=64, fp16 io, fp32 state, one call" % (Bw, Tw, H),
+                      "tok_s": Bw * Tw / (ms * 1e-3), "ms": ms,
+                      "fp32_tflops": Bw * Tw * H * 10.0 * 64 * 64 / (ms * 1e-3) / 1e12,
+                      "io_gb_s": n * 7 * 2 / (ms * 1e-3) / 1e9, "us_per_token_step": ms * 1e3 / Tw}
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -117,6 +181,14 @@ def main():
     if hip.device_count() < 1:
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.copy_calibration > 0:
+        src = hip.DeviceArray.zeros((args.copy_calibration,), np.uint8)
+        dst = hip.DeviceArray((args.copy_calibration,), np.uint8)
+        for _ in range(2):
+            dst.copy_from(src)
+        hip.device_sync()
+        print(json.dumps({"copy_calibration_bytes": args.copy_calibration}))
+        return
     dims = PRESETS[args.preset]
     fmt = {"f16": hip.FMT_F16, "w8": hip.FMT_W8, "w4": hip.FMT_W4}[args.fmt]
     B = args.batch
@@ -128,10 +200,36 @@ def main():
     state = State(dims, B)
     logits = hip.DeviceArray((B, dims.V), np.float32)
     rng = np.random.default_rng(0)
+    also = {}
     if args.prefill > 0:
+        prompt = rng.integers(0, dims.V, (B, args.prefill))
+        warm = State(dims, B)
+        sess.forward(prompt[:, :min(128, args.prefill)], warm, logits)  # sizes the arena, warms the kernels
+        del warm
+        hip.device_sync()
+        tp = time.perf_counter()
         for t0 in range(0, args.prefill, 128):
-            tn = min(128, args.prefill - t0)
-            sess.forward(rng.integers(0, dims.V, (B, tn)), state, logits)
+            sess.forward(prompt[:, t0:t0 + 128], state, logits, sync=False)
+        hip.device_sync()
+        tp = time.perf_counter() - tp
+        also["prefill_tok_s"] = B * args.prefill / tp
+        also["prefill_workload"] = "%d-token prompt x batch %d in chunks of 128 (state carried in HBM)" % (args.prefill, B)
+        if not args.no_also and args.prefill >= 128:
+            # MFMA fraction of the chunk's GEMM launches: one more chunk, eagerly, GEMM launches bracketed by events
+            scratch = State(dims, B)
+            sess.set_profile(True)
+            sess.read_profile()
+            sess.forward(prompt[:, :128], scratch, logits, sync=False)
+            launches, total_ms = sess.read_profile()
+            sess.set_profile(False)
+            del scratch
+            rows = B * 128
+            flops = 2.0 * rows * dims.L * (4 * dims.C * dims.C + 2 * dims.C * dims.F)
+            also["prefill_gemm"] = {"bound": "mfma", "achieved": flops / (total_ms * 1e-3) / 1e12,
+                                    "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                    "frac": flops / (total_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                                    "kernel": "gemm_stream_kernel (+ split-K reduce), M = %d rows" % rows,
+                                    "launches": launches, "sum_launch_ms": total_ms}
     first = rng.integers(0, dims.V, (B,))
 
     if args.warmup > 0:
@@ -157,39 +255,50 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16 activations, fp32 accumulate, %s weights" % args.fmt,
+        "dtype": "f16",
         "data": "synthetic (random-init N(0,0.02) weights quantised on load, random token ids)",
         "config": {"workload": "RWKV-7 %s-shape greedy decode, batch %d, %d-token prefill, lm_head+argmax on device"
                                % (args.preset, B, args.prefill),
                    "L": dims.L, "C": dims.C, "H": dims.H, "F": dims.F, "V": dims.V,
-                   "weight_format": args.fmt, "hip_graph": not args.no_graph, "weight_bytes_per_step": weight_bytes,
+                   "weight_format": args.fmt, "arithmetic": "fp16 activations, fp32 accumulate, fp32 WKV state",
+                   "hip_graph": not args.no_graph, "weight_bytes_per_step": weight_bytes,
                    "state_bytes_per_step": state_bytes,
                    "step_hbm_fraction": (weight_bytes + state_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                    "distinct_tokens": int(len(np.unique(toks)))},
     }
 
     if not args.no_roofline:
-        # the same steps again, eagerly, with every weight-streaming linear launch bracketed by HIP events
-        sess.set_profile(True)
+        # The weight-streaming linear launches of the same steps alone, eagerly and back to back on the session
+        # stream, each pass bracketed by one pair of HIP events (the kernels' duration does not depend on the
+        # data; the small kernels between them are skipped so that no event sits between two launches).  All
+        # 7 GB of weights stream from HBM on every pass, exactly as in the timed run.
+        scratch_state = State(dims, B)
+        sess.set_profile(2)
         sess.read_profile()
         tok = toks[-1].reshape(B, 1).astype(np.int64)
         n_prof = min(args.steps, 32)
         for _ in range(n_prof):
-            sess.forward(tok, state, logits, sync=False)
+            sess.forward(tok, scratch_state, logits, sync=False)
         launches, total_ms = sess.read_profile()
-        sess.set_profile(False)
+        sess.set_profile(0)
+        del scratch_state
         gemv_bytes, per_step = gemv_bytes_per_step(dims, args.fmt)
         assert launches == per_step * n_prof, (launches, per_step, n_prof)
         bytes_per_launch = gemv_bytes / per_step
         avg_ms = total_ms / launches
         achieved = bytes_per_launch / (avg_ms * 1e-3) / 1e9
+        traffic = MEASURED_TRAFFIC.get((args.preset, args.fmt, B))
         out["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
             "kernel": "linear_gemv_kernel (W8A16 weight-streaming GEMV; r/k/v fused, output, ffn.key, ffn.value, lm_head)",
             "bytes_per_launch": bytes_per_launch, "avg_launch_us": avg_ms * 1e3, "launches_per_step": per_step,
         }
 
+    if not args.no_also:
+        also.update(secondary_measurements(hip, model, dims, rng))
+    if also:
+        out["also"] = also
     sess.close()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(dims, args.fmt)

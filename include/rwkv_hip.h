@@ -232,11 +232,14 @@ int rwkv_hip_forward(rwkv_hip_session* s, const int64_t* tokens_host, int B, int
  * first_tokens_host [B] are the tokens of step 0. */
 int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host, int B, int steps, void* shift,
                            void* wkv, void* elapsed, void* logits, int32_t* out_tokens_host);
-/* Measurement aid: with profiling on, forward passes run eagerly (no graph replay) and every
- * weight-streaming linear launch (r/k/v, output, ffn.key, ffn.value, lm_head) is bracketed by a pair of
- * events on the session stream; read_profile waits for the stream and returns the number of bracketed
- * launches and their summed duration since the last read. */
-int rwkv_hip_session_set_profile(rwkv_hip_session* s, int on);
+/* Measurement aid (no counterpart in the reference).  While a profiling mode is on, forward passes run
+ * eagerly (no graph replay).  Mode 1: every weight-streaming linear launch (r/k/v, output, ffn.key,
+ * ffn.value, lm_head) is bracketed by its own pair of events on the session stream.  Mode 2: a pass
+ * launches ONLY those linear kernels, back to back, with one pair of events around the pass - their
+ * duration does not depend on the data, and this gives the kernels' launch-to-launch time without event
+ * overhead between them; state and logits hold garbage afterwards.  read_profile waits for the stream
+ * and returns the number of linear launches and the summed bracketed time since the last read. */
+int rwkv_hip_session_set_profile(rwkv_hip_session* s, int mode);
 int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double* total_ms);
 /* debugging/parity tap: residual stream after every layer of the last rwkv_hip_forward call,
  * f16 [L, B*T, C], valid only if enabled before the call */

@@ -106,7 +106,8 @@ struct rwkv_hip_session {
   half_t* trace = nullptr;
   std::vector<GraphEntry> graphs;
   uint64_t tick = 0;
-  bool profile = false;
+  int profile = 0;  // 0 off, 1 event pair per linear launch, 2 linear launches only with one pair per pass
+  int64_t prof_launches = 0;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;
   void* gemm_ws = nullptr;  // split-K partials of the packed GEMM
   size_t gemm_ws_bytes = 0;
@@ -254,21 +255,30 @@ int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int
     if (rc__ != RWKV_OK) return rc__; \
   } while (0)
 
-// Profiling mode: bracket a weight-streaming linear launch with a pair of events on the session stream.
+// Profiling mode 1: bracket a weight-streaming linear launch with a pair of events on the session stream.
+// Mode 2 only counts the launch (the pass as a whole is bracketed).
 #define TRY_PROF(expr)                                              \
   do {                                                              \
     hipEvent_t e0__ = nullptr, e1__ = nullptr;                      \
-    if (s->profile) {                                               \
+    if (s->profile == 1) {                                          \
       RWKV_HIP_TRY(hipEventCreate(&e0__));                          \
       RWKV_HIP_TRY(hipEventCreate(&e1__));                          \
       RWKV_HIP_TRY(hipEventRecord(e0__, st));                       \
     }                                                               \
     const int rc__ = (expr);                                        \
-    if (s->profile) {                                               \
+    if (s->profile == 1) {                                          \
       RWKV_HIP_TRY(hipEventRecord(e1__, st));                       \
       s->prof_events.push_back(std::make_pair(e0__, e1__));         \
     }                                                               \
+    if (s->profile) ++s->prof_launches;                             \
     if (rc__ != RWKV_OK) return rc__;                               \
+  } while (0)
+
+// Every launch that is not a weight-streaming linear goes through TRY_AUX: profiling mode 2 skips them, so that
+// a pass consists of the linear launches alone, back to back (their duration does not depend on the data).
+#define TRY_AUX(expr)                \
+  do {                               \
+    if (s->profile != 2) TRY(expr);  \
   } while (0)
 
 // Enqueues the whole forward pass on the session stream.  tokens are already in s->tokens_dev.
@@ -281,6 +291,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   const int64_t RC = static_cast<int64_t>(rows) * C;
   const bool step = (T == 1);
   const bool small = rows <= 8;
+  hipEvent_t pass_begin = nullptr;
+  if (s->profile == 2) {
+    RWKV_HIP_TRY(hipEventCreate(&pass_begin));
+    RWKV_HIP_TRY(hipEventRecord(pass_begin, st));
+  }
   // The single-launch time-mix core re-reads a head's LoRA rows for every batch row; with many rows the
   // row-tiled kernels of the prefill path (LoRA rows shared by 16 rows) move less data; measured crossover
   // between 32 and 64 rows.
@@ -303,13 +318,13 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     a.w = m->layers[0].t[RWKV_T_LN1_W]; a.b = m->layers[0].t[RWKV_T_LN1_B];
     a.shift = shift; a.C = C; a.T = 1; a.eps = kLnEps;
     mix6_args(m->layers[0], a);
-    TRY(ln_launch(st, kLnMix, rows, a));
+    TRY_AUX(ln_launch(st, kLnMix, rows, a));
   } else {
-    TRY(embed_gather_launch(st, rows, C, s->tokens_dev, m->emb_ln0, b.x));
+    TRY_AUX(embed_gather_launch(st, rows, C, s->tokens_dev, m->emb_ln0, b.x));
     LnArgs a = {};
     a.x = b.x; a.w = m->layers[0].t[RWKV_T_LN1_W]; a.b = m->layers[0].t[RWKV_T_LN1_B]; a.y = b.xx;
     a.C = C; a.T = 1; a.eps = kLnEps;
-    TRY(ln_launch(st, kLn, rows, a));
+    TRY_AUX(ln_launch(st, kLn, rows, a));
   }
 
   for (int l = 0; l < L; ++l) {
@@ -328,7 +343,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         a.mu[i] = w.t[ids[i]];
         a.out[i] = outs[i];
       }
-      TRY(token_shift_mix_launch(st, a));
+      TRY_AUX(token_shift_mix_launch(st, a));
     }
 
     // r, k, v projections and the LoRA rank-ins (w, a, g and, past layer 0, v)
@@ -368,7 +383,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         } else {
           for (int i = 0; i < 3; ++i) TRY_PROF(apply_matrix(s, w.m[mids[i]], rows, C, C, xs[i], RWKV_EPI_NONE, 0, ys[i]));
           for (int i = 0; i < n_lora; ++i)
-            TRY(linear_any_m(st, RWKV_FMT_F16, rows, ranks[i], C, lx[i], w.t[w1_ids[i]], nullptr, nullptr, RWKV_EPI_NONE,
+            TRY_AUX(linear_any_m(st, RWKV_FMT_F16, rows, ranks[i], C, lx[i], w.t[w1_ids[i]], nullptr, nullptr, RWKV_EPI_NONE,
                              0, lh[i]));
         }
       }
@@ -384,22 +399,22 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       p.k_a = w.t[RWKV_T_K_A]; p.r_k = w.t[RWKV_T_R_K]; p.lnx_w = w.t[RWKV_T_LNX_W]; p.lnx_b = w.t[RWKV_T_LNX_B];
       p.r = b.r; p.k = b.k; p.v = v_cur; p.v_first = b.v_first; p.v_first_out = nullptr;
       p.state = S; p.y2 = b.y2;
-      TRY(tmix_step_launch(st, p));
+      TRY_AUX(tmix_step_launch(st, p));
     } else {
       // LoRA rank-out (+ activation, + v-residual gate)
       {
         LoraOutArgs a = {};
         a.M = rows; a.C = C;
         a.h = b.hw; a.w2 = w.t[RWKV_T_W2]; a.R = m->Rw; a.act = RWKV_ACT_TANH; a.out = b.w12;
-        TRY(lora_out_launch(st, a));
+        TRY_AUX(lora_out_launch(st, a));
         a.h = b.ha; a.w2 = w.t[RWKV_T_A2]; a.R = m->Ra; a.act = RWKV_ACT_NONE; a.out = b.a12;
-        TRY(lora_out_launch(st, a));
+        TRY_AUX(lora_out_launch(st, a));
         a.h = b.hg; a.w2 = w.t[RWKV_T_G2]; a.R = m->Rg; a.act = RWKV_ACT_SIGMOID; a.out = b.g;
-        TRY(lora_out_launch(st, a));
+        TRY_AUX(lora_out_launch(st, a));
         if (l > 0) {
           a.h = b.hv; a.w2 = w.t[RWKV_T_V2]; a.R = m->Rv; a.act = RWKV_ACT_NONE; a.bias = w.t[RWKV_T_V0];
           a.vres = 1; a.v = b.v; a.v_first = b.v_first; a.out = b.xv;  // xv is free after the projections
-          TRY(lora_out_launch(st, a));
+          TRY_AUX(lora_out_launch(st, a));
           v_cur = b.xv;
         }
       }
@@ -412,11 +427,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         p.w12 = b.w12; p.w0 = w.t[RWKV_T_W0]; p.r = b.r;
         p.k32 = b.k32; p.a32 = b.a32; p.b32 = b.b32; p.d32 = b.d32; p.r32 = b.r32;
         p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
-        TRY(kk_a_gate_launch(st, p));
+        TRY_AUX(kk_a_gate_launch(st, p));
       }
-      TRY(wkv7_seq_f16_launch(st, B, T, C, H, S, b.r32, b.d32, b.k32, b.a32, b.b32, static_cast<int64_t>(T) * C, v_cur,
+      TRY_AUX(wkv7_seq_f16_launch(st, B, T, C, H, S, b.r32, b.d32, b.k32, b.a32, b.b32, static_cast<int64_t>(T) * C, v_cur,
                               b.y, static_cast<int64_t>(T) * C));
-      TRY(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
+      TRY_AUX(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
                      w.t[RWKV_T_LNX_B], b.g, b.y2));
     }
     TRY_PROF(apply_matrix(s, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
@@ -426,16 +441,16 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       LnArgs a = {};
       a.x = b.x; a.res = b.att; a.w = w.t[RWKV_T_LN2_W]; a.b = w.t[RWKV_T_LN2_B]; a.x_out = b.x1; a.shift = shift1;
       a.mu[0] = w.t[RWKV_T_FFN_X_K]; a.out[0] = b.mixed; a.n_mix = 1; a.C = C; a.T = 1; a.eps = kLnEps;
-      TRY(ln_launch(st, kAddLnMix, rows, a));
+      TRY_AUX(ln_launch(st, kAddLnMix, rows, a));
     } else {
       LnArgs a = {};
       a.x = b.x; a.res = b.att; a.w = w.t[RWKV_T_LN2_W]; a.b = w.t[RWKV_T_LN2_B]; a.x_out = b.x1; a.y = b.ln2;
       a.C = C; a.T = 1; a.eps = kLnEps;
-      TRY(ln_launch(st, kAddLn, rows, a));
+      TRY_AUX(ln_launch(st, kAddLn, rows, a));
       MixArgs mx = {};
       mx.x = b.ln2; mx.shift = shift1; mx.B = B; mx.T = T; mx.C = C; mx.n_mix = 1;
       mx.mu[0] = w.t[RWKV_T_FFN_X_K]; mx.out[0] = b.mixed;
-      TRY(token_shift_mix_launch(st, mx));
+      TRY_AUX(token_shift_mix_launch(st, mx));
     }
 
     // channel mix
@@ -451,20 +466,20 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       if (step) {
         a.shift = shift + static_cast<int64_t>(l + 1) * 2 * B * C;
         mix6_args(nx, a);
-        TRY(ln_launch(st, kAddLnMix, rows, a));
+        TRY_AUX(ln_launch(st, kAddLnMix, rows, a));
       } else {
         a.y = b.xx;
-        TRY(ln_launch(st, kAddLn, rows, a));
+        TRY_AUX(ln_launch(st, kAddLn, rows, a));
       }
     } else {
       LnArgs a = {};
       a.x = b.x1; a.res = b.cm; a.w = m->ln_out_w; a.b = m->ln_out_b; a.y = b.xf; a.C = C; a.T = T; a.eps = kLnEps;
-      TRY(ln_launch(st, kAddLastLn, B, a));
+      TRY_AUX(ln_launch(st, kAddLastLn, B, a));
       if (s->trace) {
         LnArgs t = {};
         t.x = b.x1; t.res = b.cm; t.w = m->ln_out_w; t.b = m->ln_out_b; t.x_out = b.x; t.y = b.scratch;
         t.C = C; t.T = 1; t.eps = kLnEps;
-        TRY(ln_launch(st, kAddLn, rows, t));
+        TRY_AUX(ln_launch(st, kAddLn, rows, t));
       }
     }
     if (s->trace) {
@@ -473,8 +488,14 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     }
   }
 
-  TRY(advance_launch(st, B, T, elapsed));
+  TRY_AUX(advance_launch(st, B, T, elapsed));
   TRY_PROF(apply_matrix(s, m->head, B, V, C, b.xf, RWKV_EPI_NONE, 1, logits));
+  if (pass_begin) {
+    hipEvent_t pass_end = nullptr;
+    RWKV_HIP_TRY(hipEventCreate(&pass_end));
+    RWKV_HIP_TRY(hipEventRecord(pass_end, st));
+    s->prof_events.push_back(std::make_pair(pass_begin, pass_end));
+  }
   return RWKV_OK;
 }
 
@@ -720,7 +741,8 @@ int rwkv_hip_session_set_graph(rwkv_hip_session* s, int use_graph) {
 
 int rwkv_hip_session_set_profile(rwkv_hip_session* s, int on) {
   RWKV_REQUIRE(s, "session is NULL");
-  s->profile = on != 0;
+  RWKV_REQUIRE(on >= 0 && on <= 2, "set_profile: mode must be 0, 1 or 2");
+  s->profile = on;
   return RWKV_OK;
 }
 
@@ -735,9 +757,10 @@ int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double
     (void)hipEventDestroy(pr.first);
     (void)hipEventDestroy(pr.second);
   }
-  *launches = static_cast<int64_t>(s->prof_events.size());
+  *launches = s->prof_launches;
   *total_ms = ms;
   s->prof_events.clear();
+  s->prof_launches = 0;
   return RWKV_OK;
 }
 

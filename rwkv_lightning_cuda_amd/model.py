@@ -250,8 +250,10 @@ class Session:
         self._trace = dev
         hip.check(hip.load().rwkv_hip_session_set_trace(self.handle, hip._p(dev)))
 
-    def set_profile(self, on):
-        hip.check(hip.load().rwkv_hip_session_set_profile(self.handle, ctypes.c_int(1 if on else 0)))
+    def set_profile(self, mode):
+        """0/False off; 1/True one event pair per linear launch; 2 passes launch the linear kernels only, back to
+        back, one event pair per pass (state and logits are garbage afterwards)."""
+        hip.check(hip.load().rwkv_hip_session_set_profile(self.handle, ctypes.c_int(int(mode))))
 
     def read_profile(self):
         """(launches, total_ms) of the event-bracketed linear launches since the last read."""
