@@ -472,3 +472,36 @@ def test_linear_packed_rejects_bad_arguments(gpu):
         hip.linear_packed(hip.FMT_W8, 16, 64, 256, x, x, None, None, x, ws)
     with pytest.raises(hip.RwkvHipError, match="workspace"):
         hip.linear_packed(hip.FMT_F16, 16, 64, 4096, x, x, None, None, x, None)  # split K without a workspace
+
+
+def test_wkv7_long_chunked_resume_through_host_slab_is_bitwise(gpu):
+    """BASELINE config 4 at reduced size: fp16 r,w,k,v,a,b, fp32 state, sequence run in chunks of 128 with the state
+    slab copied to the host and into a fresh device buffer at every quarter; outputs and final state must equal
+    the single uninterrupted call bit for bit."""
+    hip = gpu
+    B, T, H = 1, 1024, 6
+    C = H * 64
+    t = wkv_inputs(B, T, H, seed=5, dtype=np.float16)
+    dr, dw, dk, dv, da, db = [dev(hip, t[n]) for n in ("r", "w_raw", "k", "v", "a", "b")]
+    s_full = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y_full = hip.DeviceArray((B, T, C), np.float16)
+    hip.wkv7(B, T, C, H, hip.W_RAW_LOGIT, hip.IO_F16, s_full, dr, dw, dk, dv, da, db, y_full)
+    hip.device_sync()
+
+    state = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y = hip.DeviceArray((B, T, C), np.float16)
+    for t0 in range(0, T, 128):
+        if t0 and t0 % (T // 4) == 0:           # checkpoint: slab to the host, resume from a fresh allocation
+            slab = state.numpy()
+            state = hip.DeviceArray.from_numpy(slab)
+        off = t0 * C
+        views = [d.view(off, (1, 128, C)) for d in (dr, dw, dk, dv, da, db)]
+        hip.wkv7(1, 128, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state, views[0], views[1], views[2], views[3], views[4],
+                 views[5], y.view(off, (1, 128, C)))
+    hip.device_sync()
+    same = np.array_equal(y.numpy().view(np.uint16), y_full.numpy().view(np.uint16))
+    assert same
+    same = np.array_equal(state.numpy().view(np.uint32), s_full.numpy().view(np.uint32))
+    assert same
+    finite = bool(np.isfinite(y.numpy().astype(np.float32)).all())
+    assert finite
