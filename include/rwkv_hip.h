@@ -241,6 +241,12 @@ int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host
  * and returns the number of linear launches and the summed bracketed time since the last read. */
 int rwkv_hip_session_set_profile(rwkv_hip_session* s, int mode);
 int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double* total_ms);
+/* debugging/parity tap: device address of one of the session's activation buffers, holding what the last
+ * layer of the last rwkv_hip_forward call left there.  Ids in order: x, xx, xr, xw, xk, xv, xa, xg, r, k, v,
+ * v_first, w12, a12, g, hw, ha, hg, hv, k2, nkk, kka, y, y2, att, x1, ln2, mixed, act, cm (f16), then
+ * r32, d32, k32, a32, b32 (f32).  Which of them a pass writes depends on its shape (decode steps fuse most
+ * of them away).  No counterpart in the reference. */
+int rwkv_hip_session_debug_buffer(rwkv_hip_session* s, int id, void** ptr);
 /* debugging/parity tap: residual stream after every layer of the last rwkv_hip_forward call,
  * f16 [L, B*T, C], valid only if enabled before the call */
 int rwkv_hip_session_set_trace(rwkv_hip_session* s, void* trace);

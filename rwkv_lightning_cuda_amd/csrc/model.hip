@@ -764,6 +764,17 @@ int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double
   return RWKV_OK;
 }
 
+int rwkv_hip_session_debug_buffer(rwkv_hip_session* s, int id, void** ptr) {
+  RWKV_REQUIRE(s && ptr, "debug_buffer: NULL argument");
+  const Buffers& b = s->buf;
+  void* table[] = {b.x,  b.xx,  b.xr,  b.xw, b.xk, b.xv,  b.xa,  b.xg, b.r,   b.k,     b.v,  b.v_first,
+                   b.w12, b.a12, b.g,  b.hw, b.ha, b.hg,  b.hv,  b.k2, b.nkk, b.kka,   b.y,  b.y2,
+                   b.att, b.x1,  b.ln2, b.mixed, b.act, b.cm, b.r32, b.d32, b.k32, b.a32, b.b32};
+  RWKV_REQUIRE(id >= 0 && id < static_cast<int>(sizeof(table) / sizeof(table[0])), "debug_buffer: unknown id %d", id);
+  *ptr = table[id];
+  return RWKV_OK;
+}
+
 int rwkv_hip_session_set_trace(rwkv_hip_session* s, void* trace) {
   RWKV_REQUIRE(s, "session is NULL");
   s->trace = static_cast<half_t*>(trace);

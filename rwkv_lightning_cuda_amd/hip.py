@@ -40,6 +40,7 @@ EXPORTS = [
     "rwkv_hip_lnx_rkvres_xg", "rwkv_hip_relu_square", "rwkv_hip_add_vec", "rwkv_hip_f16_to_f32",
     "rwkv_hip_advance_i32", "rwkv_hip_sample", "rwkv_hip_argmax", "rwkv_hip_model_create", "rwkv_hip_model_destroy",
     "rwkv_hip_model_set_tensor", "rwkv_hip_model_set_matrix", "rwkv_hip_model_weight_bytes",
+    "rwkv_hip_session_debug_buffer",
     "rwkv_hip_session_create", "rwkv_hip_session_destroy", "rwkv_hip_session_stream", "rwkv_hip_session_set_graph",
     "rwkv_hip_session_set_trace", "rwkv_hip_session_set_profile", "rwkv_hip_session_read_profile", "rwkv_hip_forward", "rwkv_hip_decode_greedy",
 ]

@@ -250,6 +250,21 @@ class Session:
         self._trace = dev
         hip.check(hip.load().rwkv_hip_session_set_trace(self.handle, hip._p(dev)))
 
+    DEBUG_IDS = ["x", "xx", "xr", "xw", "xk", "xv", "xa", "xg", "r", "k", "v", "v_first", "w12", "a12", "g", "hw", "ha",
+                 "hg", "hv", "k2", "nkk", "kka", "y", "y2", "att", "x1", "ln2", "mixed", "act", "cm", "r32", "d32", "k32",
+                 "a32", "b32"]
+
+    def debug_buffer(self, name, shape):
+        """Host copy of one of the session's activation buffers (what the last layer of the last forward call
+        left there): a parity tap for tests."""
+        idx = self.DEBUG_IDS.index(name)
+        p = ctypes.c_void_p(0)
+        hip.check(hip.load().rwkv_hip_session_debug_buffer(self.handle, ctypes.c_int(idx), ctypes.byref(p)))
+        dtype = np.float32 if name.endswith("32") else np.float16
+        out = np.empty(shape, dtype)
+        hip.check(hip.load().rwkv_hip_memcpy_d2h(out.ctypes.data_as(ctypes.c_void_p), p, ctypes.c_size_t(out.nbytes)))
+        return out
+
     def set_profile(self, mode):
         """0/False off; 1/True one event pair per linear launch; 2 passes launch the linear kernels only, back to
         back, one event pair per pass (state and logits are garbage afterwards)."""
