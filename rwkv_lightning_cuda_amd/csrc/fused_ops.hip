@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float d = v[i][e] - mean;
-        sv += d * d;
+        sv = fmaf(d, d, sv);
       }
     }
   }
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
     if (c < C) {
       half8_t yv;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) yv[e] = f2h((v[i][e] - mean) * rstd * h2f(wv[i][e]) + h2f(bv[i][e]));
+      for (int e = 0; e < 8; ++e) yv[e] = f2h(fmaf((v[i][e] - mean) * rstd, h2f(wv[i][e]), h2f(bv[i][e])));
       if constexpr (MODE == kAddLn || MODE == kAddLnMix) {
         half8_t xo;
 #pragma unroll
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
               const float yf = h2f(yv[e]);
-              ov[e] = f2h(yf + (h2f(pv[i][e]) - yf) * h2f(mv[i][s][e]));
+              ov[e] = f2h(fmaf(h2f(pv[i][e]) - yf, h2f(mv[i][s][e]), yf));
             }
             *reinterpret_cast<half8_t*>(a.out[s] + dst + c) = ov;
           }

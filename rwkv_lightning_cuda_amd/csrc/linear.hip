@@ -29,7 +29,81 @@ struct LinearArgs {
   int KT;  // K tile staged in LDS (>= K when the whole x fits)
   int epilogue;
   int out_f32;
+  LnPrologue ln;
+  RowCopy copy;
 };
+
+// One row of the LayerNorm + lerp prologue into xs (K fp16 values).  Same element-to-thread assignment, two-pass
+// statistics, explicit FMAs and rounding points as ln_fused_kernel (fused_ops.hip), so the result is bit-identical
+// to running that kernel first.  The fp32 row sum s = x + res lives in LDS (sbuf, K floats; each thread re-reads
+// only what it wrote) instead of registers, so that the prologue does not cost the weight-streaming loop its
+// occupancy.  256 threads.
+__device__ __forceinline__ void ln_prologue_row(const LnPrologue& ln, const half_t* mu, int K, int m, half_t* xs,
+                                                float* sbuf, float* red, bool store) {
+  const int64_t row = static_cast<int64_t>(m) * K;
+  const int64_t xsrc = ln.mode == 2 ? ln.tokens[m] * static_cast<int64_t>(K) : row;
+  float sum = 0.0f;
+#pragma unroll 1
+  for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
+    const half8_t xv = *reinterpret_cast<const half8_t*>(ln.x + xsrc + c);
+    float v[8];
+    if (ln.mode == 1) {
+      const half8_t rv = *reinterpret_cast<const half8_t*>(ln.res + row + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = h2f(xv[e]) + h2f(rv[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = h2f(xv[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += v[e];
+    *reinterpret_cast<float4_t*>(sbuf + c) = float4_t{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<float4_t*>(sbuf + c + 4) = float4_t{v[4], v[5], v[6], v[7]};
+  }
+  sum = block_sum<4>(sum, red);
+  const float mean = sum / static_cast<float>(K);
+  float sv = 0.0f;
+#pragma unroll 1
+  for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
+    const float4_t lo = *reinterpret_cast<const float4_t*>(sbuf + c);
+    const float4_t hi = *reinterpret_cast<const float4_t*>(sbuf + c + 4);
+    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float d = v[e] - mean;
+      sv = fmaf(d, d, sv);
+    }
+  }
+  sv = block_sum<4>(sv, red);
+  const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
+#pragma unroll 1
+  for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
+    const half8_t wv = *reinterpret_cast<const half8_t*>(ln.w + c);
+    const half8_t bv = *reinterpret_cast<const half8_t*>(ln.b + c);
+    const half8_t pv = *reinterpret_cast<const half8_t*>(ln.shift + row + c);
+    const half8_t mv = *reinterpret_cast<const half8_t*>(mu + c);
+    const float4_t lo = *reinterpret_cast<const float4_t*>(sbuf + c);
+    const float4_t hi = *reinterpret_cast<const float4_t*>(sbuf + c + 4);
+    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    half8_t yv, ov;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      yv[e] = f2h(fmaf((v[e] - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
+      const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
+      ov[e] = f2h(fmaf(h2f(pv[e]) - yf, h2f(mv[e]), yf));
+    }
+    *reinterpret_cast<half8_t*>(xs + c) = ov;
+    if (store) {
+      *reinterpret_cast<half8_t*>(ln.ln_out + row + c) = yv;
+      if (ln.x_out) {
+        half8_t xo;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xo[e] = f2h(v[e]);
+        *reinterpret_cast<half8_t*>(ln.x_out + row + c) = xo;
+      }
+    }
+  }
+}
 
 // 4 signed int8 codes in a dword -> two half2 (exact).  c ^ 0x80 is the code + 128 as an unsigned
 // byte; 0x6400 | byte is the fp16 number 1024 + byte; subtracting 1152 leaves the code.
@@ -169,9 +243,9 @@ struct WaveGemv {
   }
 };
 
-template <int FMT, int M, int R, int U>
+template <int FMT, int M, int R, int U, bool LN>
 __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearProblem& prob, int block_in_problem,
-                                           half_t* xs) {
+                                           half_t* xs, float* sbuf, float* red) {
   using T = FmtTraits<FMT>;
   using W = WaveGemv<FMT, M, R, U>;
   const int K = args.K;
@@ -198,11 +272,17 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
     // request the first batch of weights, then stage x: the two latencies overlap
     if (active) W::load_batch(wa, wbase, row_bytes, kt, kn, 0, lane);
     if (kt > 0) __syncthreads();
-    for (int i = threadIdx.x * 8; i < M * kn; i += 256 * 8) {
-      const int m = i / kn;
-      const int kk = i - m * kn;
-      *reinterpret_cast<uint4_t*>(xs + m * KT + kk) =
-          *reinterpret_cast<const uint4_t*>(prob.x + static_cast<int64_t>(m) * K + kt + kk);
+    if constexpr (LN) {
+      // the launcher guarantees KT >= K here: the whole row is normalised at once
+#pragma unroll 1
+      for (int m = 0; m < M; ++m) ln_prologue_row(args.ln, prob.mu, K, m, xs + m * KT, sbuf, red, blockIdx.x == 0);
+    } else {
+      for (int i = threadIdx.x * 8; i < M * kn; i += 256 * 8) {
+        const int m = i / kn;
+        const int kk = i - m * kn;
+        *reinterpret_cast<uint4_t*>(xs + m * KT + kk) =
+            *reinterpret_cast<const uint4_t*>(prob.x + static_cast<int64_t>(m) * K + kt + kk);
+      }
     }
     __syncthreads();
     if (active) {
@@ -248,11 +328,18 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
   }
 }
 
-// grid = total blocks over all problems (each block: 4 waves x R rows); dynamic LDS = M*KT*2 bytes.
-template <int M, int R, int U>
+// grid = total blocks over all problems (each block: 4 waves x R rows); dynamic LDS = M*KT*2 bytes (+ K*4 with the
+// LayerNorm prologue, a separate instantiation so that launches without it keep their register budget).
+template <int M, int R, int U, bool LN>
 __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
+  __shared__ float red[4];
   half_t* xs = reinterpret_cast<half_t*>(lds_raw);
+  float* sbuf = reinterpret_cast<float*>(lds_raw + static_cast<size_t>(M) * args.KT * sizeof(half_t));
+  if (blockIdx.x == 0 && args.copy.n > 0) {
+    for (int i = threadIdx.x * 8; i < args.copy.n; i += 256 * 8)
+      *reinterpret_cast<uint4_t*>(args.copy.dst + i) = *reinterpret_cast<const uint4_t*>(args.copy.src + i);
+  }
   int pi = 0;
   int first = 0;
   for (int i = 0; i < args.n_problems - 1; ++i) {
@@ -264,9 +351,9 @@ __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
   const LinearProblem prob = args.p[pi];
   const int blk = blockIdx.x - first;
   switch (prob.fmt) {  // uniform per block
-    case RWKV_FMT_W8: gemv_block<RWKV_FMT_W8, M, R, U>(args, prob, blk, xs); break;
-    case RWKV_FMT_W4: gemv_block<RWKV_FMT_W4, M, R, U>(args, prob, blk, xs); break;
-    default: gemv_block<RWKV_FMT_F16, M, R, U>(args, prob, blk, xs); break;
+    case RWKV_FMT_W8: gemv_block<RWKV_FMT_W8, M, R, U, LN>(args, prob, blk, xs, sbuf, red); break;
+    case RWKV_FMT_W4: gemv_block<RWKV_FMT_W4, M, R, U, LN>(args, prob, blk, xs, sbuf, red); break;
+    default: gemv_block<RWKV_FMT_F16, M, R, U, LN>(args, prob, blk, xs, sbuf, red); break;
   }
 }
 
@@ -277,15 +364,20 @@ static int launch_one(hipStream_t st, LinearArgs& args) {
     total += ceil_div(args.p[i].N, 4 * R);
     args.block_end[i] = total;
   }
-  const size_t lds = static_cast<size_t>(M) * args.KT * sizeof(half_t);
-  hipLaunchKernelGGL((linear_gemv_kernel<M, R, U>), dim3(total), dim3(256), lds, st, args);
+  size_t lds = static_cast<size_t>(M) * args.KT * sizeof(half_t);
+  if (args.ln.mode != 0) {
+    lds += static_cast<size_t>(args.K) * sizeof(float);
+    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, true>), dim3(total), dim3(256), lds, st, args);
+  } else {
+    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, false>), dim3(total), dim3(256), lds, st, args);
+  }
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
 // Batched small-M linear: n_problems problems sharing M (<= 8), K, epilogue and output type.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
-                   int out_f32) {
+                   int out_f32, const LnPrologue* ln, const RowCopy* copy) {
   RWKV_REQUIRE(M >= 1 && M <= 8, "linear_small_m: M %d out of range", M);
   RWKV_REQUIRE(n_problems >= 1 && n_problems <= kMaxProblems, "linear_small_m: %d problems", n_problems);
   LinearArgs args = {};
@@ -299,7 +391,7 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
     RWKV_REQUIRE(K > 0 && K % elems == 0, "linear: K (%d) must be a multiple of %d for this weight format", K, elems);
     if (p.fmt == RWKV_FMT_W4) RWKV_REQUIRE(K % 128 == 0, "linear: W4 needs K %% 128 == 0 (K = %d)", K);
     RWKV_REQUIRE(p.N > 0 && p.N % 4 == 0, "linear: N (%d) must be a positive multiple of 4", p.N);
-    RWKV_REQUIRE(p.w && p.x && p.y, "linear: NULL tensor");
+    RWKV_REQUIRE(p.w && p.y && (p.x || (ln && ln->mode != 0 && p.mu)), "linear: NULL tensor");
     RWKV_REQUIRE(p.fmt == RWKV_FMT_F16 || p.scale, "linear: quantised weights need a scale tensor");
     RWKV_REQUIRE(p.fmt != RWKV_FMT_W4 || p.zp, "linear: W4 weights need a zero-point tensor");
     args.p[i] = p;
@@ -314,6 +406,18 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
   int kt = (65536 / (2 * M)) / step * step;
   if (kt < step) kt = step;
   args.KT = std::min(kt, k_round);
+  if (ln && ln->mode != 0) {
+    RWKV_REQUIRE(ln->mode == 1 || ln->mode == 2, "linear: bad LayerNorm prologue mode %d", ln->mode);
+    RWKV_REQUIRE(args.KT >= K && K % 8 == 0 && static_cast<size_t>(M) * args.KT * 2 + static_cast<size_t>(K) * 4 <= 65536,
+                 "linear: LayerNorm prologue needs the whole row in LDS (M = %d, K = %d)", M, K);
+    RWKV_REQUIRE(ln->x && ln->w && ln->b && ln->shift && ln->ln_out && (ln->mode == 2 ? ln->tokens != nullptr : ln->res != nullptr),
+                 "linear: LayerNorm prologue has a NULL tensor");
+    args.ln = *ln;
+  }
+  if (copy && copy->n > 0) {
+    RWKV_REQUIRE(copy->src && copy->dst && copy->n % 8 == 0, "linear: bad row copy");
+    args.copy = *copy;
+  }
   if (M == 1) {
     // RWKV_GEMV_RU=<R><U> picks the rows-per-wave / steps-in-flight variant for M == 1 (tuning aid)
     static const int ru = [] { const char* e = getenv("RWKV_GEMV_RU"); return e ? atoi(e) : 0; }();

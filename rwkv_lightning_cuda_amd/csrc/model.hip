@@ -300,6 +300,10 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   // row-tiled kernels of the prefill path (LoRA rows shared by 16 rows) move less data; measured crossover
   // between 32 and 64 rows.
   const bool fused_tmix = step && rows <= 32;
+  // Decode steps of up to 8 rows fold both LayerNorm + token-shift kernels of a layer into the prologue of the
+  // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key).  The residual-stream tap needs the
+  // stand-alone kernels.
+  const bool ln_in_linear = step && small && !s->trace && static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
 
   auto mix6_args = [&](const Layer& w, LnArgs& a) {
     const int ids[6] = {RWKV_T_X_R, RWKV_T_X_W, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_A, RWKV_T_X_G};
@@ -311,7 +315,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     a.n_mix = 6;
   };
 
-  if (step) {
+  if (ln_in_linear) {
+    // nothing here: layer 0's r/k/v launch gathers the embedding rows itself
+  } else if (step) {
     // embedding gather + LN1(layer 0) + six lerps + shift0 write in one kernel
     LnArgs a = {};
     a.x = m->emb_ln0; a.tokens = s->tokens_dev; a.x_out = b.x;
@@ -367,7 +373,24 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
           p[3 + i].w = w.t[w1_ids[i]]; p[3 + i].scale = nullptr; p[3 + i].zp = nullptr;
           p[3 + i].x = lx[i]; p[3 + i].y = lh[i]; p[3 + i].N = ranks[i]; p[3 + i].fmt = RWKV_FMT_F16;
         }
-        TRY_PROF(linear_small_m(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0));
+        if (ln_in_linear) {
+          const int mu_ids[7] = {RWKV_T_X_R, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_W, RWKV_T_X_A, RWKV_T_X_G, RWKV_T_X_V};
+          for (int i = 0; i < 3 + n_lora; ++i) {
+            p[i].x = nullptr;
+            p[i].mu = w.t[mu_ids[i]];
+          }
+          LnPrologue ln;
+          ln.w = w.t[RWKV_T_LN1_W]; ln.b = w.t[RWKV_T_LN1_B]; ln.shift = shift0; ln.x_out = b.x; ln.ln_out = b.xx;
+          ln.eps = kLnEps;
+          if (l == 0) {
+            ln.mode = 2; ln.x = m->emb_ln0; ln.tokens = s->tokens_dev;
+          } else {
+            ln.mode = 1; ln.x = b.x1; ln.res = b.cm;
+          }
+          TRY_PROF(linear_small_m(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0, &ln));
+        } else {
+          TRY_PROF(linear_small_m(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0));
+        }
       } else {
         bool all_packed = rows >= static_cast<int>(kPackedMinRows);
         for (int i = 0; i < 3; ++i) all_packed = all_packed && w.m[mids[i]].packed != nullptr;
@@ -399,6 +422,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       p.k_a = w.t[RWKV_T_K_A]; p.r_k = w.t[RWKV_T_R_K]; p.lnx_w = w.t[RWKV_T_LNX_W]; p.lnx_b = w.t[RWKV_T_LNX_B];
       p.r = b.r; p.k = b.k; p.v = v_cur; p.v_first = b.v_first; p.v_first_out = nullptr;
       p.state = S; p.y2 = b.y2;
+      if (ln_in_linear) {
+        p.shift_src = b.xx; p.shift_dst = shift0;
+      }
       TRY_AUX(tmix_step_launch(st, p));
     } else {
       // LoRA rank-out (+ activation, + v-residual gate)
@@ -437,7 +463,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     TRY_PROF(apply_matrix(s, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
 
     // residual add + LN2 + channel-mix token shift
-    if (step) {
+    if (ln_in_linear) {
+      // folded into the ffn.key launch below
+    } else if (step) {
       LnArgs a = {};
       a.x = b.x; a.res = b.att; a.w = w.t[RWKV_T_LN2_W]; a.b = w.t[RWKV_T_LN2_B]; a.x_out = b.x1; a.shift = shift1;
       a.mu[0] = w.t[RWKV_T_FFN_X_K]; a.out[0] = b.mixed; a.n_mix = 1; a.C = C; a.T = 1; a.eps = kLnEps;
@@ -454,11 +482,28 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     }
 
     // channel mix
-    TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
-    TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+    if (ln_in_linear) {
+      const Matrix& mk = w.m[RWKV_M_FFN_KEY];
+      LinearProblem pk = {mk.data, mk.scale, mk.zp, nullptr, b.act, F, mk.fmt, w.t[RWKV_T_FFN_X_K]};
+      LnPrologue ln;
+      ln.mode = 1; ln.x = b.x; ln.res = b.att; ln.w = w.t[RWKV_T_LN2_W]; ln.b = w.t[RWKV_T_LN2_B];
+      ln.shift = shift1; ln.x_out = b.x1; ln.ln_out = b.ln2; ln.eps = kLnEps;
+      TRY_PROF(linear_small_m(st, rows, C, 1, &pk, RWKV_EPI_RELU_SQUARE, 0, &ln));
+      // the ffn.value launch also moves the LN2 output kept above into the channel-mix shift row of the state
+      const Matrix& mv = w.m[RWKV_M_FFN_VALUE];
+      LinearProblem pv = {mv.data, mv.scale, mv.zp, b.act, b.cm, C, mv.fmt, nullptr};
+      RowCopy cp;
+      cp.src = b.ln2; cp.dst = shift1; cp.n = rows * C;
+      TRY_PROF(linear_small_m(st, rows, F, 1, &pv, RWKV_EPI_NONE, 0, nullptr, &cp));
+    } else {
+      TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
+      TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+    }
 
     // residual add + next layer's LN1 (+ lerps), or the final LN on the last token of each row
-    if (l + 1 < L) {
+    if (l + 1 < L && ln_in_linear) {
+      // the next layer's r/k/v launch adds the residual and normalises
+    } else if (l + 1 < L) {
       const Layer& nx = m->layers[l + 1];
       LnArgs a = {};
       a.x = b.x1; a.res = b.cm; a.w = nx.t[RWKV_T_LN1_W]; a.b = nx.t[RWKV_T_LN1_B]; a.x_out = b.x;

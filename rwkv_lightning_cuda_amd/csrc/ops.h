@@ -12,16 +12,44 @@ struct LinearProblem {
   const void* w;
   const half_t* scale;
   const uint8_t* zp;
-  const half_t* x;
+  const half_t* x;   // unused when the launch has a LayerNorm prologue
   void* y;
   int N;
-  int fmt;  // RWKV_FMT_*
+  int fmt;           // RWKV_FMT_*
+  const half_t* mu;  // with a LayerNorm prologue: this problem's token-shift lerp coefficients [K]
+};
+
+// LayerNorm + token-shift prologue of a small-M linear launch (decode steps): every block recomputes, for each
+// of the M rows, s = x + res (or an embedding-table row), LN(s) and the lerp of this problem against the previous
+// token's LN output, straight into its LDS copy of x - instead of a separate kernel writing six mixed copies of
+// x that the linear kernel then reads back.  Arithmetic and reduction order are those of ln_fused_kernel.
+// Block 0 also stores the residual sum and the LN output (the next shift row, written to the state by a later
+// kernel so that no block can read a shift row that another block has already replaced).
+struct LnPrologue {
+  int mode = 0;  // 0 none, 1 residual add (x + res), 2 rows of `x` as a [V,K] table gathered by tokens, no residual
+  const half_t* x = nullptr;
+  const half_t* res = nullptr;
+  const int64_t* tokens = nullptr;
+  const half_t* w = nullptr;
+  const half_t* b = nullptr;
+  const half_t* shift = nullptr;  // [M,K], read only
+  half_t* x_out = nullptr;        // [M,K] or NULL
+  half_t* ln_out = nullptr;       // [M,K]
+  float eps = 1e-5f;
+};
+
+// Extra duty of block 0 of a small-M linear launch: copy n fp16 values (the LN output kept by an earlier launch
+// into its shift-state row).
+struct RowCopy {
+  const half_t* src = nullptr;
+  half_t* dst = nullptr;
+  int n = 0;
 };
 
 // Batched small-M (<= 8) linear through the weight-streaming GEMV kernel: up to kMaxProblems problems that
 // share M and K (each with its own weight format, x and y) in one launch.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
-                   int out_f32);
+                   int out_f32, const LnPrologue* ln = nullptr, const RowCopy* copy = nullptr);
 // Any M: MFMA tiles for M >= 16 where supported, else row tiles through the GEMV kernel.
 int linear_any_m(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* w, const half_t* scale,
                  const uint8_t* zp, int epilogue, int out_f32, void* y);
@@ -153,6 +181,8 @@ struct TmixStepArgs {
   half_t* v_first_out;                      // [B,C], written when hv == NULL (layer 0), may be NULL
   float* state;                             // [B,H,64,64], updated in place
   half_t* y2;                               // [B,C] input of the output projection
+  const half_t* shift_src;                  // [B,C] LN output kept by the r/k/v launch's prologue, or NULL
+  half_t* shift_dst;                        // [B,C] time-mix shift row of the state that receives it
 };
 int tmix_step_launch(hipStream_t st, const TmixStepArgs& p);
 

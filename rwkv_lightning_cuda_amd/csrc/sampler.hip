@@ -296,19 +296,45 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
   }
 }
 
-__global__ __launch_bounds__(256) void argmax_kernel(int V, const float* __restrict__ logits, int* __restrict__ out) {
-  __shared__ float bv[4];
-  __shared__ int bi[4];
+// One 1024-thread block per row; 16-byte loads, eight in flight per thread (the row is 256 KiB at V = 65536 and
+// the kernel is pure load latency).  Lowest index among equal maxima.
+constexpr int kArgmaxThreads = 1024;
+
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(int V, const float* __restrict__ logits, int* __restrict__ out) {
+  __shared__ float bv[kArgmaxThreads / 64];
+  __shared__ int bi[kArgmaxThreads / 64];
   const float* row = logits + static_cast<int64_t>(blockIdx.x) * V;
   float best = -INFINITY;
   int idx = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += 256) {
-    const float v = row[i];
-    if (v > best) {
+  auto take = [&](float v, int i) {
+    if (v > best || (v == best && i < idx)) {
       best = v;
       idx = i;
     }
+  };
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  const int V4 = vec_ok ? V / 4 : 0;
+  constexpr int kBatch = 8;
+  for (int base = 0; base < V4; base += kArgmaxThreads * kBatch) {
+    float4_t q[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int i = base + u * kArgmaxThreads + threadIdx.x;
+      q[u] = float4_t{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      if (i < V4) q[u] = reinterpret_cast<const float4_t*>(row)[i];
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int i = (base + u * kArgmaxThreads + threadIdx.x) * 4;
+      if (i < V4 * 4) {
+        take(q[u].x, i);
+        take(q[u].y, i + 1);
+        take(q[u].z, i + 2);
+        take(q[u].w, i + 3);
+      }
+    }
   }
+  for (int i = V4 * 4 + threadIdx.x; i < V; i += kArgmaxThreads) take(row[i], i);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const float ov = __shfl_xor(best, off, 64);
@@ -324,7 +350,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(int V, const float* __restr
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int i = 1; i < 4; ++i)
+    for (int i = 1; i < kArgmaxThreads / 64; ++i)
       if (bv[i] > best || (bv[i] == best && bi[i] < idx)) {
         best = bv[i];
         idx = bi[i];
@@ -334,7 +360,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(int V, const float* __restr
 }
 
 int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out) {
-  hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(256), 0, st, V, logits, out);
+  hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(kArgmaxThreads), 0, st, V, logits, out);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }

@@ -81,6 +81,13 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
   const int c = h * kHead + i;
   const int64_t row = static_cast<int64_t>(bi) * p.C;
 
+  // the LN output that the r/k/v launch computed in its prologue becomes the shift row of the state (that
+  // launch could not store it itself: other blocks of it were still reading the old row)
+  if (p.shift_dst && tid < kHead) {
+    const int64_t o = row + h * kHead + tid;
+    p.shift_dst[o] = p.shift_src[o];
+  }
+
   // ---- all global loads up front
   float* srow = p.state + (static_cast<int64_t>(bh) * kHead + i) * kHead + 4 * q;
   float4_t S = *reinterpret_cast<const float4_t*>(srow);
