@@ -38,13 +38,17 @@ struct LinearArgs {
 // to running that kernel first.  The fp32 row sum s = x + res lives in LDS (sbuf, K floats; each thread re-reads
 // only what it wrote) instead of registers, so that the prologue does not cost the weight-streaming loop its
 // occupancy.  256 threads.
+template <int NW>
 __device__ __forceinline__ void ln_prologue_row(const LnPrologue& ln, const half_t* mu, int K, int m, half_t* xs,
                                                 float* sbuf, float* red, bool store) {
+  // Blocks of more than 256 threads: the first 256 hold the elements exactly as ln_fused_kernel's 256 threads do and
+  // the other wavefronts add zeros to the block sums, which leaves every sum bit-identical.
+  const int kend = threadIdx.x < 256 ? K : 0;
   const int64_t row = static_cast<int64_t>(m) * K;
   const int64_t xsrc = ln.mode == 2 ? ln.tokens[m] * static_cast<int64_t>(K) : row;
   float sum = 0.0f;
 #pragma unroll 1
-  for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
+  for (int c = threadIdx.x * 8; c < kend; c += 256 * 8) {
     const half8_t xv = *reinterpret_cast<const half8_t*>(ln.x + xsrc + c);
     float v[8];
     if (ln.mode == 1) {
@@ -60,11 +64,11 @@ __device__ __forceinline__ void ln_prologue_row(const LnPrologue& ln, const half
     *reinterpret_cast<float4_t*>(sbuf + c) = float4_t{v[0], v[1], v[2], v[3]};
     *reinterpret_cast<float4_t*>(sbuf + c + 4) = float4_t{v[4], v[5], v[6], v[7]};
   }
-  sum = block_sum<4>(sum, red);
+  sum = block_sum<NW>(sum, red);
   const float mean = sum / static_cast<float>(K);
   float sv = 0.0f;
 #pragma unroll 1
-  for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
+  for (int c = threadIdx.x * 8; c < kend; c += 256 * 8) {
     const float4_t lo = *reinterpret_cast<const float4_t*>(sbuf + c);
     const float4_t hi = *reinterpret_cast<const float4_t*>(sbuf + c + 4);
     const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -74,10 +78,10 @@ __device__ __forceinline__ void ln_prologue_row(const LnPrologue& ln, const half
       sv = fmaf(d, d, sv);
     }
   }
-  sv = block_sum<4>(sv, red);
+  sv = block_sum<NW>(sv, red);
   const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
 #pragma unroll 1
-  for (int c = threadIdx.x * 8; c < K; c += 256 * 8) {
+  for (int c = threadIdx.x * 8; c < kend; c += 256 * 8) {
     const half8_t wv = *reinterpret_cast<const half8_t*>(ln.w + c);
     const half8_t bv = *reinterpret_cast<const half8_t*>(ln.b + c);
     const half8_t pv = *reinterpret_cast<const half8_t*>(ln.shift + row + c);
@@ -243,7 +247,7 @@ struct WaveGemv {
   }
 };
 
-template <int FMT, int M, int R, int U, bool LN>
+template <int FMT, int M, int R, int U, bool LN, int NW>
 __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearProblem& prob, int block_in_problem,
                                            half_t* xs, float* sbuf, float* red) {
   using T = FmtTraits<FMT>;
@@ -253,7 +257,7 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
   const int N = prob.N;
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-  const int row0 = (block_in_problem * 4 + wave) * R;
+  const int row0 = (block_in_problem * NW + wave) * R;
   const bool active = row0 < N;
   const int64_t row_bytes = T::byte_off(K);
   const unsigned char* wbase =
@@ -275,9 +279,9 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
     if constexpr (LN) {
       // the launcher guarantees KT >= K here: the whole row is normalised at once
 #pragma unroll 1
-      for (int m = 0; m < M; ++m) ln_prologue_row(args.ln, prob.mu, K, m, xs + m * KT, sbuf, red, blockIdx.x == 0);
+      for (int m = 0; m < M; ++m) ln_prologue_row<NW>(args.ln, prob.mu, K, m, xs + m * KT, sbuf, red, blockIdx.x == 0);
     } else {
-      for (int i = threadIdx.x * 8; i < M * kn; i += 256 * 8) {
+      for (int i = threadIdx.x * 8; i < M * kn; i += NW * 64 * 8) {
         const int m = i / kn;
         const int kk = i - m * kn;
         *reinterpret_cast<uint4_t*>(xs + m * KT + kk) =
@@ -330,14 +334,14 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
 
 // grid = total blocks over all problems (each block: 4 waves x R rows); dynamic LDS = M*KT*2 bytes (+ K*4 with the
 // LayerNorm prologue, a separate instantiation so that launches without it keep their register budget).
-template <int M, int R, int U, bool LN>
-__global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
+template <int M, int R, int U, bool LN, int NW>
+__global__ __launch_bounds__(NW * 64) void linear_gemv_kernel(LinearArgs args) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  __shared__ float red[4];
+  __shared__ float red[NW];
   half_t* xs = reinterpret_cast<half_t*>(lds_raw);
   float* sbuf = reinterpret_cast<float*>(lds_raw + static_cast<size_t>(M) * args.KT * sizeof(half_t));
   if (blockIdx.x == 0 && args.copy.n > 0) {
-    for (int i = threadIdx.x * 8; i < args.copy.n; i += 256 * 8)
+    for (int i = threadIdx.x * 8; i < args.copy.n; i += NW * 64 * 8)
       *reinterpret_cast<uint4_t*>(args.copy.dst + i) = *reinterpret_cast<const uint4_t*>(args.copy.src + i);
   }
   int pi = 0;
@@ -351,25 +355,40 @@ __global__ __launch_bounds__(256) void linear_gemv_kernel(LinearArgs args) {
   const LinearProblem prob = args.p[pi];
   const int blk = blockIdx.x - first;
   switch (prob.fmt) {  // uniform per block
-    case RWKV_FMT_W8: gemv_block<RWKV_FMT_W8, M, R, U, LN>(args, prob, blk, xs, sbuf, red); break;
-    case RWKV_FMT_W4: gemv_block<RWKV_FMT_W4, M, R, U, LN>(args, prob, blk, xs, sbuf, red); break;
-    default: gemv_block<RWKV_FMT_F16, M, R, U, LN>(args, prob, blk, xs, sbuf, red); break;
+    case RWKV_FMT_W8: gemv_block<RWKV_FMT_W8, M, R, U, LN, NW>(args, prob, blk, xs, sbuf, red); break;
+    case RWKV_FMT_W4: gemv_block<RWKV_FMT_W4, M, R, U, LN, NW>(args, prob, blk, xs, sbuf, red); break;
+    default: gemv_block<RWKV_FMT_F16, M, R, U, LN, NW>(args, prob, blk, xs, sbuf, red); break;
   }
+}
+
+// Wavefronts per block of the LayerNorm-prologue variant.  16 (the prologue once per 32 rows, the whole grid
+// resident at once) measured slightly slower than 4 on the 7.2B shapes; RWKV_GEMV_LN_WAVES=16 selects it.
+static int ln_block_waves() {
+  static const int v = [] {
+    const char* e = getenv("RWKV_GEMV_LN_WAVES");
+    const int n = e ? atoi(e) : 0;
+    return n == 16 ? 16 : 4;
+  }();
+  return v;
 }
 
 template <int M, int R, int U>
 static int launch_one(hipStream_t st, LinearArgs& args) {
+  const bool ln = args.ln.mode != 0;
+  const int nw = (ln && M <= 2) ? ln_block_waves() : 4;  // more rows per call need more registers than 1024 threads leave
   int total = 0;
   for (int i = 0; i < args.n_problems; ++i) {
-    total += ceil_div(args.p[i].N, 4 * R);
+    total += ceil_div(args.p[i].N, nw * R);
     args.block_end[i] = total;
   }
   size_t lds = static_cast<size_t>(M) * args.KT * sizeof(half_t);
-  if (args.ln.mode != 0) {
-    lds += static_cast<size_t>(args.K) * sizeof(float);
-    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, true>), dim3(total), dim3(256), lds, st, args);
+  if (ln) lds += static_cast<size_t>(args.K) * sizeof(float);
+  if (ln && nw == 16) {
+    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, true, 16>), dim3(total), dim3(1024), lds, st, args);
+  } else if (ln) {
+    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, true, 4>), dim3(total), dim3(256), lds, st, args);
   } else {
-    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, false>), dim3(total), dim3(256), lds, st, args);
+    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, false, 4>), dim3(total), dim3(256), lds, st, args);
   }
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
