@@ -5,81 +5,135 @@
 // rank, v-residual gate fused for the v group :1118-1123); unfused variants :209-367,685-811,1132-1270;
 // dispatch src/rwkv7_fast_v4.cu:961-1014,1217-1260.
 //
-// rank-in is a plain small-N linear layer over fp16 weights [R,C] and reuses the GEMV kernel.
-// rank-out has a short reduction (R = 32..512) and many outputs: 8 lanes share one output channel,
-// each lane keeps its slice of the W2 row in registers and walks the rows of the batch, so W2 is read
-// once per block however many rows there are.
+// rank-in is a plain small-N linear layer over fp16 weights [R,C] and reuses the GEMV / streaming GEMM kernels.
+//
+// rank-out is out[M,C] = act(h[M,R]) . W2[C,R]^T: a short reduction (R = 32..512) and many outputs, on
+// v_mfma_f32_32x32x16_f16.  The activated hidden stays fp32 in the reference, so it enters the matrix core as
+// two fp16 terms, hi = f16(a) and lo = f16(a - hi): hi + lo carries 22 bits of a, both products with the fp16
+// weight are exact in fp32, and the result differs from an fp32 dot only by summation order.  Without an
+// activation the hidden is fp16 already and the lo term is skipped.  One launch takes up to four problems
+// (w, a, g, v of a layer): grid = (C/128, M/32, problems), block = 4 wavefronts x 32 output channels, the
+// 32 x 128 slice of act(h) staged in LDS once per block and K chunk.
 #include "ops.h"
 
 namespace rwkv {
 
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
 constexpr int kLoraMaxR = 512;
-constexpr int kLoraRowsPerBlock = 16;
+constexpr int kLoraRows = 32;          // rows per block: one MFMA tile
+constexpr int kLoraCols = 128;         // output channels per block: 32 per wavefront
+constexpr int kLoraKC = 128;           // reduction chunk staged in LDS
+constexpr int kLoraLd = kLoraKC + 8;   // +8 halves: ds_read_b128 of lane (j, h) at j*272 + 16h bytes is conflict-free
 
+__global__ __launch_bounds__(256) void lora_out_kernel(LoraOutMultiArgs a) {
+  __shared__ __attribute__((aligned(16))) half_t hi_s[kLoraRows][kLoraLd];
+  __shared__ __attribute__((aligned(16))) half_t lo_s[kLoraRows][kLoraLd];
+  const LoraOutProblem& p = a.p[blockIdx.z];
+  const int R = p.R;
+  const int m0 = blockIdx.y * kLoraRows;
+  const int mn = min(kLoraRows, a.M - m0);
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int j = lane & 31;
+  const int h = lane >> 5;
+  const int c = blockIdx.x * kLoraCols + wave * 32 + j;
+  const bool col_ok = c < a.C;
+  const bool split = p.act != RWKV_ACT_NONE;
+  const half_t* wrow = p.w2 + static_cast<int64_t>(col_ok ? c : 0) * R;
 
-// grid = (C/32, ceil(M/16)); block = 256: 32 output channels x 8 lanes.
-__global__ __launch_bounds__(256) void lora_out_kernel(LoraOutArgs a) {
-  __shared__ float hs[kLoraRowsPerBlock][kLoraMaxR];
-  const int R = a.R;
-  const int m0 = blockIdx.y * kLoraRowsPerBlock;
-  const int mn = min(kLoraRowsPerBlock, a.M - m0);
-  for (int i = threadIdx.x; i < mn * R; i += 256) {
-    const int m = i / R;
-    const int r = i - m * R;
-    float hv = h2f(a.h[static_cast<int64_t>(m0 + m) * R + r]);
-    if (a.act == RWKV_ACT_TANH) hv = tanhf(hv);
-    if (a.act == RWKV_ACT_SIGMOID) hv = sigmoid_f(hv);
-    hs[m][r] = hv;
-  }
-  const int g = threadIdx.x & 7;
-  const int c = blockIdx.x * 32 + (threadIdx.x >> 3);
-  // this lane's slice of W2[c]: elements g*8 + 64*i + e
-  half8_t wreg[kLoraMaxR / 64];
+  float16_t acc;
 #pragma unroll
-  for (int i = 0; i < kLoraMaxR / 64; ++i) {
-    const int r0 = g * 8 + 64 * i;
-    if (r0 < R) {
-      wreg[i] = *reinterpret_cast<const half8_t*>(a.w2 + static_cast<int64_t>(c) * R + r0);
-    } else {
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+
+  for (int kc = 0; kc < R; kc += kLoraKC) {
+    // this lane's W2 values of the chunk: k = kc + 16*kk + 8h .. +8 of output channel c
+    half8_t wreg[kLoraKC / 16];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) wreg[i][e] = static_cast<half_t>(0.0f);
-    }
-  }
-  __syncthreads();
-  const float bias = a.bias ? h2f(a.bias[c]) : 0.0f;
-  for (int m = 0; m < mn; ++m) {
-    float acc = 0.0f;
+    for (int kk = 0; kk < kLoraKC / 16; ++kk) {
+      const int k = kc + kk * 16 + h * 8;
+      if (col_ok && k < R) {
+        wreg[kk] = *reinterpret_cast<const half8_t*>(wrow + k);
+      } else {
 #pragma unroll
-    for (int i = 0; i < kLoraMaxR / 64; ++i) {
-      const int r0 = g * 8 + 64 * i;
-      if (r0 < R) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc = fmaf(hs[m][r0 + e], h2f(wreg[i][e]), acc);
+        for (int e = 0; e < 8; ++e) wreg[kk][e] = static_cast<half_t>(0.0f);
       }
     }
-    acc = group_sum<8>(acc);
-    if (g == 0) {
+    // activation of the 32 x 128 hidden slice, split into hi + lo
+    if (kc > 0) __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kLoraRows * kLoraKC / 8 / 256; ++i) {
+      const int idx = threadIdx.x + 256 * i;
+      const int m = idx / (kLoraKC / 8);
+      const int ks = (idx % (kLoraKC / 8)) * 8;
+      half8_t hi, lo;
+      if (m < mn && kc + ks < R) {
+        const half8_t hv = *reinterpret_cast<const half8_t*>(p.h + static_cast<int64_t>(m0 + m) * R + kc + ks);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float f = h2f(hv[e]);
+          if (p.act == RWKV_ACT_TANH) f = tanhf(f);
+          if (p.act == RWKV_ACT_SIGMOID) f = sigmoid_f(f);
+          hi[e] = f2h(f);
+          lo[e] = f2h(f - h2f(hi[e]));
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          hi[e] = static_cast<half_t>(0.0f);
+          lo[e] = static_cast<half_t>(0.0f);
+        }
+      }
+      *reinterpret_cast<half8_t*>(&hi_s[m][ks]) = hi;
+      if (split) *reinterpret_cast<half8_t*>(&lo_s[m][ks]) = lo;
+    }
+    __syncthreads();
+    const int kn = min(kLoraKC, R - kc);
+#pragma unroll
+    for (int kk = 0; kk < kLoraKC / 16; ++kk) {
+      if (kk * 16 < kn) {
+        const half8_t ah = *reinterpret_cast<const half8_t*>(&hi_s[j][kk * 16 + h * 8]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, wreg[kk], acc, 0, 0, 0);
+        if (split) {
+          const half8_t al = *reinterpret_cast<const half8_t*>(&lo_s[j][kk * 16 + h * 8]);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, wreg[kk], acc, 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  if (!col_ok) return;
+  const float bias = p.bias ? h2f(p.bias[c]) : 0.0f;
+  // accumulator v of lane (j, h): row 8*(v/4) + 4h + v%4, column j
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int m = 8 * (v / 4) + 4 * h + (v % 4);
+    if (m < mn) {
       const int64_t o = static_cast<int64_t>(m0 + m) * a.C + c;
       float res;
-      if (a.vres) {
-        const float vv = h2f(a.v[o]);
-        const float gate = sigmoid_f(bias + acc);
-        res = vv + (h2f(a.v_first[o]) - vv) * gate;
+      if (p.vres) {
+        const float vv = h2f(p.v[o]);
+        const float gate = sigmoid_f(bias + acc[v]);
+        res = vv + (h2f(p.v_first[o]) - vv) * gate;
       } else {
-        res = acc + bias;
+        res = acc[v] + bias;
       }
-      a.out[o] = f2h(res);
+      p.out[o] = f2h(res);
     }
   }
 }
 
-int lora_out_launch(hipStream_t st, const LoraOutArgs& a) {
+int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a) {
+  RWKV_REQUIRE(a.n >= 1 && a.n <= 4, "lora_out: %d problems (1..4)", a.n);
   RWKV_REQUIRE(a.M > 0 && a.C > 0 && a.C % 32 == 0, "lora_out: C (%d) must be a positive multiple of 32", a.C);
-  RWKV_REQUIRE(a.R > 0 && a.R % 8 == 0 && a.R <= kLoraMaxR, "lora_out: rank %d must be a multiple of 8, at most %d",
-               a.R, kLoraMaxR);
-  RWKV_REQUIRE(a.h && a.w2 && a.out, "lora_out: NULL tensor");
-  RWKV_REQUIRE(!a.vres || (a.v && a.v_first && a.bias), "lora_out: v-residual gate needs v, v_first and v0");
-  hipLaunchKernelGGL(lora_out_kernel, dim3(a.C / 32, ceil_div(a.M, kLoraRowsPerBlock)), dim3(256), 0, st, a);
+  for (int i = 0; i < a.n; ++i) {
+    const LoraOutProblem& p = a.p[i];
+    RWKV_REQUIRE(p.R > 0 && p.R % 8 == 0 && p.R <= kLoraMaxR, "lora_out: rank %d must be a multiple of 8, at most %d",
+                 p.R, kLoraMaxR);
+    RWKV_REQUIRE(p.h && p.w2 && p.out, "lora_out: NULL tensor");
+    RWKV_REQUIRE(!p.vres || (p.v && p.v_first && p.bias), "lora_out: v-residual gate needs v, v_first and v0");
+  }
+  hipLaunchKernelGGL(lora_out_kernel, dim3(ceil_div(a.C, kLoraCols), ceil_div(a.M, kLoraRows), a.n), dim3(256), 0, st, a);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
@@ -99,15 +153,17 @@ int rwkv_hip_lora_in(rwkv_stream_t s, int M, int C, int R, const void* x, const 
 int rwkv_hip_lora_out(rwkv_stream_t s, int M, int C, int R, int act, const void* h, const void* w2, const void* bias,
                       int vres, const void* v, const void* v_first, void* out) {
   RWKV_REQUIRE(act == RWKV_ACT_NONE || act == RWKV_ACT_TANH || act == RWKV_ACT_SIGMOID, "lora_out: bad act %d", act);
-  LoraOutArgs a = {};
-  a.h = static_cast<const half_t*>(h);
-  a.w2 = static_cast<const half_t*>(w2);
-  a.bias = static_cast<const half_t*>(bias);
-  a.v = static_cast<const half_t*>(v);
-  a.v_first = static_cast<const half_t*>(v_first);
-  a.out = static_cast<half_t*>(out);
-  a.M = M; a.C = C; a.R = R; a.act = act; a.vres = vres;
-  return lora_out_launch(as_stream(s), a);
+  LoraOutMultiArgs a = {};
+  LoraOutProblem& p = a.p[0];
+  p.h = static_cast<const half_t*>(h);
+  p.w2 = static_cast<const half_t*>(w2);
+  p.bias = static_cast<const half_t*>(bias);
+  p.v = static_cast<const half_t*>(v);
+  p.v_first = static_cast<const half_t*>(v_first);
+  p.out = static_cast<half_t*>(out);
+  p.R = R; p.act = act; p.vres = vres;
+  a.n = 1; a.M = M; a.C = C;
+  return lora_out_multi(as_stream(s), a);
 }
 
 }  // extern "C"

@@ -429,20 +429,18 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     } else {
       // LoRA rank-out (+ activation, + v-residual gate)
       {
-        LoraOutArgs a = {};
-        a.M = rows; a.C = C;
-        a.h = b.hw; a.w2 = w.t[RWKV_T_W2]; a.R = m->Rw; a.act = RWKV_ACT_TANH; a.out = b.w12;
-        TRY_AUX(lora_out_launch(st, a));
-        a.h = b.ha; a.w2 = w.t[RWKV_T_A2]; a.R = m->Ra; a.act = RWKV_ACT_NONE; a.out = b.a12;
-        TRY_AUX(lora_out_launch(st, a));
-        a.h = b.hg; a.w2 = w.t[RWKV_T_G2]; a.R = m->Rg; a.act = RWKV_ACT_SIGMOID; a.out = b.g;
-        TRY_AUX(lora_out_launch(st, a));
+        LoraOutMultiArgs a = {};
+        a.M = rows; a.C = C; a.n = (l > 0) ? 4 : 3;
+        a.p[0].h = b.hw; a.p[0].w2 = w.t[RWKV_T_W2]; a.p[0].R = m->Rw; a.p[0].act = RWKV_ACT_TANH; a.p[0].out = b.w12;
+        a.p[1].h = b.ha; a.p[1].w2 = w.t[RWKV_T_A2]; a.p[1].R = m->Ra; a.p[1].act = RWKV_ACT_NONE; a.p[1].out = b.a12;
+        a.p[2].h = b.hg; a.p[2].w2 = w.t[RWKV_T_G2]; a.p[2].R = m->Rg; a.p[2].act = RWKV_ACT_SIGMOID; a.p[2].out = b.g;
         if (l > 0) {
-          a.h = b.hv; a.w2 = w.t[RWKV_T_V2]; a.R = m->Rv; a.act = RWKV_ACT_NONE; a.bias = w.t[RWKV_T_V0];
-          a.vres = 1; a.v = b.v; a.v_first = b.v_first; a.out = b.xv;  // xv is free after the projections
-          TRY_AUX(lora_out_launch(st, a));
+          LoraOutProblem& pv = a.p[3];
+          pv.h = b.hv; pv.w2 = w.t[RWKV_T_V2]; pv.R = m->Rv; pv.act = RWKV_ACT_NONE; pv.bias = w.t[RWKV_T_V0];
+          pv.vres = 1; pv.v = b.v; pv.v_first = b.v_first; pv.out = b.xv;  // xv is free after the projections
           v_cur = b.xv;
         }
+        TRY_AUX(lora_out_multi(st, a));
       }
 
       // kk normalise, a-gate, decay; operands widened to fp32 for the scalar-fed WKV kernel

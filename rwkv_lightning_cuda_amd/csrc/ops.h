@@ -145,16 +145,21 @@ int advance_launch(hipStream_t st, int n, int amount, int* x);
 int embed_gather_launch(hipStream_t st, int rows, int C, const int64_t* tokens, const half_t* table, half_t* out);
 
 // ---- lora.hip -----------------------------------------------------------------------------------
-struct LoraOutArgs {
+struct LoraOutProblem {
   const half_t* h;        // [M,R]
   const half_t* w2;       // [C,R]
   const half_t* bias;     // [C] or NULL
   const half_t* v;        // [M,C] (vres)
   const half_t* v_first;  // [M,C] (vres)
   half_t* out;            // [M,C]
-  int M, C, R, act, vres;
+  int R, act, vres;
 };
-int lora_out_launch(hipStream_t st, const LoraOutArgs& a);
+struct LoraOutMultiArgs {
+  LoraOutProblem p[4];
+  int n, M, C;
+};
+// up to four rank-out products over the same rows in one launch
+int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a);
 
 // ---- sampler.hip --------------------------------------------------------------------------------
 int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out);

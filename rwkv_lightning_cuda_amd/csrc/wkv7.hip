@@ -4,12 +4,11 @@
 //   sa = sum_j S[i][j]*a[j];  S[i][j] = S[i][j]*d[j] + sa*b[j] + k[j]*v[i];  y[i] = sum_j S[i][j]*r[j]
 // with the decay map d = exp(-e^-1/2 * sigmoid(w)) of :13-14,26-28.
 //
-// Sequence kernel (any T): one wavefront per (batch, head); lane i keeps state row i in 64 VGPRs for
-// the whole call.  The per-column operands r,d,k,a,b are the same for all 64 lanes, so they are read
-// through the scalar cache into SGPRs (wave-uniform addresses) and feed the FMAs as scalar operands:
-// no LDS traffic and no cross-lane work in the inner loop, and the summation order over j is the
-// sequential one of the reference.  Operands must therefore be fp32 with the decay already applied;
-// a small element-wise pre-pass produces them when the caller passes fp16 tensors or raw decay logits.
+// Sequence kernel (any T): four wavefronts per (batch, head), each lane keeps a 4 x 4 block of the 64 x 64 state
+// in registers for the whole call.  The per-column operands r,d,k,a,b of a token are staged in LDS as fp32 and
+// each lane reads only the four columns it owns; the two row sums of a step (sa and y) are reduced over the 16
+// lanes that share a row with DPP adds.  Operands must therefore be fp32 with the decay already applied; a small
+// element-wise pre-pass produces them when the caller passes fp16 tensors or raw decay logits.
 #include "ops.h"
 
 namespace rwkv {
@@ -44,70 +43,90 @@ __global__ __launch_bounds__(256) void wkv7_prepare_kernel(int64_t n, int64_t sl
 }
 
 // ---- sequence kernel -------------------------------------------------------------------------
-// grid = B*H, block = 64 (one wavefront per head): lane i owns row i of the 64x64 state in 64 VGPRs for the
-// whole call.  r,d,k,a,b are fp32 with `op_bs` elements between batch rows; v,y are IO with `io_bs` elements
-// between batch rows.  The five operand vectors of a token are the same for every lane, so they go through
-// LDS: the wavefront stages them kSeqChunk tokens at a time with coalesced 16-byte loads (4 tokens x 256 bytes
-// per load instruction), double-buffered, and each step reads them back as broadcast 16-byte LDS reads that
-// the scheduler overlaps with the 256 FMAs of the step.  The loads of chunk c+1 are in flight while chunk c
-// computes.  Each lane keeps its own v values of the chunk in registers.  The arithmetic of a step does not
-// depend on the chunking, so splitting T over several calls is bitwise neutral.
+// grid = B*H, block = 256 (four wavefronts per head).  Wavefront q owns state rows 16q..16q+15; its lane
+// (g, c) = (lane / 16, lane % 16) owns rows 16q + 4g .. +3 and columns 4c .. 4c+3, so the 16 lanes of one DPP
+// row hold complete state rows and the wavefronts never exchange data.  r,d,k,a,b are fp32 with `op_bs`
+// elements between batch rows; v,y are IO with `io_bs` elements between batch rows.  The block stages the
+// operands kSeqChunk tokens at a time with coalesced 16-byte loads, double-buffered (the loads of chunk c+1
+// are in flight while chunk c computes); a step costs each lane six 16-byte LDS reads (its four columns of the
+// five operands and its four v values), against 112 VALU operations.  y goes back through LDS so that the
+// global stores are coalesced.  The arithmetic of a step does not depend on the chunking, so splitting T over
+// several calls is bitwise neutral.
 constexpr int kSeqChunk = 8;
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false);
+  return x + __builtin_bit_cast(float, moved);
+}
+// Sum over the 16 lanes of a DPP row.  Every exchange is between two lanes that hold each other's operands,
+// so all 16 lanes end with the bitwise same value.
+__device__ __forceinline__ float row16_sum(float x) {
+  x = dpp_add<0xB1>(x);   // quad_perm [1,0,3,2]
+  x = dpp_add<0x4E>(x);   // quad_perm [2,3,0,1]
+  x = dpp_add<0x141>(x);  // row_half_mirror: quad 0 <-> 1, 2 <-> 3
+  x = dpp_add<0x140>(x);  // row_mirror: quads (0,1) <-> (3,2)
+  return x;
+}
+
 template <typename IO>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void wkv7_seq_kernel(
-    int T, int C, int H, float* __restrict__ state,
-                                                      const float* __restrict__ r, const float* __restrict__ d,
-                                                      const float* __restrict__ k, const float* __restrict__ a,
-                                                      const float* __restrict__ b, int64_t op_bs,
-                                                      const IO* __restrict__ v, IO* __restrict__ y, int64_t io_bs) {
-  __shared__ __align__(16) float ops[2][5][kSeqChunk][kHead];  // [buffer][a,b,d,k,r][token][column]
+__global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
+                                                       const float* __restrict__ r, const float* __restrict__ d,
+                                                       const float* __restrict__ k, const float* __restrict__ a,
+                                                       const float* __restrict__ b, int64_t op_bs,
+                                                       const IO* __restrict__ v, IO* __restrict__ y, int64_t io_bs) {
+  __shared__ __align__(16) float ops[2][kSeqChunk][5][kHead];  // [buffer][token][a,b,d,k,r][column]
+  __shared__ __align__(16) float vs[2][kSeqChunk][kHead];      // [buffer][token][row]
+  __shared__ __align__(16) float ys[2][kSeqChunk][kHead];
 
   const int bh = blockIdx.x;
   const int bi = bh / H;
   const int h = bh - bi * H;
-  const int lane = threadIdx.x;
-  float* srow = state + (static_cast<int64_t>(bh) * kHead + lane) * kHead;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int i0 = 16 * (tid >> 6) + 4 * (lane >> 4);  // first of this lane's 4 rows
+  const int j0 = 4 * (lane & 15);                    // first of its 4 columns
+  float* sblk = state + (static_cast<int64_t>(bh) * kHead + i0) * kHead + j0;
 
-  float S[kHead];
+  float4_t S[4];
 #pragma unroll
-  for (int j = 0; j < kHead; j += 4) {
-    const float4_t q = *reinterpret_cast<const float4_t*>(srow + j);
-    S[j] = q.x; S[j + 1] = q.y; S[j + 2] = q.z; S[j + 3] = q.w;
-  }
+  for (int i = 0; i < 4; ++i) S[i] = *reinterpret_cast<const float4_t*>(sblk + i * kHead);
 
   const int64_t base = static_cast<int64_t>(bi) * op_bs + h * kHead;
-  const float* src[5] = {a + base, b + base, d + base, k + base, r + base};
-  const int64_t iob = static_cast<int64_t>(bi) * io_bs + h * kHead + lane;
-  const int st_tok = lane >> 4;        // staging: this lane's token within a group of 4 ...
-  const int st_col = (lane & 15) * 4;  // ... and its 4 columns
+  const int64_t iob = static_cast<int64_t>(bi) * io_bs + h * kHead;
+  // staging: 5 operands x 8 tokens x 16 float4 = 640 float4 per chunk, 256 threads x 3 slots (the third half
+  // used); slot i of thread t: operand 2i + t/128, token (t % 128) / 16, columns 4 * (t % 16)
+  const int st_half = tid >> 7;
+  const int st_tok = (tid & 127) >> 4;
+  const int st_col = (tid & 15) * 4;
+  const float* src[3] = {(st_half ? b : a) + base, (st_half ? k : d) + base, r + base};
 
-  float4_t stage[5][kSeqChunk / 4];
-  float v_next[kSeqChunk], v_cur[kSeqChunk];
+  float4_t stage[3];
+  float v_stage[2];
 
   auto request = [&](int t0) {
 #pragma unroll
-    for (int o = 0; o < 5; ++o)
-#pragma unroll
-      for (int i = 0; i < kSeqChunk / 4; ++i) {
-        const int t = t0 + st_tok + 4 * i;
-        stage[o][i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        if (t < T) stage[o][i] = *reinterpret_cast<const float4_t*>(src[o] + static_cast<int64_t>(t) * C + st_col);
+    for (int i = 0; i < 3; ++i) {
+      stage[i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      const int t = t0 + st_tok;
+      if (t < T && (i < 2 || st_half == 0)) {
+        stage[i] = *reinterpret_cast<const float4_t*>(src[i] + static_cast<int64_t>(t) * C + st_col);
       }
+    }
 #pragma unroll
-    for (int tt = 0; tt < kSeqChunk; ++tt) {
-      v_next[tt] = 0.0f;
-      if (t0 + tt < T) v_next[tt] = static_cast<float>(v[iob + static_cast<int64_t>(t0 + tt) * C]);
+    for (int i = 0; i < 2; ++i) {
+      const int t = t0 + (tid >> 6) + 4 * i;
+      v_stage[i] = 0.0f;
+      if (t < T) v_stage[i] = static_cast<float>(v[iob + static_cast<int64_t>(t) * C + lane]);
     }
   };
   auto commit = [&](int buf) {
 #pragma unroll
-    for (int o = 0; o < 5; ++o)
+    for (int i = 0; i < 3; ++i) {
+      if (i < 2 || st_half == 0) *reinterpret_cast<float4_t*>(&ops[buf][st_tok][2 * i + st_half][st_col]) = stage[i];
+    }
 #pragma unroll
-      for (int i = 0; i < kSeqChunk / 4; ++i)
-        *reinterpret_cast<float4_t*>(&ops[buf][o][st_tok + 4 * i][st_col]) = stage[o][i];
-#pragma unroll
-    for (int tt = 0; tt < kSeqChunk; ++tt) v_cur[tt] = v_next[tt];
+    for (int i = 0; i < 2; ++i) vs[buf][(tid >> 6) + 4 * i][lane] = v_stage[i];
   };
 
   request(0);
@@ -118,75 +137,73 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
     const bool more = t0 + kSeqChunk < T;
     if (more) request(t0 + kSeqChunk);
     const int n = min(kSeqChunk, T - t0);
-    // Operand reads are software-pipelined by hand (the compiler otherwise issues each LDS read right before
-    // its use and stalls on every one): the a vector of a step and its first column group are requested during
-    // the previous step; inside a step the reads of column group g+1 are issued before group g computes.
-    // __builtin_amdgcn_sched_barrier(0) keeps the scheduler from sinking the reads back down.
-    float4_t A[kHead / 4];
-    float4_t G[2][8];  // per group of 8 columns: b, d, k, r as two float4 each
-    auto load_a = [&](int tt, int lo, int hi) {
+    auto load_step = [&](int tt, float4_t (&dst)[6]) {
 #pragma unroll
-      for (int j4 = lo; j4 < hi; ++j4) A[j4] = *reinterpret_cast<const float4_t*>(&ops[buf][0][tt][4 * j4]);
+      for (int o = 0; o < 5; ++o) dst[o] = *reinterpret_cast<const float4_t*>(&ops[buf][tt][o][j0]);
+      dst[5] = *reinterpret_cast<const float4_t*>(&vs[buf][tt][i0]);
     };
-    auto load_group = [&](int tt, int g, float4_t (&dst)[8]) {
+    auto step = [&](int tt, const float4_t (&q)[6]) {
+      const float4_t av = q[0], bv = q[1], dv = q[2], kv = q[3], rv = q[4], vv = q[5];
+      float sa[4], yy[4];
 #pragma unroll
-      for (int o = 0; o < 4; ++o) {
-        dst[2 * o] = *reinterpret_cast<const float4_t*>(&ops[buf][1 + o][tt][8 * g]);
-        dst[2 * o + 1] = *reinterpret_cast<const float4_t*>(&ops[buf][1 + o][tt][8 * g + 4]);
+      for (int i = 0; i < 4; ++i) {
+        float p = S[i].x * av.x;
+        p = fmaf(S[i].y, av.y, p);
+        p = fmaf(S[i].z, av.z, p);
+        p = fmaf(S[i].w, av.w, p);
+        sa[i] = p;
       }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sa[i] = row16_sum(sa[i]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float vi = vv[i];
+        S[i].x = fmaf(S[i].x, dv.x, fmaf(sa[i], bv.x, kv.x * vi));
+        S[i].y = fmaf(S[i].y, dv.y, fmaf(sa[i], bv.y, kv.y * vi));
+        S[i].z = fmaf(S[i].z, dv.z, fmaf(sa[i], bv.z, kv.z * vi));
+        S[i].w = fmaf(S[i].w, dv.w, fmaf(sa[i], bv.w, kv.w * vi));
+        float p = S[i].x * rv.x;
+        p = fmaf(S[i].y, rv.y, p);
+        p = fmaf(S[i].z, rv.z, p);
+        p = fmaf(S[i].w, rv.w, p);
+        yy[i] = p;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) yy[i] = row16_sum(yy[i]);
+      if ((lane & 15) == 0) *reinterpret_cast<float4_t*>(&ys[buf][tt][i0]) = float4_t{yy[0], yy[1], yy[2], yy[3]};
     };
-    load_a(0, 0, kHead / 4);
-    load_group(0, 0, G[0]);
+    if (n == kSeqChunk) {
+      // Full chunk, straight-line: the operands of step tt+1 are read while step tt computes;
+      // __builtin_amdgcn_sched_barrier(0) keeps the scheduler from sinking the reads down to their first use.
+      float4_t q[2][6];
+      load_step(0, q[0]);
 #pragma unroll
-    for (int tt = 0; tt < kSeqChunk; ++tt) {
-      if (tt < n) {
-        const float vi = v_cur[tt];
-        float sa = 0.0f;
-#pragma unroll
-        for (int j4 = 0; j4 < kHead / 4; ++j4) {
-          sa = fmaf(S[4 * j4 + 0], A[j4].x, sa);
-          sa = fmaf(S[4 * j4 + 1], A[j4].y, sa);
-          sa = fmaf(S[4 * j4 + 2], A[j4].z, sa);
-          sa = fmaf(S[4 * j4 + 3], A[j4].w, sa);
-        }
-        float yy = 0.0f;
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
-          // requests for later use: next column group (or the next step's first one), a slice of the next a vector
-          if (g + 1 < 8) {
-            load_group(tt, g + 1, G[(g + 1) & 1]);
-          } else if (tt + 1 < kSeqChunk) {
-            load_group(tt + 1, 0, G[0]);
-          }
-          if (tt + 1 < kSeqChunk) load_a(tt + 1, 2 * g, 2 * g + 2);
-          __builtin_amdgcn_sched_barrier(0);
-          const float4_t(&q)[8] = G[g & 1];
-          const float bb[8] = {q[0].x, q[0].y, q[0].z, q[0].w, q[1].x, q[1].y, q[1].z, q[1].w};
-          const float dd[8] = {q[2].x, q[2].y, q[2].z, q[2].w, q[3].x, q[3].y, q[3].z, q[3].w};
-          const float kk[8] = {q[4].x, q[4].y, q[4].z, q[4].w, q[5].x, q[5].y, q[5].z, q[5].w};
-          const float rr[8] = {q[6].x, q[6].y, q[6].z, q[6].w, q[7].x, q[7].y, q[7].z, q[7].w};
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            float sv = S[8 * g + e];
-            sv = fmaf(sv, dd[e], fmaf(sa, bb[e], kk[e] * vi));
-            yy = fmaf(sv, rr[e], yy);
-            S[8 * g + e] = sv;
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        y[iob + static_cast<int64_t>(t0 + tt) * C] = static_cast<IO>(yy);
+      for (int tt = 0; tt < kSeqChunk; ++tt) {
+        if (tt + 1 < kSeqChunk) load_step(tt + 1, q[(tt + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        step(tt, q[tt & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      // the last, partial chunk (and single-token calls): same step arithmetic, rolled loop
+#pragma unroll 1
+      for (int tt = 0; tt < n; ++tt) {
+        float4_t q[6];
+        load_step(tt, q);
+        step(tt, q);
       }
     }
     if (more) commit(buf ^ 1);
     __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int tt = (tid >> 6) + 4 * i;
+      if (tt < n) y[iob + static_cast<int64_t>(t0 + tt) * C + lane] = static_cast<IO>(ys[buf][tt][lane]);
+    }
   }
 
 #pragma unroll
-  for (int j = 0; j < kHead; j += 4) {
-    float4_t q;
-    q.x = S[j]; q.y = S[j + 1]; q.z = S[j + 2]; q.w = S[j + 3];
-    *reinterpret_cast<float4_t*>(srow + j) = q;
-  }
+  for (int i = 0; i < 4; ++i) *reinterpret_cast<float4_t*>(sblk + i * kHead) = S[i];
 }
 
 template <typename IO>
@@ -194,7 +211,7 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
                        const IO* w, const IO* k, const IO* v, const IO* a, const IO* b, IO* y) {
   const int64_t row = static_cast<int64_t>(T) * C;
   if (std::is_same<IO, float>::value && w_mode == RWKV_W_DECAY) {
-    hipLaunchKernelGGL(wkv7_seq_kernel<IO>, dim3(B * H), dim3(64), 0, st, T, C, H, state,
+    hipLaunchKernelGGL(wkv7_seq_kernel<IO>, dim3(B * H), dim3(256), 0, st, T, C, H, state,
                        reinterpret_cast<const float*>(r), reinterpret_cast<const float*>(w),
                        reinterpret_cast<const float*>(k), reinterpret_cast<const float*>(a),
                        reinterpret_cast<const float*>(b), row, v, y, row);
@@ -220,7 +237,7 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
     const int64_t n = slab_row * B;
     hipLaunchKernelGGL(wkv7_prepare_kernel<IO>, dim3(ceil_div(n, 256)), dim3(256), 0, st, n, slab_row, row, w_mode,
                        r + off, w + off, k + off, a + off, b + off, r32, d32, k32, a32, b32);
-    hipLaunchKernelGGL(wkv7_seq_kernel<IO>, dim3(B * H), dim3(64), 0, st, tn, C, H, state, r32, d32, k32, a32, b32,
+    hipLaunchKernelGGL(wkv7_seq_kernel<IO>, dim3(B * H), dim3(256), 0, st, tn, C, H, state, r32, d32, k32, a32, b32,
                        slab_row, v + off, y + off, row);
   }
   hipError_t err = hipGetLastError();
@@ -235,7 +252,7 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
 int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                         const float* k, const float* a, const float* b, int64_t op_bs, const half_t* v, half_t* y,
                         int64_t io_bs) {
-  hipLaunchKernelGGL(wkv7_seq_kernel<half_t>, dim3(B * H), dim3(64), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
+  hipLaunchKernelGGL(wkv7_seq_kernel<half_t>, dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
                      io_bs);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;

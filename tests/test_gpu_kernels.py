@@ -348,6 +348,35 @@ def test_kk_gate_groupnorm_lora(gpu, orc):
             assert err <= F16_TOL
 
 
+@pytest.mark.parametrize("rows,C,R", [(1, 96, 8), (33, 256, 136), (70, 768, 480), (128, 4096, 512), (64, 4096, 96)])
+def test_lora_out_keeps_the_activated_hidden_in_fp32(gpu, rows, C, R):
+    """The rank-out product feeds act(h) to the matrix core as an fp16 hi + lo pair.  Against a float64 dot over
+    the float32 activation, the fp16 result is the correctly rounded one except at near-ties; with the lo term
+    dropped a third of the outputs would move by an ulp."""
+    hip = gpu
+    rng = np.random.default_rng(rows * 1000 + R)
+    h = (rng.standard_normal((rows, R)) * 1.5).astype(np.float16)
+    w2 = (rng.standard_normal((C, R)) * 0.1).astype(np.float16)
+    for act in (hip.ACT_TANH, hip.ACT_SIGMOID, hip.ACT_NONE):
+        hf = h.astype(np.float32)
+        if act == hip.ACT_TANH:
+            hf = np.tanh(hf)
+        elif act == hip.ACT_SIGMOID:
+            hf = (1.0 / (1.0 + np.exp(-hf))).astype(np.float32)
+        exact = hf.astype(np.float64) @ w2.astype(np.float64).T
+        want = exact.astype(np.float16)
+        o = hip.DeviceArray((rows, C), np.float16)
+        hip.lora_out(rows, C, R, act, dev(hip, h), dev(hip, w2), o)
+        hip.device_sync()
+        got = o.numpy()
+        # half an fp16 ulp of rounding + the fp32 accumulation error (a few 1e-8 of the sum of magnitudes)
+        mags = np.abs(hf).astype(np.float64) @ np.abs(w2).astype(np.float64).T
+        bound = 0.5 * np.spacing(np.abs(want)).astype(np.float64) + 1e-6 * mags
+        assert np.all(np.abs(got.astype(np.float64) - exact) <= bound)
+        off = np.mean(got.view(np.uint16) != want.view(np.uint16))
+        assert off <= 0.01, "act %d: %.4f of the outputs are not the correctly rounded value" % (act, off)
+
+
 def test_small_elementwise(gpu, orc):
     hip = gpu
     rng = np.random.default_rng(2)
