@@ -14,14 +14,14 @@
 // to the matrix core after an exact in-register expansion of the codes, without any transpose or LDS
 // traffic for the weights; every weight byte leaves HBM once per 32*MT rows of X.
 //
-// Work split.  Block = 4 wavefronts = 4 adjacent bands (128 output columns) x one K slice; the X rows of
-// the slice are staged in LDS in chunks of KC (128 or 256) and shared by the four wavefronts.  Chunks are
-// software-pipelined: while the matrix core works on chunk c out of one LDS tile and one register set, the
-// loads of chunk c+1 (first this thread's share of X, then the wavefront's weight pieces, so that waiting for
-// X does not wait for the weights) are in flight into the other set; one barrier per chunk.
-// grid = (row tiles, column blocks, K splits).  With more than one split each block writes an fp32 partial
-// tile and a second small kernel sums the partials in split order (a fixed order: results do not depend on
-// scheduling) and applies scale and epilogue.
+// Work split.  A block covers 32*MT rows x 128 output columns x one K slice with one or two groups of four
+// wavefronts: each wavefront streams one band, the groups take alternate chunks of KC = 128 k and meet in LDS at
+// the end.  The X rows of a chunk are staged in LDS and shared by the four wavefronts of the group.  Chunks
+// are software-pipelined: weight pieces are requested three chunks ahead into a ring of register sets, X two
+// chunks ahead, the X fragments of the next MFMA step are read from LDS while the current one runs; one barrier
+// per chunk.  With more than one K split each block writes an fp32 partial tile and a second small kernel
+// sums the partials in split order (a fixed order: results do not depend on scheduling) and applies scale and
+// epilogue.
 #include <algorithm>
 #include <cstdlib>
 
@@ -105,6 +105,7 @@ struct StreamArgs {
   int n_problems;
   int M, K;
   int splits, k_per_split;
+  int row_tiles, col_blocks;
   int epilogue, out_f32;
 };
 
@@ -148,6 +149,7 @@ struct Tile {
   static constexpr int XV = BM * (KC / 8) / 256;    // 16-byte vectors of X per thread per chunk
   static constexpr int QG = KC / 128;               // int4 scale groups per chunk
   static constexpr int NACC = MT == 1 ? 2 : 1;      // independent accumulation chains per row tile
+  static constexpr int DEPTH = (NW * 4 <= 16) ? 4 : (NW * 4 <= 32 ? 3 : 2);  // weight register sets in the ring
   static constexpr int kTileHalfs = BM * XSTRIDE;   // one staged X tile
   static_assert(KC % 128 == 0 && XV >= 1, "chunk must hold whole int4 groups and at least one vector per thread");
 };
@@ -161,86 +163,103 @@ __device__ __forceinline__ float finish_value(float v, int epilogue) {
   return v;
 }
 
-// One chunk's operands held by a lane between request and use.
+// One chunk's slice of X held by a thread between request and its store to LDS.
 template <int FMT, int MT, int KC>
-struct ChunkRegs {
+struct XRegs {
   using T = Tile<FMT, MT, KC>;
   uint4_t xv[T::XV];
-  uint4_t w[T::NW];
-  float sc[T::QG], zb[T::QG];
 
-  // X first, then the weights: waiting for X (to store it to LDS) does not wait for the weight pieces.
-  __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int m0, int kc, bool active,
-                                          const uint4_t* wband, int n) {
-    using P = typename T::P;
+  __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int tid, int m0, int kc) {
 #pragma unroll
     for (int i = 0; i < T::XV; ++i) {
-      const int idx = threadIdx.x + i * 256;
+      const int idx = tid + i * 256;
       const int r = idx / (KC / 8);
       const int c = (idx % (KC / 8)) * 8;
       xv[i] = uint4_t{0u, 0u, 0u, 0u};
       if (m0 + r < g.M) xv[i] = *reinterpret_cast<const uint4_t*>(pr.x + static_cast<int64_t>(m0 + r) * g.K + kc + c);
     }
-    if (active) {
-      const uint4_t* wp = wband + static_cast<int64_t>(kc / T::G) * (P::PIECES * 64);
-#pragma unroll
-      for (int i = 0; i < T::NW; ++i) w[i] = wp[i * 64];
-      if constexpr (FMT == RWKV_FMT_W4) {
-        const int64_t q0 = static_cast<int64_t>(n) * (g.K >> 7) + (kc >> 7);
-#pragma unroll
-        for (int q = 0; q < T::QG; ++q) {
-          sc[q] = h2f(pr.scale[q0 + q]);
-          zb[q] = 1024.0f + static_cast<float>(pr.zp[q0 + q]);
-        }
-      }
-    }
   }
 
-  __device__ __forceinline__ void store_x(half_t* xs) const {
+  __device__ __forceinline__ void store_x(int tid, half_t* xs) const {
 #pragma unroll
     for (int i = 0; i < T::XV; ++i) {
-      const int idx = threadIdx.x + i * 256;
+      const int idx = tid + i * 256;
       const int r = idx / (KC / 8);
       const int c = (idx % (KC / 8)) * 8;
       *reinterpret_cast<uint4_t*>(xs + r * T::XSTRIDE + c) = xv[i];
     }
   }
+};
 
+// One chunk's weight pieces (and int4 group scales) held by a lane between request and use.
+template <int FMT, int MT, int KC>
+struct WRegs {
+  using T = Tile<FMT, MT, KC>;
+  uint4_t w[T::NW];
+  float sc[T::QG], zb[T::QG];
+
+  __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int kc, const uint4_t* wband,
+                                          int n) {
+    using P = typename T::P;
+    const uint4_t* wp = wband + static_cast<int64_t>(kc / T::G) * (P::PIECES * 64);
+#pragma unroll
+    for (int i = 0; i < T::NW; ++i) w[i] = wp[i * 64];
+    if constexpr (FMT == RWKV_FMT_W4) {
+      const int64_t q0 = static_cast<int64_t>(n) * (g.K >> 7) + (kc >> 7);
+#pragma unroll
+      for (int q = 0; q < T::QG; ++q) {
+        sc[q] = h2f(pr.scale[q0 + q]);
+        zb[q] = 1024.0f + static_cast<float>(pr.zp[q0 + q]);
+      }
+    }
+  }
+
+  // The X fragments of MFMA step ks+1 are read from LDS while step ks runs (the compiler on its own issues each
+  // read right before its use, which leaves the matrix core idle for the LDS latency on every step);
+  // __builtin_amdgcn_sched_barrier(0) keeps the reads where they are written.
   __device__ __forceinline__ void multiply(const half_t* xs, int j, int h, float16_t (&acc)[MT][T::NACC],
                                            float16_t (&part)[MT][T::NACC]) const {
     using P = typename T::P;
+    constexpr int NK = T::GROUPS * T::STEPS;
+    const half_t* xlane = xs + j * T::XSTRIDE + h * P::KR;
+    half8_t a[2][MT];
+    auto load_a = [&](int ks, half8_t (&dst)[MT]) {
+      const half_t* xa = xlane + (ks / T::STEPS) * T::G + 8 * (ks % T::STEPS);
 #pragma unroll
-    for (int gi = 0; gi < T::GROUPS; ++gi) {
+      for (int mt = 0; mt < MT; ++mt) dst[mt] = *reinterpret_cast<const half8_t*>(xa + mt * 32 * T::XSTRIDE);
+    };
+    load_a(0, a[0]);
 #pragma unroll
-      for (int s = 0; s < T::STEPS; ++s) {
-        half8_t b;
-        if constexpr (FMT == RWKV_FMT_F16) {
-          const uint4_t piece = w[gi * 2 + s];
-          b = __builtin_bit_cast(half8_t, piece);
-        } else if constexpr (FMT == RWKV_FMT_W8) {
-          const uint4_t piece = w[gi];
-          b = s == 0 ? expand_w8(piece[0], piece[1]) : expand_w8(piece[2], piece[3]);
+    for (int ks = 0; ks < NK; ++ks) {
+      const int gi = ks / T::STEPS;
+      const int s = ks % T::STEPS;
+      if (ks + 1 < NK) load_a(ks + 1, a[(ks + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      half8_t b;
+      if constexpr (FMT == RWKV_FMT_F16) {
+        const uint4_t piece = w[gi * 2 + s];
+        b = __builtin_bit_cast(half8_t, piece);
+      } else if constexpr (FMT == RWKV_FMT_W8) {
+        const uint4_t piece = w[gi];
+        b = s == 0 ? expand_w8(piece[0], piece[1]) : expand_w8(piece[2], piece[3]);
+      } else {
+        const uint4_t piece = w[gi];
+        const half_t zf = static_cast<half_t>(zb[(gi * T::G) >> 7]);
+        const half2_t bias = {zf, zf};
+        b = expand_w4(piece[s], bias);
+      }
+      constexpr int kChainMask = T::NACC - 1;
+      const int chain = ks & kChainMask;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        if constexpr (FMT == RWKV_FMT_W4) {
+          part[mt][chain] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks & 1][mt], b, part[mt][chain], 0, 0, 0);
         } else {
-          const uint4_t piece = w[gi];
-          const half_t zf = static_cast<half_t>(zb[(gi * T::G) >> 7]);
-          const half2_t bias = {zf, zf};
-          b = expand_w4(piece[s], bias);
-        }
-        constexpr int kChainMask = T::NACC - 1;
-        const int chain = (gi * T::STEPS + s) & kChainMask;
-        const half_t* xa = xs + j * T::XSTRIDE + gi * T::G + h * P::KR + 8 * s;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const half8_t a = *reinterpret_cast<const half8_t*>(xa + mt * 32 * T::XSTRIDE);
-          if constexpr (FMT == RWKV_FMT_W4) {
-            part[mt][chain] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, part[mt][chain], 0, 0, 0);
-          } else {
-            acc[mt][chain] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[mt][chain], 0, 0, 0);
-          }
+          acc[mt][chain] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks & 1][mt], b, acc[mt][chain], 0, 0, 0);
         }
       }
       if constexpr (FMT == RWKV_FMT_W4) {
-        if (((gi + 1) * T::G) % 128 == 0) {  // end of a 128-group: fold with its scale
+        if (s == T::STEPS - 1 && ((gi + 1) * T::G) % 128 == 0) {  // end of a 128-group: fold with its scale
           const float s128 = sc[(gi * T::G) >> 7];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
@@ -253,29 +272,45 @@ struct ChunkRegs {
               }
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 };
 
-// One block of one problem: 128 columns x the block's K slice, which is a whole number of chunks.  Two X tiles
-// in LDS and two register sets alternate, so one barrier per chunk suffices and the next chunk's loads are in
-// flight while the matrix core works on the current one.
-template <int FMT, int MT, int KC>
-__device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamProblem& pr, int col_block, half_t* xs) {
+// One block of one problem: 128 columns x the block's K slice.  The block has KG groups of four wavefronts;
+// group kg takes chunks kg, kg + KG, ... of the slice with its own pair of X tiles in LDS, and the groups' sums
+// meet in LDS at the end (in group order), so that a CU holds two wavefronts per SIMD - one's code expansion
+// overlaps the other's matrix-core time - without more fp32 partial tiles in HBM.
+//
+// Per group and chunk c: the X slice of chunk c+2 is requested into registers, the weight pieces of chunk
+// c+D-1 into a ring of D register sets, the matrix core runs chunk c out of LDS tile c&1, then the X slice of
+// chunk c+1 (requested one iteration earlier) is stored to the other tile; one barrier per chunk.  Every load
+// of the loop is issued unconditionally - past the end of the slice it re-reads the current chunk, which is in
+// cache - because a load under a branch makes the compiler's s_waitcnt accounting assume the shorter path
+// and wait for everything in flight.  Within an iteration X is requested before the weights, so that waiting
+// for X does not wait for the younger weight loads.
+template <int FMT, int MT, int KC, int KG>
+__device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamProblem& pr, int row_tile, int col_block,
+                                             int split, half_t* xs_all) {
   using T = Tile<FMT, MT, KC>;
   using P = typename T::P;
   constexpr int BM = T::BM;
 
-  const int wave = threadIdx.x >> 6;
-  const int lane = threadIdx.x & 63;
+  const int tid = threadIdx.x & 255;  // thread within its k-group
+  const int kg = threadIdx.x >> 8;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
   const int j = lane & 31;
   const int h = lane >> 5;
-  const int m0 = blockIdx.x * BM;
-  const int band = col_block * 4 + wave;  // 32-row band of W = 32 output columns
-  const bool active = band * 32 < pr.N;
+  const int m0 = row_tile * BM;
+  const int band_here = col_block * 4 + wave;  // 32-row band of W = 32 output columns
+  const bool active = band_here * 32 < pr.N;
+  const int band = active ? band_here : pr.N / 32 - 1;  // a wavefront past the last band repeats it and stores nothing
   const int n = band * 32 + j;
-  const int kbeg = blockIdx.z * g.k_per_split;
-  const int nchunks = g.k_per_split / KC;
+  constexpr int KSTRIDE = KC * KG;  // between consecutive chunks of one group
+  const int kbeg = split * g.k_per_split + kg * KC;
+  const int nchunks = g.k_per_split / KSTRIDE;
+  half_t* xs = xs_all + kg * 2 * T::kTileHalfs;
 
   float16_t acc[MT][T::NACC], part[MT][T::NACC];
 #pragma unroll
@@ -289,26 +324,53 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
       }
 
   // this lane's first piece of the band; consecutive pieces are 64 uint4 apart
-  const uint4_t* wband = pr.wp + (static_cast<int64_t>(active ? band : 0) * (g.K / T::G)) * (P::PIECES * 64) + lane;
+  const uint4_t* wband = pr.wp + (static_cast<int64_t>(band) * (g.K / T::G)) * (P::PIECES * 64) + lane;
 
-  ChunkRegs<FMT, MT, KC> r0, r1;
-  r0.request(g, pr, m0, kbeg, active, wband, n);
-  r0.store_x(xs);
+  constexpr int D = T::DEPTH;
+  WRegs<FMT, MT, KC> wr[D];
+  XRegs<FMT, MT, KC> xr[2];
+  const int last = nchunks - 1;
+  xr[0].request(g, pr, tid, m0, kbeg);
+  xr[1].request(g, pr, tid, m0, kbeg + min(1, last) * KSTRIDE);
+#pragma unroll
+  for (int i = 0; i < D - 1; ++i) wr[i].request(g, pr, kbeg + min(i, last) * KSTRIDE, wband, n);
+  xr[0].store_x(tid, xs);
   __syncthreads();
-  for (int c = 0; c < nchunks; c += 2) {
-    // even chunk: operands in r0 / tile 0
-    if (c + 1 < nchunks) r1.request(g, pr, m0, kbeg + (c + 1) * KC, active, wband, n);
-    if (active) r0.multiply(xs, j, h, acc, part);
-    if (c + 1 >= nchunks) break;
-    r1.store_x(xs + T::kTileHalfs);
-    __syncthreads();
-    // odd chunk: operands in r1 / tile 1
-    if (c + 2 < nchunks) r0.request(g, pr, m0, kbeg + (c + 2) * KC, active, wband, n);
-    if (active) r1.multiply(xs + T::kTileHalfs, j, h, acc, part);
-    if (c + 2 < nchunks) {
-      r0.store_x(xs);
+  constexpr int U = (D % 2 == 0) ? D : 2 * D;  // unroll: register sets and LDS tiles are indexed statically
+  for (int c0 = 0; c0 < nchunks; c0 += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      if (c >= nchunks) break;
+      xr[u & 1].request(g, pr, tid, m0, kbeg + (c + 2 <= last ? c + 2 : c) * KSTRIDE);
+      wr[(u + D - 1) % D].request(g, pr, kbeg + (c + D - 1 <= last ? c + D - 1 : c) * KSTRIDE, wband, n);
+      wr[u % D].multiply(xs + (u & 1) * T::kTileHalfs, j, h, acc, part);
+      xr[(u + 1) & 1].store_x(tid, xs + ((u + 1) & 1) * T::kTileHalfs);
       __syncthreads();
     }
+  }
+
+  if constexpr (T::NACC == 2) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mt][0][v] += acc[mt][1][v];
+  }
+  if constexpr (KG == 2) {
+    // the X tiles are free after the last barrier: group 1 hands its sums to group 0 through them
+    float* red = reinterpret_cast<float*>(xs_all);
+    if (kg == 1) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[(mt * 16 + v) * 256 + tid] = acc[mt][0][v];
+    }
+    __syncthreads();
+    if (kg == 1) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mt][0][v] += red[(mt * 16 + v) * 256 + tid];
   }
   if (!active) return;
 
@@ -316,15 +378,14 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
   if constexpr (FMT == RWKV_FMT_W8) {
     if (g.splits == 1) scl = h2f(pr.scale[n]);
   }
-  float* part_out = g.splits > 1 ? pr.partial + static_cast<int64_t>(blockIdx.z) * g.M * pr.N : nullptr;
+  float* part_out = g.splits > 1 ? pr.partial + static_cast<int64_t>(split) * g.M * pr.N : nullptr;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int row = m0 + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
       if (row >= g.M) continue;
-      float sum = acc[mt][0][v];
-      if constexpr (T::NACC == 2) sum += acc[mt][1][v];
+      const float sum = acc[mt][0][v];
       const int64_t o = static_cast<int64_t>(row) * pr.N + n;
       if (part_out) {
         part_out[o] = sum;
@@ -339,18 +400,26 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
     }
 }
 
-// grid = (row tiles of 32*MT, column blocks of 128 over all problems, splits); block = 256.
-template <int MT, int KC>
-__global__ __launch_bounds__(256) void gemm_stream_kernel(StreamArgs g) {
-  __shared__ __align__(16) half_t xs[2 * 32 * MT * (KC + 8)];
+// grid = row tiles x roundup(column blocks of 128 over all problems x splits, 8), one-dimensional; block = 256 * KG.
+// Workgroups go to the eight XCDs round-robin by linear id, each XCD with its own L2: the id is decoded so that
+// the row tiles of one (column block, split) pair - which stream the same weights - land on the same XCD.
+template <int MT, int KC, int KG>
+__global__ __launch_bounds__(256 * KG) void gemm_stream_kernel(StreamArgs g) {
+  __shared__ __align__(16) half_t xs[KG * 2 * 32 * MT * (KC + 8)];
+  const int id = blockIdx.x;
+  const int row_tile = (id >> 3) % g.row_tiles;
+  const int pair = (id / (8 * g.row_tiles)) * 8 + (id & 7);
+  if (pair >= g.col_blocks * g.splits) return;
+  const int col_all = pair % g.col_blocks;
+  const int split = pair / g.col_blocks;
   int pi = 0;
-  while (pi + 1 < g.n_problems && static_cast<int>(blockIdx.y) >= g.block_end[pi]) ++pi;
-  const int col_block = blockIdx.y - (pi > 0 ? g.block_end[pi - 1] : 0);
+  while (pi + 1 < g.n_problems && col_all >= g.block_end[pi]) ++pi;
+  const int col_block = col_all - (pi > 0 ? g.block_end[pi - 1] : 0);
   const StreamProblem& pr = g.p[pi];
   switch (pr.fmt) {
-    case RWKV_FMT_W8: stream_block<RWKV_FMT_W8, MT, KC>(g, pr, col_block, xs); break;
-    case RWKV_FMT_W4: stream_block<RWKV_FMT_W4, MT, KC>(g, pr, col_block, xs); break;
-    default: stream_block<RWKV_FMT_F16, MT, KC>(g, pr, col_block, xs); break;
+    case RWKV_FMT_W8: stream_block<RWKV_FMT_W8, MT, KC, KG>(g, pr, row_tile, col_block, split, xs); break;
+    case RWKV_FMT_W4: stream_block<RWKV_FMT_W4, MT, KC, KG>(g, pr, row_tile, col_block, split, xs); break;
+    default: stream_block<RWKV_FMT_F16, MT, KC, KG>(g, pr, row_tile, col_block, split, xs); break;
   }
 }
 
@@ -404,31 +473,36 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs g) {
   }
 }
 
-static int row_tiles(int M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
-
-// Tuning hooks: RWKV_GEMM_BLOCKS = blocks wanted per launch, RWKV_GEMM_KC = 128 or 256 (chunk of K).
+// RWKV_GEMM_BLOCKS (tuning hook) = blocks wanted per launch before K is split.
 static int env_int(const char* name, int fallback) {
   const char* e = getenv(name);
   const int v = e ? atoi(e) : 0;
   return v > 0 ? v : fallback;
 }
 static int target_blocks() {
-  static const int v = env_int("RWKV_GEMM_BLOCKS", 512);
+  static const int v = env_int("RWKV_GEMM_BLOCKS", 256);
   return v;
 }
-static int chunk_k(int mt) {
-  static const int v = env_int("RWKV_GEMM_KC", 0);
-  if (v == 128 || (v == 256 && mt < 4)) return v;
-  return mt >= 4 ? 128 : 256;  // two X tiles stay within 36-70 KiB of LDS
+
+// Tile per row count (measured on 4096x4096, 16384x4096 and 4096x16384 int8 weights): up to 64 rows one 32-row
+// tile per block, so that two or more row tiles share the weights through their XCD's L2 and the split stays
+// small; up to 512 rows 64-row tiles; both with two wavefront groups per block.  Above that 128-row tiles with
+// one group (128 accumulator registers per lane leave no room for a second wavefront per SIMD).
+struct StreamConfig {
+  int mt, kc, kg;
+};
+static StreamConfig choose_config(int M) {
+  if (M <= 64) return StreamConfig{1, 128, 2};
+  if (M <= 512) return StreamConfig{2, 128, 2};
+  return StreamConfig{4, 128, 1};
 }
 
-// Split count: a power of two that gives enough blocks to occupy the CUs, K slices whole chunks.
+// Split count: a power of two that gives enough blocks to occupy the CUs, K slices whole chunks of every group.
 static int choose_splits(int M, int col_blocks, int K) {
-  const int mt = row_tiles(M);
-  const int kc = chunk_k(mt);
-  const int tiles = ceil_div(M, 32 * mt) * col_blocks;
+  const StreamConfig c = choose_config(M);
+  const int tiles = ceil_div(M, 32 * c.mt) * col_blocks;
   int splits = 1;
-  while (tiles * splits < target_blocks() && K % (splits * 2 * kc) == 0 && splits < 32) splits *= 2;
+  while (tiles * splits < target_blocks() && K % (splits * 2 * c.kc * c.kg) == 0 && splits < 32) splits *= 2;
   return splits;
 }
 
@@ -468,8 +542,7 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
     g.block_end[i] = col_blocks;
     g.p[i] = StreamProblem{q.x, static_cast<const uint4_t*>(q.packed), q.scale, q.zp, q.y, nullptr, q.N, q.fmt};
   }
-  const int mt = row_tiles(M);
-  const int kc = chunk_k(mt);
+  const StreamConfig cfg = choose_config(M);
   g.splits = r.splits = choose_splits(M, col_blocks, K);
   g.k_per_split = K / g.splits;
   if (g.splits > 1) {
@@ -489,12 +562,16 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
       at += static_cast<size_t>(g.splits) * M * problems[i].N;
     }
   }
-  const dim3 grid(ceil_div(M, 32 * mt), col_blocks, g.splits);
-  if (mt == 1 && kc == 128) hipLaunchKernelGGL((gemm_stream_kernel<1, 128>), grid, dim3(256), 0, st, g);
-  else if (mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 256>), grid, dim3(256), 0, st, g);
-  else if (mt == 2 && kc == 128) hipLaunchKernelGGL((gemm_stream_kernel<2, 128>), grid, dim3(256), 0, st, g);
-  else if (mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 256>), grid, dim3(256), 0, st, g);
-  else hipLaunchKernelGGL((gemm_stream_kernel<4, 128>), grid, dim3(256), 0, st, g);
+  RWKV_REQUIRE(g.k_per_split % (cfg.kc * cfg.kg) == 0, "linear_packed: K slice %d is not a whole number of %d-chunks",
+               g.k_per_split, cfg.kc * cfg.kg);
+  g.row_tiles = ceil_div(M, 32 * cfg.mt);
+  g.col_blocks = col_blocks;
+  const int pairs8 = ceil_div(col_blocks * g.splits, 8) * 8;
+  const dim3 grid(g.row_tiles * pairs8);
+  const dim3 block(256 * cfg.kg);
+  if (cfg.mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 2>), grid, block, 0, st, g);
+  else if (cfg.mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 128, 2>), grid, block, 0, st, g);
+  else hipLaunchKernelGGL((gemm_stream_kernel<4, 128, 1>), grid, block, 0, st, g);
   RWKV_LAUNCH_CHECK();
   if (g.splits == 1) return RWKV_OK;
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3(r.block_end[n_problems - 1]), dim3(256), 0, st, r);
