@@ -1,0 +1,225 @@
+// Channel-mix down projection of one token that reads only the rows of ffn.value whose activation is non-zero.
+//
+// Reference: rwkv7_cmix_sparse_down_relu_one_launch and cmix_sparse_spmv_relu_one_kernel
+// (cuda/rwkv7_fast_ops_fp16.cu:966-976,618-676; call site src/rwkv7_fast_v4.cu:1285-1286):
+//   vec[f] = f16(relu(preact[f])^2);  out[c] = sum over f with vec[f] != 0 of vec[f] * Wv[f][c]
+// over ffn.value stored [F,C], so that a skipped f skips a contiguous row.  The reference accumulates in half2
+// with atomicAdd (the result depends on block order); here the products are exact, the accumulation is fp32 and
+// the order is fixed, so the result is the dense product of the same codes up to fp32 summation order.
+//
+// Weights: the int8 codes of the [C,F] matrix transposed to [F,C] and stored offset by 128 (u = q + 128, one
+// byte each), with the same per-output-channel fp16 scale.
+//
+// Kernel 1: grid = (F/256, ceil(C/1024)), block = 8 wavefronts.  A wavefront owns 32 consecutive f and 1024
+// columns (16 per lane): it ballots the non-zero activations, walks the set bits eight rows at a time (missing
+// rows of the last batch repeat a row already read, with coefficient zero, so no load sits under a branch), and
+// accumulates two rows per v_dot2_f32_f16: v_perm_b32 pairs the bytes of the two rows under exponent 0x64 and
+// one packed subtract gives the exact signed codes.  The eight wavefronts' sums meet in LDS in wavefront
+// order and the block writes one fp32 partial row.  Kernel 2 sums the F/256 partial rows in a fixed order,
+// applies the scale and rounds to fp16.
+#include "ops.h"
+
+namespace rwkv {
+
+constexpr int kSparseRowsPerWave = 32;
+constexpr int kSparseWaves = 8;
+constexpr int kSparseRowsPerBlock = kSparseRowsPerWave * kSparseWaves;  // 256
+constexpr int kSparseCols = 1024;                                        // per block: 64 lanes x 16 codes
+constexpr int kSparseBatch = 8;
+
+bool ffn_sparse_supported(int C, int F) { return C >= 16 && C % 16 == 0 && F >= kSparseRowsPerBlock && F % kSparseRowsPerBlock == 0; }
+
+size_t ffn_sparse_workspace_bytes(int C, int F) { return static_cast<size_t>(F / kSparseRowsPerBlock) * C * sizeof(float); }
+
+// ---- [C,F] int8 codes -> [F,C] offset codes ------------------------------------------------------------------------------
+// grid = (F/64, C/64) tiles through LDS; C and F multiples of 64 are not required (edges are predicated).
+__global__ __launch_bounds__(256) void ffn_sparse_pack_kernel(int C, int F, const int8_t* __restrict__ w,
+                                                              uint8_t* __restrict__ wt) {
+  __shared__ uint8_t tile[64][65];
+  const int f0 = blockIdx.x * 64;
+  const int c0 = blockIdx.y * 64;
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    const int c = i >> 6;
+    const int f = i & 63;
+    uint8_t v = 0;
+    if (c0 + c < C && f0 + f < F) v = static_cast<uint8_t>(w[static_cast<int64_t>(c0 + c) * F + f0 + f]) ^ 0x80u;
+    tile[c][f] = v;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    const int f = i >> 6;
+    const int c = i & 63;
+    if (c0 + c < C && f0 + f < F) wt[static_cast<int64_t>(f0 + f) * C + c0 + c] = tile[c][f];
+  }
+}
+
+int ffn_sparse_pack_launch(hipStream_t st, int C, int F, const void* w, void* wt) {
+  RWKV_REQUIRE(ffn_sparse_supported(C, F), "ffn_sparse_pack: unsupported shape C=%d F=%d", C, F);
+  RWKV_REQUIRE(w && wt && w != wt, "ffn_sparse_pack: bad pointers");
+  hipLaunchKernelGGL(ffn_sparse_pack_kernel, dim3(ceil_div(F, 64), ceil_div(C, 64)), dim3(256), 0, st, C, F,
+                     static_cast<const int8_t*>(w), static_cast<uint8_t*>(wt));
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+// ---- kernel 1 ------------------------------------------------------------------------------------------------------------
+// `activated` != 0: `in` already holds f16(relu(preact)^2) (the model's ffn.key launch applies it).
+__global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, int F, int activated,
+                                                                       const half_t* __restrict__ in,
+                                                                       const uint4_t* __restrict__ wt,
+                                                                       float* __restrict__ partial) {
+  __shared__ __align__(16) float red[kSparseWaves][kSparseCols];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int f0 = blockIdx.x * kSparseRowsPerBlock + wave * kSparseRowsPerWave;
+  const int c0 = blockIdx.y * kSparseCols;
+  const bool col_ok = c0 + 16 * lane < C;
+  // 16-byte pieces: row f starts at f * C/16, this lane's piece of the row is (c0/16 + lane)
+  const int row_pieces = C >> 4;
+  const uint4_t* wlane = wt + (c0 >> 4) + (col_ok ? lane : 0);
+
+  float a = 0.0f;
+  if (lane < kSparseRowsPerWave) {
+    a = h2f(in[f0 + lane]);
+    if (!activated) {
+      a = fmaxf(round_h(a), 0.0f);
+      a = round_h(a * a);
+    }
+  }
+  const half_t ah = f2h(a);
+  const uint32_t abits = __builtin_bit_cast(uint16_t, ah);
+  uint64_t mask = __ballot((abits << 17) != 0u);  // +0 and -0 both count as zero
+
+  float acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+  const half2_t bias = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
+
+  while (mask != 0) {
+    int row[kSparseBatch];
+    uint32_t coef[kSparseBatch];
+    const int first = __builtin_ctzll(mask);
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p) {
+      if (mask != 0) {
+        row[p] = __builtin_ctzll(mask);
+        mask &= mask - 1;
+        coef[p] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(abits), row[p]));
+      } else {
+        row[p] = first;
+        coef[p] = 0u;
+      }
+    }
+    uint4_t q[kSparseBatch];
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p) q[p] = wlane[static_cast<int64_t>(f0 + row[p]) * row_pieces];
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; p += 2) {
+      const half2_t ap = as_half2(coef[p] | (coef[p + 1] << 16));
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t lo = q[p][d];
+        const uint32_t hi = q[p + 1][d];
+        const half2_t w0 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c040c00u) | 0x64006400u) - bias;
+        const half2_t w1 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c050c01u) | 0x64006400u) - bias;
+        const half2_t w2 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c060c02u) | 0x64006400u) - bias;
+        const half2_t w3 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c070c03u) | 0x64006400u) - bias;
+        acc[4 * d + 0] = __builtin_amdgcn_fdot2(ap, w0, acc[4 * d + 0], false);
+        acc[4 * d + 1] = __builtin_amdgcn_fdot2(ap, w1, acc[4 * d + 1], false);
+        acc[4 * d + 2] = __builtin_amdgcn_fdot2(ap, w2, acc[4 * d + 2], false);
+        acc[4 * d + 3] = __builtin_amdgcn_fdot2(ap, w3, acc[4 * d + 3], false);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    *reinterpret_cast<float4_t*>(&red[wave][16 * lane + 4 * i]) =
+        float4_t{acc[4 * i], acc[4 * i + 1], acc[4 * i + 2], acc[4 * i + 3]};
+  __syncthreads();
+  if (threadIdx.x < kSparseCols / 4) {
+    const int c = 4 * threadIdx.x;
+    float4_t sum = *reinterpret_cast<const float4_t*>(&red[0][c]);
+#pragma unroll
+    for (int w = 1; w < kSparseWaves; ++w) sum = sum + *reinterpret_cast<const float4_t*>(&red[w][c]);
+    if (c0 + c < C) *reinterpret_cast<float4_t*>(partial + static_cast<int64_t>(blockIdx.x) * C + c0 + c) = sum;
+  }
+}
+
+// ---- kernel 2: out[c] = f16(scale[c] * sum of the partial rows); block 0 also does the optional row copy --------
+// grid = ceil(C/64), block = 256 = 16 groups of partial rows x 16 column quads.  Group g sums rows g, g+16, ... (its
+// loads are independent, so they are all in flight together), the 16 group sums meet in LDS in group order.
+__global__ __launch_bounds__(256) void ffn_sparse_finish_kernel(int C, int n_partial, const float* __restrict__ partial,
+                                                                const half_t* __restrict__ scale,
+                                                                half_t* __restrict__ out, RowCopy copy) {
+  __shared__ __align__(16) float red[16][64];
+  if (blockIdx.x == 0 && copy.n > 0) {
+    for (int i = threadIdx.x * 8; i < copy.n; i += 256 * 8)
+      *reinterpret_cast<uint4_t*>(copy.dst + i) = *reinterpret_cast<const uint4_t*>(copy.src + i);
+  }
+  const int g = threadIdx.x >> 4;
+  const int cq = (threadIdx.x & 15) * 4;
+  const int c = blockIdx.x * 64 + cq;
+  float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (c < C) {
+#pragma unroll 4
+    for (int p = g; p < n_partial; p += 16) sum = sum + *reinterpret_cast<const float4_t*>(partial + static_cast<int64_t>(p) * C + c);
+  }
+  *reinterpret_cast<float4_t*>(&red[g][cq]) = sum;
+  __syncthreads();
+  if (threadIdx.x >= 16 || c >= C) return;
+  float4_t total = *reinterpret_cast<const float4_t*>(&red[0][cq]);
+#pragma unroll
+  for (int i = 1; i < 16; ++i) total = total + *reinterpret_cast<const float4_t*>(&red[i][cq]);
+  const half4_t sv = *reinterpret_cast<const half4_t*>(scale + c);
+  half4_t o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = f2h(total[i] * h2f(sv[i]));
+  *reinterpret_cast<half4_t*>(out + c) = o;
+}
+
+int ffn_sparse_launch(hipStream_t st, int C, int F, int activated, const half_t* in, const void* wt, const half_t* scale,
+                      void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy) {
+  RWKV_REQUIRE(ffn_sparse_supported(C, F), "ffn_sparse: unsupported shape C=%d F=%d", C, F);
+  RWKV_REQUIRE(in && wt && scale && out, "ffn_sparse: NULL tensor");
+  RWKV_REQUIRE(workspace && workspace_bytes >= ffn_sparse_workspace_bytes(C, F), "ffn_sparse: workspace of %zu bytes needed, got %zu",
+               ffn_sparse_workspace_bytes(C, F), workspace_bytes);
+  RowCopy cp;
+  if (copy) {
+    RWKV_REQUIRE(copy->n % 8 == 0, "ffn_sparse: row copy length %d must be a multiple of 8", copy->n);
+    cp = *copy;
+  }
+  const int n_partial = F / kSparseRowsPerBlock;
+  hipLaunchKernelGGL(ffn_sparse_kernel, dim3(n_partial, ceil_div(C, kSparseCols)), dim3(64 * kSparseWaves), 0, st, C, F,
+                     activated, in, static_cast<const uint4_t*>(wt), static_cast<float*>(workspace));
+  RWKV_LAUNCH_CHECK();
+  hipLaunchKernelGGL(ffn_sparse_finish_kernel, dim3(ceil_div(C, 64)), dim3(256), 0, st, C, n_partial,
+                     static_cast<const float*>(workspace), scale, out, cp);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+}  // namespace rwkv
+
+using namespace rwkv;
+
+extern "C" {
+
+int rwkv_hip_cmix_sparse_pack(rwkv_stream_t s, int C, int F, const void* w, void* wt) {
+  return ffn_sparse_pack_launch(as_stream(s), C, F, w, wt);
+}
+
+int rwkv_hip_cmix_sparse_workspace(int C, int F, size_t* bytes) {
+  RWKV_REQUIRE(bytes, "cmix_sparse_workspace: NULL argument");
+  RWKV_REQUIRE(ffn_sparse_supported(C, F), "cmix_sparse_workspace: unsupported shape C=%d F=%d", C, F);
+  *bytes = ffn_sparse_workspace_bytes(C, F);
+  return RWKV_OK;
+}
+
+int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int C, int F, const void* preact, const void* wt,
+                                       const void* scale, void* workspace, size_t workspace_bytes, void* out) {
+  return ffn_sparse_launch(as_stream(s), C, F, 0, static_cast<const half_t*>(preact), wt,
+                           static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr);
+}
+
+}  // extern "C"

@@ -23,6 +23,7 @@ struct Matrix {
   const half_t* scale = nullptr;
   const uint8_t* zp = nullptr;
   void* packed = nullptr;  // owned: the same codes in the MFMA-native order, for calls with >= 16 rows
+  void* sparse_t = nullptr;  // owned, ffn.value with int8 codes only: [F,C] offset codes for the one-token row-skipping product
 };
 
 struct Layer {
@@ -42,8 +43,10 @@ struct rwkv_hip_model {
   ~rwkv_hip_model() {
     if (head.packed) (void)hipFree(head.packed);
     for (Layer& l : layers) {
-      for (Matrix& mat : l.m)
+      for (Matrix& mat : l.m) {
         if (mat.packed) (void)hipFree(mat.packed);
+        if (mat.sparse_t) (void)hipFree(mat.sparse_t);
+      }
       for (void* q : l.lora_in_packed)
         if (q) (void)hipFree(q);
     }
@@ -111,6 +114,9 @@ struct rwkv_hip_session {
   std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;
   void* gemm_ws = nullptr;  // split-K partials of the packed GEMM
   size_t gemm_ws_bytes = 0;
+  void* sparse_ws = nullptr;  // partial rows of the row-skipping ffn.value product
+  size_t sparse_ws_bytes = 0;
+  bool sparse_ffn = true;     // one-token steps read only the ffn.value rows with a non-zero activation
 };
 
 namespace {
@@ -226,6 +232,11 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
       s->gemm_ws_bytes = ws;
     }
   }
+  if (!s->sparse_ws && ffn_sparse_supported(m->C, m->F)) {
+    const size_t bytes = ffn_sparse_workspace_bytes(m->C, m->F);
+    RWKV_HIP_TRY(hipMalloc(&s->sparse_ws, bytes));
+    s->sparse_ws_bytes = bytes;
+  }
   if (static_cast<int>(rows) > s->tokens_cap) {
     RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
     if (s->tokens_dev) RWKV_HIP_TRY(hipFree(s->tokens_dev));
@@ -304,6 +315,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key).  The residual-stream tap needs the
   // stand-alone kernels.
   const bool ln_in_linear = step && small && !s->trace && static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
+
+  // One-token steps read only the ffn.value rows whose relu^2 activation is non-zero (int8 weights).
+  const bool sparse_value = step && rows == 1 && s->sparse_ffn && s->sparse_ws != nullptr;
 
   auto mix6_args = [&](const Layer& w, LnArgs& a) {
     const int ids[6] = {RWKV_T_X_R, RWKV_T_X_W, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_A, RWKV_T_X_G};
@@ -489,13 +503,22 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       TRY_PROF(linear_small_m(st, rows, C, 1, &pk, RWKV_EPI_RELU_SQUARE, 0, &ln));
       // the ffn.value launch also moves the LN2 output kept above into the channel-mix shift row of the state
       const Matrix& mv = w.m[RWKV_M_FFN_VALUE];
-      LinearProblem pv = {mv.data, mv.scale, mv.zp, b.act, b.cm, C, mv.fmt, nullptr};
       RowCopy cp;
       cp.src = b.ln2; cp.dst = shift1; cp.n = rows * C;
-      TRY_PROF(linear_small_m(st, rows, F, 1, &pv, RWKV_EPI_NONE, 0, nullptr, &cp));
+      if (sparse_value && mv.sparse_t) {
+        TRY_AUX(ffn_sparse_launch(st, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm, &cp));
+      } else {
+        LinearProblem pv = {mv.data, mv.scale, mv.zp, b.act, b.cm, C, mv.fmt, nullptr};
+        TRY_PROF(linear_small_m(st, rows, F, 1, &pv, RWKV_EPI_NONE, 0, nullptr, &cp));
+      }
     } else {
       TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
-      TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_VALUE], rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+      const Matrix& mv = w.m[RWKV_M_FFN_VALUE];
+      if (sparse_value && mv.sparse_t) {
+        TRY_AUX(ffn_sparse_launch(st, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm, nullptr));
+      } else {
+        TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+      }
     }
 
     // residual add + next layer's LN1 (+ lerps), or the final LN on the last token of each row
@@ -689,10 +712,12 @@ int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, con
     RWKV_REQUIRE(K % 128 == 0, "set_matrix: W4 needs the input width (%d) to be a multiple of 128", K);
   }
   Matrix& slot = id == RWKV_M_HEAD ? m->head : m->layers[layer].m[id];
-  if (slot.packed) {
+  if (slot.packed || slot.sparse_t) {
     RWKV_HIP_TRY(hipDeviceSynchronize());
-    RWKV_HIP_TRY(hipFree(slot.packed));
+    if (slot.packed) RWKV_HIP_TRY(hipFree(slot.packed));
+    if (slot.sparse_t) RWKV_HIP_TRY(hipFree(slot.sparse_t));
     slot.packed = nullptr;
+    slot.sparse_t = nullptr;
   }
   if (linear_packed_supported(fmt, static_cast<int>(kPackedMinRows), N, K)) {
     // second copy of the codes in the order the MFMA path streams (batched decode and prefill)
@@ -702,6 +727,17 @@ int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, con
     const int rc = pack_weights_launch(nullptr, fmt, N, K, data, mat.packed);
     if (rc != RWKV_OK) {
       (void)hipFree(mat.packed);
+      return rc;
+    }
+    RWKV_HIP_TRY(hipStreamSynchronize(nullptr));
+  }
+  if (id == RWKV_M_FFN_VALUE && fmt == RWKV_FMT_W8 && ffn_sparse_supported(N, K)) {
+    // third copy: transposed, for decode steps of one sequence
+    RWKV_HIP_TRY(hipMalloc(&mat.sparse_t, static_cast<size_t>(N) * K));
+    const int rc = ffn_sparse_pack_launch(nullptr, N, K, data, mat.sparse_t);
+    if (rc != RWKV_OK) {
+      (void)hipFree(mat.sparse_t);
+      if (mat.packed) (void)hipFree(mat.packed);
       return rc;
     }
     RWKV_HIP_TRY(hipStreamSynchronize(nullptr));
@@ -761,6 +797,7 @@ int rwkv_hip_session_destroy(rwkv_hip_session* s) {
   }
   if (s->arena.base) (void)hipFree(s->arena.base);
   if (s->gemm_ws) (void)hipFree(s->gemm_ws);
+  if (s->sparse_ws) (void)hipFree(s->sparse_ws);
   if (s->tokens_dev) (void)hipFree(s->tokens_dev);
   if (s->tokens_pinned) (void)hipHostFree(s->tokens_pinned);
   if (s->argmax_dev) (void)hipFree(s->argmax_dev);
@@ -786,6 +823,21 @@ int rwkv_hip_session_set_profile(rwkv_hip_session* s, int on) {
   RWKV_REQUIRE(s, "session is NULL");
   RWKV_REQUIRE(on >= 0 && on <= 2, "set_profile: mode must be 0, 1 or 2");
   s->profile = on;
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int on) {
+  RWKV_REQUIRE(s, "session is NULL");
+  if (s->sparse_ffn != (on != 0)) {
+    // captured decode graphs hold the other kernel
+    RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+    for (auto& g : s->graphs) {
+      if (g.exec) (void)hipGraphExecDestroy(g.exec);
+      if (g.graph) (void)hipGraphDestroy(g.graph);
+    }
+    s->graphs.clear();
+    s->sparse_ffn = on != 0;
+  }
   return RWKV_OK;
 }
 

@@ -161,6 +161,16 @@ struct LoraOutMultiArgs {
 // up to four rank-out products over the same rows in one launch
 int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a);
 
+// ---- ffn_sparse.hip: one-token ffn.value product that skips the rows with a zero activation ---------------
+bool ffn_sparse_supported(int C, int F);
+size_t ffn_sparse_workspace_bytes(int C, int F);
+// [C,F] int8 codes -> [F,C] codes offset by 128
+int ffn_sparse_pack_launch(hipStream_t st, int C, int F, const void* w, void* wt);
+// activated != 0: `in` holds f16(relu(preact)^2) already; else the kernel applies it.  `copy` (optional) rides on
+// the second launch.
+int ffn_sparse_launch(hipStream_t st, int C, int F, int activated, const half_t* in, const void* wt, const half_t* scale,
+                      void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy);
+
 // ---- sampler.hip --------------------------------------------------------------------------------
 int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out);
 

@@ -79,6 +79,47 @@ def test_small_model_prefill_and_decode(gpu, orc, fmt):
     sess.close()
 
 
+def test_one_sequence_decode_with_row_skipping_ffn_value(gpu, orc):
+    """Batch-1 decode steps of a W8 model use the row-skipping ffn.value product (eager and graph replay): the
+    steps match the oracle, stay within an fp16 ulp of the dense product's logits, and the activations really
+    are sparse (else the test would not exercise the skip)."""
+    from rwkv_lightning_cuda_amd.model import Session, State
+    hip = gpu
+    dims = small_dims()
+    omodel, gmodel = build_pair(gpu, orc, dims, orc.FMT_W8, seed=33)
+    rng = np.random.default_rng(8)
+    prompt = rng.integers(0, dims.V, (1, 6))
+    steps = rng.integers(0, dims.V, (5, 1, 1))
+    results = {}
+    for mode in ("sparse", "dense"):
+        sess = Session(gmodel)
+        sess.set_sparse_ffn(mode == "sparse")
+        st = State(dims, 1)
+        lg = hip.DeviceArray((1, dims.V), np.float32)
+        sess.forward(prompt, st, lg)
+        outs = []
+        for i in range(5):
+            sess.set_graph(i != 2)
+            sess.forward(steps[i], st, lg)
+            outs.append(lg.numpy().copy())
+        if mode == "sparse":
+            act = sess.debug_buffer("act", (1, dims.F))
+            frac = float(np.mean(act == 0))
+            assert 0.2 <= frac <= 0.8, frac
+        results[mode] = (outs, st.wkv.numpy().copy())
+        sess.close()
+    ostate = omodel.new_state(1)
+    omodel.forward(prompt, ostate)
+    for i in range(5):
+        ol = omodel.forward(steps[i], ostate)
+        err = cosine(results["sparse"][0][i], ol)
+        assert err >= 0.9995
+        err = rel_err(results["sparse"][0][i], results["dense"][0][i])
+        assert err <= 2e-3
+    err = rel_err(results["sparse"][1], ostate[1])
+    assert err <= 1e-3
+
+
 def test_chunked_prefill_resume_bitwise_and_chunk_size_invariance(gpu, orc):
     """State carried in HBM across chunks.  (a) Saving the state to the host between chunks and resuming from
     the restored copy is bitwise identical to the uninterrupted run (same chunking).  (b) A different chunking
