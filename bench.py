@@ -54,10 +54,12 @@ def parse_args():
     return ap.parse_args()
 
 
-def gemv_bytes_per_step(dims, fmt):
-    """Algorithmic bytes the weight-streaming linear launches move per decode step: every code of the seven
-    big matrices once + their scales (+ zero points), the fp16 LoRA rank-in matrices that share the r/k/v launch,
-    + x in and y out (fp16).  Returns (bytes, launches)."""
+def gemv_bytes_per_step(dims, fmt, sparse_value):
+    """Algorithmic bytes the weight-streaming GEMV launches move per decode step: every code of the big
+    matrices once + their scales (+ zero points), the fp16 LoRA rank-in matrices that share the r/k/v launch,
+    + x in and y out (fp16).  With `sparse_value` the ffn.value product is not a GEMV launch (a one-sequence
+    step reads only the rows with a non-zero activation through another kernel) and is left out.
+    Returns (bytes, launches)."""
     C, F, V, L = dims.C, dims.F, dims.V, dims.L
 
     def mat(N, K):
@@ -76,8 +78,8 @@ def gemv_bytes_per_step(dims, fmt):
     total = mat(V, C)
     for l in range(L):
         # launch 1: r/k/v + the LoRA rank-ins (one launch); 2: output; 3: ffn.key; 4: ffn.value
-        total += 3 * mat(C, C) + lora_in(l) + mat(C, C) + mat(F, C) + mat(C, F)
-    launches = 4 * L + 1
+        total += 3 * mat(C, C) + lora_in(l) + mat(C, C) + mat(F, C) + (0 if sparse_value else mat(C, F))
+    launches = (3 if sparse_value else 4) * L + 1
     return total, launches
 
 
@@ -242,6 +244,21 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     value = args.steps * B / elapsed
 
+    # one-sequence steps over int8 weights skip the ffn.value rows with a zero activation (the reference's default
+    # for rows == 1, include/rwkv7_fast_v4_common.hpp:198-211); the dense product is timed beside it below
+    sparse_value = B == 1 and args.fmt == "w8" and dims.F % 256 == 0 and dims.C % 16 == 0
+    if sparse_value and not args.no_also:
+        sess.set_sparse_ffn(False)
+        sess.decode_greedy(first, min(args.warmup, 8) or 1, state, logits)
+        hip.device_sync()
+        td = time.perf_counter()
+        sess.decode_greedy(first, min(args.steps, 64), state, logits)
+        hip.device_sync()
+        also["decode_dense_ffn_value_tok_s"] = min(args.steps, 64) * B / (time.perf_counter() - td)
+        sess.set_sparse_ffn(True)
+        act = sess.debug_buffer("act", (B, dims.F))
+        also["ffn_value_rows_skipped_fraction_last_layer"] = float(np.mean(act == 0))
+
     weight_bytes = model.weight_bytes()
     state_bytes = B * (2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2)
     out = {
@@ -261,7 +278,8 @@ def main():
                                % (args.preset, B, args.prefill),
                    "L": dims.L, "C": dims.C, "H": dims.H, "F": dims.F, "V": dims.V,
                    "weight_format": args.fmt, "arithmetic": "fp16 activations, fp32 accumulate, fp32 WKV state",
-                   "hip_graph": not args.no_graph, "weight_bytes_per_step": weight_bytes,
+                   "hip_graph": not args.no_graph, "sparse_ffn_value": sparse_value,
+                   "weight_bytes_per_step": weight_bytes,
                    "state_bytes_per_step": state_bytes,
                    "step_hbm_fraction": (weight_bytes + state_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                    "distinct_tokens": int(len(np.unique(toks)))},
@@ -282,7 +300,7 @@ def main():
         launches, total_ms = sess.read_profile()
         sess.set_profile(0)
         del scratch_state
-        gemv_bytes, per_step = gemv_bytes_per_step(dims, args.fmt)
+        gemv_bytes, per_step = gemv_bytes_per_step(dims, args.fmt, sparse_value)
         assert launches == per_step * n_prof, (launches, per_step, n_prof)
         bytes_per_launch = gemv_bytes / per_step
         avg_ms = total_ms / launches
@@ -291,7 +309,8 @@ def main():
         out["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-            "kernel": "linear_gemv_kernel (W8A16 weight-streaming GEMV; r/k/v fused, output, ffn.key, ffn.value, lm_head)",
+            "kernel": "linear_gemv_kernel (weight-streaming GEMV: r/k/v + LoRA rank-ins, output, ffn.key%s, lm_head)"
+                      % ("" if sparse_value else ", ffn.value"),
             "bytes_per_launch": bytes_per_launch, "avg_launch_us": avg_ms * 1e3, "launches_per_step": per_step,
         }
 

@@ -259,6 +259,11 @@ int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double
  * (CmixMode::NoFcOne of the reference, src/rwkv7_fast_v4.cu:1285-1286); on by default, 0 selects the dense
  * product. */
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int on);
+/* Decode steps of up to 8 rows can fold the two LayerNorm + token-shift kernels of a layer into the prologue of
+ * the linear launches that consume them (bitwise the same results).  Off by default: on this chip the extra
+ * work inside every GEMV block costs more than the two small launches it saves.  No counterpart in the
+ * reference. */
+int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on);
 /* debugging/parity tap: device address of one of the session's activation buffers, holding what the last
  * layer of the last rwkv_hip_forward call left there.  Ids in order: x, xx, xr, xw, xk, xv, xa, xg, r, k, v,
  * v_first, w12, a12, g, hw, ha, hg, hv, k2, nkk, kka, y, y2, att, x1, ln2, mixed, act, cm (f16), then

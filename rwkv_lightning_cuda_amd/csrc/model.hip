@@ -13,6 +13,8 @@
 #include <mutex>
 #include <vector>
 
+#include <cstdlib>
+
 #include "ops.h"
 
 using namespace rwkv;
@@ -117,6 +119,7 @@ struct rwkv_hip_session {
   void* sparse_ws = nullptr;  // partial rows of the row-skipping ffn.value product
   size_t sparse_ws_bytes = 0;
   bool sparse_ffn = true;     // one-token steps read only the ffn.value rows with a non-zero activation
+  bool fused_ln = false;      // decode steps fold LayerNorm + token shift into the linear launches (measured slower)
 };
 
 namespace {
@@ -314,7 +317,8 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   // Decode steps of up to 8 rows fold both LayerNorm + token-shift kernels of a layer into the prologue of the
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key).  The residual-stream tap needs the
   // stand-alone kernels.
-  const bool ln_in_linear = step && small && !s->trace && static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
+  const bool ln_in_linear = s->fused_ln && step && small && !s->trace &&
+                            static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
 
   // One-token steps read only the ffn.value rows whose relu^2 activation is non-zero (int8 weights).
   const bool sparse_value = step && rows == 1 && s->sparse_ffn && s->sparse_ws != nullptr;
@@ -826,16 +830,29 @@ int rwkv_hip_session_set_profile(rwkv_hip_session* s, int on) {
   return RWKV_OK;
 }
 
+static int drop_graphs(rwkv_hip_session* s) {
+  RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
+  for (auto& g : s->graphs) {
+    if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    if (g.graph) (void)hipGraphDestroy(g.graph);
+  }
+  s->graphs.clear();
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on) {
+  RWKV_REQUIRE(s, "session is NULL");
+  if (s->fused_ln != (on != 0)) {
+    TRY(drop_graphs(s));  // captured decode graphs hold the other kernels
+    s->fused_ln = on != 0;
+  }
+  return RWKV_OK;
+}
+
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int on) {
   RWKV_REQUIRE(s, "session is NULL");
   if (s->sparse_ffn != (on != 0)) {
-    // captured decode graphs hold the other kernel
-    RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
-    for (auto& g : s->graphs) {
-      if (g.exec) (void)hipGraphExecDestroy(g.exec);
-      if (g.graph) (void)hipGraphDestroy(g.graph);
-    }
-    s->graphs.clear();
+    TRY(drop_graphs(s));  // captured decode graphs hold the other kernel
     s->sparse_ffn = on != 0;
   }
   return RWKV_OK;

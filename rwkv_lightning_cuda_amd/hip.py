@@ -36,7 +36,7 @@ EXPORTS = [
     "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",
     "rwkv_hip_pack_weights", "rwkv_hip_linear_packed_workspace", "rwkv_hip_linear_packed", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
     "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
-    "rwkv_hip_session_set_sparse_ffn",
+    "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln",
     "rwkv_hip_layer_norm", "rwkv_hip_add_layer_norm", "rwkv_hip_add_last_layer_norm", "rwkv_hip_token_shift_mix",
     "rwkv_hip_add_layer_norm_cmix_mix", "rwkv_hip_add_layer_norm_tmix_mix6", "rwkv_hip_kk_a_gate",
     "rwkv_hip_lnx_rkvres_xg", "rwkv_hip_relu_square", "rwkv_hip_add_vec", "rwkv_hip_f16_to_f32",

@@ -265,6 +265,10 @@ class Session:
         hip.check(hip.load().rwkv_hip_memcpy_d2h(out.ctypes.data_as(ctypes.c_void_p), p, ctypes.c_size_t(out.nbytes)))
         return out
 
+    def set_fused_ln(self, on):
+        """Decode steps fold LayerNorm + token shift into the linear launches (bitwise the same; default off)."""
+        hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(1 if on else 0)))
+
     def set_sparse_ffn(self, on):
         """One-sequence decode steps read only the ffn.value rows with a non-zero activation (default on)."""
         hip.check(hip.load().rwkv_hip_session_set_sparse_ffn(self.handle, ctypes.c_int(1 if on else 0)))

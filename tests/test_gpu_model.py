@@ -327,9 +327,9 @@ def test_config3_7p2b_width_two_layers_quantised(gpu, orc, fmt_name):
 
 @pytest.mark.parametrize("B", [1, 3, 8])
 def test_decode_step_with_layernorm_folded_into_linear_is_bitwise_the_unfused_step(gpu, B):
-    """Decode steps of up to 8 rows compute LayerNorm + token shift inside the linear kernels' prologue; with the
-    residual-stream tap on, the stand-alone kernels run instead.  Same arithmetic and reduction order: logits,
-    shift rows and WKV state must be bit-identical, step after step."""
+    """Decode steps of up to 8 rows can compute LayerNorm + token shift inside the linear kernels' prologue
+    (session option, off by default) instead of the stand-alone kernels.  Same arithmetic and reduction order:
+    logits, shift rows and WKV state must be bit-identical, step after step."""
     from rwkv_lightning_cuda_amd.model import HipModel, Session, State, synth_weights
     hip = gpu
     dims = small_dims()
@@ -341,16 +341,14 @@ def test_decode_step_with_layernorm_folded_into_linear_is_bitwise_the_unfused_st
     s_fused, s_plain = State(dims, B), State(dims, B)
     l_fused = hip.DeviceArray((B, dims.V), np.float32)
     l_plain = hip.DeviceArray((B, dims.V), np.float32)
-    trace = hip.DeviceArray((dims.L, B, dims.C), np.float16)
     sess.forward(prompt, s_fused, l_fused)
     sess.forward(prompt, s_plain, l_plain)
     for step in range(4):
         tok = rng.integers(0, dims.V, (B, 1))
-        sess.set_trace(None)
+        sess.set_fused_ln(True)
         sess.forward(tok, s_fused, l_fused)
-        sess.set_trace(trace)
+        sess.set_fused_ln(False)
         sess.forward(tok, s_plain, l_plain)
-        sess.set_trace(None)
         same = np.array_equal(l_fused.numpy().view(np.uint32), l_plain.numpy().view(np.uint32))
         assert same, "logits differ at step %d" % step
         same = np.array_equal(s_fused.shift.numpy().view(np.uint16), s_plain.shift.numpy().view(np.uint16))
