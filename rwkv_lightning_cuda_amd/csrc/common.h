@@ -67,7 +67,15 @@ __device__ __forceinline__ float round_h(float f) { return static_cast<float>(st
 // element 0 for every i.
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// The reference is built with --use_fast_math (approximate division, __expf, fast tanhf); these are the
+// gfx950 counterparts: v_rcp_f32 (1 ulp) and v_exp_f32.
+__device__ __forceinline__ float rcp_f(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float sigmoid_f(float x) { return rcp_f(1.0f + __expf(-x)); }
+// tanh through e^(-2|x|): absolute error of a few 1e-8 (the library tanhf costs some 80 instructions)
+__device__ __forceinline__ float tanh_f(float x) {
+  const float t = __expf(-2.0f * fabsf(x));
+  return copysignf((1.0f - t) * rcp_f(1.0f + t), x);
+}
 
 // Sum over the 64 lanes of a wave, result in every lane.
 __device__ __forceinline__ float wave_sum(float v) {

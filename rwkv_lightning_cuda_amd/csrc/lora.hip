@@ -13,7 +13,7 @@
 // weight are exact in fp32, and the result differs from an fp32 dot only by summation order.  Without an
 // activation the hidden is fp16 already and the lo term is skipped.  One launch takes up to four problems
 // (w, a, g, v of a layer): grid = (C/128, M/32, problems), block = 4 wavefronts x 32 output channels, the
-// 32 x 128 slice of act(h) staged in LDS once per block and K chunk.
+// 32 x R slice of act(h) staged in LDS once per block.
 #include "ops.h"
 
 namespace rwkv {
@@ -21,16 +21,23 @@ namespace rwkv {
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kLoraMaxR = 512;
-constexpr int kLoraRows = 32;          // rows per block: one MFMA tile
-constexpr int kLoraCols = 128;         // output channels per block: 32 per wavefront
-constexpr int kLoraKC = 128;           // reduction chunk staged in LDS
-constexpr int kLoraLd = kLoraKC + 8;   // +8 halves: ds_read_b128 of lane (j, h) at j*272 + 16h bytes is conflict-free
+constexpr int kLoraRows = 32;   // rows per block: one MFMA tile
+constexpr int kLoraCols = 128;  // output channels per block: 32 per wavefront
+constexpr int kLoraThreads = 2 * kLoraCols;
+constexpr int kLoraStage = (kLoraRows * (kLoraMaxR / 8 + 1) + kLoraThreads - 1) / kLoraThreads;  // pieces per thread
 
-__global__ __launch_bounds__(256) void lora_out_kernel(LoraOutMultiArgs a) {
-  __shared__ __attribute__((aligned(16))) half_t hi_s[kLoraRows][kLoraLd];
-  __shared__ __attribute__((aligned(16))) half_t lo_s[kLoraRows][kLoraLd];
+// Every lane first requests its whole weight row (up to 32 pieces of 8), the block turns its 32 x R slice of the
+// hidden into hi / lo fp16 in LDS while those loads are in flight (one barrier), then each wavefront runs its MFMA
+// steps.  Rows are R + 8 halves apart:
+// for ranks that are multiples of 16 the ds_read_b128 of lane (j, h) at j * (2R + 16) + 16h bytes is
+// conflict-free (other ranks lose some LDS bandwidth), and the zeroed 8-half pad is what the last MFMA step of
+// a rank that is not a multiple of 16 reads.
+__global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs a) {
+  __shared__ __attribute__((aligned(16))) half_t hi_s[kLoraRows * (kLoraMaxR + 8)];
+  __shared__ __attribute__((aligned(16))) half_t lo_s[kLoraRows * (kLoraMaxR + 8)];
   const LoraOutProblem& p = a.p[blockIdx.z];
   const int R = p.R;
+  const int ld = R + 8;
   const int m0 = blockIdx.y * kLoraRows;
   const int mn = min(kLoraRows, a.M - m0);
   const int wave = threadIdx.x >> 6;
@@ -42,62 +49,68 @@ __global__ __launch_bounds__(256) void lora_out_kernel(LoraOutMultiArgs a) {
   const bool split = p.act != RWKV_ACT_NONE;
   const half_t* wrow = p.w2 + static_cast<int64_t>(col_ok ? c : 0) * R;
 
+  // this lane's W2 values, all requested before the activation work: k = 16*kk + 8h .. +8 of output channel c
+  half8_t w[kLoraMaxR / 16];
+#pragma unroll
+  for (int kk = 0; kk < kLoraMaxR / 16; ++kk) {
+    const int k = kk * 16 + h * 8;
+    if (k < R) {
+      w[kk] = *reinterpret_cast<const half8_t*>(wrow + k);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w[kk][e] = static_cast<half_t>(0.0f);
+    }
+  }
+
+  // activation of the 32 x R hidden slice, split into hi + lo; R/8 pieces of 8 per row + the zeroed pad.  All of
+  // a thread's pieces are requested before the first is used.
+  const int pieces = (R >> 3) + 1;
+  half8_t hv[kLoraStage];
+#pragma unroll
+  for (int i = 0; i < kLoraStage; ++i) {
+    const int idx = threadIdx.x + i * kLoraThreads;
+    const int m = idx / pieces;
+    const int ks = (idx - m * pieces) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) hv[i][e] = static_cast<half_t>(0.0f);
+    if (m < mn && ks < R) hv[i] = *reinterpret_cast<const half8_t*>(p.h + static_cast<int64_t>(m0 + m) * R + ks);
+  }
+#pragma unroll
+  for (int i = 0; i < kLoraStage; ++i) {
+    const int idx = threadIdx.x + i * kLoraThreads;
+    const int m = idx / pieces;
+    const int ks = (idx - m * pieces) * 8;
+    if (m < kLoraRows) {
+      half8_t hi, lo;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        // rows past M and the pad hold zeros: every activation here maps them to values whose weights are zero
+        // or whose rows are never stored, but the pad must be exactly zero
+        float f = h2f(hv[i][e]);
+        if (p.act == RWKV_ACT_TANH) f = tanh_f(f);
+        if (p.act == RWKV_ACT_SIGMOID) f = sigmoid_f(f);
+        if (ks >= R) f = 0.0f;
+        hi[e] = f2h(f);
+        lo[e] = f2h(f - h2f(hi[e]));
+      }
+      *reinterpret_cast<half8_t*>(&hi_s[m * ld + ks]) = hi;
+      if (split) *reinterpret_cast<half8_t*>(&lo_s[m * ld + ks]) = lo;
+    }
+  }
+  __syncthreads();
+
   float16_t acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-
-  for (int kc = 0; kc < R; kc += kLoraKC) {
-    // this lane's W2 values of the chunk: k = kc + 16*kk + 8h .. +8 of output channel c
-    half8_t wreg[kLoraKC / 16];
 #pragma unroll
-    for (int kk = 0; kk < kLoraKC / 16; ++kk) {
-      const int k = kc + kk * 16 + h * 8;
-      if (col_ok && k < R) {
-        wreg[kk] = *reinterpret_cast<const half8_t*>(wrow + k);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) wreg[kk][e] = static_cast<half_t>(0.0f);
-      }
-    }
-    // activation of the 32 x 128 hidden slice, split into hi + lo
-    if (kc > 0) __syncthreads();
-#pragma unroll
-    for (int i = 0; i < kLoraRows * kLoraKC / 8 / 256; ++i) {
-      const int idx = threadIdx.x + 256 * i;
-      const int m = idx / (kLoraKC / 8);
-      const int ks = (idx % (kLoraKC / 8)) * 8;
-      half8_t hi, lo;
-      if (m < mn && kc + ks < R) {
-        const half8_t hv = *reinterpret_cast<const half8_t*>(p.h + static_cast<int64_t>(m0 + m) * R + kc + ks);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float f = h2f(hv[e]);
-          if (p.act == RWKV_ACT_TANH) f = tanhf(f);
-          if (p.act == RWKV_ACT_SIGMOID) f = sigmoid_f(f);
-          hi[e] = f2h(f);
-          lo[e] = f2h(f - h2f(hi[e]));
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          hi[e] = static_cast<half_t>(0.0f);
-          lo[e] = static_cast<half_t>(0.0f);
-        }
-      }
-      *reinterpret_cast<half8_t*>(&hi_s[m][ks]) = hi;
-      if (split) *reinterpret_cast<half8_t*>(&lo_s[m][ks]) = lo;
-    }
-    __syncthreads();
-    const int kn = min(kLoraKC, R - kc);
-#pragma unroll
-    for (int kk = 0; kk < kLoraKC / 16; ++kk) {
-      if (kk * 16 < kn) {
-        const half8_t ah = *reinterpret_cast<const half8_t*>(&hi_s[j][kk * 16 + h * 8]);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, wreg[kk], acc, 0, 0, 0);
-        if (split) {
-          const half8_t al = *reinterpret_cast<const half8_t*>(&lo_s[j][kk * 16 + h * 8]);
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, wreg[kk], acc, 0, 0, 0);
-        }
+  for (int kk = 0; kk < kLoraMaxR / 16; ++kk) {
+    const int k = kk * 16;
+    if (k < R) {
+      const half8_t ah = *reinterpret_cast<const half8_t*>(&hi_s[j * ld + k + h * 8]);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, w[kk], acc, 0, 0, 0);
+      if (split) {
+        const half8_t al = *reinterpret_cast<const half8_t*>(&lo_s[j * ld + k + h * 8]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, w[kk], acc, 0, 0, 0);
       }
     }
   }
@@ -133,7 +146,8 @@ int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a) {
     RWKV_REQUIRE(p.h && p.w2 && p.out, "lora_out: NULL tensor");
     RWKV_REQUIRE(!p.vres || (p.v && p.v_first && p.bias), "lora_out: v-residual gate needs v, v_first and v0");
   }
-  hipLaunchKernelGGL(lora_out_kernel, dim3(ceil_div(a.C, kLoraCols), ceil_div(a.M, kLoraRows), a.n), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(lora_out_kernel, dim3(ceil_div(a.C, kLoraCols), ceil_div(a.M, kLoraRows), a.n), dim3(kLoraThreads), 0, st,
+                     a);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }

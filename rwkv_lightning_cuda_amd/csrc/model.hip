@@ -310,10 +310,10 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     RWKV_HIP_TRY(hipEventCreate(&pass_begin));
     RWKV_HIP_TRY(hipEventRecord(pass_begin, st));
   }
-  // The single-launch time-mix core re-reads a head's LoRA rows for every batch row; with many rows the
-  // row-tiled kernels of the prefill path (LoRA rows shared by 16 rows) move less data; measured crossover
-  // between 32 and 64 rows.
-  const bool fused_tmix = step && rows <= 32;
+  // The single-launch time-mix core re-reads a head's LoRA rows for every batch row; from 16 rows on the
+  // row-tiled kernels of the prefill path (LoRA rank-outs on the matrix core) are faster (measured: 4.2 -> 4.0 ms
+  // per step at 16 rows, 5.5 -> 4.6 ms at 32).
+  const bool fused_tmix = step && rows <= 8;
   // Decode steps of up to 8 rows fold both LayerNorm + token-shift kernels of a layer into the prologue of the
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key).  The residual-stream tap needs the
   // stand-alone kernels.

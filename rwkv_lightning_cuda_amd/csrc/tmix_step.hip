@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
     if (hid[gidx] == nullptr) continue;
     for (int r = tid; r < ranks[gidx]; r += kStepThreads) {
       float hv = h2f(hid[gidx][r]);
-      if (gidx == 0) hv = tanhf(hv);
+      if (gidx == 0) hv = tanh_f(hv);
       if (gidx == 2) hv = sigmoid_f(hv);
       hs[gidx][r] = hv;
     }
