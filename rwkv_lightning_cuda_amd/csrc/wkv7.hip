@@ -43,15 +43,17 @@ __global__ __launch_bounds__(256) void wkv7_prepare_kernel(int64_t n, int64_t sl
 }
 
 // ---- sequence kernel -------------------------------------------------------------------------
-// grid = B*H, block = 256 (four wavefronts per head).  Wavefront q owns state rows 16q..16q+15; its lane
-// (g, c) = (lane / 16, lane % 16) owns rows 16q + 4g .. +3 and columns 4c .. 4c+3, so the 16 lanes of one DPP
-// row hold complete state rows and the wavefronts never exchange data.  r,d,k,a,b are fp32 with `op_bs`
-// elements between batch rows; v,y are IO with `io_bs` elements between batch rows.  The block stages the
-// operands kSeqChunk tokens at a time with coalesced 16-byte loads, double-buffered (the loads of chunk c+1
-// are in flight while chunk c computes); a step costs each lane six 16-byte LDS reads (its four columns of the
-// five operands and its four v values), against 112 VALU operations.  y goes back through LDS so that the
-// global stores are coalesced.  The arithmetic of a step does not depend on the chunking, so splitting T over
-// several calls is bitwise neutral.
+// grid = B*H, block = 1024/RPL threads: 16/RPL wavefronts per head, RPL = 4 or 2 state rows per lane.  Lane
+// (g, c) = (lane / 16, lane % 16) of wavefront q owns rows 4*RPL*q + RPL*g .. +RPL-1 and columns 4c .. 4c+3, so
+// the 16 lanes of one DPP row hold complete state rows and the wavefronts never exchange data.  r,d,k,a,b are
+// fp32 with `op_bs` elements between batch rows; v,y are IO with `io_bs` elements between batch rows.  The
+// block stages the operands kSeqChunk tokens at a time with coalesced 16-byte loads, double-buffered (the
+// loads of chunk c+1 are in flight while chunk c computes); a step costs each lane six LDS reads (its four
+// columns of the five operands and its v values) against 28*RPL VALU operations.  y goes back through LDS so
+// that the global stores are coalesced.  The arithmetic of a state element does not depend on RPL or on the
+// chunking: every variant and every split of T over several calls gives bitwise the same result.  RPL = 2
+// halves the serial work per token of a wavefront and is used while the grid is small enough to leave CUs
+// idle; RPL = 4 reads each operand half as often.
 constexpr int kSeqChunk = 8;
 
 template <int CTRL>
@@ -69,12 +71,18 @@ __device__ __forceinline__ float row16_sum(float x) {
   return x;
 }
 
-template <typename IO>
-__global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
-                                                       const float* __restrict__ r, const float* __restrict__ d,
-                                                       const float* __restrict__ k, const float* __restrict__ a,
-                                                       const float* __restrict__ b, int64_t op_bs,
-                                                       const IO* __restrict__ v, IO* __restrict__ y, int64_t io_bs) {
+template <typename IO, int RPL>
+__global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
+                                                              const float* __restrict__ r, const float* __restrict__ d,
+                                                              const float* __restrict__ k, const float* __restrict__ a,
+                                                              const float* __restrict__ b, int64_t op_bs,
+                                                              const IO* __restrict__ v, IO* __restrict__ y,
+                                                              int64_t io_bs) {
+  constexpr int NT = 1024 / RPL;
+  constexpr int kOpVecs = 5 * kSeqChunk * (kHead / 4);         // float4 of operands per chunk
+  constexpr int kOpSlots = (kOpVecs + NT - 1) / NT;
+  constexpr int kVSlots = (kSeqChunk * kHead + NT - 1) / NT;
+  typedef float rows_t __attribute__((ext_vector_type(RPL)));
   __shared__ __align__(16) float ops[2][kSeqChunk][5][kHead];  // [buffer][token][a,b,d,k,r][column]
   __shared__ __align__(16) float vs[2][kSeqChunk][kHead];      // [buffer][token][row]
   __shared__ __align__(16) float ys[2][kSeqChunk][kHead];
@@ -84,49 +92,53 @@ __global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, floa
   const int h = bh - bi * H;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int i0 = 16 * (tid >> 6) + 4 * (lane >> 4);  // first of this lane's 4 rows
-  const int j0 = 4 * (lane & 15);                    // first of its 4 columns
+  const int i0 = 4 * RPL * (tid >> 6) + RPL * (lane >> 4);  // first of this lane's rows
+  const int j0 = 4 * (lane & 15);                           // first of its 4 columns
   float* sblk = state + (static_cast<int64_t>(bh) * kHead + i0) * kHead + j0;
 
-  float4_t S[4];
+  float4_t S[RPL];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) S[i] = *reinterpret_cast<const float4_t*>(sblk + i * kHead);
+  for (int i = 0; i < RPL; ++i) S[i] = *reinterpret_cast<const float4_t*>(sblk + i * kHead);
 
   const int64_t base = static_cast<int64_t>(bi) * op_bs + h * kHead;
   const int64_t iob = static_cast<int64_t>(bi) * io_bs + h * kHead;
-  // staging: 5 operands x 8 tokens x 16 float4 = 640 float4 per chunk, 256 threads x 3 slots (the third half
-  // used); slot i of thread t: operand 2i + t/128, token (t % 128) / 16, columns 4 * (t % 16)
-  const int st_half = tid >> 7;
-  const int st_tok = (tid & 127) >> 4;
-  const int st_col = (tid & 15) * 4;
-  const float* src[3] = {(st_half ? b : a) + base, (st_half ? k : d) + base, r + base};
+  // staging slot i of thread t: float4 number t + i*NT of the chunk = (operand, token, 4 columns)
+  const float* st_src[kOpSlots];
+  int st_dst[kOpSlots];  // offset inside ops[buf], -1: slot unused
+#pragma unroll
+  for (int i = 0; i < kOpSlots; ++i) {
+    const int idx = tid + i * NT;
+    const int o = idx / (kSeqChunk * 16);
+    const int tok = (idx >> 4) % kSeqChunk;
+    const int col = (idx & 15) * 4;
+    const float* src = o == 0 ? a : (o == 1 ? b : (o == 2 ? d : (o == 3 ? k : r)));
+    st_src[i] = src + base + static_cast<int64_t>(tok) * C + col;
+    st_dst[i] = idx < kOpVecs ? (tok * 5 + o) * kHead + col : -1;
+  }
 
-  float4_t stage[3];
-  float v_stage[2];
+  float4_t stage[kOpSlots];
+  float v_stage[kVSlots];
 
   auto request = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < 3; ++i) {
+    for (int i = 0; i < kOpSlots; ++i) {
+      const int tok = ((tid + i * NT) >> 4) % kSeqChunk;
       stage[i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-      const int t = t0 + st_tok;
-      if (t < T && (i < 2 || st_half == 0)) {
-        stage[i] = *reinterpret_cast<const float4_t*>(src[i] + static_cast<int64_t>(t) * C + st_col);
-      }
+      if (st_dst[i] >= 0 && t0 + tok < T) stage[i] = *reinterpret_cast<const float4_t*>(st_src[i] + static_cast<int64_t>(t0) * C);
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int t = t0 + (tid >> 6) + 4 * i;
+    for (int i = 0; i < kVSlots; ++i) {
+      const int t = t0 + ((tid + i * NT) >> 6);
       v_stage[i] = 0.0f;
       if (t < T) v_stage[i] = static_cast<float>(v[iob + static_cast<int64_t>(t) * C + lane]);
     }
   };
   auto commit = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 3; ++i) {
-      if (i < 2 || st_half == 0) *reinterpret_cast<float4_t*>(&ops[buf][st_tok][2 * i + st_half][st_col]) = stage[i];
-    }
+    for (int i = 0; i < kOpSlots; ++i)
+      if (st_dst[i] >= 0) *reinterpret_cast<float4_t*>(&ops[buf][0][0][0] + st_dst[i]) = stage[i];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) vs[buf][(tid >> 6) + 4 * i][lane] = v_stage[i];
+    for (int i = 0; i < kVSlots; ++i) vs[buf][(tid + i * NT) >> 6][lane] = v_stage[i];
   };
 
   request(0);
@@ -137,16 +149,24 @@ __global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, floa
     const bool more = t0 + kSeqChunk < T;
     if (more) request(t0 + kSeqChunk);
     const int n = min(kSeqChunk, T - t0);
-    auto load_step = [&](int tt, float4_t (&dst)[6]) {
-#pragma unroll
-      for (int o = 0; o < 5; ++o) dst[o] = *reinterpret_cast<const float4_t*>(&ops[buf][tt][o][j0]);
-      dst[5] = *reinterpret_cast<const float4_t*>(&vs[buf][tt][i0]);
+    struct StepOps {
+      float4_t av, bv, dv, kv, rv;
+      rows_t vv;
     };
-    auto step = [&](int tt, const float4_t (&q)[6]) {
-      const float4_t av = q[0], bv = q[1], dv = q[2], kv = q[3], rv = q[4], vv = q[5];
-      float sa[4], yy[4];
+    auto load_step = [&](int tt, StepOps& q) {
+      q.av = *reinterpret_cast<const float4_t*>(&ops[buf][tt][0][j0]);
+      q.bv = *reinterpret_cast<const float4_t*>(&ops[buf][tt][1][j0]);
+      q.dv = *reinterpret_cast<const float4_t*>(&ops[buf][tt][2][j0]);
+      q.kv = *reinterpret_cast<const float4_t*>(&ops[buf][tt][3][j0]);
+      q.rv = *reinterpret_cast<const float4_t*>(&ops[buf][tt][4][j0]);
+      q.vv = *reinterpret_cast<const rows_t*>(&vs[buf][tt][i0]);
+    };
+    auto step = [&](int tt, const StepOps& q) {
+      const float4_t av = q.av, bv = q.bv, dv = q.dv, kv = q.kv, rv = q.rv;
+      float sa[RPL];
+      rows_t yy;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < RPL; ++i) {
         float p = S[i].x * av.x;
         p = fmaf(S[i].y, av.y, p);
         p = fmaf(S[i].z, av.z, p);
@@ -154,10 +174,10 @@ __global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, floa
         sa[i] = p;
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sa[i] = row16_sum(sa[i]);
+      for (int i = 0; i < RPL; ++i) sa[i] = row16_sum(sa[i]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float vi = vv[i];
+      for (int i = 0; i < RPL; ++i) {
+        const float vi = q.vv[i];
         S[i].x = fmaf(S[i].x, dv.x, fmaf(sa[i], bv.x, kv.x * vi));
         S[i].y = fmaf(S[i].y, dv.y, fmaf(sa[i], bv.y, kv.y * vi));
         S[i].z = fmaf(S[i].z, dv.z, fmaf(sa[i], bv.z, kv.z * vi));
@@ -169,13 +189,13 @@ __global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, floa
         yy[i] = p;
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) yy[i] = row16_sum(yy[i]);
-      if ((lane & 15) == 0) *reinterpret_cast<float4_t*>(&ys[buf][tt][i0]) = float4_t{yy[0], yy[1], yy[2], yy[3]};
+      for (int i = 0; i < RPL; ++i) yy[i] = row16_sum(yy[i]);
+      if ((lane & 15) == 0) *reinterpret_cast<rows_t*>(&ys[buf][tt][i0]) = yy;
     };
     if (n == kSeqChunk) {
       // Full chunk, straight-line: the operands of step tt+1 are read while step tt computes;
       // __builtin_amdgcn_sched_barrier(0) keeps the scheduler from sinking the reads down to their first use.
-      float4_t q[2][6];
+      StepOps q[2];
       load_step(0, q[0]);
 #pragma unroll
       for (int tt = 0; tt < kSeqChunk; ++tt) {
@@ -188,7 +208,7 @@ __global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, floa
       // the last, partial chunk (and single-token calls): same step arithmetic, rolled loop
 #pragma unroll 1
       for (int tt = 0; tt < n; ++tt) {
-        float4_t q[6];
+        StepOps q;
         load_step(tt, q);
         step(tt, q);
       }
@@ -196,14 +216,29 @@ __global__ __launch_bounds__(256) void wkv7_seq_kernel(int T, int C, int H, floa
     if (more) commit(buf ^ 1);
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int tt = (tid >> 6) + 4 * i;
+    for (int i = 0; i < kVSlots; ++i) {
+      const int tt = (tid + i * NT) >> 6;
       if (tt < n) y[iob + static_cast<int64_t>(t0 + tt) * C + lane] = static_cast<IO>(ys[buf][tt][lane]);
     }
   }
 
 #pragma unroll
-  for (int i = 0; i < 4; ++i) *reinterpret_cast<float4_t*>(sblk + i * kHead) = S[i];
+  for (int i = 0; i < RPL; ++i) *reinterpret_cast<float4_t*>(sblk + i * kHead) = S[i];
+}
+
+// Heads in flight below which the chip has idle CUs with four wavefronts per head.
+constexpr int kSeqSmallGrid = 128;
+
+template <typename IO>
+static void launch_seq(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
+                       const float* k, const float* a, const float* b, int64_t op_bs, const IO* v, IO* y, int64_t io_bs) {
+  if (B * H <= kSeqSmallGrid && T > 1) {
+    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 2>), dim3(B * H), dim3(512), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
+                       io_bs);
+  } else {
+    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
+                       io_bs);
+  }
 }
 
 template <typename IO>
@@ -211,10 +246,9 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
                        const IO* w, const IO* k, const IO* v, const IO* a, const IO* b, IO* y) {
   const int64_t row = static_cast<int64_t>(T) * C;
   if (std::is_same<IO, float>::value && w_mode == RWKV_W_DECAY) {
-    hipLaunchKernelGGL(wkv7_seq_kernel<IO>, dim3(B * H), dim3(256), 0, st, T, C, H, state,
-                       reinterpret_cast<const float*>(r), reinterpret_cast<const float*>(w),
-                       reinterpret_cast<const float*>(k), reinterpret_cast<const float*>(a),
-                       reinterpret_cast<const float*>(b), row, v, y, row);
+    launch_seq<IO>(st, B, T, C, H, state, reinterpret_cast<const float*>(r), reinterpret_cast<const float*>(w),
+                   reinterpret_cast<const float*>(k), reinterpret_cast<const float*>(a),
+                   reinterpret_cast<const float*>(b), row, v, y, row);
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
   }
@@ -237,8 +271,7 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
     const int64_t n = slab_row * B;
     hipLaunchKernelGGL(wkv7_prepare_kernel<IO>, dim3(ceil_div(n, 256)), dim3(256), 0, st, n, slab_row, row, w_mode,
                        r + off, w + off, k + off, a + off, b + off, r32, d32, k32, a32, b32);
-    hipLaunchKernelGGL(wkv7_seq_kernel<IO>, dim3(B * H), dim3(256), 0, st, tn, C, H, state, r32, d32, k32, a32, b32,
-                       slab_row, v + off, y + off, row);
+    launch_seq<IO>(st, B, tn, C, H, state, r32, d32, k32, a32, b32, slab_row, v + off, y + off, row);
   }
   hipError_t err = hipGetLastError();
   hipError_t ferr = hipFreeAsync(ws, st);
@@ -252,8 +285,7 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
 int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                         const float* k, const float* a, const float* b, int64_t op_bs, const half_t* v, half_t* y,
                         int64_t io_bs) {
-  hipLaunchKernelGGL(wkv7_seq_kernel<half_t>, dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
-                     io_bs);
+  launch_seq<half_t>(st, B, T, C, H, state, r, d, k, a, b, op_bs, v, y, io_bs);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
