@@ -62,6 +62,15 @@ __device__ __forceinline__ half_t f2h(float f) { return static_cast<half_t>(f); 
 // value after a round trip through fp16: the rounding point where the reference stores fp16
 __device__ __forceinline__ float round_h(float f) { return static_cast<float>(static_cast<half_t>(f)); }
 
+// a * b rounded to fp32 as a step of its own.  Without the barrier the compiler may fuse a product and the
+// fp16 conversion that follows it into one mixed-precision instruction with a single rounding, and whether it
+// does depends on the surrounding code: kernels that must agree bitwise on f16(a * b) go through this.
+__device__ __forceinline__ float mul_f32(float a, float b) {
+  float p = a * b;
+  asm volatile("" : "+v"(p));
+  return p;
+}
+
 // Reinterpret a dword as two fp16 values.  Always go through this by-value helper: applying
 // __builtin_bit_cast directly to a vector element (`bit_cast<half2>(vec[i])`) makes this compiler read
 // element 0 for every i.

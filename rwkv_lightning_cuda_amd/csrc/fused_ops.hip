@@ -44,7 +44,33 @@ __global__ __launch_bounds__(kLnThreads) void ln_fused_kernel(LnArgs a) {
     if (c < C) {
       const half8_t xv = *reinterpret_cast<const half8_t*>(a.x + xsrc + c);
       half8_t rv = {};
-      if constexpr (MODE != kLn && MODE != kLnMix) rv = *reinterpret_cast<const half8_t*>(a.res + src + c);
+      if constexpr (MODE != kLn && MODE != kLnMix) {
+        if (a.res_partial) {
+          const float* pp = a.res_partial + src + c;
+          float4_t s0 = *reinterpret_cast<const float4_t*>(pp);
+          float4_t s1 = *reinterpret_cast<const float4_t*>(pp + 4);
+#pragma unroll 4
+          for (int sp = 1; sp < a.res_splits; ++sp) {
+            s0 = s0 + *reinterpret_cast<const float4_t*>(pp + sp * a.res_plane);
+            s1 = s1 + *reinterpret_cast<const float4_t*>(pp + sp * a.res_plane + 4);
+          }
+          float scl[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) scl[e] = 1.0f;
+          if (a.res_scale) {
+            const half8_t sv8 = *reinterpret_cast<const half8_t*>(a.res_scale + c);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) scl[e] = h2f(sv8[e]);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            rv[e] = f2h(mul_f32(s0[e], scl[e]));
+            rv[4 + e] = f2h(mul_f32(s1[e], scl[4 + e]));
+          }
+        } else {
+          rv = *reinterpret_cast<const half8_t*>(a.res + src + c);
+        }
+      }
       wv[i] = *reinterpret_cast<const half8_t*>(a.w + c);
       bv[i] = *reinterpret_cast<const half8_t*>(a.b + c);
       if constexpr (kMix) {
@@ -147,9 +173,8 @@ int ln_launch(hipStream_t st, int mode, int rows, const LnArgs& a) {
 }
 
 // ---- token shift: out_s = x + (prev - x) * mu_s with prev = shift[b] at t == 0, else x[b,t-1];
-// then shift[b] = x[b,T-1].  One thread per (row, 8 channels).  For T == 1 the same thread reads and
-// then overwrites its shift slice; for T > 1 the shift rows are rewritten by a second launch so no
-// thread can overwrite a slice another one still has to read. ----------------------------------
+// then shift[b] = x[b,T-1].  One thread per (row, 8 channels); the thread of token 0 reads the old shift slice
+// and then overwrites it, so no thread can overwrite a slice another one still has to read. ------------
 
 __global__ __launch_bounds__(256) void token_shift_mix_kernel(MixArgs a) {
   const int cvecs = a.C / 8;
@@ -173,18 +198,11 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(MixArgs a) {
     }
     *reinterpret_cast<half8_t*>(a.out[s] + o) = ov;
   }
-  if (a.T == 1) *reinterpret_cast<half8_t*>(a.shift + static_cast<int64_t>(b) * a.C + c) = cur;
-}
-
-__global__ __launch_bounds__(256) void shift_update_kernel(int B, int T, int C, const half_t* __restrict__ x,
-                                                           half_t* __restrict__ shift) {
-  const int cvecs = C / 8;
-  const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= B * cvecs) return;
-  const int b = idx / cvecs;
-  const int c = (idx - b * cvecs) * 8;
-  *reinterpret_cast<half8_t*>(shift + static_cast<int64_t>(b) * C + c) =
-      *reinterpret_cast<const half8_t*>(x + (static_cast<int64_t>(b) * T + (T - 1)) * C + c);
+  // the thread that read the old shift slice replaces it with the last token's slice: no other thread touches it
+  if (t == 0) {
+    const half8_t last = (a.T == 1) ? cur : *reinterpret_cast<const half8_t*>(a.x + o + static_cast<int64_t>(a.T - 1) * a.C);
+    *reinterpret_cast<half8_t*>(a.shift + static_cast<int64_t>(b) * a.C + c) = last;
+  }
 }
 
 int token_shift_mix_launch(hipStream_t st, const MixArgs& a) {
@@ -192,10 +210,6 @@ int token_shift_mix_launch(hipStream_t st, const MixArgs& a) {
   RWKV_REQUIRE(a.n_mix >= 1 && a.n_mix <= 6, "token shift: n_mix %d out of range", a.n_mix);
   const int64_t n = static_cast<int64_t>(a.B) * a.T * (a.C / 8);
   hipLaunchKernelGGL(token_shift_mix_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, st, a);
-  if (a.T > 1) {
-    hipLaunchKernelGGL(shift_update_kernel, dim3(ceil_div(a.B * (a.C / 8), 256)), dim3(256), 0, st, a.B, a.T, a.C,
-                       a.x, a.shift);
-  }
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }

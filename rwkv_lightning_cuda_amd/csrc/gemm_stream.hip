@@ -390,7 +390,7 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
       if (part_out) {
         part_out[o] = sum;
       } else {
-        const float val = finish_value(sum * scl, g.epilogue);
+        const float val = finish_value(mul_f32(sum, scl), g.epilogue);
         if (g.out_f32) {
           static_cast<float*>(pr.y)[o] = val;
         } else {
@@ -462,7 +462,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs g) {
   }
   float4_t val;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) val[c] = finish_value(sum[c] * scl[c], g.epilogue);
+  for (int c = 0; c < 4; ++c) val[c] = finish_value(mul_f32(sum[c], scl[c]), g.epilogue);
   if (g.out_f32) {
     static_cast<float4_t*>(pr.y)[i] = val;
   } else {
@@ -520,7 +520,7 @@ size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const i
 size_t linear_packed_workspace_bytes(int M, int N, int K) { return linear_packed_multi_workspace_bytes(M, K, 1, &N); }
 
 int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const PackedProblem* problems, int epilogue,
-                        int out_f32, void* workspace, size_t workspace_bytes) {
+                        int out_f32, void* workspace, size_t workspace_bytes, DeferredReduce* defer) {
   RWKV_REQUIRE(n_problems >= 1 && n_problems <= kMaxProblems, "linear_packed: %d problems (1..%d allowed)", n_problems,
                kMaxProblems);
   StreamArgs g;
@@ -573,16 +573,27 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
   else if (cfg.mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 128, 2>), grid, block, 0, st, g);
   else hipLaunchKernelGGL((gemm_stream_kernel<4, 128, 1>), grid, block, 0, st, g);
   RWKV_LAUNCH_CHECK();
+  if (defer) *defer = DeferredReduce{};
   if (g.splits == 1) return RWKV_OK;
+  if (defer) {
+    RWKV_REQUIRE(n_problems == 1 && epilogue == RWKV_EPI_NONE && !out_f32,
+                 "linear_packed: a deferred reduce takes one problem, fp16 output and no epilogue");
+    defer->partial = g.p[0].partial;
+    defer->scale = problems[0].fmt == RWKV_FMT_W8 ? problems[0].scale : nullptr;
+    defer->plane = static_cast<int64_t>(M) * problems[0].N;
+    defer->splits = g.splits;
+    return RWKV_OK;
+  }
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3(r.block_end[n_problems - 1]), dim3(256), 0, st, r);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
 int linear_packed(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* packed, const half_t* scale,
-                  const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes) {
+                  const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes,
+                  DeferredReduce* defer) {
   const PackedProblem q = {packed, scale, zp, x, y, N, fmt};
-  return linear_packed_multi(st, M, K, 1, &q, epilogue, out_f32, workspace, workspace_bytes);
+  return linear_packed_multi(st, M, K, 1, &q, epilogue, out_f32, workspace, workspace_bytes, defer);
 }
 
 }  // namespace rwkv

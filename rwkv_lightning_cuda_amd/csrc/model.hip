@@ -254,13 +254,23 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
   return RWKV_OK;
 }
 
+// With `defer` the split-K partials of a packed call stay in the session workspace for the LayerNorm kernel that
+// consumes the result (defer->partial != NULL afterwards); the workspace is rewritten by the next packed call.
 int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int K, const half_t* x, int epilogue,
-                 int out_f32, void* y) {
+                 int out_f32, void* y, DeferredReduce* defer = nullptr) {
+  if (defer) *defer = DeferredReduce{};
   if (M >= kPackedMinRows && mat.packed) {
     return linear_packed(s->stream, mat.fmt, M, N, K, x, mat.packed, mat.scale, mat.zp, epilogue, out_f32, y, s->gemm_ws,
-                         s->gemm_ws_bytes);
+                         s->gemm_ws_bytes, defer);
   }
   return linear_any_m(s->stream, mat.fmt, M, N, K, x, mat.data, mat.scale, mat.zp, epilogue, out_f32, y);
+}
+
+void take_deferred(LnArgs& a, const DeferredReduce& d) {
+  a.res_partial = d.partial;
+  a.res_scale = d.scale;
+  a.res_plane = d.plane;
+  a.res_splits = d.splits;
 }
 
 #define TRY(expr)                  \
@@ -476,7 +486,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       TRY_AUX(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
                      w.t[RWKV_T_LNX_B], b.g, b.y2));
     }
-    TRY_PROF(apply_matrix(s, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att));
+    // From 16 rows on (the streaming GEMM) the LayerNorm kernels that consume the output projection and
+    // ffn.value sum the split-K partials themselves instead of a reduce launch; att / cm then stay unwritten.
+    const bool defer_ok = !s->trace && !ln_in_linear;
+    DeferredReduce att_partial;
+    TRY_PROF(apply_matrix(s, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att, defer_ok ? &att_partial : nullptr));
 
     // residual add + LN2 + channel-mix token shift
     if (ln_in_linear) {
@@ -485,11 +499,13 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       LnArgs a = {};
       a.x = b.x; a.res = b.att; a.w = w.t[RWKV_T_LN2_W]; a.b = w.t[RWKV_T_LN2_B]; a.x_out = b.x1; a.shift = shift1;
       a.mu[0] = w.t[RWKV_T_FFN_X_K]; a.out[0] = b.mixed; a.n_mix = 1; a.C = C; a.T = 1; a.eps = kLnEps;
+      take_deferred(a, att_partial);
       TRY_AUX(ln_launch(st, kAddLnMix, rows, a));
     } else {
       LnArgs a = {};
       a.x = b.x; a.res = b.att; a.w = w.t[RWKV_T_LN2_W]; a.b = w.t[RWKV_T_LN2_B]; a.x_out = b.x1; a.y = b.ln2;
       a.C = C; a.T = 1; a.eps = kLnEps;
+      take_deferred(a, att_partial);
       TRY_AUX(ln_launch(st, kAddLn, rows, a));
       MixArgs mx = {};
       mx.x = b.ln2; mx.shift = shift1; mx.B = B; mx.T = T; mx.C = C; mx.n_mix = 1;
@@ -498,6 +514,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     }
 
     // channel mix
+    DeferredReduce cm_partial;
     if (ln_in_linear) {
       const Matrix& mk = w.m[RWKV_M_FFN_KEY];
       LinearProblem pk = {mk.data, mk.scale, mk.zp, nullptr, b.act, F, mk.fmt, w.t[RWKV_T_FFN_X_K]};
@@ -521,7 +538,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       if (sparse_value && mv.sparse_t) {
         TRY_AUX(ffn_sparse_launch(st, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm, nullptr));
       } else {
-        TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm));
+        TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm, defer_ok ? &cm_partial : nullptr));
       }
     }
 
@@ -533,6 +550,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       LnArgs a = {};
       a.x = b.x1; a.res = b.cm; a.w = nx.t[RWKV_T_LN1_W]; a.b = nx.t[RWKV_T_LN1_B]; a.x_out = b.x;
       a.C = C; a.T = 1; a.eps = kLnEps;
+      take_deferred(a, cm_partial);
       if (step) {
         a.shift = shift + static_cast<int64_t>(l + 1) * 2 * B * C;
         mix6_args(nx, a);
@@ -544,6 +562,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     } else {
       LnArgs a = {};
       a.x = b.x1; a.res = b.cm; a.w = m->ln_out_w; a.b = m->ln_out_b; a.y = b.xf; a.C = C; a.T = T; a.eps = kLnEps;
+      take_deferred(a, cm_partial);
       TRY_AUX(ln_launch(st, kAddLastLn, B, a));
       if (s->trace) {
         LnArgs t = {};

@@ -59,11 +59,21 @@ bool linear_mfma_supported(int fmt, int M, int N, int K);
 
 // ---- gemm_stream.hip: weights in the MFMA-native packed order ------------------------------------------------
 bool linear_packed_supported(int fmt, int M, int N, int K);
+// A packed linear call whose split-K partials are left for the consumer to sum (see LnArgs::res_partial).
+// partial == NULL after the call: the shape needed no split and y holds the result.
+struct DeferredReduce {
+  const float* partial = nullptr;
+  const half_t* scale = nullptr;
+  int64_t plane = 0;
+  int splits = 0;
+};
 int pack_weights_launch(hipStream_t st, int fmt, int N, int K, const void* w, void* packed);
 // Workspace for one call: fp32 split-K partials (0 when the shape needs no split).
 size_t linear_packed_workspace_bytes(int M, int N, int K);
+// defer (single problem, fp16 output, no epilogue): the consumer sums the partials instead of a reduce launch.
 int linear_packed(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* packed, const half_t* scale,
-                  const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes);
+                  const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes,
+                  DeferredReduce* defer = nullptr);
 // Up to kMaxProblems products sharing M and K (own weights, format, x, y each) in one launch (+ one reduce launch).
 struct PackedProblem {
   const void* packed;
@@ -76,7 +86,7 @@ struct PackedProblem {
 };
 size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const int* Ns);
 int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const PackedProblem* problems, int epilogue,
-                        int out_f32, void* workspace, size_t workspace_bytes);
+                        int out_f32, void* workspace, size_t workspace_bytes, DeferredReduce* defer = nullptr);
 
 // ---- fused_ops.hip ------------------------------------------------------------------------------
 enum LnMode {
@@ -102,6 +112,13 @@ struct LnArgs {
   int T;
   int n_mix;
   float eps;
+  // If res_partial is not NULL the residual is still the split-K partial tiles of a packed linear call:
+  // res = f16(scale[c] * sum over splits of partial[s][row][c]), summed in split order (what the reduce
+  // kernel of that call would have stored); `res` is then unused.
+  const float* res_partial;
+  const half_t* res_scale;  // NULL: no scale
+  int64_t res_plane;        // elements between splits
+  int res_splits;
 };
 
 int ln_launch(hipStream_t st, int mode, int rows, const LnArgs& a);

@@ -120,6 +120,40 @@ def test_one_sequence_decode_with_row_skipping_ffn_value(gpu, orc):
     assert err <= 1e-3
 
 
+@pytest.mark.parametrize("fmt", [1, 2])
+@pytest.mark.parametrize("B,T", [(2, 16), (40, 1)])
+def test_split_k_partials_summed_by_the_layernorm_kernels_bitwise(gpu, fmt, B, T):
+    """From 16 rows on, the LayerNorm kernels after the output projection and after ffn.value sum the fp32
+    split-K partials of the streaming GEMM themselves; with the residual-stream tap on, the reduce kernel runs
+    instead.  Same sums in the same order: logits, shift rows and WKV state are bit-identical (prefill chunk and
+    batched decode step)."""
+    from rwkv_lightning_cuda_amd.model import HipModel, ModelDims, Session, State, synth_weights
+    hip = gpu
+    dims = ModelDims(L=2, C=512, H=8, F=2048, V=1024, Rw=32, Ra=32, Rg=64, Rv=32)
+    gmodel = HipModel.from_host_weights(dims, synth_weights(dims, 4), fmt)
+    rng = np.random.default_rng(B + T)
+    tokens = rng.integers(0, dims.V, (B, T))
+    sess = Session(gmodel)
+    sess.set_graph(False)
+    outs = []
+    for tapped in (False, True):
+        st = State(dims, B)
+        lg = hip.DeviceArray((B, dims.V), np.float32)
+        trace = hip.DeviceArray((dims.L, B * T, dims.C), np.float16)
+        sess.set_trace(trace if tapped else None)
+        sess.forward(tokens, st, lg)
+        sess.set_trace(None)
+        outs.append((lg.numpy().copy(), st.shift.numpy().copy(), st.wkv.numpy().copy()))
+    same = np.array_equal(outs[0][0].view(np.uint32), outs[1][0].view(np.uint32))
+    assert same
+    same = np.array_equal(outs[0][1].view(np.uint16), outs[1][1].view(np.uint16))
+    assert same
+    same = np.array_equal(outs[0][2].view(np.uint32), outs[1][2].view(np.uint32))
+    assert same
+    assert np.isfinite(outs[0][0]).all() and np.abs(outs[0][0]).max() > 0
+    sess.close()
+
+
 def test_chunked_prefill_resume_bitwise_and_chunk_size_invariance(gpu, orc):
     """State carried in HBM across chunks.  (a) Saving the state to the host between chunks and resuming from
     the restored copy is bitwise identical to the uninterrupted run (same chunking).  (b) A different chunking
