@@ -12,7 +12,8 @@ whole-job tokens/s plus
                   launch / average launch duration from HIP events on the session stream
   cpu_baseline -- the scalar C++ oracle timed on the host cores on a bounded slice of the same workload
   also         -- the other figures the metric names, measured in the same run: prefill tokens/s of the
-                  4096-token prompt (and the MFMA fraction of its GEMM launches), batch-64 decode tokens/s,
+                  4096-token prompt (and the MFMA fraction of its GEMM launches), batch-16 and batch-64 decode tokens/s,
+                  batch-1 decode with int4 weights,
                   and the WKV7 op alone on a long sequence.
 """
 import argparse
@@ -31,7 +32,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak, published
 # HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled
 # by what the same counter reads for a 1 GiB device-to-device copy (FETCH_SIZE reads half the bytes copied,
 # WRITE_SIZE all of them); the summary of those runs is kept under profiles/.  Keyed by (preset, format, batch).
-MEASURED_TRAFFIC = {("7.2B", "w8", 1): 2.0 * 26445.1 * 1024 + 1.0 * 38.5 * 1024}
+MEASURED_TRAFFIC = {("7.2B", "w8", 1): 2.0 * 24294.0 * 1024 + 1.0 * 46.0 * 1024}
 
 
 def parse_args():
@@ -44,7 +45,7 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--prefill", type=int, default=4096, help="tokens prefilled (chunk 128) before the decode loop")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary measurements (prefill MFMA fraction, "
-                    "batch-64 decode, WKV7 op)")
+                    "batch-16/64 decode, W4 decode, WKV7 op)")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps eagerly instead of replaying a HIP graph")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run a device-to-device copy of BYTES (twice) and exit: the known-size kernel that "
@@ -124,25 +125,25 @@ def secondary_measurements(hip, model, dims, rng):
     """Batch-64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7 op alone."""
     from rwkv_lightning_cuda_amd.model import Session, State
     res = {}
-    B = 64
-    sess = Session(model)
-    state = State(dims, B)
-    logits = hip.DeviceArray((B, dims.V), np.float32)
-    sess.forward(rng.integers(0, dims.V, (B, 128)), state, logits)
-    first = rng.integers(0, dims.V, (B,))
-    sess.decode_greedy(first, 8, state, logits)
-    hip.device_sync()
-    t0 = time.perf_counter()
-    steps = 64
-    sess.decode_greedy(first, steps, state, logits)
-    hip.device_sync()
-    dt = time.perf_counter() - t0
-    state_bytes = B * (2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2)
-    res["decode_bs64_tok_s"] = steps * B / dt
-    res["decode_bs64_ms_per_step"] = dt * 1e3 / steps
-    res["decode_bs64_hbm_fraction"] = (model.weight_bytes() + state_bytes) / (dt / steps) / 1e9 / HBM_PEAK_GBPS
-    sess.close()
-    del state, logits
+    for B in (16, 64):
+        sess = Session(model)
+        state = State(dims, B)
+        logits = hip.DeviceArray((B, dims.V), np.float32)
+        sess.forward(rng.integers(0, dims.V, (B, 128)), state, logits)
+        first = rng.integers(0, dims.V, (B,))
+        sess.decode_greedy(first, 8, state, logits)
+        hip.device_sync()
+        t0 = time.perf_counter()
+        steps = 64
+        sess.decode_greedy(first, steps, state, logits)
+        hip.device_sync()
+        dt = time.perf_counter() - t0
+        state_bytes = B * (2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2)
+        res["decode_bs%d_tok_s" % B] = steps * B / dt
+        res["decode_bs%d_ms_per_step" % B] = dt * 1e3 / steps
+        res["decode_bs%d_hbm_fraction" % B] = (model.weight_bytes() + state_bytes) / (dt / steps) / 1e9 / HBM_PEAK_GBPS
+        sess.close()
+        del state, logits
 
     # WKV7 op alone: fp16 r,w,k,v,a,b [B,T,C], fp32 state, raw-logit decay, one call
     Bw, Tw, H = 16, 2048, dims.H
@@ -316,9 +317,29 @@ def main():
 
     if not args.no_also:
         also.update(secondary_measurements(hip, model, dims, rng))
+    sess.close()
+    if not args.no_also and args.fmt == "w8":
+        # the same shape with int4 weights (asymmetric, groups of 128), batch 1
+        del model
+        m4 = HipModel.random_on_device(dims, hip.FMT_W4, seed=1)
+        s4 = Session(m4)
+        st4 = State(dims, 1)
+        lg4 = hip.DeviceArray((1, dims.V), np.float32)
+        s4.forward(rng.integers(0, dims.V, (1, 128)), st4, lg4)
+        f4 = rng.integers(0, dims.V, (1,))
+        s4.decode_greedy(f4, 8, st4, lg4)
+        hip.device_sync()
+        t4 = time.perf_counter()
+        s4.decode_greedy(f4, 64, st4, lg4)
+        hip.device_sync()
+        t4 = time.perf_counter() - t4
+        also["decode_w4_bs1_tok_s"] = 64 / t4
+        sb4 = 2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2
+        also["decode_w4_bs1_hbm_fraction"] = (m4.weight_bytes() + sb4) / (t4 / 64) / 1e9 / HBM_PEAK_GBPS
+        s4.close()
+        del m4
     if also:
         out["also"] = also
-    sess.close()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(dims, args.fmt)
     print(json.dumps(out))

@@ -156,23 +156,33 @@ struct WeightVec<RWKV_FMT_F16> {
 template <>
 struct WeightVec<RWKV_FMT_W4> {
   static constexpr int kElems = 32;
-  // returns sum_k code_k * x_k (codes 0..15, exact in fp16); the zero point is folded by the caller
-  __device__ static __forceinline__ float dot(const uint4_t& wv, const half2_t* x, float acc) {
+  // sum_k (code_k - zp) * x_k over the lane's 32 codes (all in one 128-group), exact products.  A dword holds
+  // elements 0..7 as nibbles n0..n7; (d >> 4j) & 0x000f000f picks (n_j, n_{j+4}), OR 0x6400 makes them the fp16
+  // numbers 1024 + code, one packed subtract of 1024 + zp leaves code - zp.  xp[4i + j] must hold
+  // (x_{8i+j}, x_{8i+j+4}).
+  __device__ static __forceinline__ float dot(const uint4_t& wv, const half2_t* xp, half2_t zb, float acc) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t d = wv[i];
-      const uint32_t even = d & 0x0f0f0f0fu;        // elements 0,2,4,6 of this dword
-      const uint32_t odd = (d >> 4) & 0x0f0f0f0fu;  // elements 1,3,5,7
-      const half2_t bias = {static_cast<half_t>(1024.0f), static_cast<half_t>(1024.0f)};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        // half2 (element 2j, element 2j+1) = bytes j of `even` and `odd`, each OR 0x6400
-        const uint32_t sel = 0x0c040c00u + j * 0x00010001u;
-        const uint32_t pk = __builtin_amdgcn_perm(odd, even, sel) | 0x64006400u;
-        acc = dot2(as_half2(pk) - bias, x[4 * i + j], acc);
+        const uint32_t pk = ((d >> (4 * j)) & 0x000f000fu) | 0x64006400u;
+        acc = dot2(as_half2(pk) - zb, xp[4 * i + j], acc);
       }
     }
     return acc;
+  }
+  // (x0,x1)(x2,x3)(x4,x5)(x6,x7) per 8 elements -> (x0,x4)(x1,x5)(x2,x6)(x3,x7)
+  __device__ static __forceinline__ void pair_x(const half2_t* xv, half2_t* xp) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = __builtin_bit_cast(uint32_t, xv[4 * i + j / 2]);
+        const uint32_t hi = __builtin_bit_cast(uint32_t, xv[4 * i + 2 + j / 2]);
+        xp[4 * i + j] = as_half2(__builtin_amdgcn_perm(hi, lo, (j & 1) ? 0x07060302u : 0x05040100u));
+      }
+    }
   }
 };
 
@@ -191,22 +201,35 @@ template <int FMT, int M, int R, int U>
 struct WaveGemv {
   using T = FmtTraits<FMT>;
 
-  __device__ static __forceinline__ void load_batch(uint4_t (&w)[U][R], const unsigned char* wbase, int64_t row_bytes,
-                                                    int k_lo, int kn, int step0, int lane) {
+  // One batch of weight vectors in flight; for int4 codes also the (row, 128-group) scale and zero point of each
+  // vector (the lane's 32 codes all lie in one group), requested together with it.
+  struct Batch {
+    uint4_t w[U][R];
+    half_t sc[U][R];
+    uint8_t zp[U][R];
+  };
+
+  __device__ static __forceinline__ void load_batch(Batch& bt, const unsigned char* wbase, int64_t row_bytes, int k_lo, int kn,
+                                                    int step0, int lane, const LinearProblem& prob, int row0, int K) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k0 = (step0 + u) * T::kStep + lane * T::kElems;
       if (k0 < kn) {
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-          w[u][r] = *reinterpret_cast<const uint4_t*>(wbase + r * row_bytes + T::byte_off(k_lo + k0));
+        for (int r = 0; r < R; ++r) {
+          bt.w[u][r] = *reinterpret_cast<const uint4_t*>(wbase + r * row_bytes + T::byte_off(k_lo + k0));
+          if constexpr (FMT == RWKV_FMT_W4) {
+            const int64_t gi = static_cast<int64_t>(row0 + r) * (K >> 7) + ((k_lo + k0) >> 7);
+            bt.sc[u][r] = prob.scale[gi];
+            bt.zp[u][r] = prob.zp[gi];
+          }
+        }
       }
     }
   }
 
-  __device__ static __forceinline__ void compute_batch(float (&acc)[R][M], const uint4_t (&w)[U][R], const half_t* xs,
-                                                       int KT, int k_lo, int kn, int step0, int lane,
-                                                       const LinearProblem& prob, int row0, int K) {
+  __device__ static __forceinline__ void compute_batch(float (&acc)[R][M], const Batch& bt, const half_t* xs, int KT,
+                                                       int kn, int step0, int lane) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k0 = (step0 + u) * T::kStep + lane * T::kElems;
@@ -222,24 +245,18 @@ struct WaveGemv {
             for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
           }
           if constexpr (FMT == RWKV_FMT_W4) {
-            // 32 codes per lane all lie in one 128-group: scale and zero point are per (row, group)
-            const int g = (k_lo + k0) >> 7;
-            const int G = K >> 7;
-            float xsum = 0.0f;
-            const half2_t ones = {static_cast<half_t>(1.0f), static_cast<half_t>(1.0f)};
-#pragma unroll
-            for (int e = 0; e < XV; ++e) xsum = dot2(xv[e], ones, xsum);
+            half2_t xp[XV];
+            WeightVec<FMT>::pair_x(xv, xp);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-              const int64_t gi = static_cast<int64_t>(row0 + r) * G + g;
-              const float sc = h2f(prob.scale[gi]);
-              const float z = static_cast<float>(prob.zp[gi]);
-              const float part = WeightVec<FMT>::dot(w[u][r], xv, 0.0f) - z * xsum;
-              acc[r][m] = fmaf(part, sc, acc[r][m]);
+              const half_t zf = static_cast<half_t>(1024.0f + static_cast<float>(bt.zp[u][r]));
+              const half2_t zb = {zf, zf};
+              const float part = WeightVec<FMT>::dot(bt.w[u][r], xp, zb, 0.0f);
+              acc[r][m] = fmaf(part, h2f(bt.sc[u][r]), acc[r][m]);
             }
           } else {
 #pragma unroll
-            for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(w[u][r], xv, acc[r][m]);
+            for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(bt.w[u][r], xv, acc[r][m]);
           }
         }
       }
@@ -269,12 +286,12 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
 
-  uint4_t wa[U][R], wb[U][R];
+  typename W::Batch wa, wb;
   for (int kt = 0; kt < K; kt += KT) {
     const int kn = min(KT, K - kt);
     const int nsteps = (kn + T::kStep - 1) / T::kStep;
     // request the first batch of weights, then stage x: the two latencies overlap
-    if (active) W::load_batch(wa, wbase, row_bytes, kt, kn, 0, lane);
+    if (active) W::load_batch(wa, wbase, row_bytes, kt, kn, 0, lane, prob, row0, K);
     if (kt > 0) __syncthreads();
     if constexpr (LN) {
       // the launcher guarantees KT >= K here: the whole row is normalised at once
@@ -292,11 +309,11 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
     if (active) {
       // ping-pong over batches of U steps
       for (int s0 = 0; s0 < nsteps; s0 += 2 * U) {
-        if (s0 + U < nsteps) W::load_batch(wb, wbase, row_bytes, kt, kn, s0 + U, lane);
-        W::compute_batch(acc, wa, xs, KT, kt, kn, s0, lane, prob, row0, K);
+        if (s0 + U < nsteps) W::load_batch(wb, wbase, row_bytes, kt, kn, s0 + U, lane, prob, row0, K);
+        W::compute_batch(acc, wa, xs, KT, kn, s0, lane);
         if (s0 + U < nsteps) {
-          if (s0 + 2 * U < nsteps) W::load_batch(wa, wbase, row_bytes, kt, kn, s0 + 2 * U, lane);
-          W::compute_batch(acc, wb, xs, KT, kt, kn, s0 + U, lane, prob, row0, K);
+          if (s0 + 2 * U < nsteps) W::load_batch(wa, wbase, row_bytes, kt, kn, s0 + 2 * U, lane, prob, row0, K);
+          W::compute_batch(acc, wb, xs, KT, kn, s0 + U, lane);
         }
       }
     }
