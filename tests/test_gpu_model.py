@@ -298,6 +298,56 @@ def test_config1_0p1b_prefill_512_then_128_greedy_steps(gpu, orc):
     sess.close()
 
 
+@pytest.mark.parametrize("B", [1, 8, 64])
+def test_config2_1p5b_width_w8_decode_batches(gpu, orc, B):
+    """BASELINE config 2 at full width (C 2048, H 32, F 8192, LoRA ranks 96/96/256/64; two layers, reduced
+    vocabulary), W8A16 quantised on load: per-sequence state from a random prefill (48 tokens in chunks of 16; 16
+    tokens at batch 64 to bound the oracle's time),
+    then decode steps at batch 1 (GEMV + row-skipping ffn.value), 8 (GEMV, fused time-mix step) and 64
+    (streaming MFMA GEMM with split-K partials summed by the LayerNorm kernels, row-tiled time-mix kernels),
+    every step's logits against the oracle."""
+    import os
+    from rwkv_lightning_cuda_amd.model import PRESETS, HipModel, ModelDims, Session, State, synth_weights
+    hip = gpu
+    big = PRESETS["1.5B"]
+    dims = ModelDims(L=2, C=big.C, H=big.H, F=big.F, V=4096, Rw=big.Rw, Ra=big.Ra, Rg=big.Rg, Rv=big.Rv)
+    weights = synth_weights(dims, 52)
+    orc.set_threads(min(16, os.cpu_count() or 1))
+    omodel = orc.Model(dims, weights, orc.FMT_W8)
+    gmodel = HipModel.from_host_weights(dims, weights, hip.FMT_W8)
+    rng = np.random.default_rng(B)
+    P = 48 if B <= 8 else 16
+    steps = 4 if B <= 8 else 2
+    prompt = rng.integers(0, dims.V, (B, P))
+    sess = Session(gmodel)
+    gstate = State(dims, B)
+    glogits = hip.DeviceArray((B, dims.V), np.float32)
+    ostate = omodel.new_state(B)
+    for t0 in range(0, P, 16):
+        sess.forward(prompt[:, t0:t0 + 16], gstate, glogits)
+        ologits = omodel.forward(prompt[:, t0:t0 + 16], ostate)
+    cos = cosine(glogits.numpy(), ologits)
+    assert cos >= 0.9995
+    nxt = np.argmax(ologits, axis=1).reshape(B, 1)
+    for step in range(steps):
+        sess.forward(nxt, gstate, glogits)
+        ologits = omodel.forward(nxt, ostate)
+        g = glogits.numpy()
+        for b in range(B):
+            cos = cosine(g[b], ologits[b])
+            assert cos >= 0.9995, "step %d row %d" % (step, b)
+        err = rel_err(g, ologits)
+        assert err <= 4e-3
+        nxt = np.argmax(ologits, axis=1).reshape(B, 1)
+    orc.set_threads(1)
+    err = rel_err(gstate.wkv.numpy(), ostate[1])
+    assert err <= 5e-3
+    err = rel_err(gstate.shift.numpy().astype(np.float32), ostate[0].astype(np.float32))
+    assert err <= 4e-3
+    assert gstate.elapsed.numpy().tolist() == [P + steps] * B
+    sess.close()
+
+
 @pytest.mark.parametrize("fmt_name", ["w8", "w4"])
 def test_config3_7p2b_width_two_layers_quantised(gpu, orc, fmt_name):
     """BASELINE config 3 at full width (C 4096, H 64, F 16384, LoRA ranks 128/128/480/96) with two layers and a
