@@ -378,21 +378,10 @@ __global__ __launch_bounds__(NW * 64) void linear_gemv_kernel(LinearArgs args) {
   }
 }
 
-// Wavefronts per block of the LayerNorm-prologue variant.  16 (the prologue once per 32 rows, the whole grid
-// resident at once) measured slightly slower than 4 on the 7.2B shapes; RWKV_GEMV_LN_WAVES=16 selects it.
-static int ln_block_waves() {
-  static const int v = [] {
-    const char* e = getenv("RWKV_GEMV_LN_WAVES");
-    const int n = e ? atoi(e) : 0;
-    return n == 16 ? 16 : 4;
-  }();
-  return v;
-}
-
 template <int M, int R, int U>
 static int launch_one(hipStream_t st, LinearArgs& args) {
   const bool ln = args.ln.mode != 0;
-  const int nw = (ln && M <= 2) ? ln_block_waves() : 4;  // more rows per call need more registers than 1024 threads leave
+  const int nw = 4;
   int total = 0;
   for (int i = 0; i < args.n_problems; ++i) {
     total += ceil_div(args.p[i].N, nw * R);
@@ -400,9 +389,7 @@ static int launch_one(hipStream_t st, LinearArgs& args) {
   }
   size_t lds = static_cast<size_t>(M) * args.KT * sizeof(half_t);
   if (ln) lds += static_cast<size_t>(args.K) * sizeof(float);
-  if (ln && nw == 16) {
-    hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, true, 16>), dim3(total), dim3(1024), lds, st, args);
-  } else if (ln) {
+  if (ln) {
     hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, true, 4>), dim3(total), dim3(256), lds, st, args);
   } else {
     hipLaunchKernelGGL((linear_gemv_kernel<M, R, U, false, 4>), dim3(total), dim3(256), lds, st, args);
@@ -453,22 +440,6 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
   if (copy && copy->n > 0) {
     RWKV_REQUIRE(copy->src && copy->dst && copy->n % 8 == 0, "linear: bad row copy");
     args.copy = *copy;
-  }
-  if (M == 1) {
-    // RWKV_GEMV_RU=<R><U> picks the rows-per-wave / steps-in-flight variant for M == 1 (tuning aid)
-    static const int ru = [] { const char* e = getenv("RWKV_GEMV_RU"); return e ? atoi(e) : 0; }();
-    switch (ru) {
-      case 11: return launch_one<1, 1, 1>(st, args);
-      case 12: return launch_one<1, 1, 2>(st, args);
-      case 14: return launch_one<1, 1, 4>(st, args);
-      case 24: return launch_one<1, 2, 4>(st, args);
-      case 22: return launch_one<1, 2, 2>(st, args);
-      case 41: return launch_one<1, 4, 1>(st, args);
-      case 42: return launch_one<1, 4, 2>(st, args);
-      case 44: return launch_one<1, 4, 4>(st, args);
-      case 81: return launch_one<1, 8, 1>(st, args);
-      default: break;
-    }
   }
   switch (M) {
     case 1: return launch_one<1, 2, 1>(st, args);
