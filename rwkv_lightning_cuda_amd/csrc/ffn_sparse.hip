@@ -7,14 +7,14 @@
 // with atomicAdd (the result depends on block order); here the products are exact, the accumulation is fp32 and
 // the order is fixed, so the result is the dense product of the same codes up to fp32 summation order.
 //
-// Weights: the int8 codes of the [C,F] matrix transposed to [F,C] and stored offset by 128 (u = q + 128, one
-// byte each), with the same per-output-channel fp16 scale.
+// Weights: the [C,F] matrix transposed to [F,C]: fp16 values as they are, or int8 codes stored offset by 128
+// (u = q + 128, one byte each) with the same per-output-channel fp16 scale.
 //
-// Kernel 1: grid = (F/256, ceil(C/1024)), block = 8 wavefronts.  A wavefront owns 32 consecutive f and 1024
-// columns (16 per lane): it ballots the non-zero activations, walks the set bits eight rows at a time (missing
-// rows of the last batch repeat a row already read, with coefficient zero, so no load sits under a branch), and
-// accumulates two rows per v_dot2_f32_f16: v_perm_b32 pairs the bytes of the two rows under exponent 0x64 and
-// one packed subtract gives the exact signed codes.  The eight wavefronts' sums meet in LDS in wavefront
+// Kernel 1: grid = (F/256, column chunks), block = 8 wavefronts.  A wavefront owns 32 consecutive f and one 16-byte
+// piece of the row per lane (1024 int8 or 512 fp16 columns per chunk): it ballots the non-zero activations, walks
+// the set bits eight rows at a time (missing rows of the last batch repeat a row already read, with coefficient
+// zero, so no load sits under a branch), and accumulates two rows per v_dot2_f32_f16: v_perm_b32 pairs the
+// values of the two rows (int8: bytes under exponent 0x64, then one packed subtract gives the exact codes).  The eight wavefronts' sums meet in LDS in wavefront
 // order and the block writes one fp32 partial row.  Kernel 2 sums the F/256 partial rows in a fixed order,
 // applies the scale and rounds to fp16.
 #include "ops.h"
@@ -24,25 +24,31 @@ namespace rwkv {
 constexpr int kSparseRowsPerWave = 32;
 constexpr int kSparseWaves = 8;
 constexpr int kSparseRowsPerBlock = kSparseRowsPerWave * kSparseWaves;  // 256
-constexpr int kSparseCols = 1024;                                        // per block: 64 lanes x 16 codes
 constexpr int kSparseBatch = 8;
 
-bool ffn_sparse_supported(int C, int F) { return C >= 16 && C % 16 == 0 && F >= kSparseRowsPerBlock && F % kSparseRowsPerBlock == 0; }
+// columns per lane = values in a 16-byte piece
+constexpr int sparse_lane_cols(int fmt) { return fmt == RWKV_FMT_W8 ? 16 : 8; }
+
+bool ffn_sparse_supported(int fmt, int C, int F) {
+  if (fmt != RWKV_FMT_W8 && fmt != RWKV_FMT_F16) return false;
+  return C >= 16 && C % 16 == 0 && F >= kSparseRowsPerBlock && F % kSparseRowsPerBlock == 0;
+}
 
 size_t ffn_sparse_workspace_bytes(int C, int F) { return static_cast<size_t>(F / kSparseRowsPerBlock) * C * sizeof(float); }
 
-// ---- [C,F] int8 codes -> [F,C] offset codes ------------------------------------------------------------------------------
+// ---- [C,F] -> [F,C] (int8 codes get the offset) ----------------------------------------------------------------------
 // grid = (F/64, C/64) tiles through LDS; C and F multiples of 64 are not required (edges are predicated).
-__global__ __launch_bounds__(256) void ffn_sparse_pack_kernel(int C, int F, const int8_t* __restrict__ w,
-                                                              uint8_t* __restrict__ wt) {
-  __shared__ uint8_t tile[64][65];
+template <typename E>
+__global__ __launch_bounds__(256) void ffn_sparse_pack_kernel(int C, int F, const E* __restrict__ w, E* __restrict__ wt) {
+  __shared__ E tile[64][65];
   const int f0 = blockIdx.x * 64;
   const int c0 = blockIdx.y * 64;
   for (int i = threadIdx.x; i < 64 * 64; i += 256) {
     const int c = i >> 6;
     const int f = i & 63;
-    uint8_t v = 0;
-    if (c0 + c < C && f0 + f < F) v = static_cast<uint8_t>(w[static_cast<int64_t>(c0 + c) * F + f0 + f]) ^ 0x80u;
+    E v = 0;
+    if (c0 + c < C && f0 + f < F) v = w[static_cast<int64_t>(c0 + c) * F + f0 + f];
+    if constexpr (sizeof(E) == 1) v ^= 0x80u;
     tile[c][f] = v;
   }
   __syncthreads();
@@ -53,30 +59,39 @@ __global__ __launch_bounds__(256) void ffn_sparse_pack_kernel(int C, int F, cons
   }
 }
 
-int ffn_sparse_pack_launch(hipStream_t st, int C, int F, const void* w, void* wt) {
-  RWKV_REQUIRE(ffn_sparse_supported(C, F), "ffn_sparse_pack: unsupported shape C=%d F=%d", C, F);
+int ffn_sparse_pack_launch(hipStream_t st, int fmt, int C, int F, const void* w, void* wt) {
+  RWKV_REQUIRE(ffn_sparse_supported(fmt, C, F), "ffn_sparse_pack: unsupported format %d or shape C=%d F=%d", fmt, C, F);
   RWKV_REQUIRE(w && wt && w != wt, "ffn_sparse_pack: bad pointers");
-  hipLaunchKernelGGL(ffn_sparse_pack_kernel, dim3(ceil_div(F, 64), ceil_div(C, 64)), dim3(256), 0, st, C, F,
-                     static_cast<const int8_t*>(w), static_cast<uint8_t*>(wt));
+  const dim3 grid(ceil_div(F, 64), ceil_div(C, 64));
+  if (fmt == RWKV_FMT_W8) {
+    hipLaunchKernelGGL(ffn_sparse_pack_kernel<uint8_t>, grid, dim3(256), 0, st, C, F, static_cast<const uint8_t*>(w),
+                       static_cast<uint8_t*>(wt));
+  } else {
+    hipLaunchKernelGGL(ffn_sparse_pack_kernel<uint16_t>, grid, dim3(256), 0, st, C, F, static_cast<const uint16_t*>(w),
+                       static_cast<uint16_t*>(wt));
+  }
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
 // ---- kernel 1 ------------------------------------------------------------------------------------------------------------
 // `activated` != 0: `in` already holds f16(relu(preact)^2) (the model's ffn.key launch applies it).
+template <int FMT>
 __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, int F, int activated,
                                                                        const half_t* __restrict__ in,
                                                                        const uint4_t* __restrict__ wt,
                                                                        float* __restrict__ partial) {
-  __shared__ __align__(16) float red[kSparseWaves][kSparseCols];
+  constexpr int LC = sparse_lane_cols(FMT);  // columns per lane
+  constexpr int kCols = 64 * LC;             // columns per block
+  __shared__ __align__(16) float red[kSparseWaves][kCols];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
   const int f0 = blockIdx.x * kSparseRowsPerBlock + wave * kSparseRowsPerWave;
-  const int c0 = blockIdx.y * kSparseCols;
-  const bool col_ok = c0 + 16 * lane < C;
-  // 16-byte pieces: row f starts at f * C/16, this lane's piece of the row is (c0/16 + lane)
-  const int row_pieces = C >> 4;
-  const uint4_t* wlane = wt + (c0 >> 4) + (col_ok ? lane : 0);
+  const int c0 = blockIdx.y * kCols;
+  const bool col_ok = c0 + LC * lane < C;
+  // 16-byte pieces: row f has C/LC of them, this lane's piece of the row is (c0/LC + lane)
+  const int row_pieces = C / LC;
+  const uint4_t* wlane = wt + c0 / LC + (col_ok ? lane : 0);
 
   float a = 0.0f;
   if (lane < kSparseRowsPerWave) {
@@ -90,9 +105,9 @@ __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, in
   const uint32_t abits = __builtin_bit_cast(uint16_t, ah);
   uint64_t mask = __ballot((abits << 17) != 0u);  // +0 and -0 both count as zero
 
-  float acc[16];
+  float acc[LC];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+  for (int i = 0; i < LC; ++i) acc[i] = 0.0f;
   const half2_t bias = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
 
   while (mask != 0) {
@@ -120,24 +135,32 @@ __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, in
       for (int d = 0; d < 4; ++d) {
         const uint32_t lo = q[p][d];
         const uint32_t hi = q[p + 1][d];
-        const half2_t w0 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c040c00u) | 0x64006400u) - bias;
-        const half2_t w1 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c050c01u) | 0x64006400u) - bias;
-        const half2_t w2 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c060c02u) | 0x64006400u) - bias;
-        const half2_t w3 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c070c03u) | 0x64006400u) - bias;
-        acc[4 * d + 0] = __builtin_amdgcn_fdot2(ap, w0, acc[4 * d + 0], false);
-        acc[4 * d + 1] = __builtin_amdgcn_fdot2(ap, w1, acc[4 * d + 1], false);
-        acc[4 * d + 2] = __builtin_amdgcn_fdot2(ap, w2, acc[4 * d + 2], false);
-        acc[4 * d + 3] = __builtin_amdgcn_fdot2(ap, w3, acc[4 * d + 3], false);
+        if constexpr (FMT == RWKV_FMT_W8) {
+          const half2_t w0 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c040c00u) | 0x64006400u) - bias;
+          const half2_t w1 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c050c01u) | 0x64006400u) - bias;
+          const half2_t w2 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c060c02u) | 0x64006400u) - bias;
+          const half2_t w3 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c070c03u) | 0x64006400u) - bias;
+          acc[4 * d + 0] = __builtin_amdgcn_fdot2(ap, w0, acc[4 * d + 0], false);
+          acc[4 * d + 1] = __builtin_amdgcn_fdot2(ap, w1, acc[4 * d + 1], false);
+          acc[4 * d + 2] = __builtin_amdgcn_fdot2(ap, w2, acc[4 * d + 2], false);
+          acc[4 * d + 3] = __builtin_amdgcn_fdot2(ap, w3, acc[4 * d + 3], false);
+        } else {
+          // a dword holds two fp16 columns of a row: pair the low halves and the high halves of the two rows
+          const half2_t w0 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x05040100u));
+          const half2_t w1 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x07060302u));
+          acc[2 * d + 0] = __builtin_amdgcn_fdot2(ap, w0, acc[2 * d + 0], false);
+          acc[2 * d + 1] = __builtin_amdgcn_fdot2(ap, w1, acc[2 * d + 1], false);
+        }
       }
     }
   }
 
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-    *reinterpret_cast<float4_t*>(&red[wave][16 * lane + 4 * i]) =
+  for (int i = 0; i < LC / 4; ++i)
+    *reinterpret_cast<float4_t*>(&red[wave][LC * lane + 4 * i]) =
         float4_t{acc[4 * i], acc[4 * i + 1], acc[4 * i + 2], acc[4 * i + 3]};
   __syncthreads();
-  if (threadIdx.x < kSparseCols / 4) {
+  if (threadIdx.x < kCols / 4) {
     const int c = 4 * threadIdx.x;
     float4_t sum = *reinterpret_cast<const float4_t*>(&red[0][c]);
 #pragma unroll
@@ -171,17 +194,18 @@ __global__ __launch_bounds__(256) void ffn_sparse_finish_kernel(int C, int n_par
   float4_t total = *reinterpret_cast<const float4_t*>(&red[0][cq]);
 #pragma unroll
   for (int i = 1; i < 16; ++i) total = total + *reinterpret_cast<const float4_t*>(&red[i][cq]);
-  const half4_t sv = *reinterpret_cast<const half4_t*>(scale + c);
+  half4_t sv = {static_cast<half_t>(1.0f), static_cast<half_t>(1.0f), static_cast<half_t>(1.0f), static_cast<half_t>(1.0f)};
+  if (scale) sv = *reinterpret_cast<const half4_t*>(scale + c);
   half4_t o;
 #pragma unroll
   for (int i = 0; i < 4; ++i) o[i] = f2h(total[i] * h2f(sv[i]));
   *reinterpret_cast<half4_t*>(out + c) = o;
 }
 
-int ffn_sparse_launch(hipStream_t st, int C, int F, int activated, const half_t* in, const void* wt, const half_t* scale,
-                      void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy) {
-  RWKV_REQUIRE(ffn_sparse_supported(C, F), "ffn_sparse: unsupported shape C=%d F=%d", C, F);
-  RWKV_REQUIRE(in && wt && scale && out, "ffn_sparse: NULL tensor");
+int ffn_sparse_launch(hipStream_t st, int fmt, int C, int F, int activated, const half_t* in, const void* wt,
+                      const half_t* scale, void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy) {
+  RWKV_REQUIRE(ffn_sparse_supported(fmt, C, F), "ffn_sparse: unsupported format %d or shape C=%d F=%d", fmt, C, F);
+  RWKV_REQUIRE(in && wt && out && (fmt != RWKV_FMT_W8 || scale), "ffn_sparse: NULL tensor");
   RWKV_REQUIRE(workspace && workspace_bytes >= ffn_sparse_workspace_bytes(C, F), "ffn_sparse: workspace of %zu bytes needed, got %zu",
                ffn_sparse_workspace_bytes(C, F), workspace_bytes);
   RowCopy cp;
@@ -190,11 +214,17 @@ int ffn_sparse_launch(hipStream_t st, int C, int F, int activated, const half_t*
     cp = *copy;
   }
   const int n_partial = F / kSparseRowsPerBlock;
-  hipLaunchKernelGGL(ffn_sparse_kernel, dim3(n_partial, ceil_div(C, kSparseCols)), dim3(64 * kSparseWaves), 0, st, C, F,
-                     activated, in, static_cast<const uint4_t*>(wt), static_cast<float*>(workspace));
+  const dim3 grid(n_partial, ceil_div(C, 64 * sparse_lane_cols(fmt)));
+  if (fmt == RWKV_FMT_W8) {
+    hipLaunchKernelGGL(ffn_sparse_kernel<RWKV_FMT_W8>, grid, dim3(64 * kSparseWaves), 0, st, C, F, activated, in,
+                       static_cast<const uint4_t*>(wt), static_cast<float*>(workspace));
+  } else {
+    hipLaunchKernelGGL(ffn_sparse_kernel<RWKV_FMT_F16>, grid, dim3(64 * kSparseWaves), 0, st, C, F, activated, in,
+                       static_cast<const uint4_t*>(wt), static_cast<float*>(workspace));
+  }
   RWKV_LAUNCH_CHECK();
   hipLaunchKernelGGL(ffn_sparse_finish_kernel, dim3(ceil_div(C, 64)), dim3(256), 0, st, C, n_partial,
-                     static_cast<const float*>(workspace), scale, out, cp);
+                     static_cast<const float*>(workspace), fmt == RWKV_FMT_W8 ? scale : nullptr, out, cp);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
@@ -205,20 +235,20 @@ using namespace rwkv;
 
 extern "C" {
 
-int rwkv_hip_cmix_sparse_pack(rwkv_stream_t s, int C, int F, const void* w, void* wt) {
-  return ffn_sparse_pack_launch(as_stream(s), C, F, w, wt);
+int rwkv_hip_cmix_sparse_pack(rwkv_stream_t s, int fmt, int C, int F, const void* w, void* wt) {
+  return ffn_sparse_pack_launch(as_stream(s), fmt, C, F, w, wt);
 }
 
 int rwkv_hip_cmix_sparse_workspace(int C, int F, size_t* bytes) {
   RWKV_REQUIRE(bytes, "cmix_sparse_workspace: NULL argument");
-  RWKV_REQUIRE(ffn_sparse_supported(C, F), "cmix_sparse_workspace: unsupported shape C=%d F=%d", C, F);
+  RWKV_REQUIRE(ffn_sparse_supported(RWKV_FMT_W8, C, F), "cmix_sparse_workspace: unsupported shape C=%d F=%d", C, F);
   *bytes = ffn_sparse_workspace_bytes(C, F);
   return RWKV_OK;
 }
 
-int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int C, int F, const void* preact, const void* wt,
+int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int fmt, int C, int F, const void* preact, const void* wt,
                                        const void* scale, void* workspace, size_t workspace_bytes, void* out) {
-  return ffn_sparse_launch(as_stream(s), C, F, 0, static_cast<const half_t*>(preact), wt,
+  return ffn_sparse_launch(as_stream(s), fmt, C, F, 0, static_cast<const half_t*>(preact), wt,
                            static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr);
 }
 

@@ -25,7 +25,7 @@ struct Matrix {
   const half_t* scale = nullptr;
   const uint8_t* zp = nullptr;
   void* packed = nullptr;  // owned: the same codes in the MFMA-native order, for calls with >= 16 rows
-  void* sparse_t = nullptr;  // owned, ffn.value with int8 codes only: [F,C] offset codes for the one-token row-skipping product
+  void* sparse_t = nullptr;  // owned, ffn.value with int8 codes or fp16 only: the [F,C] copy for the one-token row-skipping product
 };
 
 struct Layer {
@@ -235,7 +235,7 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
       s->gemm_ws_bytes = ws;
     }
   }
-  if (!s->sparse_ws && ffn_sparse_supported(m->C, m->F)) {
+  if (!s->sparse_ws && ffn_sparse_supported(RWKV_FMT_W8, m->C, m->F)) {
     const size_t bytes = ffn_sparse_workspace_bytes(m->C, m->F);
     RWKV_HIP_TRY(hipMalloc(&s->sparse_ws, bytes));
     s->sparse_ws_bytes = bytes;
@@ -330,7 +330,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   const bool ln_in_linear = s->fused_ln && step && small && !s->trace &&
                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
 
-  // One-token steps read only the ffn.value rows whose relu^2 activation is non-zero (int8 weights).
+  // One-token steps read only the ffn.value rows whose relu^2 activation is non-zero (int8 or fp16 weights).
   const bool sparse_value = step && rows == 1 && s->sparse_ffn && s->sparse_ws != nullptr;
 
   auto mix6_args = [&](const Layer& w, LnArgs& a) {
@@ -527,7 +527,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       RowCopy cp;
       cp.src = b.ln2; cp.dst = shift1; cp.n = rows * C;
       if (sparse_value && mv.sparse_t) {
-        TRY_AUX(ffn_sparse_launch(st, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm, &cp));
+        TRY_AUX(ffn_sparse_launch(st, mv.fmt, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm, &cp));
       } else {
         LinearProblem pv = {mv.data, mv.scale, mv.zp, b.act, b.cm, C, mv.fmt, nullptr};
         TRY_PROF(linear_small_m(st, rows, F, 1, &pv, RWKV_EPI_NONE, 0, nullptr, &cp));
@@ -536,7 +536,8 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
       const Matrix& mv = w.m[RWKV_M_FFN_VALUE];
       if (sparse_value && mv.sparse_t) {
-        TRY_AUX(ffn_sparse_launch(st, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm, nullptr));
+        TRY_AUX(ffn_sparse_launch(st, mv.fmt, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
+                                  nullptr));
       } else {
         TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm, defer_ok ? &cm_partial : nullptr));
       }
@@ -754,10 +755,10 @@ int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, con
     }
     RWKV_HIP_TRY(hipStreamSynchronize(nullptr));
   }
-  if (id == RWKV_M_FFN_VALUE && fmt == RWKV_FMT_W8 && ffn_sparse_supported(N, K)) {
+  if (id == RWKV_M_FFN_VALUE && ffn_sparse_supported(fmt, N, K)) {
     // third copy: transposed, for decode steps of one sequence
-    RWKV_HIP_TRY(hipMalloc(&mat.sparse_t, static_cast<size_t>(N) * K));
-    const int rc = ffn_sparse_pack_launch(nullptr, N, K, data, mat.sparse_t);
+    RWKV_HIP_TRY(hipMalloc(&mat.sparse_t, static_cast<size_t>(N) * K * (fmt == RWKV_FMT_F16 ? 2 : 1)));
+    const int rc = ffn_sparse_pack_launch(nullptr, fmt, N, K, data, mat.sparse_t);
     if (rc != RWKV_OK) {
       (void)hipFree(mat.sparse_t);
       if (mat.packed) (void)hipFree(mat.packed);

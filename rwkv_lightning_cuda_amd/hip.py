@@ -239,8 +239,8 @@ def lora_in(M, C, R, x, w1, h, stream=None):
     check(load().rwkv_hip_lora_in(_p(stream), _i(M), _i(C), _i(R), _p(x), _p(w1), _p(h)))
 
 
-def cmix_sparse_pack(C, F, w, wt, stream=None):
-    check(load().rwkv_hip_cmix_sparse_pack(_p(stream), _i(C), _i(F), _p(w), _p(wt)))
+def cmix_sparse_pack(fmt, C, F, w, wt, stream=None):
+    check(load().rwkv_hip_cmix_sparse_pack(_p(stream), _i(fmt), _i(C), _i(F), _p(w), _p(wt)))
 
 
 def cmix_sparse_workspace(C, F):
@@ -249,9 +249,9 @@ def cmix_sparse_workspace(C, F):
     return n.value
 
 
-def cmix_sparse_down_relu_one(C, F, preact, wt, scale, workspace, out, stream=None):
-    check(load().rwkv_hip_cmix_sparse_down_relu_one(_p(stream), _i(C), _i(F), _p(preact), _p(wt), _p(scale), _p(workspace),
-                                                    ctypes.c_size_t(workspace.nbytes), _p(out)))
+def cmix_sparse_down_relu_one(fmt, C, F, preact, wt, scale, workspace, out, stream=None):
+    check(load().rwkv_hip_cmix_sparse_down_relu_one(_p(stream), _i(fmt), _i(C), _i(F), _p(preact), _p(wt), _p(scale),
+                                                    _p(workspace), ctypes.c_size_t(workspace.nbytes), _p(out)))
 
 
 def lora_out(M, C, R, act, h, w2, out, bias=None, vres=0, v=None, v_first=None, stream=None):

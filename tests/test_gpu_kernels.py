@@ -403,20 +403,30 @@ def test_lora_out_keeps_the_activated_hidden_in_fp32(gpu, rows, C, R):
         assert off <= 0.01, "act %d: %.4f of the outputs are not the correctly rounded value" % (act, off)
 
 
+@pytest.mark.parametrize("fmt_name", ["w8", "f16"])
 @pytest.mark.parametrize("C,F", [(768, 3072), (2560, 10240), (4096, 16384)])
-def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F):
-    """ffn.value of one token over the transposed int8 copy, skipping rows with a zero activation: against the
-    oracle's dense product of the same codes and against the dense GEMV on the GPU; edge patterns of the
+def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F, fmt_name):
+    """ffn.value of one token over the transposed copy, skipping rows with a zero activation: against the
+    oracle's dense product of the same weights and against the dense GEMV on the GPU; edge patterns of the
     activation (none, one, all non-zero; a wavefront's 32 rows all zero); repeat calls bitwise equal."""
     hip = gpu
     rng = np.random.default_rng(C + F)
     w = (rng.standard_normal((C, F)) * 0.02).astype(np.float16)
-    q, s = orc.quantize_w8(w)
-    qd, sd = dev(hip, q), dev(hip, s)
-    wt = hip.DeviceArray((F, C), np.uint8)
-    hip.cmix_sparse_pack(C, F, qd, wt)
+    if fmt_name == "w8":
+        fmt = hip.FMT_W8
+        q, s = orc.quantize_w8(w)
+        qd, sd = dev(hip, q), dev(hip, s)
+        wt = hip.DeviceArray((F, C), np.uint8)
+        want_t = (q.T.astype(np.int16) + 128).astype(np.uint8)
+    else:
+        fmt = hip.FMT_F16
+        q, s = w, None
+        qd, sd = dev(hip, w), None
+        wt = hip.DeviceArray((F, C), np.float16)
+        want_t = np.ascontiguousarray(w.T)
+    hip.cmix_sparse_pack(fmt, C, F, qd, wt)
     hip.device_sync()
-    same = np.array_equal(wt.numpy(), (q.T.astype(np.int16) + 128).astype(np.uint8))
+    same = np.array_equal(wt.numpy().view(np.uint8), want_t.view(np.uint8))
     assert same
     ws = hip.DeviceArray.zeros((hip.cmix_sparse_workspace(C, F),), np.uint8)
 
@@ -431,9 +441,9 @@ def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F):
     }
     for name, pre in patterns.items():
         act = orc.relu_square(pre.reshape(1, F))
-        want = orc.gemv(orc.FMT_W8, act, q, s)
+        want = orc.gemv(fmt, act, q, s)
         out = hip.DeviceArray((1, C), np.float16)
-        hip.cmix_sparse_down_relu_one(C, F, dev(hip, pre), wt, sd, ws, out)
+        hip.cmix_sparse_down_relu_one(fmt, C, F, dev(hip, pre), wt, sd, ws, out)
         hip.device_sync()
         got = out.numpy()
         if name == "none":
@@ -442,9 +452,9 @@ def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F):
             err = rel_err(got.astype(np.float32), want.astype(np.float32))
             assert err <= F16_TOL, name
         dense = hip.DeviceArray((1, C), np.float16)
-        hip.linear(hip.FMT_W8, 1, C, F, dev(hip, act), qd, sd, None, dense)
+        hip.linear(fmt, 1, C, F, dev(hip, act), qd, sd, None, dense)
         out2 = hip.DeviceArray((1, C), np.float16)
-        hip.cmix_sparse_down_relu_one(C, F, dev(hip, pre), wt, sd, ws, out2)
+        hip.cmix_sparse_down_relu_one(fmt, C, F, dev(hip, pre), wt, sd, ws, out2)
         hip.device_sync()
         # two fp32 sums of the same exact products in different orders: at most an fp16 ulp apart at the output scale
         d = np.abs(got.astype(np.float32) - dense.numpy().astype(np.float32)).max()
@@ -461,7 +471,9 @@ def test_cmix_sparse_rejects_bad_arguments(gpu):
         hip.cmix_sparse_workspace(100, 1024)  # C not a multiple of 16
     buf = hip.DeviceArray.zeros((1024,), np.uint8)
     with pytest.raises(hip.RwkvHipError):
-        hip.cmix_sparse_down_relu_one(256, 1024, buf, buf, buf, buf, buf)  # workspace too small
+        hip.cmix_sparse_down_relu_one(hip.FMT_W8, 256, 1024, buf, buf, buf, buf, buf)  # workspace too small
+    with pytest.raises(hip.RwkvHipError):
+        hip.cmix_sparse_pack(hip.FMT_W4, 256, 1024, buf, hip.DeviceArray.zeros((1024,), np.uint8))  # no int4 variant
 
 
 def test_small_elementwise(gpu, orc):

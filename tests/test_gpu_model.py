@@ -79,14 +79,15 @@ def test_small_model_prefill_and_decode(gpu, orc, fmt):
     sess.close()
 
 
-def test_one_sequence_decode_with_row_skipping_ffn_value(gpu, orc):
-    """Batch-1 decode steps of a W8 model use the row-skipping ffn.value product (eager and graph replay): the
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_one_sequence_decode_with_row_skipping_ffn_value(gpu, orc, fmt):
+    """Batch-1 decode steps of an fp16 or W8 model use the row-skipping ffn.value product (eager and graph replay): the
     steps match the oracle, stay within an fp16 ulp of the dense product's logits, and the activations really
     are sparse (else the test would not exercise the skip)."""
     from rwkv_lightning_cuda_amd.model import Session, State
     hip = gpu
     dims = small_dims()
-    omodel, gmodel = build_pair(gpu, orc, dims, orc.FMT_W8, seed=33)
+    omodel, gmodel = build_pair(gpu, orc, dims, fmt, seed=33)
     rng = np.random.default_rng(8)
     prompt = rng.integers(0, dims.V, (1, 6))
     steps = rng.integers(0, dims.V, (5, 1, 1))
