@@ -249,14 +249,14 @@ def main():
     # for rows == 1, include/rwkv7_fast_v4_common.hpp:198-211); the dense product is timed beside it below
     sparse_value = B == 1 and args.fmt in ("w8", "f16") and dims.F % 256 == 0 and dims.C % 16 == 0
     if sparse_value and not args.no_also:
-        sess.set_sparse_ffn(False)
+        sess.set_sparse_ffn(0)
         sess.decode_greedy(first, min(args.warmup, 8) or 1, state, logits)
         hip.device_sync()
         td = time.perf_counter()
         sess.decode_greedy(first, min(args.steps, 64), state, logits)
         hip.device_sync()
         also["decode_dense_ffn_value_tok_s"] = min(args.steps, 64) * B / (time.perf_counter() - td)
-        sess.set_sparse_ffn(True)
+        sess.set_sparse_ffn(1)
         act = sess.debug_buffer("act", (B, dims.F))
         also["ffn_value_rows_skipped_fraction_last_layer"] = float(np.mean(act == 0))
 

@@ -119,20 +119,24 @@ int rwkv_hip_linear_packed(rwkv_stream_t s, int fmt, int M, int N, int K, const 
                            const void* scale, const void* zp, int epilogue, int out_f32, void* y,
                            void* workspace, size_t workspace_bytes);
 
-/* ---- ffn.value of one token, reading only the rows with a non-zero activation.  Replaces
- * rwkv7_cmix_sparse_down_relu_one_launch (cuda/rwkv7_fast_v4_kernels.cuh:90-92,
- * cuda/rwkv7_fast_ops_fp16.cu:966-976,618-676):
+/* ---- ffn.value of a few tokens, reading per token only the rows with a non-zero activation.  Replaces
+ * rwkv7_cmix_sparse_down_relu_one_launch and rwkv7_cmix_sparse_down_relu_rows_launch
+ * (cuda/rwkv7_fast_v4_kernels.cuh:90-100, cuda/rwkv7_fast_ops_fp16.cu:966-992,618-737), per token:
  *   vec[f] = f16(relu(preact[f])^2);  out[c] = f16(sum over f with vec[f] != 0 of vec[f] * W[c][f])
  * for fmt = RWKV_FMT_F16 (the reference's case), or with int8 codes (RWKV_FMT_W8)
  *   out[c] = f16(scale[c] * sum over f with vec[f] != 0 of vec[f] * q[c][f]).
- * The reference accumulates in half2 with atomicAdd; this one accumulates exact products in fp32 in a fixed
- * order, so it equals the dense product up to fp32 summation order and repeats bitwise.
+ * preact [rows,F], out [rows,C], rows 1..12.  The reference accumulates in half2 with atomicAdd; this one
+ * accumulates exact products in fp32 in a fixed order, so it equals the dense product up to fp32 summation order
+ * and repeats bitwise.
  * cmix_sparse_pack turns the [C,F] matrix (fp16 values, or the codes of rwkv_hip_quantize_w8) into the [F,C]
  * copy `wt` (same size) that the product reads - the layout the reference keeps ffn.value in
  * (include/rwkv7_fast_v4_common.hpp:313-321); `scale` is the per-output-channel tensor of the codes (unused
  * for fp16).  C % 16 == 0, F % 256 == 0.  workspace: fp32 partial rows, size from cmix_sparse_workspace. */
 int rwkv_hip_cmix_sparse_pack(rwkv_stream_t s, int fmt, int C, int F, const void* w, void* wt);
-int rwkv_hip_cmix_sparse_workspace(int C, int F, size_t* bytes);
+int rwkv_hip_cmix_sparse_workspace(int rows, int C, int F, size_t* bytes);
+int rwkv_hip_cmix_sparse_down_relu_rows(rwkv_stream_t s, int fmt, int rows, int C, int F, const void* preact,
+                                        const void* wt, const void* scale, void* workspace, size_t workspace_bytes,
+                                        void* out);
 int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int fmt, int C, int F, const void* preact, const void* wt,
                                        const void* scale, void* workspace, size_t workspace_bytes, void* out);
 
@@ -258,10 +262,12 @@ int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host
  * and returns the number of linear launches and the summed bracketed time since the last read. */
 int rwkv_hip_session_set_profile(rwkv_hip_session* s, int mode);
 int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double* total_ms);
-/* Decode steps of one sequence use the row-skipping ffn.value product when the matrix is fp16 or int8 codes
- * (CmixMode::NoFcOne of the reference, src/rwkv7_fast_v4.cu:1285-1286); on by default, 0 selects the dense
- * product. */
-int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int on);
+/* Decode steps of up to max_rows rows (0..12) use the row-skipping ffn.value product when the matrix is fp16 or
+ * int8 codes (CmixMode::NoFcOne / NoFcRows2 of the reference, include/rwkv7_fast_v4_common.hpp:198-211, whose
+ * default is 12 rows at C = 4096).  Default 1: every extra row re-reads its share of the matrix, which pays
+ * only while rows x (fraction of non-zero activations) stays below 1 - about half the activations are
+ * non-zero with random-init weights, far fewer with trained ones.  0 selects the dense product. */
+int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
 /* Decode steps of up to 8 rows can fold the two LayerNorm + token-shift kernels of a layer into the prologue of
  * the linear launches that consume them (bitwise the same results).  Off by default: on this chip the extra
  * work inside every GEMV block costs more than the two small launches it saves.  No counterpart in the

@@ -1,7 +1,8 @@
-// Channel-mix down projection of one token that reads only the rows of ffn.value whose activation is non-zero.
+// Channel-mix down projection of a few tokens that reads, per token, only the rows of ffn.value whose activation
+// is non-zero.
 //
-// Reference: rwkv7_cmix_sparse_down_relu_one_launch and cmix_sparse_spmv_relu_one_kernel
-// (cuda/rwkv7_fast_ops_fp16.cu:966-976,618-676; call site src/rwkv7_fast_v4.cu:1285-1286):
+// Reference: rwkv7_cmix_sparse_down_relu_one_launch / _rows_launch and cmix_sparse_spmv_relu_one_kernel / _rows_kernel
+// (cuda/rwkv7_fast_ops_fp16.cu:966-992,618-737; call site src/rwkv7_fast_v4.cu:1285-1292), per token:
 //   vec[f] = f16(relu(preact[f])^2);  out[c] = sum over f with vec[f] != 0 of vec[f] * Wv[f][c]
 // over ffn.value stored [F,C], so that a skipped f skips a contiguous row.  The reference accumulates in half2
 // with atomicAdd (the result depends on block order); here the products are exact, the accumulation is fp32 and
@@ -10,7 +11,7 @@
 // Weights: the [C,F] matrix transposed to [F,C]: fp16 values as they are, or int8 codes stored offset by 128
 // (u = q + 128, one byte each) with the same per-output-channel fp16 scale.
 //
-// Kernel 1: grid = (F/256, column chunks), block = 8 wavefronts.  A wavefront owns 32 consecutive f and one 16-byte
+// Kernel 1: grid = (F/256, column chunks, tokens), block = 8 wavefronts.  A wavefront owns 32 consecutive f and one 16-byte
 // piece of the row per lane (1024 int8 or 512 fp16 columns per chunk): it ballots the non-zero activations, walks
 // the set bits eight rows at a time (missing rows of the last batch repeat a row already read, with coefficient
 // zero, so no load sits under a branch), and accumulates two rows per v_dot2_f32_f16: v_perm_b32 pairs the
@@ -34,7 +35,9 @@ bool ffn_sparse_supported(int fmt, int C, int F) {
   return C >= 16 && C % 16 == 0 && F >= kSparseRowsPerBlock && F % kSparseRowsPerBlock == 0;
 }
 
-size_t ffn_sparse_workspace_bytes(int C, int F) { return static_cast<size_t>(F / kSparseRowsPerBlock) * C * sizeof(float); }
+size_t ffn_sparse_workspace_bytes(int rows, int C, int F) {
+  return static_cast<size_t>(rows) * (F / kSparseRowsPerBlock) * C * sizeof(float);
+}
 
 // ---- [C,F] -> [F,C] (int8 codes get the offset) ----------------------------------------------------------------------
 // grid = (F/64, C/64) tiles through LDS; C and F multiples of 64 are not required (edges are predicated).
@@ -92,6 +95,8 @@ __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, in
   // 16-byte pieces: row f has C/LC of them, this lane's piece of the row is (c0/LC + lane)
   const int row_pieces = C / LC;
   const uint4_t* wlane = wt + c0 / LC + (col_ok ? lane : 0);
+  in += static_cast<int64_t>(blockIdx.z) * F;                       // this token's activations ...
+  partial += static_cast<int64_t>(blockIdx.z) * gridDim.x * C;      // ... and partial rows
 
   float a = 0.0f;
   if (lane < kSparseRowsPerWave) {
@@ -170,19 +175,21 @@ __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, in
 }
 
 // ---- kernel 2: out[c] = f16(scale[c] * sum of the partial rows); block 0 also does the optional row copy --------
-// grid = ceil(C/64), block = 256 = 16 groups of partial rows x 16 column quads.  Group g sums rows g, g+16, ... (its
+// grid = (ceil(C/64), tokens), block = 256 = 16 groups of partial rows x 16 column quads.  Group g sums rows g, g+16, ... (its
 // loads are independent, so they are all in flight together), the 16 group sums meet in LDS in group order.
 __global__ __launch_bounds__(256) void ffn_sparse_finish_kernel(int C, int n_partial, const float* __restrict__ partial,
                                                                 const half_t* __restrict__ scale,
                                                                 half_t* __restrict__ out, RowCopy copy) {
   __shared__ __align__(16) float red[16][64];
-  if (blockIdx.x == 0 && copy.n > 0) {
+  if (blockIdx.x == 0 && blockIdx.y == 0 && copy.n > 0) {
     for (int i = threadIdx.x * 8; i < copy.n; i += 256 * 8)
       *reinterpret_cast<uint4_t*>(copy.dst + i) = *reinterpret_cast<const uint4_t*>(copy.src + i);
   }
   const int g = threadIdx.x >> 4;
   const int cq = (threadIdx.x & 15) * 4;
   const int c = blockIdx.x * 64 + cq;
+  partial += static_cast<int64_t>(blockIdx.y) * n_partial * C;  // this token's partial rows ...
+  out += static_cast<int64_t>(blockIdx.y) * C;                  // ... and output row
   float4_t sum = {0.0f, 0.0f, 0.0f, 0.0f};
   if (c < C) {
 #pragma unroll 4
@@ -202,19 +209,20 @@ __global__ __launch_bounds__(256) void ffn_sparse_finish_kernel(int C, int n_par
   *reinterpret_cast<half4_t*>(out + c) = o;
 }
 
-int ffn_sparse_launch(hipStream_t st, int fmt, int C, int F, int activated, const half_t* in, const void* wt,
+int ffn_sparse_launch(hipStream_t st, int fmt, int rows, int C, int F, int activated, const half_t* in, const void* wt,
                       const half_t* scale, void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy) {
   RWKV_REQUIRE(ffn_sparse_supported(fmt, C, F), "ffn_sparse: unsupported format %d or shape C=%d F=%d", fmt, C, F);
+  RWKV_REQUIRE(rows >= 1 && rows <= kSparseMaxRows, "ffn_sparse: %d rows (1..%d)", rows, kSparseMaxRows);
   RWKV_REQUIRE(in && wt && out && (fmt != RWKV_FMT_W8 || scale), "ffn_sparse: NULL tensor");
-  RWKV_REQUIRE(workspace && workspace_bytes >= ffn_sparse_workspace_bytes(C, F), "ffn_sparse: workspace of %zu bytes needed, got %zu",
-               ffn_sparse_workspace_bytes(C, F), workspace_bytes);
+  RWKV_REQUIRE(workspace && workspace_bytes >= ffn_sparse_workspace_bytes(rows, C, F),
+               "ffn_sparse: workspace of %zu bytes needed, got %zu", ffn_sparse_workspace_bytes(rows, C, F), workspace_bytes);
   RowCopy cp;
   if (copy) {
     RWKV_REQUIRE(copy->n % 8 == 0, "ffn_sparse: row copy length %d must be a multiple of 8", copy->n);
     cp = *copy;
   }
   const int n_partial = F / kSparseRowsPerBlock;
-  const dim3 grid(n_partial, ceil_div(C, 64 * sparse_lane_cols(fmt)));
+  const dim3 grid(n_partial, ceil_div(C, 64 * sparse_lane_cols(fmt)), rows);
   if (fmt == RWKV_FMT_W8) {
     hipLaunchKernelGGL(ffn_sparse_kernel<RWKV_FMT_W8>, grid, dim3(64 * kSparseWaves), 0, st, C, F, activated, in,
                        static_cast<const uint4_t*>(wt), static_cast<float*>(workspace));
@@ -223,7 +231,7 @@ int ffn_sparse_launch(hipStream_t st, int fmt, int C, int F, int activated, cons
                        static_cast<const uint4_t*>(wt), static_cast<float*>(workspace));
   }
   RWKV_LAUNCH_CHECK();
-  hipLaunchKernelGGL(ffn_sparse_finish_kernel, dim3(ceil_div(C, 64)), dim3(256), 0, st, C, n_partial,
+  hipLaunchKernelGGL(ffn_sparse_finish_kernel, dim3(ceil_div(C, 64), rows), dim3(256), 0, st, C, n_partial,
                      static_cast<const float*>(workspace), fmt == RWKV_FMT_W8 ? scale : nullptr, out, cp);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
@@ -239,17 +247,24 @@ int rwkv_hip_cmix_sparse_pack(rwkv_stream_t s, int fmt, int C, int F, const void
   return ffn_sparse_pack_launch(as_stream(s), fmt, C, F, w, wt);
 }
 
-int rwkv_hip_cmix_sparse_workspace(int C, int F, size_t* bytes) {
+int rwkv_hip_cmix_sparse_workspace(int rows, int C, int F, size_t* bytes) {
   RWKV_REQUIRE(bytes, "cmix_sparse_workspace: NULL argument");
   RWKV_REQUIRE(ffn_sparse_supported(RWKV_FMT_W8, C, F), "cmix_sparse_workspace: unsupported shape C=%d F=%d", C, F);
-  *bytes = ffn_sparse_workspace_bytes(C, F);
+  RWKV_REQUIRE(rows >= 1 && rows <= kSparseMaxRows, "cmix_sparse_workspace: %d rows (1..%d)", rows, kSparseMaxRows);
+  *bytes = ffn_sparse_workspace_bytes(rows, C, F);
   return RWKV_OK;
+}
+
+int rwkv_hip_cmix_sparse_down_relu_rows(rwkv_stream_t s, int fmt, int rows, int C, int F, const void* preact,
+                                        const void* wt, const void* scale, void* workspace, size_t workspace_bytes,
+                                        void* out) {
+  return ffn_sparse_launch(as_stream(s), fmt, rows, C, F, 0, static_cast<const half_t*>(preact), wt,
+                           static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr);
 }
 
 int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int fmt, int C, int F, const void* preact, const void* wt,
                                        const void* scale, void* workspace, size_t workspace_bytes, void* out) {
-  return ffn_sparse_launch(as_stream(s), fmt, C, F, 0, static_cast<const half_t*>(preact), wt,
-                           static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr);
+  return rwkv_hip_cmix_sparse_down_relu_rows(s, fmt, 1, C, F, preact, wt, scale, workspace, workspace_bytes, out);
 }
 
 }  // extern "C"

@@ -118,7 +118,7 @@ struct rwkv_hip_session {
   size_t gemm_ws_bytes = 0;
   void* sparse_ws = nullptr;  // partial rows of the row-skipping ffn.value product
   size_t sparse_ws_bytes = 0;
-  bool sparse_ffn = true;     // one-token steps read only the ffn.value rows with a non-zero activation
+  int sparse_ffn_rows = 1;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
   bool fused_ln = false;      // decode steps fold LayerNorm + token shift into the linear launches (measured slower)
 };
 
@@ -236,7 +236,7 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
     }
   }
   if (!s->sparse_ws && ffn_sparse_supported(RWKV_FMT_W8, m->C, m->F)) {
-    const size_t bytes = ffn_sparse_workspace_bytes(m->C, m->F);
+    const size_t bytes = ffn_sparse_workspace_bytes(kSparseMaxRows, m->C, m->F);
     RWKV_HIP_TRY(hipMalloc(&s->sparse_ws, bytes));
     s->sparse_ws_bytes = bytes;
   }
@@ -330,8 +330,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   const bool ln_in_linear = s->fused_ln && step && small && !s->trace &&
                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
 
-  // One-token steps read only the ffn.value rows whose relu^2 activation is non-zero (int8 or fp16 weights).
-  const bool sparse_value = step && rows == 1 && s->sparse_ffn && s->sparse_ws != nullptr;
+  // Decode steps of a few rows (one by default) read, per row, only the ffn.value rows whose relu^2 activation is
+  // non-zero (int8 or fp16 weights).
+  const bool sparse_value = step && rows <= s->sparse_ffn_rows && s->sparse_ws != nullptr;
 
   auto mix6_args = [&](const Layer& w, LnArgs& a) {
     const int ids[6] = {RWKV_T_X_R, RWKV_T_X_W, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_A, RWKV_T_X_G};
@@ -527,7 +528,8 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       RowCopy cp;
       cp.src = b.ln2; cp.dst = shift1; cp.n = rows * C;
       if (sparse_value && mv.sparse_t) {
-        TRY_AUX(ffn_sparse_launch(st, mv.fmt, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm, &cp));
+        TRY_AUX(ffn_sparse_launch(st, mv.fmt, rows, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
+                                  &cp));
       } else {
         LinearProblem pv = {mv.data, mv.scale, mv.zp, b.act, b.cm, C, mv.fmt, nullptr};
         TRY_PROF(linear_small_m(st, rows, F, 1, &pv, RWKV_EPI_NONE, 0, nullptr, &cp));
@@ -536,7 +538,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       TRY_PROF(apply_matrix(s, w.m[RWKV_M_FFN_KEY], rows, F, C, b.mixed, RWKV_EPI_RELU_SQUARE, 0, b.act));
       const Matrix& mv = w.m[RWKV_M_FFN_VALUE];
       if (sparse_value && mv.sparse_t) {
-        TRY_AUX(ffn_sparse_launch(st, mv.fmt, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
+        TRY_AUX(ffn_sparse_launch(st, mv.fmt, rows, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
                                   nullptr));
       } else {
         TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm, defer_ok ? &cm_partial : nullptr));
@@ -869,11 +871,13 @@ int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on) {
   return RWKV_OK;
 }
 
-int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int on) {
+int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows) {
   RWKV_REQUIRE(s, "session is NULL");
-  if (s->sparse_ffn != (on != 0)) {
+  RWKV_REQUIRE(max_rows >= 0 && max_rows <= kSparseMaxRows, "set_sparse_ffn: max_rows %d out of range (0..%d)", max_rows,
+               kSparseMaxRows);
+  if (s->sparse_ffn_rows != max_rows) {
     TRY(drop_graphs(s));  // captured decode graphs hold the other kernel
-    s->sparse_ffn = on != 0;
+    s->sparse_ffn_rows = max_rows;
   }
   return RWKV_OK;
 }

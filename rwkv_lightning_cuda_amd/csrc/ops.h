@@ -180,12 +180,13 @@ int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a);
 
 // ---- ffn_sparse.hip: one-token ffn.value product that skips the rows with a zero activation ---------------
 bool ffn_sparse_supported(int fmt, int C, int F);  // int8 codes or fp16
-size_t ffn_sparse_workspace_bytes(int C, int F);
+constexpr int kSparseMaxRows = 12;  // the reference's largest row count for this path (default_cmix_nofc_max_rows)
+size_t ffn_sparse_workspace_bytes(int rows, int C, int F);
 // [C,F] -> [F,C]; int8 codes are stored offset by 128
 int ffn_sparse_pack_launch(hipStream_t st, int fmt, int C, int F, const void* w, void* wt);
-// activated != 0: `in` holds f16(relu(preact)^2) already; else the kernel applies it.  `copy` (optional) rides on
-// the second launch.  scale: per output channel for int8 codes, unused for fp16.
-int ffn_sparse_launch(hipStream_t st, int fmt, int C, int F, int activated, const half_t* in, const void* wt,
+// `in` [rows,F], `out` [rows,C].  activated != 0: `in` holds f16(relu(preact)^2) already; else the kernel applies it.
+// `copy` (optional) rides on the second launch.  scale: per output channel for int8 codes, unused for fp16.
+int ffn_sparse_launch(hipStream_t st, int fmt, int rows, int C, int F, int activated, const half_t* in, const void* wt,
                       const half_t* scale, void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy);
 
 // ---- sampler.hip --------------------------------------------------------------------------------

@@ -269,9 +269,10 @@ class Session:
         """Decode steps fold LayerNorm + token shift into the linear launches (bitwise the same; default off)."""
         hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(1 if on else 0)))
 
-    def set_sparse_ffn(self, on):
-        """One-sequence decode steps read only the ffn.value rows with a non-zero activation (default on)."""
-        hip.check(hip.load().rwkv_hip_session_set_sparse_ffn(self.handle, ctypes.c_int(1 if on else 0)))
+    def set_sparse_ffn(self, max_rows):
+        """Decode steps of up to max_rows rows (0..12; True = 1, False = 0) read only the ffn.value rows with a
+        non-zero activation (default 1)."""
+        hip.check(hip.load().rwkv_hip_session_set_sparse_ffn(self.handle, ctypes.c_int(int(max_rows))))
 
     def set_profile(self, mode):
         """0/False off; 1/True one event pair per linear launch; 2 passes launch the linear kernels only, back to

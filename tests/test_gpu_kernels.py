@@ -463,6 +463,48 @@ def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F, fmt_n
         assert same, name
 
 
+@pytest.mark.parametrize("fmt_name", ["w8", "f16"])
+def test_cmix_sparse_down_rows_matches_the_one_row_product(gpu, orc, fmt_name):
+    """Several tokens per call: each row of the output is bitwise what the one-row call gives for that token, and
+    matches the oracle's dense product."""
+    hip = gpu
+    C, F, rows = 768, 3072, 5
+    rng = np.random.default_rng(17)
+    w = (rng.standard_normal((C, F)) * 0.02).astype(np.float16)
+    if fmt_name == "w8":
+        fmt = hip.FMT_W8
+        q, s = orc.quantize_w8(w)
+        sd = dev(hip, s)
+        wt = hip.DeviceArray((F, C), np.uint8)
+    else:
+        fmt = hip.FMT_F16
+        q, s, sd = w, None, None
+        wt = hip.DeviceArray((F, C), np.float16)
+    hip.cmix_sparse_pack(fmt, C, F, dev(hip, q), wt)
+    pre = rng.standard_normal((rows, F)).astype(np.float16)
+    pre[2] = -np.abs(pre[2])  # a token with no active row at all
+    ws = hip.DeviceArray.zeros((hip.cmix_sparse_workspace(C, F, rows),), np.uint8)
+    out = hip.DeviceArray((rows, C), np.float16)
+    hip.cmix_sparse_down_relu_rows(fmt, rows, C, F, dev(hip, pre), wt, sd, ws, out)
+    hip.device_sync()
+    got = out.numpy()
+    want = orc.gemv(fmt, orc.relu_square(pre), q, s)
+    err = rel_err(got.astype(np.float32), want.astype(np.float32))
+    assert err <= F16_TOL
+    assert not got[2].any()
+    ws1 = hip.DeviceArray.zeros((hip.cmix_sparse_workspace(C, F),), np.uint8)
+    for r in range(rows):
+        one = hip.DeviceArray((1, C), np.float16)
+        hip.cmix_sparse_down_relu_one(fmt, C, F, dev(hip, pre[r]), wt, sd, ws1, one)
+        hip.device_sync()
+        same = np.array_equal(one.numpy().view(np.uint16)[0], got.view(np.uint16)[r])
+        assert same, r
+    with pytest.raises(hip.RwkvHipError):
+        hip.cmix_sparse_down_relu_rows(fmt, 13, C, F, dev(hip, pre), wt, sd, ws, out)  # more rows than the path takes
+    with pytest.raises(hip.RwkvHipError):
+        hip.cmix_sparse_down_relu_rows(fmt, rows, C, F, dev(hip, pre), wt, sd, ws1, out)  # workspace of one row
+
+
 def test_cmix_sparse_rejects_bad_arguments(gpu):
     hip = gpu
     with pytest.raises(hip.RwkvHipError):

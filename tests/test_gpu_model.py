@@ -79,24 +79,24 @@ def test_small_model_prefill_and_decode(gpu, orc, fmt):
     sess.close()
 
 
-@pytest.mark.parametrize("fmt", [0, 1])
-def test_one_sequence_decode_with_row_skipping_ffn_value(gpu, orc, fmt):
-    """Batch-1 decode steps of an fp16 or W8 model use the row-skipping ffn.value product (eager and graph replay): the
-    steps match the oracle, stay within an fp16 ulp of the dense product's logits, and the activations really
-    are sparse (else the test would not exercise the skip)."""
+@pytest.mark.parametrize("fmt,B", [(0, 1), (1, 1), (1, 3)])
+def test_decode_with_row_skipping_ffn_value(gpu, orc, fmt, B):
+    """Decode steps of an fp16 or W8 model with the row-skipping ffn.value product (one row by default, up to 12 by
+    session option; eager and graph replay): the steps match the oracle, stay within an fp16 ulp of the dense
+    product's logits, and the activations really are sparse (else the test would not exercise the skip)."""
     from rwkv_lightning_cuda_amd.model import Session, State
     hip = gpu
     dims = small_dims()
     omodel, gmodel = build_pair(gpu, orc, dims, fmt, seed=33)
     rng = np.random.default_rng(8)
-    prompt = rng.integers(0, dims.V, (1, 6))
-    steps = rng.integers(0, dims.V, (5, 1, 1))
+    prompt = rng.integers(0, dims.V, (B, 6))
+    steps = rng.integers(0, dims.V, (5, B, 1))
     results = {}
     for mode in ("sparse", "dense"):
         sess = Session(gmodel)
-        sess.set_sparse_ffn(mode == "sparse")
-        st = State(dims, 1)
-        lg = hip.DeviceArray((1, dims.V), np.float32)
+        sess.set_sparse_ffn(B if mode == "sparse" else 0)
+        st = State(dims, B)
+        lg = hip.DeviceArray((B, dims.V), np.float32)
         sess.forward(prompt, st, lg)
         outs = []
         for i in range(5):
@@ -104,12 +104,12 @@ def test_one_sequence_decode_with_row_skipping_ffn_value(gpu, orc, fmt):
             sess.forward(steps[i], st, lg)
             outs.append(lg.numpy().copy())
         if mode == "sparse":
-            act = sess.debug_buffer("act", (1, dims.F))
+            act = sess.debug_buffer("act", (B, dims.F))
             frac = float(np.mean(act == 0))
             assert 0.2 <= frac <= 0.8, frac
         results[mode] = (outs, st.wkv.numpy().copy())
         sess.close()
-    ostate = omodel.new_state(1)
+    ostate = omodel.new_state(B)
     omodel.forward(prompt, ostate)
     for i in range(5):
         ol = omodel.forward(steps[i], ostate)
