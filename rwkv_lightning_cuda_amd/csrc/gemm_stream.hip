@@ -356,8 +356,14 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mt][0][v] += acc[mt][1][v];
   }
+  // The X tiles are free after the last barrier.  Group 1 hands its sums to group 0 through them; group 0 then lays
+  // the finished 32*MT x 128 tile out in LDS (rows 136 floats apart: conflict-free for both access patterns) and
+  // all threads write it to memory in 16/32-byte pieces along the rows - the accumulator layout itself would
+  // give 2-byte stores 64 bytes apart.
+  constexpr int kStageLd = 136;
+  float* stage = reinterpret_cast<float*>(xs_all) + (KG == 2 ? MT * 16 * 256 : 0);
+  static_assert((KG == 2 ? MT * 16 * 256 : 0) * 4 + BM * kStageLd * 4 <= KG * 2 * T::kTileHalfs * 2, "epilogue tile exceeds the LDS tiles");
   if constexpr (KG == 2) {
-    // the X tiles are free after the last barrier: group 1 hands its sums to group 0 through them
     float* red = reinterpret_cast<float*>(xs_all);
     if (kg == 1) {
 #pragma unroll
@@ -366,38 +372,47 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
         for (int v = 0; v < 16; ++v) red[(mt * 16 + v) * 256 + tid] = acc[mt][0][v];
     }
     __syncthreads();
-    if (kg == 1) return;
+  }
+  const bool partial_out = g.splits > 1;
+  if (kg == 0) {
+    float scl = 1.0f;
+    if constexpr (FMT == RWKV_FMT_W8) {
+      if (!partial_out) scl = h2f(pr.scale[n]);
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mt][0][v] += red[(mt * 16 + v) * 256 + tid];
-  }
-  if (!active) return;
-
-  float scl = 1.0f;
-  if constexpr (FMT == RWKV_FMT_W8) {
-    if (g.splits == 1) scl = h2f(pr.scale[n]);
-  }
-  float* part_out = g.splits > 1 ? pr.partial + static_cast<int64_t>(split) * g.M * pr.N : nullptr;
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = m0 + mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-      if (row >= g.M) continue;
-      const float sum = acc[mt][0][v];
-      const int64_t o = static_cast<int64_t>(row) * pr.N + n;
-      if (part_out) {
-        part_out[o] = sum;
-      } else {
-        const float val = finish_value(mul_f32(sum, scl), g.epilogue);
-        if (g.out_f32) {
-          static_cast<float*>(pr.y)[o] = val;
-        } else {
-          static_cast<half_t*>(pr.y)[o] = f2h(val);
-        }
+      for (int v = 0; v < 16; ++v) {
+        float sum = acc[mt][0][v];
+        if constexpr (KG == 2) sum += reinterpret_cast<const float*>(xs_all)[(mt * 16 + v) * 256 + tid];
+        const int row = mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        stage[row * kStageLd + wave * 32 + j] = partial_out ? sum : finish_value(mul_f32(sum, scl), g.epilogue);
       }
+  }
+  __syncthreads();
+  float* part_out = partial_out ? pr.partial + static_cast<int64_t>(split) * g.M * pr.N : nullptr;
+  const int col0 = col_block * 128;
+  for (int idx = threadIdx.x; idx < BM * 16; idx += 256 * KG) {
+    const int row = idx >> 4;
+    const int col = col0 + (idx & 15) * 8;
+    if (m0 + row >= g.M || col >= pr.N) continue;
+    const float4_t lo = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + (idx & 15) * 8);
+    const float4_t hi = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + (idx & 15) * 8 + 4);
+    const int64_t o = static_cast<int64_t>(m0 + row) * pr.N + col;
+    if (partial_out || g.out_f32) {
+      float* dst = partial_out ? part_out + o : static_cast<float*>(pr.y) + o;
+      *reinterpret_cast<float4_t*>(dst) = lo;
+      *reinterpret_cast<float4_t*>(dst + 4) = hi;
+    } else {
+      half8_t hv;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        hv[e] = f2h(lo[e]);
+        hv[4 + e] = f2h(hi[e]);
+      }
+      *reinterpret_cast<half8_t*>(static_cast<half_t*>(pr.y) + o) = hv;
     }
+  }
 }
 
 // grid = row tiles x roundup(column blocks of 128 over all problems x splits, 8), one-dimensional; block = 256 * KG.
