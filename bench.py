@@ -232,7 +232,10 @@ def main():
                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                     "frac": flops / (total_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
                                     "kernel": "gemm_stream_kernel (+ split-K reduce), M = %d rows" % rows,
-                                    "launches": launches, "sum_launch_ms": total_ms}
+                                    "launches": launches, "sum_launch_ms": total_ms,
+                                    # at M = 128 the launches are weight-streaming bound: the same time against HBM
+                                    "weights_gb_s": model.weight_bytes() / (total_ms * 1e-3) / 1e9,
+                                    "hbm_frac": model.weight_bytes() / (total_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
     first = rng.integers(0, dims.V, (B,))
 
     if args.warmup > 0:
