@@ -553,10 +553,11 @@ def _quant_parts(orc, hip, fmt, w):
 
 @pytest.mark.parametrize("fmt_name", ["f16", "w8", "w4"])
 @pytest.mark.parametrize("M,N,K", [(16, 128, 512), (33, 96, 256), (64, 256, 1024), (128, 160, 2048), (200, 64, 768),
-                                   (17, 4096, 256)])
+                                   (17, 4096, 256), (64, 128, 2560), (600, 256, 1024), (1030, 96, 512)])
 def test_linear_packed_matches_oracle(gpu, orc, fmt_name, M, N, K):
-    """Every row-tile variant (M <= 32, <= 64, > 64, several row tiles), with and without K splits, ragged M and
-    a column count that is not a multiple of the 128-column block."""
+    """Every tile variant (32-, 64- and 128-row tiles; one and two wavefront groups; several row tiles), with and
+    without K splits, chunk counts that are not a power of two, ragged M and a column count that is not a multiple
+    of the 128-column block."""
     hip = gpu
     if fmt_name == "w4" and K % 128:
         pytest.skip("W4 groups are 128 wide")
