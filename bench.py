@@ -12,7 +12,7 @@ whole-job tokens/s plus
                   launch / average launch duration from HIP events on the session stream
   cpu_baseline -- the scalar C++ oracle timed on the host cores on a bounded slice of the same workload
   also         -- the other figures the metric names, measured in the same run: prefill tokens/s of the
-                  4096-token prompt (and the MFMA fraction of its GEMM launches), batch-16 and batch-64 decode tokens/s,
+                  4096-token prompt (and the MFMA fraction of its GEMM launches), batch-8, -16 and -64 decode tokens/s,
                   batch-1 decode with int4 weights,
                   and the WKV7 op alone on a long sequence.
 """
@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--prefill", type=int, default=4096, help="tokens prefilled (chunk 128) before the decode loop")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary measurements (prefill MFMA fraction, "
-                    "batch-16/64 decode, W4 decode, WKV7 op)")
+                    "batch-8/16/64 decode, W4 decode, WKV7 op)")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps eagerly instead of replaying a HIP graph")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run a device-to-device copy of BYTES (twice) and exit: the known-size kernel that "
@@ -122,10 +122,10 @@ def cpu_baseline(dims, fmt_name):
 
 
 def secondary_measurements(hip, model, dims, rng):
-    """Batch-64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7 op alone."""
+    """Batch-8, -16 and -64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7 op alone."""
     from rwkv_lightning_cuda_amd.model import Session, State
     res = {}
-    for B in (16, 64):
+    for B in (8, 16, 64):
         sess = Session(model)
         state = State(dims, B)
         logits = hip.DeviceArray((B, dims.V), np.float32)

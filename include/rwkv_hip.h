@@ -268,8 +268,8 @@ int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double
  * only while rows x (fraction of non-zero activations) stays below 1 - about half the activations are
  * non-zero with random-init weights, far fewer with trained ones.  0 selects the dense product. */
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
-/* Decode steps of up to 8 rows can fold the two LayerNorm + token-shift kernels of a layer into the prologue of
- * the linear launches that consume them (bitwise the same results).  Off by default: on this chip the extra
+/* Decode steps on the GEMV path (one or two rows) can fold the two LayerNorm + token-shift kernels of a layer
+ * into the prologue of the linear launches that consume them (bitwise the same results).  Off by default: on this chip the extra
  * work inside every GEMV block costs more than the two small launches it saves.  No counterpart in the
  * reference. */
 int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on);

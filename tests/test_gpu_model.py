@@ -410,9 +410,10 @@ def test_config3_7p2b_width_two_layers_quantised(gpu, orc, fmt_name):
     sess.close()
 
 
-@pytest.mark.parametrize("B", [1, 3, 8])
+@pytest.mark.parametrize("B", [1, 2])
 def test_decode_step_with_layernorm_folded_into_linear_is_bitwise_the_unfused_step(gpu, B):
-    """Decode steps of up to 8 rows can compute LayerNorm + token shift inside the linear kernels' prologue
+    """Decode steps on the GEMV path (one or two rows) can compute LayerNorm + token shift inside the linear
+    kernels' prologue
     (session option, off by default) instead of the stand-alone kernels.  Same arithmetic and reduction order:
     logits, shift rows and WKV state must be bit-identical, step after step."""
     from rwkv_lightning_cuda_amd.model import HipModel, Session, State, synth_weights
