@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void wkv7_prepare_kernel(int64_t n, int64_t sl
 }
 
 // ---- sequence kernel -------------------------------------------------------------------------
-// grid = B*H, block = 1024/RPL threads: 16/RPL wavefronts per head, RPL = 4 or 2 state rows per lane.  Lane
+// grid = B*H, block = 1024/RPL threads: 16/RPL wavefronts per head, RPL = 4, 2 or 1 state rows per lane.  Lane
 // (g, c) = (lane / 16, lane % 16) of wavefront q owns rows 4*RPL*q + RPL*g .. +RPL-1 and columns 4c .. 4c+3, so
 // the 16 lanes of one DPP row hold complete state rows and the wavefronts never exchange data.  r,d,k,a,b are
 // fp32 with `op_bs` elements between batch rows; v,y are IO with `io_bs` elements between batch rows.  The
@@ -51,9 +51,9 @@ __global__ __launch_bounds__(256) void wkv7_prepare_kernel(int64_t n, int64_t sl
 // loads of chunk c+1 are in flight while chunk c computes); a step costs each lane six LDS reads (its four
 // columns of the five operands and its v values) against 28*RPL VALU operations.  y goes back through LDS so
 // that the global stores are coalesced.  The arithmetic of a state element does not depend on RPL or on the
-// chunking: every variant and every split of T over several calls gives bitwise the same result.  RPL = 2
-// halves the serial work per token of a wavefront and is used while the grid is small enough to leave CUs
-// idle; RPL = 4 reads each operand half as often.
+// chunking: every variant and every split of T over several calls gives bitwise the same result.  Smaller RPL
+// means less serial work per token and wavefront and is used while the grid is small enough to leave SIMDs
+// idle (RPL = 1 up to 64 heads, 2 up to 128); RPL = 4 reads each operand least often.
 constexpr int kSeqChunk = 8;
 
 template <int CTRL>
@@ -128,9 +128,9 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
     }
 #pragma unroll
     for (int i = 0; i < kVSlots; ++i) {
-      const int t = t0 + ((tid + i * NT) >> 6);
+      const int tok = (tid + i * NT) >> 6;
       v_stage[i] = 0.0f;
-      if (t < T) v_stage[i] = static_cast<float>(v[iob + static_cast<int64_t>(t) * C + lane]);
+      if (tok < kSeqChunk && t0 + tok < T) v_stage[i] = static_cast<float>(v[iob + static_cast<int64_t>(t0 + tok) * C + lane]);
     }
   };
   auto commit = [&](int buf) {
@@ -138,7 +138,10 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
     for (int i = 0; i < kOpSlots; ++i)
       if (st_dst[i] >= 0) *reinterpret_cast<float4_t*>(&ops[buf][0][0][0] + st_dst[i]) = stage[i];
 #pragma unroll
-    for (int i = 0; i < kVSlots; ++i) vs[buf][(tid + i * NT) >> 6][lane] = v_stage[i];
+    for (int i = 0; i < kVSlots; ++i) {
+      const int tok = (tid + i * NT) >> 6;
+      if (tok < kSeqChunk) vs[buf][tok][lane] = v_stage[i];
+    }
   };
 
   request(0);
@@ -226,13 +229,17 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
   for (int i = 0; i < RPL; ++i) *reinterpret_cast<float4_t*>(sblk + i * kHead) = S[i];
 }
 
-// Heads in flight below which the chip has idle CUs with four wavefronts per head.
+// Heads in flight below which the chip has idle SIMDs with four (eight) wavefronts per head.
 constexpr int kSeqSmallGrid = 128;
+constexpr int kSeqTinyGrid = 64;
 
 template <typename IO>
 static void launch_seq(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                        const float* k, const float* a, const float* b, int64_t op_bs, const IO* v, IO* y, int64_t io_bs) {
-  if (B * H <= kSeqSmallGrid && T > 1) {
+  if (B * H <= kSeqTinyGrid && T > 1) {
+    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 1>), dim3(B * H), dim3(1024), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
+                       io_bs);
+  } else if (B * H <= kSeqSmallGrid && T > 1) {
     hipLaunchKernelGGL((wkv7_seq_kernel<IO, 2>), dim3(B * H), dim3(512), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
                        io_bs);
   } else {

@@ -77,16 +77,16 @@ def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):
 
 
 def test_wkv7_small_and_large_grids_agree_bitwise(gpu):
-    """Small grids run with eight wavefronts per head, large ones with four; a state element sees the same
-    arithmetic either way, so the same sequence gives bitwise the same outputs and state inside a batch of 1
-    and inside a batch of 70."""
+    """Grids of up to 64 heads run with sixteen wavefronts per head, up to 128 with eight, larger ones with four;
+    a state element sees the same arithmetic in each, so the same sequence gives bitwise the same outputs and
+    state inside a batch of 1, of 40 and of 70 (two heads each)."""
     hip = gpu
     T, H = 37, 2
     C = H * 64
     one = wkv_inputs(1, T, H, seed=5, dtype=np.float16)
     names = ["r", "w_raw", "k", "v", "a", "b"]
     outs = []
-    for B in (1, 70):
+    for B in (1, 40, 70):
         rng = np.random.default_rng(B)
         full = {n: np.concatenate([one[n]] + [rng.permutation(one[n].reshape(-1)).reshape(one[n].shape)
                                               for _ in range(B - 1)], axis=0) for n in names}
@@ -96,10 +96,11 @@ def test_wkv7_small_and_large_grids_agree_bitwise(gpu):
         hip.wkv7(B, T, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state, *[d[n] for n in names], y)
         hip.device_sync()
         outs.append((y.numpy()[0].copy(), state.numpy()[0].copy()))
-    same = np.array_equal(outs[0][0].view(np.uint16), outs[1][0].view(np.uint16))
-    assert same
-    same = np.array_equal(outs[0][1].view(np.uint32), outs[1][1].view(np.uint32))
-    assert same
+    for other in outs[1:]:
+        same = np.array_equal(outs[0][0].view(np.uint16), other[0].view(np.uint16))
+        assert same
+        same = np.array_equal(outs[0][1].view(np.uint32), other[1].view(np.uint32))
+        assert same
 
 
 # ------------------------------------------------------------------------------------------- formats
