@@ -44,7 +44,7 @@ class ModelDims:
                 "ffn_value": (C, F), "head": (V, C)}[name]
 
 
-# Shapes of BASELINE.json's configs.  LoRA ranks (w, a, v, g): 0.1B as given there; the larger
+# Shapes of the benchmark configurations.  LoRA ranks (w, a, v, g): 0.1B as given there; the larger
 # ones follow the upstream RWKV-7 convention.
 PRESETS = {
     "0.1B": ModelDims(L=12, C=768, H=12, F=3072, V=65536, Rw=64, Ra=64, Rg=128, Rv=32),

@@ -647,7 +647,7 @@ def test_linear_packed_rejects_bad_arguments(gpu):
 
 
 def test_wkv7_long_chunked_resume_through_host_slab_is_bitwise(gpu):
-    """BASELINE config 4 at reduced size: fp16 r,w,k,v,a,b, fp32 state, sequence run in chunks of 128 with the state
+    """Benchmark configuration 4 at reduced size: fp16 r,w,k,v,a,b, fp32 state, sequence run in chunks of 128 with the state
     slab copied to the host and into a fresh device buffer at every quarter; outputs and final state must equal
     the single uninterrupted call bit for bit."""
     hip = gpu

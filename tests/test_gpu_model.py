@@ -243,7 +243,7 @@ def test_forward_argument_errors(gpu, orc):
 
 
 def test_config1_0p1b_prefill_512_then_128_greedy_steps(gpu, orc):
-    """BASELINE config 1: 0.1B shape, fp16 weights N(0, 0.02), 512 random tokens prefilled in chunks of 128, then
+    """Benchmark configuration 1: 0.1B shape, fp16 weights N(0, 0.02), 512 random tokens prefilled in chunks of 128, then
     128 greedy steps at batch 1.  The greedy token stream must equal the oracle's (up to exact ties), the logits after the prompt
     and after the last step must agree (cosine >= 0.9995), the fp32 WKV state within 2e-3 of its scale."""
     from rwkv_lightning_cuda_amd.model import PRESETS, HipModel, Session, State, synth_weights
@@ -301,7 +301,7 @@ def test_config1_0p1b_prefill_512_then_128_greedy_steps(gpu, orc):
 
 @pytest.mark.parametrize("B", [1, 8, 64])
 def test_config2_1p5b_width_w8_decode_batches(gpu, orc, B):
-    """BASELINE config 2 at full width (C 2048, H 32, F 8192, LoRA ranks 96/96/256/64; two layers, reduced
+    """Benchmark configuration 2 at full width (C 2048, H 32, F 8192, LoRA ranks 96/96/256/64; two layers, reduced
     vocabulary), W8A16 quantised on load: per-sequence state from a random prefill (48 tokens in chunks of 16; 16
     tokens at batch 64 to bound the oracle's time),
     then decode steps at batch 1 (GEMV + row-skipping ffn.value), 8 (GEMV, fused time-mix step) and 64
@@ -351,7 +351,7 @@ def test_config2_1p5b_width_w8_decode_batches(gpu, orc, B):
 
 @pytest.mark.parametrize("fmt_name", ["w8", "w4"])
 def test_config3_7p2b_width_two_layers_quantised(gpu, orc, fmt_name):
-    """BASELINE config 3 at full width (C 4096, H 64, F 16384, LoRA ranks 128/128/480/96) with two layers and a
+    """Benchmark configuration 3 at full width (C 4096, H 64, F 16384, LoRA ranks 128/128/480/96) with two layers and a
     reduced vocabulary, W8A16 and W4A16 quantised from the same fp16 weights on both sides: one prefill call of
     2 x 16 tokens (streaming MFMA GEMM, row-tiled time-mix kernels) and decode steps at batch 2 (GEMV, fused
     time-mix kernel), per-layer residual streams and logits against the oracle."""
