@@ -479,8 +479,16 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         TRY_AUX(lora_out_multi(st, a));
       }
 
-      // kk normalise, a-gate, decay; operands widened to fp32 for the scalar-fed WKV kernel
-      {
+      if (!s->trace && tmix_seq_whole_heads(B, T, H)) {
+        // kk normalise / a-gate / decay, the WKV recurrence and GroupNorm / bonus / gate in one launch
+        TmixSeqArgs fa;
+        fa.r = b.r; fa.k = b.k; fa.a12 = b.a12; fa.w12 = b.w12; fa.g = b.g;
+        fa.k_k = w.t[RWKV_T_K_K]; fa.a0 = w.t[RWKV_T_A0]; fa.k_a = w.t[RWKV_T_K_A]; fa.w0 = w.t[RWKV_T_W0];
+        fa.r_k = w.t[RWKV_T_R_K]; fa.lnx_w = w.t[RWKV_T_LNX_W]; fa.lnx_b = w.t[RWKV_T_LNX_B];
+        TRY_AUX(tmix_seq_launch(st, B, T, C, H, S, fa, v_cur, b.y2));
+      } else {
+        // with the residual-stream tap on, or few heads in flight: the three stand-alone kernels (same arithmetic,
+        // bitwise the same)
         KkArgs p = {};
         p.k = b.k; p.k_k = w.t[RWKV_T_K_K]; p.a0 = w.t[RWKV_T_A0]; p.a12 = b.a12; p.k_a = w.t[RWKV_T_K_A];
         p.new_k = b.k2; p.neg_kk = nullptr; p.kka = nullptr;
@@ -488,11 +496,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         p.k32 = b.k32; p.a32 = b.a32; p.b32 = b.b32; p.d32 = b.d32; p.r32 = b.r32;
         p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
         TRY_AUX(kk_a_gate_launch(st, p));
+        TRY_AUX(wkv7_seq_f16_launch(st, B, T, C, H, S, b.r32, b.d32, b.k32, b.a32, b.b32, static_cast<int64_t>(T) * C, v_cur,
+                                b.y, static_cast<int64_t>(T) * C));
+        TRY_AUX(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
+                       w.t[RWKV_T_LNX_B], b.g, b.y2));
       }
-      TRY_AUX(wkv7_seq_f16_launch(st, B, T, C, H, S, b.r32, b.d32, b.k32, b.a32, b.b32, static_cast<int64_t>(T) * C, v_cur,
-                              b.y, static_cast<int64_t>(T) * C));
-      TRY_AUX(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
-                     w.t[RWKV_T_LNX_B], b.g, b.y2));
     }
     // From 16 rows on (the streaming GEMM) the LayerNorm kernels that consume the output projection and
     // ffn.value sum the split-K partials themselves instead of a reduce launch; att / cm then stay unwritten.

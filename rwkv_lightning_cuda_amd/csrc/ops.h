@@ -195,6 +195,17 @@ int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out);
 // ---- wkv7.hip -----------------------------------------------------------------------------------
 // T tokens of the recurrence from fp32 operands (decay applied); v, y fp16.  op_bs / io_bs: elements
 // between batch rows of the operand / io tensors.
+// The model's row-tiled time-mix pass in one launch: kk normalise / a-gate / decay while staging, the WKV recurrence,
+// then per-head GroupNorm + (r.k.r_k) v bonus + gate on the way out.  All fp16 tensors [B,T,C] contiguous.
+struct TmixSeqArgs {
+  const half_t *r, *k, *a12, *w12, *g;
+  const half_t *k_k, *a0, *k_a, *w0, *r_k, *lnx_w, *lnx_b;  // [C]
+};
+int tmix_seq_launch(hipStream_t st, int B, int T, int C, int H, float* state, const TmixSeqArgs& fa, const half_t* v,
+                    half_t* y2);
+// false: few heads in flight and more than one token - the stand-alone kernels are faster there (the recurrence
+// then runs a head's row ranges on separate CUs, which the fused pass cannot: its GroupNorm needs whole heads)
+bool tmix_seq_whole_heads(int B, int T, int H);
 int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                         const float* k, const float* a, const float* b, int64_t op_bs, const half_t* v, half_t* y,
                         int64_t io_bs);

@@ -9,6 +9,7 @@
 // each lane reads only the four columns it owns; the two row sums of a step (sa and y) are reduced over the 16
 // lanes that share a row with DPP adds.  Operands must therefore be fp32 with the decay already applied; a small
 // element-wise pre-pass produces them when the caller passes fp16 tensors or raw decay logits.
+#include <type_traits>
 #include "ops.h"
 
 namespace rwkv {
@@ -71,14 +72,25 @@ __device__ __forceinline__ float row16_sum(float x) {
   return x;
 }
 
-template <typename IO, int RPL>
-__global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
+// FUSED (the model's row-tiled time-mix path, fp16 io): the operands are not read as fp32 tensors but derived
+// while staging from the fp16 rows r, k, a12, w12 - the arithmetic of kk_a_gate_kernel, one wavefront per token,
+// lane = channel - and y is not stored but taken through the per-head GroupNorm, the (r.k.r_k) v bonus and the
+// gate - the arithmetic of lnx_rkvres_xg_kernel on the fp16-rounded y - so that three launches and the fp32
+// operand tensors between them become one launch.  Bitwise the same results as the three kernels.
+//
+// PARTS > 1: the rows of a head's state are independent of each other (row i needs only its own sum over the
+// columns, v_i and the per-column operands), so a head is cut into PARTS row ranges that run as separate blocks on
+// separate CUs - with few heads in flight the step is bound by one CU's VALU rate, not by memory.  Not with FUSED
+// (the GroupNorm needs the whole head's y).  Same lanes, same rows, same arithmetic: bitwise the same results.
+template <typename IO, int RPL, int PARTS, bool FUSED>
+__global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
                                                               const float* __restrict__ r, const float* __restrict__ d,
                                                               const float* __restrict__ k, const float* __restrict__ a,
                                                               const float* __restrict__ b, int64_t op_bs,
                                                               const IO* __restrict__ v, IO* __restrict__ y,
-                                                              int64_t io_bs) {
-  constexpr int NT = 1024 / RPL;
+                                                              int64_t io_bs, TmixSeqArgs fa) {
+  static_assert(PARTS == 1 || !FUSED, "the fused pass needs whole heads");
+  constexpr int NT = 1024 / RPL / PARTS;
   constexpr int kOpVecs = 5 * kSeqChunk * (kHead / 4);         // float4 of operands per chunk
   constexpr int kOpSlots = (kOpVecs + NT - 1) / NT;
   constexpr int kVSlots = (kSeqChunk * kHead + NT - 1) / NT;
@@ -86,13 +98,17 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
   __shared__ __align__(16) float ops[2][kSeqChunk][5][kHead];  // [buffer][token][a,b,d,k,r][column]
   __shared__ __align__(16) float vs[2][kSeqChunk][kHead];      // [buffer][token][row]
   __shared__ __align__(16) float ys[2][kSeqChunk][kHead];
+  __shared__ __align__(16) float spare[NT * RPL];
+  __shared__ __align__(16) float gs[FUSED ? 2 : 1][FUSED ? kSeqChunk : 1][kHead];  // FUSED: the gate rows
 
-  const int bh = blockIdx.x;
+  const int bh = blockIdx.x / PARTS;
+  const int part = blockIdx.x % PARTS;
   const int bi = bh / H;
   const int h = bh - bi * H;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int i0 = 4 * RPL * (tid >> 6) + RPL * (lane >> 4);  // first of this lane's rows
+  const int row_lo = part * (kHead / PARTS);                         // this block's rows
+  const int i0 = row_lo + 4 * RPL * (tid >> 6) + RPL * (lane >> 4);  // first of this lane's rows
   const int j0 = 4 * (lane & 15);                           // first of its 4 columns
   float* sblk = state + (static_cast<int64_t>(bh) * kHead + i0) * kHead + j0;
 
@@ -104,6 +120,7 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
   const int64_t iob = static_cast<int64_t>(bi) * io_bs + h * kHead;
   // staging slot i of thread t: float4 number t + i*NT of the chunk = (operand, token, 4 columns)
   const float* st_src[kOpSlots];
+  int st_tok[kOpSlots];
   int st_dst[kOpSlots];  // offset inside ops[buf], -1: slot unused
 #pragma unroll
   for (int i = 0; i < kOpSlots; ++i) {
@@ -112,45 +129,118 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
     const int tok = (idx >> 4) % kSeqChunk;
     const int col = (idx & 15) * 4;
     const float* src = o == 0 ? a : (o == 1 ? b : (o == 2 ? d : (o == 3 ? k : r)));
-    st_src[i] = src + base + static_cast<int64_t>(tok) * C + col;
+    st_src[i] = src + base + col;
+    st_tok[i] = tok;
     st_dst[i] = idx < kOpVecs ? (tok * 5 + o) * kHead + col : -1;
   }
 
-  float4_t stage[kOpSlots];
-  float v_stage[kVSlots];
+  // Two sets of staging registers: a chunk is requested two chunks before it is needed - eight steps are shorter
+  // than a trip to memory.
+  float4_t stage[2][kOpSlots];
+  float v_stage[2][kVSlots];
+  // FUSED: raw fp16 values of this thread's (token, channel) slots: r, k, a12, w12, g; and its channel's constants
+  half_t raw[2][kVSlots][5];
+  float c_kk = 0.0f, c_a0 = 0.0f, c_ka = 0.0f, c_w0 = 0.0f, c_rk = 0.0f, c_lnw = 0.0f, c_lnb = 0.0f;
+  if constexpr (FUSED) {
+    const int c = h * kHead + lane;
+    c_kk = h2f(fa.k_k[c]); c_a0 = h2f(fa.a0[c]); c_ka = h2f(fa.k_a[c]); c_w0 = h2f(fa.w0[c]);
+    c_rk = h2f(fa.r_k[c]); c_lnw = h2f(fa.lnx_w[c]); c_lnb = h2f(fa.lnx_b[c]);
+  }
 
-  auto request = [&](int t0) {
+  // Every load is issued unconditionally (tokens past the end repeat the last one; their steps never run): a load
+  // under a branch makes the compiler's s_waitcnt accounting wait for everything in flight, the younger set too.
+  auto request = [&](int t0, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
+    if constexpr (!FUSED) {
 #pragma unroll
-    for (int i = 0; i < kOpSlots; ++i) {
-      const int tok = ((tid + i * NT) >> 4) % kSeqChunk;
-      stage[i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-      if (st_dst[i] >= 0 && t0 + tok < T) stage[i] = *reinterpret_cast<const float4_t*>(st_src[i] + static_cast<int64_t>(t0) * C);
+      for (int i = 0; i < kOpSlots; ++i) {
+        stage[set][i] = *reinterpret_cast<const float4_t*>(st_src[i] + static_cast<int64_t>(min(t0 + st_tok[i], T - 1)) * C);
+      }
     }
 #pragma unroll
     for (int i = 0; i < kVSlots; ++i) {
-      const int tok = (tid + i * NT) >> 6;
-      v_stage[i] = 0.0f;
-      if (tok < kSeqChunk && t0 + tok < T) v_stage[i] = static_cast<float>(v[iob + static_cast<int64_t>(t0 + tok) * C + lane]);
+      const int tok = min((tid + i * NT) >> 6, kSeqChunk - 1);
+      const int64_t at = iob + static_cast<int64_t>(min(t0 + tok, T - 1)) * C + lane;
+      v_stage[set][i] = static_cast<float>(v[at]);
+      if constexpr (FUSED) {
+        raw[set][i][0] = fa.r[at]; raw[set][i][1] = fa.k[at]; raw[set][i][2] = fa.a12[at]; raw[set][i][3] = fa.w12[at];
+        raw[set][i][4] = fa.g[at];
+      }
     }
   };
-  auto commit = [&](int buf) {
+  auto commit = [&](int buf, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
+    if constexpr (!FUSED) {
 #pragma unroll
-    for (int i = 0; i < kOpSlots; ++i)
-      if (st_dst[i] >= 0) *reinterpret_cast<float4_t*>(&ops[buf][0][0][0] + st_dst[i]) = stage[i];
+      for (int i = 0; i < kOpSlots; ++i)
+        if (st_dst[i] >= 0) *reinterpret_cast<float4_t*>(&ops[buf][0][0][0] + st_dst[i]) = stage[set][i];
+    }
 #pragma unroll
     for (int i = 0; i < kVSlots; ++i) {
-      const int tok = (tid + i * NT) >> 6;
-      if (tok < kSeqChunk) vs[buf][tok][lane] = v_stage[i];
+      const int tok = (tid + i * NT) >> 6;  // wave-uniform: one wavefront per token, lane = channel
+      if (tok < kSeqChunk) {
+        vs[buf][tok][lane] = v_stage[set][i];
+        if constexpr (FUSED) {
+          // kk normalise, a-gate, new k, decay: the statements of kk_a_gate_kernel
+          const float kv = h2f(raw[set][i][1]);
+          const float u = kv * c_kk;
+          const float total = wave_sum(u * u);
+          const float inv = 1.0f / fmaxf(sqrtf(total), kKkEps);
+          const float kk = u * inv;
+          const float av = sigmoid_f(c_a0 + h2f(raw[set][i][2]));
+          const half_t nk = f2h(kv * fmaf(av, c_ka, 1.0f - c_ka));
+          const half_t nkk = f2h(-kk);
+          const half_t kka = f2h(kk * av);
+          const float wraw = round_h(h2f(raw[set][i][3]) + c_w0);
+          ops[buf][tok][0][lane] = h2f(nkk);
+          ops[buf][tok][1][lane] = h2f(kka);
+          ops[buf][tok][2][lane] = exp2f(-0.8750387749145276f / (1.0f + exp2f(-1.4426950408889634f * wraw)));
+          ops[buf][tok][3][lane] = h2f(nk);
+          ops[buf][tok][4][lane] = h2f(raw[set][i][0]);
+          gs[buf][tok][lane] = h2f(raw[set][i][4]);
+        }
+      }
     }
   };
 
-  request(0);
-  commit(0);
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  request(0, Set0{});
+  if (T > kSeqChunk) request(kSeqChunk, Set1{});
+  commit(0, Set0{});
   __syncthreads();
-  for (int t0 = 0; t0 < T; t0 += kSeqChunk) {
-    const int buf = (t0 / kSeqChunk) & 1;
+  // The y rows of a finished chunk (tokens t0 .. t0+n-1, LDS buffer buf) go to memory: one wavefront per token,
+  // lane = channel.  It runs in the middle of the next chunk, where its LDS and memory latencies hide behind the
+  // steps; ys[buf] is next written a barrier later.  FUSED also reads the chunk's operand, v and gate rows: each
+  // thread reads exactly the (token, channel) slots that it overwrites itself in the commit that follows.
+  auto write_out = [&](int t0, int n, int buf) {
+#pragma unroll
+    for (int i = 0; i < kVSlots; ++i) {
+      const int tt = (tid + i * NT) >> 6;
+      if (tt < n) {
+        if constexpr (FUSED) {
+          // GroupNorm over the head, (r.k.r_k) v bonus, gate: the statements of lnx_rkvres_xg_kernel on the
+          // fp16-rounded y
+          const float yv = round_h(ys[buf][tt][lane]);
+          const float mean = wave_sum(yv) * (1.0f / 64.0f);
+          const float dd = yv - mean;
+          const float var = wave_sum(dd * dd) * (1.0f / 64.0f);
+          const float rstd = rsqrtf(var + kLnxEps);
+          const float rkv = wave_sum(ops[buf][tt][4][lane] * ops[buf][tt][3][lane] * c_rk);
+          const float o = (dd * rstd * c_lnw + c_lnb + rkv * vs[buf][tt][lane]) * gs[buf][tt][lane];
+          y[iob + static_cast<int64_t>(t0 + tt) * C + lane] = static_cast<IO>(o);
+        } else if (PARTS == 1 || (lane >= row_lo && lane < row_lo + kHead / PARTS)) {
+          y[iob + static_cast<int64_t>(t0 + tt) * C + lane] = static_cast<IO>(ys[buf][tt][lane]);
+        }
+      }
+    }
+  };
+  // chunk c: LDS buffer c&1, staging set c&1 - both static inside the two-chunk body
+  auto run_chunk = [&](int t0, auto set_c) {
+    constexpr int buf = decltype(set_c)::value;
+    using Other = std::integral_constant<int, 1 - buf>;
     const bool more = t0 + kSeqChunk < T;
-    if (more) request(t0 + kSeqChunk);
+    request(t0 + 2 * kSeqChunk, set_c);  // this chunk's set was committed a chunk ago
     const int n = min(kSeqChunk, T - t0);
     struct StepOps {
       float4_t av, bv, dv, kv, rv;
@@ -164,10 +254,11 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
       q.rv = *reinterpret_cast<const float4_t*>(&ops[buf][tt][4][j0]);
       q.vv = *reinterpret_cast<const rows_t*>(&vs[buf][tt][i0]);
     };
-    auto step = [&](int tt, const StepOps& q) {
-      const float4_t av = q.av, bv = q.bv, dv = q.dv, kv = q.kv, rv = q.rv;
+    // A step in two halves.  step_state carries the recurrence: row sums of S a, then the update - the only chain
+    // from one token to the next.  step_out reads the new state: y = S r.
+    auto step_state = [&](const StepOps& q) {
+      const float4_t av = q.av, bv = q.bv, dv = q.dv, kv = q.kv;
       float sa[RPL];
-      rows_t yy;
 #pragma unroll
       for (int i = 0; i < RPL; ++i) {
         float p = S[i].x * av.x;
@@ -185,6 +276,13 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
         S[i].y = fmaf(S[i].y, dv.y, fmaf(sa[i], bv.y, kv.y * vi));
         S[i].z = fmaf(S[i].z, dv.z, fmaf(sa[i], bv.z, kv.z * vi));
         S[i].w = fmaf(S[i].w, dv.w, fmaf(sa[i], bv.w, kv.w * vi));
+      }
+    };
+    auto step_out = [&](int tt, const StepOps& q) {
+      const float4_t rv = q.rv;
+      rows_t yy;
+#pragma unroll
+      for (int i = 0; i < RPL; ++i) {
         float p = S[i].x * rv.x;
         p = fmaf(S[i].y, rv.y, p);
         p = fmaf(S[i].z, rv.z, p);
@@ -193,19 +291,28 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
       }
 #pragma unroll
       for (int i = 0; i < RPL; ++i) yy[i] = row16_sum(yy[i]);
-      if ((lane & 15) == 0) *reinterpret_cast<rows_t*>(&ys[buf][tt][i0]) = yy;
+      // the 16 lanes of a row hold the same sums: the first stores them, the others store to a spare area - a
+      // store under a branch would end the scheduling region here
+      float* dst = (lane & 15) == 0 ? &ys[buf][tt][i0] : &spare[tid * RPL];
+      *reinterpret_cast<rows_t*>(dst) = yy;
     };
     if (n == kSeqChunk) {
-      // Full chunk, straight-line: the operands of step tt+1 are read while step tt computes;
-      // __builtin_amdgcn_sched_barrier(0) keeps the scheduler from sinking the reads down to their first use.
+      // Full chunk, straight-line.  The operands of step tt+1 are read from LDS while step tt computes, and the
+      // scheduling regions run from the middle of one step to the middle of the next
+      // (__builtin_amdgcn_sched_barrier(0) between the halves), so that the compiler fills the latency bubbles
+      // of step tt's output sums with the independent recurrence half of step tt+1.
       StepOps q[2];
       load_step(0, q[0]);
 #pragma unroll
       for (int tt = 0; tt < kSeqChunk; ++tt) {
         if (tt + 1 < kSeqChunk) load_step(tt + 1, q[(tt + 1) & 1]);
+        step_state(q[tt & 1]);
         __builtin_amdgcn_sched_barrier(0);
-        step(tt, q[tt & 1]);
-        __builtin_amdgcn_sched_barrier(0);
+        step_out(tt, q[tt & 1]);
+        if (tt == kSeqChunk / 2 - 1) {
+          if (t0 > 0) write_out(t0 - kSeqChunk, kSeqChunk, buf ^ 1);
+          if (more) commit(buf ^ 1, Other{});
+        }
       }
     } else {
       // the last, partial chunk (and single-token calls): same step arithmetic, rolled loop
@@ -213,39 +320,50 @@ __global__ __launch_bounds__(1024 / RPL) void wkv7_seq_kernel(int T, int C, int 
       for (int tt = 0; tt < n; ++tt) {
         StepOps q;
         load_step(tt, q);
-        step(tt, q);
+        step_state(q);
+        step_out(tt, q);
       }
+      if (t0 > 0) write_out(t0 - kSeqChunk, kSeqChunk, buf ^ 1);  // (nothing follows a partial chunk: no commit)
     }
-    if (more) commit(buf ^ 1);
     __syncthreads();
-#pragma unroll
-    for (int i = 0; i < kVSlots; ++i) {
-      const int tt = (tid + i * NT) >> 6;
-      if (tt < n) y[iob + static_cast<int64_t>(t0 + tt) * C + lane] = static_cast<IO>(ys[buf][tt][lane]);
-    }
+  };
+  for (int t0 = 0; t0 < T; t0 += 2 * kSeqChunk) {
+    run_chunk(t0, Set0{});
+    if (t0 + kSeqChunk < T) run_chunk(t0 + kSeqChunk, Set1{});
   }
+  const int t_last = (T - 1) / kSeqChunk * kSeqChunk;
+  write_out(t_last, T - t_last, (t_last / kSeqChunk) & 1);
 
 #pragma unroll
   for (int i = 0; i < RPL; ++i) *reinterpret_cast<float4_t*>(sblk + i * kHead) = S[i];
 }
 
-// Heads in flight below which the chip has idle SIMDs with four (eight) wavefronts per head.
+// Heads in flight up to which a head is cut into four (two) row ranges of four wavefronts each, one block per
+// range; above, one block of four wavefronts per head fills the chip.  Single-token calls move a head's state once
+// and are bound by that traffic: whole heads.
 constexpr int kSeqSmallGrid = 128;
 constexpr int kSeqTinyGrid = 64;
 
-template <typename IO>
+bool tmix_seq_whole_heads(int B, int T, int H) { return !(B * H <= kSeqSmallGrid && T > 1); }
+
+template <typename IO, bool FUSED>
 static void launch_seq(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
-                       const float* k, const float* a, const float* b, int64_t op_bs, const IO* v, IO* y, int64_t io_bs) {
-  if (B * H <= kSeqTinyGrid && T > 1) {
-    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 1>), dim3(B * H), dim3(1024), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
-                       io_bs);
-  } else if (B * H <= kSeqSmallGrid && T > 1) {
-    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 2>), dim3(B * H), dim3(512), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
-                       io_bs);
-  } else {
-    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs, v, y,
-                       io_bs);
+                       const float* k, const float* a, const float* b, int64_t op_bs, const IO* v, IO* y, int64_t io_bs,
+                       const TmixSeqArgs& fa) {
+  if constexpr (!FUSED) {
+    if (B * H <= kSeqTinyGrid && T > 1) {
+      hipLaunchKernelGGL((wkv7_seq_kernel<IO, 1, 4, false>), dim3(B * H * 4), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
+                         op_bs, v, y, io_bs, fa);
+      return;
+    }
+    if (B * H <= kSeqSmallGrid && T > 1) {
+      hipLaunchKernelGGL((wkv7_seq_kernel<IO, 2, 2, false>), dim3(B * H * 2), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
+                         op_bs, v, y, io_bs, fa);
+      return;
+    }
   }
+  hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, FUSED>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs,
+                     v, y, io_bs, fa);
 }
 
 template <typename IO>
@@ -253,9 +371,9 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
                        const IO* w, const IO* k, const IO* v, const IO* a, const IO* b, IO* y) {
   const int64_t row = static_cast<int64_t>(T) * C;
   if (std::is_same<IO, float>::value && w_mode == RWKV_W_DECAY) {
-    launch_seq<IO>(st, B, T, C, H, state, reinterpret_cast<const float*>(r), reinterpret_cast<const float*>(w),
-                   reinterpret_cast<const float*>(k), reinterpret_cast<const float*>(a),
-                   reinterpret_cast<const float*>(b), row, v, y, row);
+    launch_seq<IO, false>(st, B, T, C, H, state, reinterpret_cast<const float*>(r), reinterpret_cast<const float*>(w),
+                          reinterpret_cast<const float*>(k), reinterpret_cast<const float*>(a),
+                          reinterpret_cast<const float*>(b), row, v, y, row, TmixSeqArgs{});
     RWKV_LAUNCH_CHECK();
     return RWKV_OK;
   }
@@ -278,7 +396,7 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
     const int64_t n = slab_row * B;
     hipLaunchKernelGGL(wkv7_prepare_kernel<IO>, dim3(ceil_div(n, 256)), dim3(256), 0, st, n, slab_row, row, w_mode,
                        r + off, w + off, k + off, a + off, b + off, r32, d32, k32, a32, b32);
-    launch_seq<IO>(st, B, tn, C, H, state, r32, d32, k32, a32, b32, slab_row, v + off, y + off, row);
+    launch_seq<IO, false>(st, B, tn, C, H, state, r32, d32, k32, a32, b32, slab_row, v + off, y + off, row, TmixSeqArgs{});
   }
   hipError_t err = hipGetLastError();
   hipError_t ferr = hipFreeAsync(ws, st);
@@ -292,7 +410,17 @@ static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, f
 int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                         const float* k, const float* a, const float* b, int64_t op_bs, const half_t* v, half_t* y,
                         int64_t io_bs) {
-  launch_seq<half_t>(st, B, T, C, H, state, r, d, k, a, b, op_bs, v, y, io_bs);
+  launch_seq<half_t, false>(st, B, T, C, H, state, r, d, k, a, b, op_bs, v, y, io_bs, TmixSeqArgs{});
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+int tmix_seq_launch(hipStream_t st, int B, int T, int C, int H, float* state, const TmixSeqArgs& fa, const half_t* v,
+                    half_t* y2) {
+  RWKV_REQUIRE(fa.r && fa.k && fa.a12 && fa.w12 && fa.g && fa.k_k && fa.a0 && fa.k_a && fa.w0 && fa.r_k && fa.lnx_w && fa.lnx_b,
+               "tmix_seq: NULL tensor");
+  const int64_t row = static_cast<int64_t>(T) * C;
+  launch_seq<half_t, true>(st, B, T, C, H, state, nullptr, nullptr, nullptr, nullptr, nullptr, 0, v, y2, row, fa);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }

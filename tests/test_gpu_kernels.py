@@ -77,9 +77,10 @@ def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):
 
 
 def test_wkv7_small_and_large_grids_agree_bitwise(gpu):
-    """Grids of up to 64 heads run with sixteen wavefronts per head, up to 128 with eight, larger ones with four;
-    a state element sees the same arithmetic in each, so the same sequence gives bitwise the same outputs and
-    state inside a batch of 1, of 40 and of 70 (two heads each)."""
+    """With up to 64 heads in flight a head runs as four blocks of 16 state rows each (sixteen wavefronts per head),
+    up to 128 as two blocks of 32 rows (eight), above as one block (four); a state element sees the same
+    arithmetic in each, so the same sequence gives bitwise the same outputs and state inside a batch of 1, of 40
+    and of 70 (two heads each)."""
     hip = gpu
     T, H = 37, 2
     C = H * 64

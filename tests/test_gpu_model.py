@@ -122,12 +122,14 @@ def test_decode_with_row_skipping_ffn_value(gpu, orc, fmt, B):
 
 
 @pytest.mark.parametrize("fmt", [1, 2])
-@pytest.mark.parametrize("B,T", [(2, 16), (40, 1)])
-def test_split_k_partials_summed_by_the_layernorm_kernels_bitwise(gpu, fmt, B, T):
-    """From 16 rows on, the LayerNorm kernels after the output projection and after ffn.value sum the fp32
-    split-K partials of the streaming GEMM themselves; with the residual-stream tap on, the reduce kernel runs
-    instead.  Same sums in the same order: logits, shift rows and WKV state are bit-identical (prefill chunk and
-    batched decode step)."""
+@pytest.mark.parametrize("B,T", [(2, 16), (20, 21), (36, 11), (40, 1)])
+def test_fused_launches_match_the_standalone_kernels_bitwise(gpu, fmt, B, T):
+    """Two fusions of the row-tiled path are switched off while the residual-stream tap is on.  (1) The LayerNorm
+    kernels after the output projection and after ffn.value sum the fp32 split-K partials of the streaming GEMM
+    themselves; tapped, the reduce kernel runs instead.  (2) kk normalise / a-gate / decay, the WKV recurrence and
+    GroupNorm / bonus / gate run as one launch; tapped, as the three stand-alone kernels.  Same arithmetic in the
+    same order: logits, shift rows and WKV state are bit-identical (prefill chunks with and without a ragged tail,
+    at each of the sequence kernel's three wavefronts-per-head variants, and a batched decode step)."""
     from rwkv_lightning_cuda_amd.model import HipModel, ModelDims, Session, State, synth_weights
     hip = gpu
     dims = ModelDims(L=2, C=512, H=8, F=2048, V=1024, Rw=32, Ra=32, Rg=64, Rv=32)
