@@ -137,7 +137,7 @@ __device__ __forceinline__ half8_t expand_w4(uint32_t d, half2_t bias) {
                     as_half2(__builtin_amdgcn_perm(odd, even, 0x0c070c03u) | 0x64006400u) - bias);
 }
 
-template <int FMT, int MT, int KC>
+template <int FMT, int MT, int KC, int WG = 4>
 struct Tile {
   using P = PackTraits<FMT>;
   static constexpr int BM = 32 * MT;
@@ -146,7 +146,8 @@ struct Tile {
   static constexpr int NW = GROUPS * P::PIECES;     // weight pieces per lane per chunk
   static constexpr int STEPS = P::KR / 8;
   static constexpr int XSTRIDE = KC + 8;            // fp16 per staged row: 16-byte pad keeps b128 reads conflict-free
-  static constexpr int XV = BM * (KC / 8) / 256;    // 16-byte vectors of X per thread per chunk
+  static constexpr int GT = 64 * WG;                // threads of a wavefront group
+  static constexpr int XV = BM * (KC / 8) / GT;     // 16-byte vectors of X per thread per chunk
   static constexpr int QG = KC / 128;               // int4 scale groups per chunk
   static constexpr int NACC = MT == 1 ? 2 : 1;      // independent accumulation chains per row tile
   static constexpr int DEPTH = (NW * 4 <= 16) ? 4 : (NW * 4 <= 32 ? 3 : 2);  // weight register sets in the ring
@@ -164,15 +165,15 @@ __device__ __forceinline__ float finish_value(float v, int epilogue) {
 }
 
 // One chunk's slice of X held by a thread between request and its store to LDS.
-template <int FMT, int MT, int KC>
+template <int FMT, int MT, int KC, int WG>
 struct XRegs {
-  using T = Tile<FMT, MT, KC>;
+  using T = Tile<FMT, MT, KC, WG>;
   uint4_t xv[T::XV];
 
   __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int tid, int m0, int kc) {
 #pragma unroll
     for (int i = 0; i < T::XV; ++i) {
-      const int idx = tid + i * 256;
+      const int idx = tid + i * T::GT;
       const int r = idx / (KC / 8);
       const int c = (idx % (KC / 8)) * 8;
       xv[i] = uint4_t{0u, 0u, 0u, 0u};
@@ -183,7 +184,7 @@ struct XRegs {
   __device__ __forceinline__ void store_x(int tid, half_t* xs) const {
 #pragma unroll
     for (int i = 0; i < T::XV; ++i) {
-      const int idx = tid + i * 256;
+      const int idx = tid + i * T::GT;
       const int r = idx / (KC / 8);
       const int c = (idx % (KC / 8)) * 8;
       *reinterpret_cast<uint4_t*>(xs + r * T::XSTRIDE + c) = xv[i];
@@ -277,10 +278,11 @@ struct WRegs {
   }
 };
 
-// One block of one problem: 128 columns x the block's K slice.  The block has KG groups of four wavefronts;
-// group kg takes chunks kg, kg + KG, ... of the slice with its own pair of X tiles in LDS, and the groups' sums
-// meet in LDS at the end (in group order), so that a CU holds two wavefronts per SIMD - one's code expansion
-// overlaps the other's matrix-core time - without more fp32 partial tiles in HBM.
+// One block of one problem: 32 * WG columns x the block's K slice.  The block has KG groups of WG wavefronts (one
+// 32-column band of the weights per wavefront); group kg takes chunks kg, kg + KG, ... of the slice with its own
+// pair of X tiles in LDS, and the groups' sums meet in LDS at the end (in group order), so that a CU holds two
+// wavefronts per SIMD - one's code expansion overlaps the other's matrix-core time - without more fp32 partial
+// tiles in HBM.
 //
 // Per group and chunk c: the X slice of chunk c+2 is requested into registers, the weight pieces of chunk
 // c+D-1 into a ring of D register sets, the matrix core runs chunk c out of LDS tile c&1, then the X slice of
@@ -289,21 +291,22 @@ struct WRegs {
 // cache - because a load under a branch makes the compiler's s_waitcnt accounting assume the shorter path
 // and wait for everything in flight.  Within an iteration X is requested before the weights, so that waiting
 // for X does not wait for the younger weight loads.
-template <int FMT, int MT, int KC, int KG>
+template <int FMT, int MT, int KC, int KG, int WG>
 __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamProblem& pr, int row_tile, int col_block,
                                              int split, half_t* xs_all) {
-  using T = Tile<FMT, MT, KC>;
+  using T = Tile<FMT, MT, KC, WG>;
   using P = typename T::P;
   constexpr int BM = T::BM;
+  constexpr int GT = T::GT;
 
-  const int tid = threadIdx.x & 255;  // thread within its k-group
-  const int kg = threadIdx.x >> 8;
+  const int tid = threadIdx.x % GT;  // thread within its k-group
+  const int kg = threadIdx.x / GT;
   const int wave = tid >> 6;
   const int lane = tid & 63;
   const int j = lane & 31;
   const int h = lane >> 5;
   const int m0 = row_tile * BM;
-  const int band_here = col_block * 4 + wave;  // 32-row band of W = 32 output columns
+  const int band_here = col_block * WG + wave;  // 32-row band of W = 32 output columns
   const bool active = band_here * 32 < pr.N;
   const int band = active ? band_here : pr.N / 32 - 1;  // a wavefront past the last band repeats it and stores nothing
   const int n = band * 32 + j;
@@ -328,7 +331,7 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
 
   constexpr int D = T::DEPTH;
   WRegs<FMT, MT, KC> wr[D];
-  XRegs<FMT, MT, KC> xr[2];
+  XRegs<FMT, MT, KC, WG> xr[2];
   const int last = nchunks - 1;
   xr[0].request(g, pr, tid, m0, kbeg);
   xr[1].request(g, pr, tid, m0, kbeg + min(1, last) * KSTRIDE);
@@ -356,20 +359,22 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mt][0][v] += acc[mt][1][v];
   }
-  // The X tiles are free after the last barrier.  Group 1 hands its sums to group 0 through them; group 0 then lays
-  // the finished 32*MT x 128 tile out in LDS (rows 136 floats apart: conflict-free for both access patterns) and
-  // all threads write it to memory in 16/32-byte pieces along the rows - the accumulator layout itself would
-  // give 2-byte stores 64 bytes apart.
-  constexpr int kStageLd = 136;
-  float* stage = reinterpret_cast<float*>(xs_all) + (KG == 2 ? MT * 16 * 256 : 0);
-  static_assert((KG == 2 ? MT * 16 * 256 : 0) * 4 + BM * kStageLd * 4 <= KG * 2 * T::kTileHalfs * 2, "epilogue tile exceeds the LDS tiles");
-  if constexpr (KG == 2) {
+  // The X tiles are free after the last barrier.  The other groups hand their sums to group 0 through them; group 0
+  // then lays the finished 32*MT x 32*WG tile out in LDS (rows padded by 8 floats) and all threads write it to
+  // memory in 16/32-byte pieces along the rows - the accumulator layout itself would give 2-byte stores 64 bytes
+  // apart.
+  constexpr int kCols = 32 * WG;         // columns of the block
+  constexpr int kStageLd = kCols + 8;
+  constexpr int kRedFloats = (KG - 1) * MT * 16 * GT;
+  float* stage = reinterpret_cast<float*>(xs_all) + kRedFloats;
+  static_assert(kRedFloats * 4 + BM * kStageLd * 4 <= KG * 2 * T::kTileHalfs * 2, "epilogue tile exceeds the LDS tiles");
+  if constexpr (KG > 1) {
     float* red = reinterpret_cast<float*>(xs_all);
-    if (kg == 1) {
+    if (kg > 0) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) red[(mt * 16 + v) * 256 + tid] = acc[mt][0][v];
+        for (int v = 0; v < 16; ++v) red[((kg - 1) * MT * 16 + mt * 16 + v) * GT + tid] = acc[mt][0][v];
     }
     __syncthreads();
   }
@@ -384,20 +389,23 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         float sum = acc[mt][0][v];
-        if constexpr (KG == 2) sum += reinterpret_cast<const float*>(xs_all)[(mt * 16 + v) * 256 + tid];
+#pragma unroll
+        for (int q = 1; q < KG; ++q) sum += reinterpret_cast<const float*>(xs_all)[((q - 1) * MT * 16 + mt * 16 + v) * GT + tid];
         const int row = mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
         stage[row * kStageLd + wave * 32 + j] = partial_out ? sum : finish_value(mul_f32(sum, scl), g.epilogue);
       }
   }
   __syncthreads();
   float* part_out = partial_out ? pr.partial + static_cast<int64_t>(split) * g.M * pr.N : nullptr;
-  const int col0 = col_block * 128;
-  for (int idx = threadIdx.x; idx < BM * 16; idx += 256 * KG) {
-    const int row = idx >> 4;
-    const int col = col0 + (idx & 15) * 8;
+  const int col0 = col_block * kCols;
+  constexpr int kPieces = kCols / 8;  // 8-column pieces per row
+  for (int idx = threadIdx.x; idx < BM * kPieces; idx += GT * KG) {
+    const int row = idx / kPieces;
+    const int piece = idx % kPieces;
+    const int col = col0 + piece * 8;
     if (m0 + row >= g.M || col >= pr.N) continue;
-    const float4_t lo = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + (idx & 15) * 8);
-    const float4_t hi = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + (idx & 15) * 8 + 4);
+    const float4_t lo = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + piece * 8);
+    const float4_t hi = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + piece * 8 + 4);
     const int64_t o = static_cast<int64_t>(m0 + row) * pr.N + col;
     if (partial_out || g.out_f32) {
       float* dst = partial_out ? part_out + o : static_cast<float*>(pr.y) + o;
@@ -415,11 +423,11 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
   }
 }
 
-// grid = row tiles x roundup(column blocks of 128 over all problems x splits, 8), one-dimensional; block = 256 * KG.
+// grid = row tiles x roundup(column blocks over all problems x splits, 8), one-dimensional; block = 64 * WG * KG.
 // Workgroups go to the eight XCDs round-robin by linear id, each XCD with its own L2: the id is decoded so that
 // the row tiles of one (column block, split) pair - which stream the same weights - land on the same XCD.
-template <int MT, int KC, int KG>
-__global__ __launch_bounds__(256 * KG) void gemm_stream_kernel(StreamArgs g) {
+template <int MT, int KC, int KG, int WG>
+__global__ __launch_bounds__(64 * WG * KG) void gemm_stream_kernel(StreamArgs g) {
   __shared__ __align__(16) half_t xs[KG * 2 * 32 * MT * (KC + 8)];
   const int id = blockIdx.x;
   const int row_tile = (id >> 3) % g.row_tiles;
@@ -432,9 +440,9 @@ __global__ __launch_bounds__(256 * KG) void gemm_stream_kernel(StreamArgs g) {
   const int col_block = col_all - (pi > 0 ? g.block_end[pi - 1] : 0);
   const StreamProblem& pr = g.p[pi];
   switch (pr.fmt) {
-    case RWKV_FMT_W8: stream_block<RWKV_FMT_W8, MT, KC, KG>(g, pr, row_tile, col_block, split, xs); break;
-    case RWKV_FMT_W4: stream_block<RWKV_FMT_W4, MT, KC, KG>(g, pr, row_tile, col_block, split, xs); break;
-    default: stream_block<RWKV_FMT_F16, MT, KC, KG>(g, pr, row_tile, col_block, split, xs); break;
+    case RWKV_FMT_W8: stream_block<RWKV_FMT_W8, MT, KC, KG, WG>(g, pr, row_tile, col_block, split, xs); break;
+    case RWKV_FMT_W4: stream_block<RWKV_FMT_W4, MT, KC, KG, WG>(g, pr, row_tile, col_block, split, xs); break;
+    default: stream_block<RWKV_FMT_F16, MT, KC, KG, WG>(g, pr, row_tile, col_block, split, xs); break;
   }
 }
 
@@ -504,21 +512,33 @@ static int target_blocks() {
 // tile per block, so that two or more row tiles share the weights through their XCD's L2 and the split stays
 // small; up to 512 rows 64-row tiles; both with two wavefront groups per block.  Above that 128-row tiles with
 // one group (128 accumulator registers per lane leave no room for a second wavefront per SIMD).
-struct StreamConfig {
-  int mt, kc, kg;
-};
 // 33..64 rows against enough column blocks to occupy the CUs without a K split (the head): one 64-row tile, so that
 // no weight is requested by two blocks (268 MB of int8 codes at 64 rows: 95 -> 75 us).
-static StreamConfig choose_config(int M, int col_blocks) {
-  if (M > 32 && M <= 64 && col_blocks >= target_blocks()) return StreamConfig{2, 128, 2};
-  if (M <= 64) return StreamConfig{1, 128, 2};
-  if (M <= 512) return StreamConfig{2, 128, 2};
-  return StreamConfig{4, 128, 1};
+// Up to 32 rows, where 128-column blocks would need a K split: blocks of 64 columns with four groups of two
+// wavefronts - twice the blocks per matrix, so half the split (less partial-sum traffic) or none (no reduce
+// launch): 16 rows x 16384 columns 23.4 -> 19.6 us; decode steps of 8 / 16 / 32 rows 7 / 5 / 3 % faster.  At 64
+// rows the narrow blocks lose (24.5 -> 30 us): every block reads all of X.
+struct StreamConfig {
+  int mt, kc, kg, wg;
+  int cols() const { return 32 * wg; }
+};
+static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns) {
+  int cb128 = 0;
+  for (int i = 0; i < n_problems; ++i) cb128 += ceil_div(Ns[i], 128);
+  if (M <= 32 && K % (128 * 4) == 0 && cb128 < target_blocks()) return StreamConfig{1, 128, 4, 2};
+  if (M > 32 && M <= 64 && cb128 >= target_blocks()) return StreamConfig{2, 128, 2, 4};
+  if (M <= 64) return StreamConfig{1, 128, 2, 4};
+  if (M <= 512) return StreamConfig{2, 128, 2, 4};
+  return StreamConfig{4, 128, 1, 4};
+}
+static int count_col_blocks(const StreamConfig& c, int n_problems, const int* Ns) {
+  int col_blocks = 0;
+  for (int i = 0; i < n_problems; ++i) col_blocks += ceil_div(Ns[i], c.cols());
+  return col_blocks;
 }
 
 // Split count: a power of two that gives enough blocks to occupy the CUs, K slices whole chunks of every group.
-static int choose_splits(int M, int col_blocks, int K) {
-  const StreamConfig c = choose_config(M, col_blocks);
+static int choose_splits(const StreamConfig& c, int M, int col_blocks, int K) {
   const int tiles = ceil_div(M, 32 * c.mt) * col_blocks;
   int splits = 1;
   while (tiles * splits < target_blocks() && K % (splits * 2 * c.kc * c.kg) == 0 && splits < 32) splits *= 2;
@@ -526,13 +546,10 @@ static int choose_splits(int M, int col_blocks, int K) {
 }
 
 size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const int* Ns) {
-  int col_blocks = 0;
   int64_t n_total = 0;
-  for (int i = 0; i < n_problems; ++i) {
-    col_blocks += ceil_div(Ns[i], 128);
-    n_total += Ns[i];
-  }
-  const int splits = choose_splits(M, col_blocks, K);
+  for (int i = 0; i < n_problems; ++i) n_total += Ns[i];
+  const StreamConfig c = choose_config(M, K, n_problems, Ns);
+  const int splits = choose_splits(c, M, count_col_blocks(c, n_problems, Ns), K);
   return splits > 1 ? static_cast<size_t>(splits) * M * n_total * sizeof(float) : 0;
 }
 
@@ -549,6 +566,9 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
   g.K = K;
   g.epilogue = r.epilogue = epilogue;
   g.out_f32 = r.out_f32 = out_f32;
+  int Ns[kMaxProblems];
+  for (int i = 0; i < n_problems; ++i) Ns[i] = problems[i].N;
+  const StreamConfig cfg = choose_config(M, K, n_problems, Ns);
   int col_blocks = 0;
   for (int i = 0; i < n_problems; ++i) {
     const PackedProblem& q = problems[i];
@@ -557,12 +577,11 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
     RWKV_REQUIRE(q.x && q.packed && q.y, "linear_packed: NULL tensor");
     RWKV_REQUIRE(q.fmt == RWKV_FMT_F16 || q.scale, "linear_packed: quantised weights need a scale tensor");
     RWKV_REQUIRE(q.fmt != RWKV_FMT_W4 || q.zp, "linear_packed: W4 weights need a zero-point tensor");
-    col_blocks += ceil_div(q.N, 128);
+    col_blocks += ceil_div(q.N, cfg.cols());
     g.block_end[i] = col_blocks;
     g.p[i] = StreamProblem{q.x, static_cast<const uint4_t*>(q.packed), q.scale, q.zp, q.y, nullptr, q.N, q.fmt};
   }
-  const StreamConfig cfg = choose_config(M, col_blocks);
-  g.splits = r.splits = choose_splits(M, col_blocks, K);
+  g.splits = r.splits = choose_splits(cfg, M, col_blocks, K);
   g.k_per_split = K / g.splits;
   if (g.splits > 1) {
     size_t need = 0;
@@ -587,10 +606,11 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
   g.col_blocks = col_blocks;
   const int pairs8 = ceil_div(col_blocks * g.splits, 8) * 8;
   const dim3 grid(g.row_tiles * pairs8);
-  const dim3 block(256 * cfg.kg);
-  if (cfg.mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 2>), grid, block, 0, st, g);
-  else if (cfg.mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 128, 2>), grid, block, 0, st, g);
-  else hipLaunchKernelGGL((gemm_stream_kernel<4, 128, 1>), grid, block, 0, st, g);
+  const dim3 block(64 * cfg.wg * cfg.kg);
+  if (cfg.wg == 2) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 4, 2>), grid, block, 0, st, g);
+  else if (cfg.mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 2, 4>), grid, block, 0, st, g);
+  else if (cfg.mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 128, 2, 4>), grid, block, 0, st, g);
+  else hipLaunchKernelGGL((gemm_stream_kernel<4, 128, 1, 4>), grid, block, 0, st, g);
   RWKV_LAUNCH_CHECK();
   if (defer) *defer = DeferredReduce{};
   if (g.splits == 1) return RWKV_OK;
