@@ -400,20 +400,24 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
       half_t* ys[3] = {b.r, b.k, v_cur};
       if (small) {
         // one launch: three big matrices (any format) + the rank-in matrices (fp16), all with K = C
+        // The rank-in blocks come first: with fp16 weights against int8 they are the longest of the launch, and
+        // blocks start in id order - at the end they would run on alone.
         LinearProblem p[7];
-        for (int i = 0; i < 3; ++i) {
-          p[i].w = w.m[mids[i]].data; p[i].scale = w.m[mids[i]].scale; p[i].zp = w.m[mids[i]].zp;
-          p[i].x = xs[i]; p[i].y = ys[i]; p[i].N = C; p[i].fmt = w.m[mids[i]].fmt;
-        }
         for (int i = 0; i < n_lora; ++i) {
-          p[3 + i].w = w.t[w1_ids[i]]; p[3 + i].scale = nullptr; p[3 + i].zp = nullptr;
-          p[3 + i].x = lx[i]; p[3 + i].y = lh[i]; p[3 + i].N = ranks[i]; p[3 + i].fmt = RWKV_FMT_F16;
+          p[i].w = w.t[w1_ids[i]]; p[i].scale = nullptr; p[i].zp = nullptr;
+          p[i].x = lx[i]; p[i].y = lh[i]; p[i].N = ranks[i]; p[i].fmt = RWKV_FMT_F16;
+        }
+        for (int i = 0; i < 3; ++i) {
+          LinearProblem& q = p[n_lora + i];
+          q.w = w.m[mids[i]].data; q.scale = w.m[mids[i]].scale; q.zp = w.m[mids[i]].zp;
+          q.x = xs[i]; q.y = ys[i]; q.N = C; q.fmt = w.m[mids[i]].fmt;
         }
         if (ln_in_linear) {
-          const int mu_ids[7] = {RWKV_T_X_R, RWKV_T_X_K, RWKV_T_X_V, RWKV_T_X_W, RWKV_T_X_A, RWKV_T_X_G, RWKV_T_X_V};
+          const int lora_mu[4] = {RWKV_T_X_W, RWKV_T_X_A, RWKV_T_X_G, RWKV_T_X_V};
+          const int dense_mu[3] = {RWKV_T_X_R, RWKV_T_X_K, RWKV_T_X_V};
           for (int i = 0; i < 3 + n_lora; ++i) {
             p[i].x = nullptr;
-            p[i].mu = w.t[mu_ids[i]];
+            p[i].mu = w.t[i < n_lora ? lora_mu[i] : dense_mu[i - n_lora]];
           }
           LnPrologue ln;
           ln.w = w.t[RWKV_T_LN1_W]; ln.b = w.t[RWKV_T_LN1_B]; ln.shift = shift0; ln.x_out = b.x; ln.ln_out = b.xx;
