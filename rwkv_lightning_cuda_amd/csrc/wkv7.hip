@@ -82,7 +82,10 @@ __device__ __forceinline__ float row16_sum(float x) {
 // columns, v_i and the per-column operands), so a head is cut into PARTS row ranges that run as separate blocks on
 // separate CUs - with few heads in flight the step is bound by one CU's VALU rate, not by memory.  Not with FUSED
 // (the GroupNorm needs the whole head's y).  Same lanes, same rows, same arithmetic: bitwise the same results.
-template <typename IO, int RPL, int PARTS, bool FUSED>
+//
+// STRAIGHT = false leaves out the unrolled eight-step body: single-token calls move a head's state once and are
+// bound by that traffic, so they want the registers for more blocks per CU instead (148 -> under 100 VGPRs).
+template <typename IO, int RPL, int PARTS, bool FUSED, bool STRAIGHT = true>
 __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
                                                               const float* __restrict__ r, const float* __restrict__ d,
                                                               const float* __restrict__ k, const float* __restrict__ a,
@@ -98,7 +101,10 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
   __shared__ __align__(16) float ops[2][kSeqChunk][5][kHead];  // [buffer][token][a,b,d,k,r][column]
   __shared__ __align__(16) float vs[2][kSeqChunk][kHead];      // [buffer][token][row]
   __shared__ __align__(16) float ys[2][kSeqChunk][kHead];
-  __shared__ __align__(16) float spare[NT * RPL];
+  // Where to the 15 idle lanes of a row store in step_out.  The single-token variant keeps to 32 KB of LDS instead
+  // (five blocks per CU) and stores under a branch.
+  constexpr bool kSpare = STRAIGHT;
+  __shared__ __align__(16) float spare[kSpare ? NT * RPL : 4];
   __shared__ __align__(16) float gs[FUSED ? 2 : 1][FUSED ? kSeqChunk : 1][kHead];  // FUSED: the gate rows
 
   const int bh = blockIdx.x / PARTS;
@@ -293,10 +299,14 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
       for (int i = 0; i < RPL; ++i) yy[i] = row16_sum(yy[i]);
       // the 16 lanes of a row hold the same sums: the first stores them, the others store to a spare area - a
       // store under a branch would end the scheduling region here
-      float* dst = (lane & 15) == 0 ? &ys[buf][tt][i0] : &spare[tid * RPL];
-      *reinterpret_cast<rows_t*>(dst) = yy;
+      if constexpr (kSpare) {
+        float* dst = (lane & 15) == 0 ? &ys[buf][tt][i0] : &spare[tid * RPL];
+        *reinterpret_cast<rows_t*>(dst) = yy;
+      } else {
+        if ((lane & 15) == 0) *reinterpret_cast<rows_t*>(&ys[buf][tt][i0]) = yy;
+      }
     };
-    if (n == kSeqChunk) {
+    if (STRAIGHT && n == kSeqChunk) {
       // Full chunk, straight-line.  The operands of step tt+1 are read from LDS while step tt computes, and the
       // scheduling regions run from the middle of one step to the middle of the next
       // (__builtin_amdgcn_sched_barrier(0) between the halves), so that the compiler fills the latency bubbles
@@ -362,8 +372,13 @@ static void launch_seq(hipStream_t st, int B, int T, int C, int H, float* state,
       return;
     }
   }
-  hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, FUSED>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs,
-                     v, y, io_bs, fa);
+  if (T == 1) {
+    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, FUSED, false>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
+                       op_bs, v, y, io_bs, fa);
+  } else {
+    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, FUSED>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs,
+                       v, y, io_bs, fa);
+  }
 }
 
 template <typename IO>
