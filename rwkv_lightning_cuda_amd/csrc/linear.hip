@@ -33,53 +33,75 @@ struct LinearArgs {
   RowCopy copy;
 };
 
-// One row of the LayerNorm + lerp prologue into xs (K fp16 values).  Same element-to-thread assignment, two-pass
-// statistics, explicit FMAs and rounding points as ln_fused_kernel (fused_ops.hip), so the result is bit-identical
-// to running that kernel first.  The fp32 row sum s = x + res lives in LDS (sbuf, K floats; each thread re-reads
-// only what it wrote) instead of registers, so that the prologue does not cost the weight-streaming loop its
-// occupancy.  256 threads.
+// One row of the LayerNorm + lerp prologue into xs (K fp16 values).  Same two-pass statistics, explicit FMAs and
+// rounding points as ln_fused_kernel (fused_ops.hip), and the same order of summation, so the result is
+// bit-identical to running that kernel first: that kernel gives each of its 256, 512 or 1024 threads (by row
+// length) one 8-element slice and adds wavefront sums in wavefront order; here thread t of 256 stands in for
+// its threads t, t + 256, ... with one partial sum each, and the block sum walks the same list of wavefront sums
+// (slots of absent threads hold zero, which changes no bit).  The fp32 row sum s = x + res lives in LDS (sbuf, K
+// floats; each thread re-reads only what it wrote) instead of registers, so that the prologue does not cost the
+// weight-streaming loop its occupancy.  256 threads; red holds 16 floats.
+__device__ __forceinline__ float ln_block_sum4(float (&x)[4], float* red) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) x[j] = wave_sum(x[j]);
+  __syncthreads();  // red may still be read from a previous call
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) red[j * 4 + (threadIdx.x >> 6)] = x[j];
+  }
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) t += red[i];
+  return t;
+}
+
 template <int NW>
 __device__ __forceinline__ void ln_prologue_row(const LnPrologue& ln, const half_t* mu, int K, int m, half_t* xs,
                                                 float* sbuf, float* red, bool store) {
-  // Blocks of more than 256 threads: the first 256 hold the elements exactly as ln_fused_kernel's 256 threads do and
-  // the other wavefronts add zeros to the block sums, which leaves every sum bit-identical.
-  const int kend = threadIdx.x < 256 ? K : 0;
+  static_assert(NW == 4, "the prologue mirrors the LayerNorm kernel with 256 threads");
+  const int kend = K;
   const int64_t row = static_cast<int64_t>(m) * K;
   const int64_t xsrc = ln.mode == 2 ? ln.tokens[m] * static_cast<int64_t>(K) : row;
-  float sum = 0.0f;
-#pragma unroll 1
-  for (int c = threadIdx.x * 8; c < kend; c += 256 * 8) {
-    const half8_t xv = *reinterpret_cast<const half8_t*>(ln.x + xsrc + c);
-    float v[8];
-    if (ln.mode == 1) {
-      const half8_t rv = *reinterpret_cast<const half8_t*>(ln.res + row + c);
+  float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = h2f(xv[e]) + h2f(rv[e]);
-    } else {
+  for (int j = 0; j < 4; ++j) {
+    const int c = (threadIdx.x + 256 * j) * 8;
+    if (c < kend) {
+      const half8_t xv = *reinterpret_cast<const half8_t*>(ln.x + xsrc + c);
+      float v[8];
+      if (ln.mode == 1) {
+        const half8_t rv = *reinterpret_cast<const half8_t*>(ln.res + row + c);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = h2f(xv[e]);
-    }
+        for (int e = 0; e < 8; ++e) v[e] = h2f(xv[e]) + h2f(rv[e]);
+      } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) sum += v[e];
-    *reinterpret_cast<float4_t*>(sbuf + c) = float4_t{v[0], v[1], v[2], v[3]};
-    *reinterpret_cast<float4_t*>(sbuf + c + 4) = float4_t{v[4], v[5], v[6], v[7]};
-  }
-  sum = block_sum<NW>(sum, red);
-  const float mean = sum / static_cast<float>(K);
-  float sv = 0.0f;
-#pragma unroll 1
-  for (int c = threadIdx.x * 8; c < kend; c += 256 * 8) {
-    const float4_t lo = *reinterpret_cast<const float4_t*>(sbuf + c);
-    const float4_t hi = *reinterpret_cast<const float4_t*>(sbuf + c + 4);
-    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        for (int e = 0; e < 8; ++e) v[e] = h2f(xv[e]);
+      }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float d = v[e] - mean;
-      sv = fmaf(d, d, sv);
+      for (int e = 0; e < 8; ++e) sum[j] += v[e];
+      *reinterpret_cast<float4_t*>(sbuf + c) = float4_t{v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<float4_t*>(sbuf + c + 4) = float4_t{v[4], v[5], v[6], v[7]};
     }
   }
-  sv = block_sum<NW>(sv, red);
-  const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
+  const float mean = ln_block_sum4(sum, red) / static_cast<float>(K);
+  float sv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = (threadIdx.x + 256 * j) * 8;
+    if (c < kend) {
+      const float4_t lo = *reinterpret_cast<const float4_t*>(sbuf + c);
+      const float4_t hi = *reinterpret_cast<const float4_t*>(sbuf + c + 4);
+      const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = v[e] - mean;
+        sv[j] = fmaf(d, d, sv[j]);
+      }
+    }
+  }
+  const float sv_total = ln_block_sum4(sv, red);
+  const float rstd = rsqrtf(sv_total / static_cast<float>(K) + ln.eps);
 #pragma unroll 1
   for (int c = threadIdx.x * 8; c < kend; c += 256 * 8) {
     const half8_t wv = *reinterpret_cast<const half8_t*>(ln.w + c);
@@ -354,7 +376,7 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
 template <int M, int R, int U, bool LN, int NW>
 __global__ __launch_bounds__(NW * 64) void linear_gemv_kernel(LinearArgs args) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  __shared__ float red[NW];
+  __shared__ float red[16];
   half_t* xs = reinterpret_cast<half_t*>(lds_raw);
   float* sbuf = reinterpret_cast<float*>(lds_raw + static_cast<size_t>(M) * args.KT * sizeof(half_t));
   if (blockIdx.x == 0 && args.copy.n > 0) {

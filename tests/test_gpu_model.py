@@ -412,15 +412,16 @@ def test_config3_7p2b_width_two_layers_quantised(gpu, orc, fmt_name):
     sess.close()
 
 
-@pytest.mark.parametrize("B", [1, 2])
-def test_decode_step_with_layernorm_folded_into_linear_is_bitwise_the_unfused_step(gpu, B):
+@pytest.mark.parametrize("B,wide", [(1, False), (2, False), (1, True)])
+def test_decode_step_with_layernorm_folded_into_linear_is_bitwise_the_unfused_step(gpu, B, wide):
     """Decode steps on the GEMV path (one or two rows) can compute LayerNorm + token shift inside the linear
     kernels' prologue
     (session option, off by default) instead of the stand-alone kernels.  Same arithmetic and reduction order:
-    logits, shift rows and WKV state must be bit-identical, step after step."""
-    from rwkv_lightning_cuda_amd.model import HipModel, Session, State, synth_weights
+    logits, shift rows and WKV state must be bit-identical, step after step - also at a row length where the
+    stand-alone kernel runs with 512 threads (C = 2560) and the prologue's 256 threads each stand in for two."""
+    from rwkv_lightning_cuda_amd.model import HipModel, ModelDims, Session, State, synth_weights
     hip = gpu
-    dims = small_dims()
+    dims = ModelDims(L=2, C=2560, H=40, F=5120, V=512, Rw=32, Ra=32, Rg=64, Rv=32) if wide else small_dims()
     gmodel = HipModel.from_host_weights(dims, synth_weights(dims, 9), hip.FMT_W8)
     rng = np.random.default_rng(B)
     prompt = rng.integers(0, dims.V, (B, 5))
