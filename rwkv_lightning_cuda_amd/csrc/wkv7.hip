@@ -21,28 +21,6 @@ __device__ __forceinline__ float decay_from_logit(float w) {
   return exp2f(kWScaleLog2e / (1.0f + exp2f(kNLog2e * w)));
 }
 
-// ---- pre-pass: any io type -> fp32 operands, decay applied -----------------------------------
-// Source tensors are [B,T,C]; the pre-pass takes tokens [t0, t0+tn) of every batch row and writes
-// compact fp32 [B,tn,C] operands.
-template <typename IO>
-__global__ __launch_bounds__(256) void wkv7_prepare_kernel(int64_t n, int64_t slab_row, int64_t src_row, int w_mode,
-                                                           const IO* __restrict__ r, const IO* __restrict__ w,
-                                                           const IO* __restrict__ k, const IO* __restrict__ a,
-                                                           const IO* __restrict__ b, float* __restrict__ r32,
-                                                           float* __restrict__ d32, float* __restrict__ k32,
-                                                           float* __restrict__ a32, float* __restrict__ b32) {
-  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int64_t bi = i / slab_row;            // slab_row = tn*C, src_row = T*C
-  const int64_t src = bi * src_row + (i - bi * slab_row);
-  const float wv = static_cast<float>(w[src]);
-  r32[i] = static_cast<float>(r[src]);
-  d32[i] = (w_mode == RWKV_W_RAW_LOGIT) ? decay_from_logit(wv) : wv;
-  k32[i] = static_cast<float>(k[src]);
-  a32[i] = static_cast<float>(a[src]);
-  b32[i] = static_cast<float>(b[src]);
-}
-
 // ---- sequence kernel -------------------------------------------------------------------------
 // grid = B*H, block = 1024/RPL threads: 16/RPL wavefronts per head, RPL = 4, 2 or 1 state rows per lane.  Lane
 // (g, c) = (lane / 16, lane % 16) of wavefront q owns rows 4*RPL*q + RPL*g .. +RPL-1 and columns 4c .. 4c+3, so
@@ -72,6 +50,21 @@ __device__ __forceinline__ float row16_sum(float x) {
   return x;
 }
 
+// Where the five operand vectors of a token come from (SRC):
+//   kSrcFp32  - fp32 tensors r, d, k, a, b (decay applied), `op_bs` elements between batch rows, staged with 16-byte
+//               loads: what kk_a_gate_kernel writes for the model's stand-alone path;
+//   kSrcRaw   - the caller's r, w, k, a, b in the io type, converted (and the decay derived from w, by w_mode)
+//               while staging, one wavefront per token, lane = channel: the C-ABI operator, which so reads every
+//               operand once instead of through an fp32 copy (14 instead of 56 bytes per token and channel);
+//   kSrcFused - the model's fused pass, below.
+constexpr int kSrcFp32 = 0;
+constexpr int kSrcFused = 1;
+constexpr int kSrcRaw = 2;
+struct RawOperands {
+  const void *r, *w, *k, *a, *b;
+  int w_mode;
+};
+
 // FUSED (the model's row-tiled time-mix path, fp16 io): the operands are not read as fp32 tensors but derived
 // while staging from the fp16 rows r, k, a12, w12 - the arithmetic of kk_a_gate_kernel, one wavefront per token,
 // lane = channel - and y is not stored but taken through the per-head GroupNorm, the (r.k.r_k) v bonus and the
@@ -85,13 +78,15 @@ __device__ __forceinline__ float row16_sum(float x) {
 //
 // STRAIGHT = false leaves out the unrolled eight-step body: single-token calls move a head's state once and are
 // bound by that traffic, so they want the registers for more blocks per CU instead (148 -> under 100 VGPRs).
-template <typename IO, int RPL, int PARTS, bool FUSED, bool STRAIGHT = true>
+template <typename IO, int RPL, int PARTS, int SRC, bool STRAIGHT = true>
 __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int C, int H, float* __restrict__ state,
                                                               const float* __restrict__ r, const float* __restrict__ d,
                                                               const float* __restrict__ k, const float* __restrict__ a,
                                                               const float* __restrict__ b, int64_t op_bs,
                                                               const IO* __restrict__ v, IO* __restrict__ y,
-                                                              int64_t io_bs, TmixSeqArgs fa) {
+                                                              int64_t io_bs, TmixSeqArgs fa, RawOperands ro) {
+  constexpr bool FUSED = SRC == kSrcFused;
+  constexpr bool RAW = SRC == kSrcRaw;
   static_assert(PARTS == 1 || !FUSED, "the fused pass needs whole heads");
   constexpr int NT = 1024 / RPL / PARTS;
   constexpr int kOpVecs = 5 * kSeqChunk * (kHead / 4);         // float4 of operands per chunk
@@ -146,6 +141,13 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
   float v_stage[2][kVSlots];
   // FUSED: raw fp16 values of this thread's (token, channel) slots: r, k, a12, w12, g; and its channel's constants
   half_t raw[2][kVSlots][5];
+  // RAW: the caller's r, w, k, a, b values of the slots, still in the io type
+  IO rio[2][RAW ? kVSlots : 1][5];
+  const IO* ro_r = static_cast<const IO*>(ro.r);
+  const IO* ro_w = static_cast<const IO*>(ro.w);
+  const IO* ro_k = static_cast<const IO*>(ro.k);
+  const IO* ro_a = static_cast<const IO*>(ro.a);
+  const IO* ro_b = static_cast<const IO*>(ro.b);
   float c_kk = 0.0f, c_a0 = 0.0f, c_ka = 0.0f, c_w0 = 0.0f, c_rk = 0.0f, c_lnw = 0.0f, c_lnb = 0.0f;
   if constexpr (FUSED) {
     const int c = h * kHead + lane;
@@ -157,7 +159,7 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
   // under a branch makes the compiler's s_waitcnt accounting wait for everything in flight, the younger set too.
   auto request = [&](int t0, auto set_c) {
     constexpr int set = decltype(set_c)::value;
-    if constexpr (!FUSED) {
+    if constexpr (SRC == kSrcFp32) {
 #pragma unroll
       for (int i = 0; i < kOpSlots; ++i) {
         stage[set][i] = *reinterpret_cast<const float4_t*>(st_src[i] + static_cast<int64_t>(min(t0 + st_tok[i], T - 1)) * C);
@@ -172,11 +174,15 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
         raw[set][i][0] = fa.r[at]; raw[set][i][1] = fa.k[at]; raw[set][i][2] = fa.a12[at]; raw[set][i][3] = fa.w12[at];
         raw[set][i][4] = fa.g[at];
       }
+      if constexpr (RAW) {
+        rio[set][i][0] = ro_a[at]; rio[set][i][1] = ro_b[at]; rio[set][i][2] = ro_w[at]; rio[set][i][3] = ro_k[at];
+        rio[set][i][4] = ro_r[at];
+      }
     }
   };
   auto commit = [&](int buf, auto set_c) {
     constexpr int set = decltype(set_c)::value;
-    if constexpr (!FUSED) {
+    if constexpr (SRC == kSrcFp32) {
 #pragma unroll
       for (int i = 0; i < kOpSlots; ++i)
         if (st_dst[i] >= 0) *reinterpret_cast<float4_t*>(&ops[buf][0][0][0] + st_dst[i]) = stage[set][i];
@@ -204,6 +210,14 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
           ops[buf][tok][3][lane] = h2f(nk);
           ops[buf][tok][4][lane] = h2f(raw[set][i][0]);
           gs[buf][tok][lane] = h2f(raw[set][i][4]);
+        }
+        if constexpr (RAW) {
+          const float wv = static_cast<float>(rio[set][i][2]);
+          ops[buf][tok][0][lane] = static_cast<float>(rio[set][i][0]);
+          ops[buf][tok][1][lane] = static_cast<float>(rio[set][i][1]);
+          ops[buf][tok][2][lane] = (ro.w_mode == RWKV_W_RAW_LOGIT) ? decay_from_logit(wv) : wv;
+          ops[buf][tok][3][lane] = static_cast<float>(rio[set][i][3]);
+          ops[buf][tok][4][lane] = static_cast<float>(rio[set][i][4]);
         }
       }
     }
@@ -356,76 +370,46 @@ constexpr int kSeqTinyGrid = 64;
 
 bool tmix_seq_whole_heads(int B, int T, int H) { return !(B * H <= kSeqSmallGrid && T > 1); }
 
-template <typename IO, bool FUSED>
+template <typename IO, int SRC>
 static void launch_seq(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                        const float* k, const float* a, const float* b, int64_t op_bs, const IO* v, IO* y, int64_t io_bs,
-                       const TmixSeqArgs& fa) {
-  if constexpr (!FUSED) {
+                       const TmixSeqArgs& fa, const RawOperands& ro) {
+  if constexpr (SRC != kSrcFused) {
     if (B * H <= kSeqTinyGrid && T > 1) {
-      hipLaunchKernelGGL((wkv7_seq_kernel<IO, 1, 4, false>), dim3(B * H * 4), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
-                         op_bs, v, y, io_bs, fa);
+      hipLaunchKernelGGL((wkv7_seq_kernel<IO, 1, 4, SRC>), dim3(B * H * 4), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
+                         op_bs, v, y, io_bs, fa, ro);
       return;
     }
     if (B * H <= kSeqSmallGrid && T > 1) {
-      hipLaunchKernelGGL((wkv7_seq_kernel<IO, 2, 2, false>), dim3(B * H * 2), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
-                         op_bs, v, y, io_bs, fa);
+      hipLaunchKernelGGL((wkv7_seq_kernel<IO, 2, 2, SRC>), dim3(B * H * 2), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
+                         op_bs, v, y, io_bs, fa, ro);
       return;
     }
   }
   if (T == 1) {
-    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, FUSED, false>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
-                       op_bs, v, y, io_bs, fa);
+    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, SRC, false>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b,
+                       op_bs, v, y, io_bs, fa, ro);
   } else {
-    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, FUSED>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs,
-                       v, y, io_bs, fa);
+    hipLaunchKernelGGL((wkv7_seq_kernel<IO, 4, 1, SRC>), dim3(B * H), dim3(256), 0, st, T, C, H, state, r, d, k, a, b, op_bs,
+                       v, y, io_bs, fa, ro);
   }
 }
 
+// The C-ABI operator: operands in the io type, read once by the sequence kernel itself.
 template <typename IO>
 static int launch_wkv7(hipStream_t st, int B, int T, int C, int H, int w_mode, float* state, const IO* r,
                        const IO* w, const IO* k, const IO* v, const IO* a, const IO* b, IO* y) {
   const int64_t row = static_cast<int64_t>(T) * C;
-  if (std::is_same<IO, float>::value && w_mode == RWKV_W_DECAY) {
-    launch_seq<IO, false>(st, B, T, C, H, state, reinterpret_cast<const float*>(r), reinterpret_cast<const float*>(w),
-                          reinterpret_cast<const float*>(k), reinterpret_cast<const float*>(a),
-                          reinterpret_cast<const float*>(b), row, v, y, row, TmixSeqArgs{});
-    RWKV_LAUNCH_CHECK();
-    return RWKV_OK;
-  }
-  // Pre-pass in slabs of tokens so the fp32 workspace stays bounded (5 operands x 256 MiB); the
-  // state carries across slabs in HBM, which keeps the result bitwise independent of the slab size.
-  const int64_t slab_budget = 64ll << 20;  // fp32 elements per operand
-  const int t_slab = static_cast<int>(std::min<int64_t>(T, std::max<int64_t>(1, slab_budget / (static_cast<int64_t>(B) * C))));
-  const int64_t slab_elems = static_cast<int64_t>(B) * t_slab * C;
-  float* ws = nullptr;
-  RWKV_HIP_TRY(hipMallocAsync(reinterpret_cast<void**>(&ws), sizeof(float) * 5 * slab_elems, st));
-  float* r32 = ws;
-  float* d32 = ws + slab_elems;
-  float* k32 = ws + 2 * slab_elems;
-  float* a32 = ws + 3 * slab_elems;
-  float* b32 = ws + 4 * slab_elems;
-  for (int t0 = 0; t0 < T; t0 += t_slab) {
-    const int tn = std::min(t_slab, T - t0);
-    const int64_t off = static_cast<int64_t>(t0) * C;
-    const int64_t slab_row = static_cast<int64_t>(tn) * C;
-    const int64_t n = slab_row * B;
-    hipLaunchKernelGGL(wkv7_prepare_kernel<IO>, dim3(ceil_div(n, 256)), dim3(256), 0, st, n, slab_row, row, w_mode,
-                       r + off, w + off, k + off, a + off, b + off, r32, d32, k32, a32, b32);
-    launch_seq<IO, false>(st, B, tn, C, H, state, r32, d32, k32, a32, b32, slab_row, v + off, y + off, row, TmixSeqArgs{});
-  }
-  hipError_t err = hipGetLastError();
-  hipError_t ferr = hipFreeAsync(ws, st);
-  if (err != hipSuccess || ferr != hipSuccess) {
-    set_error("wkv7 launch failed: %s", hipGetErrorString(err != hipSuccess ? err : ferr));
-    return RWKV_E_RUNTIME;
-  }
+  const RawOperands ro = {r, w, k, a, b, w_mode};
+  launch_seq<IO, kSrcRaw>(st, B, T, C, H, state, nullptr, nullptr, nullptr, nullptr, nullptr, 0, v, y, row, TmixSeqArgs{}, ro);
+  RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
 int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                         const float* k, const float* a, const float* b, int64_t op_bs, const half_t* v, half_t* y,
                         int64_t io_bs) {
-  launch_seq<half_t, false>(st, B, T, C, H, state, r, d, k, a, b, op_bs, v, y, io_bs, TmixSeqArgs{});
+  launch_seq<half_t, kSrcFp32>(st, B, T, C, H, state, r, d, k, a, b, op_bs, v, y, io_bs, TmixSeqArgs{}, RawOperands{});
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
@@ -435,7 +419,8 @@ int tmix_seq_launch(hipStream_t st, int B, int T, int C, int H, float* state, co
   RWKV_REQUIRE(fa.r && fa.k && fa.a12 && fa.w12 && fa.g && fa.k_k && fa.a0 && fa.k_a && fa.w0 && fa.r_k && fa.lnx_w && fa.lnx_b,
                "tmix_seq: NULL tensor");
   const int64_t row = static_cast<int64_t>(T) * C;
-  launch_seq<half_t, true>(st, B, T, C, H, state, nullptr, nullptr, nullptr, nullptr, nullptr, 0, v, y2, row, fa);
+  launch_seq<half_t, kSrcFused>(st, B, T, C, H, state, nullptr, nullptr, nullptr, nullptr, nullptr, 0, v, y2, row, fa,
+                                RawOperands{});
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
