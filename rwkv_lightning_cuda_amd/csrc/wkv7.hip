@@ -4,11 +4,11 @@
 //   sa = sum_j S[i][j]*a[j];  S[i][j] = S[i][j]*d[j] + sa*b[j] + k[j]*v[i];  y[i] = sum_j S[i][j]*r[j]
 // with the decay map d = exp(-e^-1/2 * sigmoid(w)) of :13-14,26-28.
 //
-// Sequence kernel (any T): four wavefronts per (batch, head), each lane keeps a 4 x 4 block of the 64 x 64 state
-// in registers for the whole call.  The per-column operands r,d,k,a,b of a token are staged in LDS as fp32 and
-// each lane reads only the four columns it owns; the two row sums of a step (sa and y) are reduced over the 16
-// lanes that share a row with DPP adds.  Operands must therefore be fp32 with the decay already applied; a small
-// element-wise pre-pass produces them when the caller passes fp16 tensors or raw decay logits.
+// Sequence kernel (any T): four to sixteen wavefronts per (batch, head), each lane keeps a few rows x 4 columns of
+// the 64 x 64 state in registers for the whole call.  The per-column operands r,d,k,a,b of a token are staged in
+// LDS as fp32 and each lane reads only the four columns it owns; the two row sums of a step (sa and y) are
+// reduced over the 16 lanes that share a row with DPP adds.  The staging converts what the caller has (fp16 or
+// fp32 tensors, raw decay logits or decays, or the model's own fp16 rows) on the way into LDS.
 #include <type_traits>
 #include "ops.h"
 
@@ -347,7 +347,8 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
         step_state(q);
         step_out(tt, q);
       }
-      if (t0 > 0) write_out(t0 - kSeqChunk, kSeqChunk, buf ^ 1);  // (nothing follows a partial chunk: no commit)
+      if (t0 > 0) write_out(t0 - kSeqChunk, kSeqChunk, buf ^ 1);
+      if (more) commit(buf ^ 1, Other{});  // (only without the straight-line body: a partial chunk is the last)
     }
     __syncthreads();
   };
