@@ -122,7 +122,7 @@ def test_decode_with_row_skipping_ffn_value(gpu, orc, fmt, B):
 
 
 @pytest.mark.parametrize("fmt", [1, 2])
-@pytest.mark.parametrize("B,T", [(2, 16), (20, 21), (36, 11), (40, 1)])
+@pytest.mark.parametrize("B,T", [(2, 16), (20, 21), (36, 11), (40, 1), (12, 1)])
 def test_fused_launches_match_the_standalone_kernels_bitwise(gpu, fmt, B, T):
     """Two fusions of the row-tiled path are switched off while the residual-stream tap is on.  (1) The LayerNorm
     kernels after the output projection and after ffn.value sum the fp32 split-K partials of the streaming GEMM
