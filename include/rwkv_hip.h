@@ -88,6 +88,16 @@ int rwkv_hip_quantize_w4(rwkv_stream_t s, int N, int K, const void* w_f16, void*
 int rwkv_hip_dequant_w4(rwkv_stream_t s, int N, int K, const void* q, const void* scale, const void* zp,
                         void* w_f16);
 
+/* ---- checkpoint tensors: bf16 in the file, fp16 on the device.  Replace rwkv7_v4_bf16_to_f16_launch,
+ * rwkv7_v4_bf16_to_f16_transpose_launch and rwkv7_v4_emb_ln0_bf16_to_f16_launch
+ * (cuda/rwkv7_fast_v4_kernels.cuh:8-29): widening to fp32 is exact, the fp16 result is rounded to nearest even.
+ * transpose: src [rows,cols] -> dst [cols,rows].  emb_ln0: out[v] = f16(LayerNorm(emb[v]) * weight + bias) with
+ * two-pass fp32 statistics, emb [V,C], weight / bias [C] all bf16. ---- */
+int rwkv_hip_bf16_to_f16(rwkv_stream_t s, int64_t n, const void* src_bf16, void* dst_f16);
+int rwkv_hip_bf16_to_f16_transpose(rwkv_stream_t s, int rows, int cols, const void* src_bf16, void* dst_f16);
+int rwkv_hip_emb_ln0_bf16_to_f16(rwkv_stream_t s, int V, int C, const void* emb_bf16, const void* weight_bf16,
+                                 const void* bias_bf16, float eps, void* out_f16);
+
 /* Synthetic fp16 weights ~ mean + std*N(0,1) from a counter-based hash of (seed, index): random-init
  * models for benchmarks without a checkpoint (no counterpart in the reference, which loads .pth files). */
 int rwkv_hip_fill_normal_f16(rwkv_stream_t s, int64_t n, uint64_t seed, float mean, float stdv, void* out);

@@ -132,6 +132,51 @@ void orc_f16_to_f32_array(const uint16_t* src, float* dst, int64_t n) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Checkpoint tensors, bf16 -> fp16.  cuda/rwkv7_v3a_ops.cu:70-116 (bf16_bits_to_float_dev, bf16_to_f16_kernel,
+// bf16_to_f16_transpose_kernel): the bf16 pattern is the upper half of an fp32, the fp16 is that fp32 rounded to
+// nearest even.  :153-185 (emb_ln0_bf16_to_f16_kernel): per embedding row, mean and variance in fp32 over the
+// widened values (two passes), y = f16((x - mean) * rstd * w + b) with w, b widened from bf16.  Sums run
+// c = 0..C-1 in order (the kernel's own order over 256 threads is not restated: tolerance-level only).
+// ---------------------------------------------------------------------------------------------
+static inline float bf16_widen(uint16_t bits) {
+  const uint32_t wide = static_cast<uint32_t>(bits) << 16;
+  float f;
+  std::memcpy(&f, &wide, sizeof(f));
+  return f;
+}
+
+void orc_bf16_to_f16(int rows, int cols, int transpose, const uint16_t* src, uint16_t* dst) {
+  for (int r = 0; r < rows; ++r) {
+    for (int c = 0; c < cols; ++c) {
+      const uint16_t h = orc_f32_to_f16(bf16_widen(src[static_cast<int64_t>(r) * cols + c]));
+      if (transpose) {
+        dst[static_cast<int64_t>(c) * rows + r] = h;
+      } else {
+        dst[static_cast<int64_t>(r) * cols + c] = h;
+      }
+    }
+  }
+}
+
+void orc_emb_ln0(int V, int C, const uint16_t* emb, const uint16_t* w, const uint16_t* b, float eps, uint16_t* out) {
+  parallel_for(V, [&](int64_t v) {
+    const uint16_t* row = emb + v * C;
+    float sum = 0.0f;
+    for (int c = 0; c < C; ++c) sum += bf16_widen(row[c]);
+    const float mean = sum / static_cast<float>(C);
+    float sq = 0.0f;
+    for (int c = 0; c < C; ++c) {
+      const float d = bf16_widen(row[c]) - mean;
+      sq += d * d;
+    }
+    const float rstd = 1.0f / std::sqrt(sq / static_cast<float>(C) + eps);
+    for (int c = 0; c < C; ++c) {
+      out[v * C + c] = orc_f32_to_f16((bf16_widen(row[c]) - mean) * rstd * bf16_widen(w[c]) + bf16_widen(b[c]));
+    }
+  });
+}
+
+// ---------------------------------------------------------------------------------------------
 // WKV7.  cuda/rwkv7_wkv_fp32_v2.cu:13-14,26-28 (decay map), :100-126 (per-token recurrence of
 // wkv_fp32_v2_kernel): thread i owns state row i;
 //   sa = sum_j S[i][j]*a[j];  S[i][j] = S[i][j]*d[j] + sa*b[j] + k[j]*v[i];  y[i] = sum_j S[i][j]*r[j].

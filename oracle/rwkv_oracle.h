@@ -39,6 +39,11 @@ float orc_f16_to_f32(uint16_t h);
 void orc_f32_to_f16_array(const float* src, uint16_t* dst, int64_t n);
 void orc_f16_to_f32_array(const uint16_t* src, float* dst, int64_t n);
 
+/* checkpoint tensors: bf16 [rows,cols] -> fp16 (round to nearest even), optionally into [cols,rows];
+ * embedding rows through LayerNorm(ln0) (cuda/rwkv7_v3a_ops.cu:70-116,153-185) */
+void orc_bf16_to_f16(int rows, int cols, int transpose, const uint16_t* src, uint16_t* dst);
+void orc_emb_ln0(int V, int C, const uint16_t* emb, const uint16_t* w, const uint16_t* b, float eps, uint16_t* out);
+
 /* ---- WKV7 ---------------------------------------------------------------------------
  * state [B,H,64,64] f32 (row = value index i, column = key index j), in/out.
  * r,w,k,v,a,b,y [B,T,C].  w_mode 0: w is the raw decay logit, decay = exp(-e^-1/2 * sigmoid(w));

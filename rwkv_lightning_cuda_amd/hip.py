@@ -33,7 +33,8 @@ EXPORTS = [
     "rwkv_hip_mem_info", "rwkv_hip_stream_create", "rwkv_hip_stream_destroy", "rwkv_hip_stream_sync",
     "rwkv_hip_device_sync", "rwkv_hip_event_create", "rwkv_hip_event_destroy", "rwkv_hip_event_record",
     "rwkv_hip_event_elapsed_ms", "rwkv_hip_wkv7", "rwkv_hip_quantize_w8", "rwkv_hip_dequant_w8",
-    "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",
+    "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_bf16_to_f16", "rwkv_hip_bf16_to_f16_transpose",
+    "rwkv_hip_emb_ln0_bf16_to_f16", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",
     "rwkv_hip_pack_weights", "rwkv_hip_linear_packed_workspace", "rwkv_hip_linear_packed", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
     "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
     "rwkv_hip_cmix_sparse_down_relu_rows",
@@ -192,6 +193,19 @@ def _ptr_array(items):
 def wkv7(B, T, C, H, w_mode, io, state, r, w, k, v, a, b, y, stream=None):
     check(load().rwkv_hip_wkv7(_p(stream), _i(B), _i(T), _i(C), _i(H), _i(w_mode), _i(io), _p(state), _p(r), _p(w),
                                _p(k), _p(v), _p(a), _p(b), _p(y)))
+
+
+def bf16_to_f16(n, src, dst, stream=None):
+    check(load().rwkv_hip_bf16_to_f16(_p(stream), ctypes.c_int64(n), _p(src), _p(dst)))
+
+
+def bf16_to_f16_transpose(rows, cols, src, dst, stream=None):
+    check(load().rwkv_hip_bf16_to_f16_transpose(_p(stream), _i(rows), _i(cols), _p(src), _p(dst)))
+
+
+def emb_ln0_bf16_to_f16(V, C, emb, weight, bias, eps, out, stream=None):
+    check(load().rwkv_hip_emb_ln0_bf16_to_f16(_p(stream), _i(V), _i(C), _p(emb), _p(weight), _p(bias),
+                                              ctypes.c_float(eps), _p(out)))
 
 
 def quantize_w8(N, K, w, q, scale, stream=None):

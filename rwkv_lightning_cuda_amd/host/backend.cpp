@@ -3,16 +3,21 @@
 // Mirrors ModelBackend in the reference (src/rwkv7_fast_v4.cu:1349-1592): argument checks and their
 // messages, the state layout and zero-initialisation of create_state (:1373-1400), the per-layer strided
 // slice copies of copy_state_slice (:1421-1504), copy_logits_slice (:1506-1532) and the capacity formula of
-// query_prefill_capacity (:1534-1580).  Differences: weights are synthetic random-init (no .pth reader
-// here), only the fp32-state mode exists, device errors throw instead of exiting, and forward passes run
-// through pooled sessions (stream + arena + decode graphs) so concurrent callers do not allocate per call.
+// query_prefill_capacity (:1534-1580), and its load pipeline (:110-701): the checkpoint's bf16 tensors are
+// uploaded as they are and converted on the device (fp16, LoRA matrices transposed, embedding through ln0),
+// the seven big matrices then quantised on load when a weight format is asked for.  Differences: a model_path
+// of the form synthetic:<preset>... builds random-init weights without a file, only the fp32-state mode
+// exists, device errors throw instead of exiting, and forward passes run through pooled sessions (stream +
+// arena + decode graphs) so concurrent callers do not allocate per call.
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
 #include <mutex>
 #include <sstream>
 #include <stdexcept>
 #include <unordered_map>
 
+#include "pth_tensor.hpp"
 #include "rwkv_server_backend.hpp"
 
 namespace rwkv7_server {
@@ -27,6 +32,7 @@ struct Spec {
   int fmt = RWKV_FMT_F16;
   std::uint64_t seed = 1;
   std::string name;
+  std::string checkpoint;  // empty: synthetic weights
 };
 
 ModelDims preset(const std::string& name) {
@@ -49,12 +55,31 @@ ModelDims preset(const std::string& name) {
   return d;
 }
 
+// <file>.pth[:f16|:w8|:w4] - the weight format the big matrices are quantised to on load (default fp16, the
+// reference's only one); the model name is the file stem, as in the reference (src/rwkv7_fast_v4.cu:1353-1362).
+Spec parse_checkpoint_spec(const std::string& path) {
+  Spec spec;
+  spec.checkpoint = path;
+  const std::size_t colon = path.rfind(':');
+  if (colon != std::string::npos) {
+    const std::string tail = path.substr(colon + 1);
+    const int fmt = tail == "f16" ? RWKV_FMT_F16 : tail == "w8" ? RWKV_FMT_W8 : tail == "w4" ? RWKV_FMT_W4 : -1;
+    if (fmt >= 0) {
+      spec.fmt = fmt;
+      spec.checkpoint = path.substr(0, colon);
+    }
+  }
+  const std::size_t slash = spec.checkpoint.find_last_of('/');
+  std::string stem = slash == std::string::npos ? spec.checkpoint : spec.checkpoint.substr(slash + 1);
+  const std::size_t dot = stem.rfind('.');
+  if (dot != std::string::npos && dot > 0) stem.resize(dot);
+  spec.name = stem;
+  return spec;
+}
+
 Spec parse_spec(const std::string& path) {
   const std::string prefix = "synthetic:";
-  if (path.compare(0, prefix.size(), prefix) != 0) {
-    throw std::runtime_error(
-        "this backend has no checkpoint reader: model_path must be synthetic:<preset>[:f16|w8|w4][:seed=<n>], got " + path);
-  }
+  if (path.compare(0, prefix.size(), prefix) != 0) return parse_checkpoint_spec(path);
   Spec spec;
   std::stringstream ss(path.substr(prefix.size()));
   std::string part;
@@ -89,12 +114,16 @@ struct ModelBackend::Impl {
   rwkv_hip_model* model = nullptr;
   std::vector<DeviceBuffer<std::uint8_t>> storage;  // owns every weight tensor
   std::uint64_t fill_counter = 0;
+  std::string archive_folder;       // "<folder>/data.pkl" names the checkpoint's top folder
+  void* pinned = nullptr;           // host staging of the checkpoint loader
+  std::size_t pinned_bytes = 0;
 
   mutable std::mutex pool_mutex;
   mutable std::vector<rwkv_hip_session*> idle_sessions;
 
   ~Impl() {
     for (auto* s : idle_sessions) rwkv_hip_session_destroy(s);
+    if (pinned) rwkv_hip_host_free(pinned);
     if (model) rwkv_hip_model_destroy(model);
   }
 
@@ -112,8 +141,10 @@ struct ModelBackend::Impl {
     return p;
   }
 
-  void set_matrix(int layer, int id, int N, int K) {
-    void* w16 = fill(static_cast<std::size_t>(N) * K, 0.0f, 0.02f);
+  void set_matrix(int layer, int id, int N, int K) { install_matrix(layer, id, N, K, fill(static_cast<std::size_t>(N) * K, 0.0f, 0.02f)); }
+
+  // w16: fp16 [N,K] in `storage`; kept as the weight for fp16, else quantised on the device and released
+  void install_matrix(int layer, int id, int N, int K, void* w16) {
     if (spec.fmt == RWKV_FMT_F16) {
       check_hip(rwkv_hip_model_set_matrix(model, layer, id, RWKV_FMT_F16, w16, nullptr, nullptr), "set matrix");
       return;
@@ -138,6 +169,210 @@ struct ModelBackend::Impl {
         break;
       }
     }
+  }
+
+  // ---- checkpoint ------------------------------------------------------------------------------------------
+  [[noreturn]] static void load_error(const std::string& what) { throw std::runtime_error("load model: " + what); }
+
+  // The tensor's bf16 patterns in logical order on the device (a temporary the caller releases with the sync
+  // after its conversion kernel).
+  DeviceBuffer<std::uint16_t> upload_bf16(const llm_infer::PthArchive& archive, const llm_infer::TensorRecord& rec) {
+    // Row-major tensors (all of a normal checkpoint): the byte range goes from the file into a pinned buffer and
+    // from there to the device, no per-element pass on the host.
+    std::uint64_t n = 1;
+    std::int64_t expect = 1;
+    bool dense = rec.shape.size() == rec.stride.size();
+    for (std::size_t i = rec.shape.size(); dense && i-- > 0;) {
+      if (rec.shape[i] < 0) dense = false;
+      if (rec.shape[i] != 1 && rec.stride[i] != expect) dense = false;
+      expect *= rec.shape[i];
+      n *= static_cast<std::uint64_t>(rec.shape[i]);
+    }
+    const llm_infer::PthEntry* entry = dense && n > 0 ? archive.find_entry(archive_folder + "/data/" + rec.storage_key) : nullptr;
+    if (entry != nullptr && entry->is_stored() && entry->uncompressed_size == rec.storage_size * 2 &&
+        rec.storage_offset + n <= rec.storage_size) {
+      const std::size_t bytes = static_cast<std::size_t>(n) * 2;
+      if (bytes > pinned_bytes) {
+        if (pinned) check_hip(rwkv_hip_host_free(pinned), "free pinned staging");
+        pinned = nullptr;
+        pinned_bytes = 0;
+        check_hip(rwkv_hip_host_alloc(&pinned, bytes), "alloc pinned staging");
+        pinned_bytes = bytes;
+      }
+      llm_infer::Status rd = archive.read_stored_entry_range(*entry, rec.storage_offset * 2, pinned, bytes);
+      if (!rd.ok_status()) load_error(rd.message());
+      DeviceBuffer<std::uint16_t> dev;
+      dev.resize(static_cast<std::size_t>(n), "alloc bf16 staging");
+      check_hip(rwkv_hip_memcpy_h2d(dev.p, pinned, bytes), "copy bf16 weight");
+      return dev;
+    }
+    auto data = llm_infer::load_bf16_tensor_select(archive, rec, true, false, false);
+    if (!data.ok()) load_error(data.status().message());
+    DeviceBuffer<std::uint16_t> dev;
+    dev.resize(data.value().values_bf16.size(), "alloc bf16 staging");
+    if (dev.n) {
+      check_hip(rwkv_hip_memcpy_h2d(dev.p, data.value().values_bf16.data(), dev.n * sizeof(std::uint16_t)), "copy bf16 weight");
+    }
+    return dev;
+  }
+
+  // fp16 copy of a checkpoint tensor in `storage`: elements as they are, or a [rows,cols] matrix into [cols,rows]
+  void* convert(const llm_infer::PthArchive& archive, const llm_infer::TensorRecord& rec, std::size_t elems, int t_rows,
+                int t_cols) {
+    std::size_t n = 1;
+    for (std::int64_t d : rec.shape) n *= static_cast<std::size_t>(d);
+    if (n != elems) {
+      load_error("tensor " + rec.name + " has shape " + llm_infer::shape_string(rec.shape) + ", expected " +
+                 std::to_string(elems) + " elements");
+    }
+    if (t_rows > 0 && (rec.shape.size() != 2 || rec.shape[0] != t_rows || rec.shape[1] != t_cols)) {
+      load_error("tensor " + rec.name + " has shape " + llm_infer::shape_string(rec.shape) + ", expected [" +
+                 std::to_string(t_rows) + "," + std::to_string(t_cols) + "]");
+    }
+    DeviceBuffer<std::uint16_t> raw = upload_bf16(archive, rec);
+    void* out = alloc(elems * sizeof(half), "alloc weight tensor");
+    if (t_rows > 0) {
+      check_hip(rwkv_hip_bf16_to_f16_transpose(nullptr, t_rows, t_cols, raw.p, out), "bf16 -> f16 transpose");
+    } else {
+      check_hip(rwkv_hip_bf16_to_f16(nullptr, static_cast<int64_t>(elems), raw.p, out), "bf16 -> f16");
+    }
+    check_hip(rwkv_hip_device_sync(), "sync weight preprocess");  // raw is released on return
+    return out;
+  }
+
+  void load_checkpoint(bool chunk_load) {
+    auto opened = llm_infer::PthArchive::open(spec.checkpoint, chunk_load);
+    if (!opened.ok()) load_error(opened.status().message());
+    const llm_infer::PthArchive& archive = opened.value();
+    auto parsed = llm_infer::parse_pth_tensor_records(archive);
+    if (!parsed.ok()) load_error(parsed.status().message());
+    for (const auto& e : archive.entries()) {
+      static const std::string kTail = "/data.pkl";
+      if (e.name.size() >= kTail.size() && e.name.compare(e.name.size() - kTail.size(), kTail.size(), kTail) == 0) {
+        archive_folder = e.name.substr(0, e.name.size() - kTail.size());
+        break;
+      }
+    }
+    std::unordered_map<std::string, const llm_infer::TensorRecord*> by_name;
+    for (const auto& rec : parsed.value()) by_name[rec.name] = &rec;
+    auto find = [&](const std::string& name) -> const llm_infer::TensorRecord* {
+      auto it = by_name.find(name);
+      return it == by_name.end() ? nullptr : it->second;
+    };
+    auto need = [&](const std::string& name) -> const llm_infer::TensorRecord& {
+      const llm_infer::TensorRecord* rec = find(name);
+      if (rec == nullptr) load_error("missing tensor: " + name);
+      return *rec;
+    };
+
+    // dimensions from tensor shapes (infer_model_dims, include/rwkv7_fast_v4_common.hpp:262-288; LoRA ranks from
+    // the rank-in matrices, src/rwkv7_fast_v4.cu:1168-1172)
+    ModelDims d;
+    for (const auto& rec : parsed.value()) {
+      if (rec.name.compare(0, 7, "blocks.") == 0) {
+        char* end = nullptr;
+        const long layer = std::strtol(rec.name.c_str() + 7, &end, 10);
+        if (end && *end == '.' && layer >= 0) d.layers = std::max(d.layers, static_cast<int>(layer) + 1);
+      }
+    }
+    if (const auto* emb = find("emb.weight"); emb && emb->shape.size() == 2) {
+      d.vocab = static_cast<int>(emb->shape[0]);
+      d.channels = static_cast<int>(emb->shape[1]);
+    }
+    if (const auto* rk = find("blocks.0.att.r_k"); rk && rk->shape.size() == 2) {
+      d.heads = static_cast<int>(rk->shape[0]);
+      d.head_size = static_cast<int>(rk->shape[1]);
+    }
+    if (const auto* key = find("blocks.0.ffn.key.weight"); key && key->shape.size() == 2) d.ffn = static_cast<int>(key->shape[0]);
+    if (!(d.layers > 0 && d.channels > 0 && d.heads > 0 && d.head_size > 0 && d.vocab > 0 && d.ffn > 0)) {
+      load_error("could not infer model dimensions");
+    }
+    if (d.channels != d.heads * d.head_size) load_error("C must equal H*N");
+    if (d.head_size != 64) load_error("current kernels require head size 64");
+    auto rank_of = [&](const std::string& name) {
+      const llm_infer::TensorRecord* rec = find(name);
+      if (rec == nullptr || rec->shape.size() != 2 || rec->shape[0] != d.channels) load_error("missing or misshapen tensor: " + name);
+      if (rec->shape[1] <= 0 || rec->shape[1] > 512) load_error("LoRA rank of " + name + " must be in 1..512");
+      return static_cast<int>(rec->shape[1]);
+    };
+    d.rank_w = rank_of("blocks.0.att.w1");
+    d.rank_a = rank_of("blocks.0.att.a1");
+    d.rank_g = rank_of("blocks.0.att.g1");
+    d.rank_v = rank_of(d.layers > 1 ? "blocks.1.att.v1" : "blocks.0.att.v1");
+    spec.dims = d;
+
+    check_hip(rwkv_hip_model_create(&model, d.layers, d.channels, d.heads, d.ffn, d.vocab, d.rank_w, d.rank_a, d.rank_g,
+                                    d.rank_v),
+              "create model");
+    const std::size_t C = static_cast<std::size_t>(d.channels);
+    const int Ci = d.channels;
+    auto vector = [&](int layer, int id, const std::string& name) {
+      check_hip(rwkv_hip_model_set_tensor(model, layer, id, convert(archive, need(name), C, 0, 0)), "set tensor");
+    };
+    auto matrix = [&](int layer, int id, const std::string& name, int N, int K) {
+      const llm_infer::TensorRecord& rec = need(name);
+      if (rec.shape.size() != 2 || rec.shape[0] != N || rec.shape[1] != K) {
+        load_error("tensor " + name + " has shape " + llm_infer::shape_string(rec.shape) + ", expected [" + std::to_string(N) +
+                   "," + std::to_string(K) + "]");
+      }
+      install_matrix(layer, id, N, K, convert(archive, rec, static_cast<std::size_t>(N) * K, 0, 0));
+    };
+
+    {  // embedding rows through ln0, once (build_cpu_emb_ln0_f16, src/rwkv7_fast_v4.cu:450-572)
+      const llm_infer::TensorRecord& emb = need("emb.weight");
+      const llm_infer::TensorRecord& w = need("blocks.0.ln0.weight");
+      const llm_infer::TensorRecord& b = need("blocks.0.ln0.bias");
+      DeviceBuffer<std::uint16_t> emb_raw = upload_bf16(archive, emb);
+      DeviceBuffer<std::uint16_t> w_raw = upload_bf16(archive, w);
+      DeviceBuffer<std::uint16_t> b_raw = upload_bf16(archive, b);
+      if (emb_raw.n != static_cast<std::size_t>(d.vocab) * C || w_raw.n != C || b_raw.n != C) {
+        load_error("emb/ln0 shape mismatch for emb+ln0 preprocessing");
+      }
+      void* out = alloc(emb_raw.n * sizeof(half), "alloc emb+ln0");
+      check_hip(rwkv_hip_emb_ln0_bf16_to_f16(nullptr, d.vocab, Ci, emb_raw.p, w_raw.p, b_raw.p, 1e-5f, out), "emb+ln0 preprocess");
+      check_hip(rwkv_hip_device_sync(), "sync emb+ln0 preprocess");
+      check_hip(rwkv_hip_model_set_tensor(model, -1, RWKV_T_EMB_LN0, out), "set tensor");
+    }
+    vector(-1, RWKV_T_LN_OUT_W, "ln_out.weight");
+    vector(-1, RWKV_T_LN_OUT_B, "ln_out.bias");
+    matrix(-1, RWKV_M_HEAD, "head.weight", d.vocab, Ci);
+
+    struct Named { int id; const char* suffix; };
+    static const Named vectors[] = {
+        {RWKV_T_LN1_W, "ln1.weight"}, {RWKV_T_LN1_B, "ln1.bias"}, {RWKV_T_LN2_W, "ln2.weight"}, {RWKV_T_LN2_B, "ln2.bias"},
+        {RWKV_T_X_R, "att.x_r"}, {RWKV_T_X_W, "att.x_w"}, {RWKV_T_X_K, "att.x_k"}, {RWKV_T_X_V, "att.x_v"},
+        {RWKV_T_X_A, "att.x_a"}, {RWKV_T_X_G, "att.x_g"}, {RWKV_T_W0, "att.w0"}, {RWKV_T_A0, "att.a0"},
+        {RWKV_T_K_K, "att.k_k"}, {RWKV_T_K_A, "att.k_a"}, {RWKV_T_R_K, "att.r_k"}, {RWKV_T_LNX_W, "att.ln_x.weight"},
+        {RWKV_T_LNX_B, "att.ln_x.bias"}, {RWKV_T_FFN_X_K, "ffn.x_k"}};
+    // LoRA pairs: the file has the rank-in as [C,R] and the rank-out as [R,C]; the kernels read both transposed
+    // ("out,in": [R,C] and [C,R] - the reference's `_t` copies, include/rwkv7_fast_v4_common.hpp:326-338)
+    struct Lora { int in_id, out_id; const char* in_name; const char* out_name; int ModelDims::*rank; };
+    static const Lora loras[] = {{RWKV_T_W1, RWKV_T_W2, "att.w1", "att.w2", &ModelDims::rank_w},
+                                 {RWKV_T_A1, RWKV_T_A2, "att.a1", "att.a2", &ModelDims::rank_a},
+                                 {RWKV_T_G1, RWKV_T_G2, "att.g1", "att.g2", &ModelDims::rank_g},
+                                 {RWKV_T_V1, RWKV_T_V2, "att.v1", "att.v2", &ModelDims::rank_v}};
+    for (int l = 0; l < d.layers; ++l) {
+      const std::string p = "blocks." + std::to_string(l) + ".";
+      for (const Named& v : vectors) vector(l, v.id, p + v.suffix);
+      for (const Lora& lo : loras) {
+        const bool value_residual = lo.in_id == RWKV_T_V1;
+        if (value_residual && l == 0) continue;  // unused in the first layer (unused_weight_like_v3a, :318-323)
+        const int R = d.*(lo.rank);
+        check_hip(rwkv_hip_model_set_tensor(model, l, lo.in_id, convert(archive, need(p + lo.in_name), C * R, Ci, R)), "set tensor");
+        check_hip(rwkv_hip_model_set_tensor(model, l, lo.out_id, convert(archive, need(p + lo.out_name), C * R, R, Ci)), "set tensor");
+        if (value_residual) vector(l, RWKV_T_V0, p + "att.v0");
+      }
+      matrix(l, RWKV_M_ATT_R, p + "att.receptance.weight", Ci, Ci);
+      matrix(l, RWKV_M_ATT_K, p + "att.key.weight", Ci, Ci);
+      matrix(l, RWKV_M_ATT_V, p + "att.value.weight", Ci, Ci);
+      matrix(l, RWKV_M_ATT_O, p + "att.output.weight", Ci, Ci);
+      matrix(l, RWKV_M_FFN_KEY, p + "ffn.key.weight", d.ffn, Ci);
+      matrix(l, RWKV_M_FFN_VALUE, p + "ffn.value.weight", Ci, d.ffn);  // the file's own [C,F] layout
+    }
+    check_hip(rwkv_hip_device_sync(), "sync model build");
+    if (pinned) check_hip(rwkv_hip_host_free(pinned), "free pinned staging");
+    pinned = nullptr;
+    pinned_bytes = 0;
   }
 
   void build() {
@@ -209,14 +444,18 @@ struct ModelBackend::Impl {
   }
 };
 
-ModelBackend::ModelBackend(std::string model_path, bool use_wkv32, bool /*chunk_load*/) : impl_(std::make_unique<Impl>()) {
+ModelBackend::ModelBackend(std::string model_path, bool use_wkv32, bool chunk_load) : impl_(std::make_unique<Impl>()) {
   if (!use_wkv32) {
     throw std::runtime_error("this backend provides the fp32 WKV state only: construct it with use_wkv32 = true");
   }
   impl_->model_path = std::move(model_path);
   impl_->spec = parse_spec(impl_->model_path);
   impl_->model_name = impl_->spec.name;
-  impl_->build();
+  if (impl_->spec.checkpoint.empty()) {
+    impl_->build();
+  } else {
+    impl_->load_checkpoint(chunk_load);
+  }
 }
 
 ModelBackend::~ModelBackend() = default;

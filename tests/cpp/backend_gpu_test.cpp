@@ -32,7 +32,7 @@ double cosine(const std::vector<float>& a, const std::vector<float>& b, std::siz
 }  // namespace
 
 HOST_TEST(construction_and_spec_errors) {
-  CHECK_THROWS(ModelBackend("/some/model.pth", true), "no checkpoint reader");
+  CHECK_THROWS(ModelBackend("/some/model.pth", true), "load model: failed to open file");
   CHECK_THROWS(ModelBackend("synthetic:13B", true), "unknown synthetic model preset");
   CHECK_THROWS(ModelBackend("synthetic:tiny:w9", true), "bad synthetic model option");
   CHECK_THROWS(ModelBackend("synthetic:tiny", false), "fp32 WKV state only");

@@ -63,6 +63,24 @@ def f32_to_f16(x):
     return out
 
 
+def bf16_to_f16(bits, transpose=False):
+    """bits: uint16 [rows, cols] of bf16 patterns -> float16 [rows, cols] (or [cols, rows])."""
+    bits = _c(bits, np.uint16)
+    rows, cols = bits.shape
+    out = np.empty((cols, rows) if transpose else (rows, cols), np.float16)
+    lib().orc_bf16_to_f16(rows, cols, int(bool(transpose)), _p(bits), _p(out))
+    return out
+
+
+def emb_ln0(emb_bits, w_bits, b_bits, eps=1e-5):
+    """bf16 patterns (uint16) of the embedding [V,C] and ln0 weight / bias [C] -> float16 [V,C]."""
+    emb_bits = _c(emb_bits, np.uint16)
+    V, C = emb_bits.shape
+    out = np.empty((V, C), np.float16)
+    lib().orc_emb_ln0(V, C, _p(emb_bits), _p(_c(w_bits, np.uint16)), _p(_c(b_bits, np.uint16)), ctypes.c_float(eps), _p(out))
+    return out
+
+
 def f16_to_f32(x):
     x = _c(x, np.float16)
     out = np.empty(x.shape, np.float32)

@@ -104,6 +104,49 @@ def test_wkv7_small_and_large_grids_agree_bitwise(gpu):
         assert same
 
 
+# ------------------------------------------------------------------------------- checkpoint tensors
+def test_bf16_to_f16_every_pattern_and_transposes_bit_exact(gpu, orc):
+    hip = gpu
+    bits = np.arange(65536, dtype=np.uint16).reshape(256, 256)
+    want = orc.bf16_to_f16(bits)
+    out = hip.DeviceArray((256, 256), np.float16)
+    hip.bf16_to_f16(bits.size, dev(hip, bits), out)
+    hip.device_sync()
+    got = out.numpy()
+    nan = np.isnan(want)
+    same = np.array_equal(np.isnan(got), nan) and np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+    assert same
+    # a length that is not a multiple of the 8-element vectors
+    tail = hip.DeviceArray((1003,), np.float16)
+    hip.bf16_to_f16(1003, dev(hip, bits.reshape(-1)[:1003].copy()), tail)
+    for rows, cols in [(37, 70), (64, 16), (1, 200), (96, 33)]:
+        src = np.random.default_rng(rows).integers(0, 0x7f00, (rows, cols)).astype(np.uint16)   # finite values
+        t = hip.DeviceArray((cols, rows), np.float16)
+        hip.bf16_to_f16_transpose(rows, cols, dev(hip, src), t)
+        hip.device_sync()
+        same = np.array_equal(t.numpy().view(np.uint16), orc.bf16_to_f16(src, transpose=True).view(np.uint16))
+        assert same
+    hip.device_sync()
+    same = np.array_equal(tail.numpy().view(np.uint16)[:1000], want.reshape(-1).view(np.uint16)[:1000])
+    assert same
+    with pytest.raises(hip.RwkvHipError):
+        hip.bf16_to_f16_transpose(0, 4, dev(hip, bits), out)
+
+
+def test_emb_ln0_matches_oracle(gpu, orc):
+    hip = gpu
+    rng = np.random.default_rng(21)
+    V, C = 50, 768
+    to_bf16 = lambda a: (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    emb = to_bf16(rng.standard_normal((V, C)))
+    w, b = to_bf16(1 + 0.1 * rng.standard_normal(C)), to_bf16(0.1 * rng.standard_normal(C))
+    out = hip.DeviceArray((V, C), np.float16)
+    hip.emb_ln0_bf16_to_f16(V, C, dev(hip, emb), dev(hip, w), dev(hip, b), 1e-5, out)
+    hip.device_sync()
+    err = rel_err(out.numpy().astype(np.float32), orc.emb_ln0(emb, w, b).astype(np.float32))
+    assert err <= F16_TOL
+
+
 # ------------------------------------------------------------------------------------------- formats
 def test_quantize_dequant_bit_exact(gpu, orc):
     hip = gpu

@@ -479,3 +479,48 @@ def test_chunked_prefill_equals_one_call_in_oracle():
     assert np.array_equal(l1, l2) and np.array_equal(s1[1], s2[1]) and np.array_equal(s1[0], s2[0])
     with pytest.raises(ValueError):
         om.forward(np.array([[dims.V]]), om.new_state(1))
+
+
+# ------------------------------------------------------------------------------- checkpoint tensors (bf16 -> fp16)
+def _bf16_bits_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def test_bf16_to_f16_over_every_pattern_against_numpy():
+    """Widening a bf16 pattern is exact by construction of the format; rounding the fp32 to fp16 is IEEE
+    round-to-nearest-even, which numpy implements independently.  All 65536 patterns, plain and transposed."""
+    bits = np.arange(65536, dtype=np.uint16).reshape(256, 256)
+    with np.errstate(over="ignore"):   # bf16 values beyond 65504 become infinity, as they should
+        want = _bf16_bits_to_f32(bits).astype(np.float16)
+    got = orc.bf16_to_f16(bits)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+    got_t = orc.bf16_to_f16(bits[:37, :70].copy(), transpose=True)
+    assert got_t.shape == (70, 37)
+    keep = ~np.isnan(want[:37, :70].T)
+    assert np.array_equal(got_t.view(np.uint16)[keep], want[:37, :70].T.view(np.uint16)[keep])
+    # inside fp16's normal range a bf16 value has few enough fraction bits to be exact
+    f = _bf16_bits_to_f32(bits)
+    normal = np.isfinite(f) & (np.abs(f) >= 2.0 ** -14) & (np.abs(f) <= 65504.0)
+    assert np.array_equal(got[normal].astype(np.float32), f[normal])
+
+
+def test_emb_ln0_against_float64_and_invariants():
+    rng = np.random.default_rng(20)
+    V, C = 19, 192
+    to_bf16 = lambda a: (a.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)  # truncation: still a bf16 value
+    emb, w, b = to_bf16(rng.standard_normal((V, C))), to_bf16(1 + 0.1 * rng.standard_normal(C)), to_bf16(0.1 * rng.standard_normal(C))
+    e64, w64, b64 = (f64(_bf16_bits_to_f32(a)) for a in (emb, w, b))
+    mu = e64.mean(axis=1, keepdims=True)
+    var = ((e64 - mu) ** 2).mean(axis=1, keepdims=True)
+    want = (e64 - mu) / np.sqrt(var + 1e-5) * w64 + b64
+    got = f64(orc.emb_ln0(emb, w, b))
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1e-2)) <= 1.5e-3           # fp16 rounding of the result
+    # weight 1, bias 0: every row comes out with mean 0 and variance 1 (up to eps and fp16 rounding)
+    one, zero = to_bf16(np.ones(C)), to_bf16(np.zeros(C))
+    plain = f64(orc.emb_ln0(emb, one, zero))
+    assert np.max(np.abs(plain.mean(axis=1))) <= 2e-3 and np.max(np.abs(plain.var(axis=1) - 1)) <= 5e-3
+    # a constant row has no variance: the output is the bias
+    const = to_bf16(np.full((2, C), 3.0))
+    assert np.array_equal(orc.emb_ln0(const, w, b), np.broadcast_to(_bf16_bits_to_f32(b).astype(np.float16), (2, C)))
