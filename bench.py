@@ -259,6 +259,18 @@ def main():
                                     # at M = 128 the launches are weight-streaming bound: the same time against HBM
                                     "weights_gb_s": model.weight_bytes() / (total_ms * 1e-3) / 1e9,
                                     "hbm_frac": model.weight_bytes() / (total_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+            # the same prompt in chunks of 512 (the chunk width is the caller's choice: wider chunks stream the
+            # weights once per 512 tokens), into a scratch state
+            wide = State(dims, B)
+            sess.forward(prompt[:, :min(512, args.prefill)], wide, logits)
+            hip.device_sync()
+            tw = time.perf_counter()
+            for t0 in range(0, args.prefill, 512):
+                sess.forward(prompt[:, t0:t0 + 512], wide, logits, sync=False)
+            hip.device_sync()
+            tw = time.perf_counter() - tw
+            also["prefill_chunk512_tok_s"] = B * args.prefill / tw
+            del wide
     first = rng.integers(0, dims.V, (B,))
 
     if args.warmup > 0:
