@@ -446,6 +446,179 @@ __global__ __launch_bounds__(64 * WG * KG) void gemm_stream_kernel(StreamArgs g)
   }
 }
 
+// ---- many rows: 128 rows x 256 columns per block, two bands per wavefront -------------------------------------------
+// From a few hundred rows on the product is bound by the matrix core and by LDS, not by the weights: with one band
+// per wavefront every MFMA needs its own 1 KiB X fragment from LDS, and LDS delivers 128 bytes per clock against
+// 32 clocks per MFMA and SIMD - four wavefronts saturate both at once.  Here a wavefront keeps two 32-column bands
+// (wave w: bands w and w + 4 of the block), so each X fragment feeds two MFMAs and a block reads X from L2 half as
+// often.  One group of four wavefronts, one wavefront per SIMD (128 accumulator registers per lane); int8 and
+// fp16 weights (the int4 path would double the accumulators once more and stays on the narrower tile).
+template <int FMT>
+__device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const StreamProblem& pr, int row_tile, int col_block,
+                                                  int split, half_t* xs) {
+  constexpr int MT = 4, KC = 128, NB = 2;
+  using T = Tile<FMT, MT, KC, 4>;
+  using P = typename T::P;
+  constexpr int BM = T::BM;
+  static_assert(FMT != RWKV_FMT_W4, "the wide tile takes int8 and fp16 weights");
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int j = lane & 31;
+  const int h = lane >> 5;
+  const int m0 = row_tile * BM;
+  const int kbeg = split * g.k_per_split;
+  const int nchunks = g.k_per_split / KC;
+
+  bool active[NB];
+  int n[NB];
+  const uint4_t* wband[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int band_here = col_block * (4 * NB) + nb * 4 + wave;
+    active[nb] = band_here * 32 < pr.N;
+    const int band = active[nb] ? band_here : pr.N / 32 - 1;  // past the last band: repeat it, store nothing
+    n[nb] = band * 32 + j;
+    wband[nb] = pr.wp + (static_cast<int64_t>(band) * (g.K / T::G)) * (P::PIECES * 64) + lane;
+  }
+
+  float16_t acc[NB][MT];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[nb][mt][v] = 0.0f;
+
+  constexpr int D = FMT == RWKV_FMT_F16 ? 2 : 3;  // weight register sets per band
+  WRegs<FMT, MT, KC> wr[D][NB];
+  XRegs<FMT, MT, KC, 4> xr;  // one chunk ahead: a chunk is 64 MFMAs per wavefront, longer than a trip to L2
+  const int last = nchunks - 1;
+  xr.request(g, pr, tid, m0, kbeg);
+#pragma unroll
+  for (int i = 0; i < D - 1; ++i)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) wr[i][nb].request(g, pr, kbeg + min(i, last) * KC, wband[nb], n[nb]);
+  xr.store_x(tid, xs);
+  __syncthreads();
+
+  constexpr int NK = T::GROUPS * T::STEPS;
+  auto multiply = [&](const half_t* tile, const WRegs<FMT, MT, KC> (&w)[NB]) {
+    const half_t* xlane = tile + j * T::XSTRIDE + h * P::KR;
+    half8_t a[2][MT];
+    auto load_a = [&](int ks, half8_t (&dst)[MT]) {
+      const half_t* xa = xlane + (ks / T::STEPS) * T::G + 8 * (ks % T::STEPS);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) dst[mt] = *reinterpret_cast<const half8_t*>(xa + mt * 32 * T::XSTRIDE);
+    };
+    load_a(0, a[0]);
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      const int gi = ks / T::STEPS;
+      const int st = ks % T::STEPS;
+      if (ks + 1 < NK) load_a(ks + 1, a[(ks + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        half8_t b;
+        if constexpr (FMT == RWKV_FMT_F16) {
+          b = __builtin_bit_cast(half8_t, w[nb].w[gi * 2 + st]);
+        } else {
+          const uint4_t piece = w[nb].w[gi];
+          b = st == 0 ? expand_w8(piece[0], piece[1]) : expand_w8(piece[2], piece[3]);
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nb][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks & 1][mt], b, acc[nb][mt], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  constexpr int U = (D % 2 == 0) ? D : 2 * D;
+  for (int c0 = 0; c0 < nchunks; c0 += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      if (c >= nchunks) break;
+      xr.request(g, pr, tid, m0, kbeg + (c + 1 <= last ? c + 1 : c) * KC);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        wr[(u + D - 1) % D][nb].request(g, pr, kbeg + (c + D - 1 <= last ? c + D - 1 : c) * KC, wband[nb], n[nb]);
+      multiply(xs + (u & 1) * T::kTileHalfs, wr[u % D]);
+      xr.store_x(tid, xs + ((u + 1) & 1) * T::kTileHalfs);
+      __syncthreads();
+    }
+  }
+
+  // output: one 128-column half of the tile at a time through LDS (the X tiles are free), written in 16/32-byte
+  // pieces along the rows
+  constexpr int kStageLd = 128 + 8;
+  static_assert(BM * kStageLd * 4 <= 2 * T::kTileHalfs * 2, "epilogue tile exceeds the LDS tiles");
+  float* stage = reinterpret_cast<float*>(xs);
+  const bool partial_out = g.splits > 1;
+  float* part_out = partial_out ? pr.partial + static_cast<int64_t>(split) * g.M * pr.N : nullptr;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    if (nb > 0) __syncthreads();  // the previous half has been read
+    float scl = 1.0f;
+    if constexpr (FMT == RWKV_FMT_W8) {
+      if (!partial_out) scl = h2f(pr.scale[n[nb]]);
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float sum = acc[nb][mt][v];
+        const int row = mt * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        stage[row * kStageLd + wave * 32 + j] = partial_out ? sum : finish_value(mul_f32(sum, scl), g.epilogue);
+      }
+    __syncthreads();
+    const int col0 = col_block * (128 * NB) + nb * 128;
+    for (int idx = tid; idx < BM * 16; idx += 256) {
+      const int row = idx >> 4;
+      const int piece = idx & 15;
+      const int col = col0 + piece * 8;
+      if (m0 + row >= g.M || col >= pr.N) continue;
+      const float4_t lo = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + piece * 8);
+      const float4_t hi = *reinterpret_cast<const float4_t*>(stage + row * kStageLd + piece * 8 + 4);
+      const int64_t o = static_cast<int64_t>(m0 + row) * pr.N + col;
+      if (partial_out || g.out_f32) {
+        float* dst = partial_out ? part_out + o : static_cast<float*>(pr.y) + o;
+        *reinterpret_cast<float4_t*>(dst) = lo;
+        *reinterpret_cast<float4_t*>(dst + 4) = hi;
+      } else {
+        half8_t hv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          hv[e] = f2h(lo[e]);
+          hv[4 + e] = f2h(hi[e]);
+        }
+        *reinterpret_cast<half8_t*>(static_cast<half_t*>(pr.y) + o) = hv;
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void gemm_stream_wide_kernel(StreamArgs g) {
+  __shared__ __align__(16) half_t xs[2 * 128 * (128 + 8)];
+  const int id = blockIdx.x;
+  const int row_tile = (id >> 3) % g.row_tiles;
+  const int pair = (id / (8 * g.row_tiles)) * 8 + (id & 7);
+  if (pair >= g.col_blocks * g.splits) return;
+  const int col_all = pair % g.col_blocks;
+  const int split = pair / g.col_blocks;
+  int pi = 0;
+  while (pi + 1 < g.n_problems && col_all >= g.block_end[pi]) ++pi;
+  const int col_block = col_all - (pi > 0 ? g.block_end[pi - 1] : 0);
+  const StreamProblem& pr = g.p[pi];
+  if (pr.fmt == RWKV_FMT_W8) {
+    stream_block_wide<RWKV_FMT_W8>(g, pr, row_tile, col_block, split, xs);
+  } else {
+    stream_block_wide<RWKV_FMT_F16>(g, pr, row_tile, col_block, split, xs);
+  }
+}
+
 struct ReduceProblem {
   const float4_t* partial;
   const half_t* scale;  // NULL unless the problem's weights are int8 codes
@@ -518,16 +691,30 @@ static int target_blocks() {
 // wavefronts - twice the blocks per matrix, so half the split (less partial-sum traffic) or none (no reduce
 // launch): 16 rows x 16384 columns 23.4 -> 19.6 us; decode steps of 8 / 16 / 32 rows 7 / 5 / 3 % faster.  At 64
 // rows the narrow blocks lose (24.5 -> 30 us): every block reads all of X.
+// From 385 rows on, int8 and fp16 weights, when 128 x 256 tiles alone give 128 blocks or more: the wide tile, whose
+// wavefronts feed two MFMAs from every X fragment they read from LDS and whose blocks request half the X bytes per
+// flop (int8 codes, 2048 rows: 16384x4096 436 -> 345 us, 4096x16384 400 -> 317 us; 512 rows x 16384 columns
+// 138 -> 104 us).  With fewer blocks it would need a K split where the 64-row tiles need none (512 rows x 4096
+// columns: 35 us against 42).  Its registers have no room for the int4 codes' zero points.
+constexpr int kWideMinRows = 384, kWideMinBlocks = 128;
 struct StreamConfig {
   int mt, kc, kg, wg;
-  int cols() const { return 32 * wg; }
+  int nb = 1;  // bands per wavefront
+  int cols() const { return 32 * wg * nb; }
 };
-static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns) {
+static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns, const int* fmts) {
   int cb128 = 0;
   for (int i = 0; i < n_problems; ++i) cb128 += ceil_div(Ns[i], 128);
   if (M <= 32 && K % (128 * 4) == 0 && cb128 < target_blocks()) return StreamConfig{1, 128, 4, 2};
   if (M > 32 && M <= 64 && cb128 >= target_blocks()) return StreamConfig{2, 128, 2, 4};
   if (M <= 64) return StreamConfig{1, 128, 2, 4};
+  bool any_w4 = false;
+  int cb256 = 0;
+  for (int i = 0; i < n_problems; ++i) {
+    any_w4 = any_w4 || fmts[i] == RWKV_FMT_W4;
+    cb256 += ceil_div(Ns[i], 256);
+  }
+  if (M > kWideMinRows && !any_w4 && ceil_div(M, 128) * cb256 >= kWideMinBlocks) return StreamConfig{4, 128, 1, 4, 2};
   if (M <= 512) return StreamConfig{2, 128, 2, 4};
   return StreamConfig{4, 128, 1, 4};
 }
@@ -545,12 +732,19 @@ static int choose_splits(const StreamConfig& c, int M, int col_blocks, int K) {
   return splits;
 }
 
+// The formats are not known here: the larger of what the tiles with and without int4 weights would need.
 size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const int* Ns) {
   int64_t n_total = 0;
   for (int i = 0; i < n_problems; ++i) n_total += Ns[i];
-  const StreamConfig c = choose_config(M, K, n_problems, Ns);
-  const int splits = choose_splits(c, M, count_col_blocks(c, n_problems, Ns), K);
-  return splits > 1 ? static_cast<size_t>(splits) * M * n_total * sizeof(float) : 0;
+  int fmts[kMaxProblems];
+  size_t need = 0;
+  for (int fmt : {RWKV_FMT_W8, RWKV_FMT_W4}) {
+    for (int i = 0; i < n_problems && i < kMaxProblems; ++i) fmts[i] = fmt;
+    const StreamConfig c = choose_config(M, K, n_problems, Ns, fmts);
+    const int splits = choose_splits(c, M, count_col_blocks(c, n_problems, Ns), K);
+    if (splits > 1) need = std::max(need, static_cast<size_t>(splits) * M * n_total * sizeof(float));
+  }
+  return need;
 }
 
 size_t linear_packed_workspace_bytes(int M, int N, int K) { return linear_packed_multi_workspace_bytes(M, K, 1, &N); }
@@ -566,9 +760,12 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
   g.K = K;
   g.epilogue = r.epilogue = epilogue;
   g.out_f32 = r.out_f32 = out_f32;
-  int Ns[kMaxProblems];
-  for (int i = 0; i < n_problems; ++i) Ns[i] = problems[i].N;
-  const StreamConfig cfg = choose_config(M, K, n_problems, Ns);
+  int Ns[kMaxProblems], fmts[kMaxProblems];
+  for (int i = 0; i < n_problems; ++i) {
+    Ns[i] = problems[i].N;
+    fmts[i] = problems[i].fmt;
+  }
+  const StreamConfig cfg = choose_config(M, K, n_problems, Ns, fmts);
   int col_blocks = 0;
   for (int i = 0; i < n_problems; ++i) {
     const PackedProblem& q = problems[i];
@@ -607,7 +804,8 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
   const int pairs8 = ceil_div(col_blocks * g.splits, 8) * 8;
   const dim3 grid(g.row_tiles * pairs8);
   const dim3 block(64 * cfg.wg * cfg.kg);
-  if (cfg.wg == 2) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 4, 2>), grid, block, 0, st, g);
+  if (cfg.nb == 2) hipLaunchKernelGGL(gemm_stream_wide_kernel, grid, block, 0, st, g);
+  else if (cfg.wg == 2) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 4, 2>), grid, block, 0, st, g);
   else if (cfg.mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 2, 4>), grid, block, 0, st, g);
   else if (cfg.mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 128, 2, 4>), grid, block, 0, st, g);
   else hipLaunchKernelGGL((gemm_stream_kernel<4, 128, 1, 4>), grid, block, 0, st, g);

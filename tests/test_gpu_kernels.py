@@ -599,9 +599,11 @@ def _quant_parts(orc, hip, fmt, w):
 @pytest.mark.parametrize("fmt_name", ["f16", "w8", "w4"])
 @pytest.mark.parametrize("M,N,K", [(16, 128, 512), (33, 96, 256), (64, 256, 1024), (128, 160, 2048), (200, 64, 768),
                                    (17, 4096, 256), (64, 128, 2560), (600, 256, 1024), (1030, 96, 512),
-                                   (20, 96, 1024), (32, 4160, 512), (5, 64, 2048)])
+                                   (20, 96, 1024), (32, 4160, 512), (5, 64, 2048),
+                                   (1030, 3872, 512), (3000, 2336, 256)])
 def test_linear_packed_matches_oracle(gpu, orc, fmt_name, M, N, K):
-    """Every tile variant (32-, 64- and 128-row tiles; one, two and four wavefront groups; 128- and 64-column blocks;
+    """Every tile variant (32-, 64- and 128-row tiles; one, two and four wavefront groups; 64-, 128- and 256-column
+    blocks - the last two shapes take the 128 x 256 tile for int8 and fp16 weights, once split and once not;
     several row tiles), with and without K splits, chunk counts that are not a power of two, ragged M and column
     counts that are not a multiple of the column block."""
     hip = gpu
