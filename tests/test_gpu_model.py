@@ -79,6 +79,34 @@ def test_small_model_prefill_and_decode(gpu, orc, fmt):
     sess.close()
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_many_row_prefill_chunk_on_the_wide_gemm_tile(gpu, orc, fmt):
+    """13 sequences x 128 tokens = 1664 rows: the r/k/v + rank-in launch (seven problems, int8 or fp16 next to fp16,
+    column counts of 512 and 32..64) has 13 x 10 tiles of 128 x 256 and takes the two-band tile; the other launches
+    stay on the 64- and 128-row tiles."""
+    from rwkv_lightning_cuda_amd.model import ModelDims, Session, State
+    hip = gpu
+    dims = ModelDims(L=1, C=512, H=8, F=2048, V=256, Rw=32, Ra=32, Rg=64, Rv=32)
+    omodel, gmodel = build_pair(gpu, orc, dims, fmt, seed=33)
+    B, T = 13, 128
+    tokens = np.random.default_rng(8).integers(0, dims.V, (B, T))
+    sess = Session(gmodel)
+    gstate = State(dims, B)
+    glogits = hip.DeviceArray((B, dims.V), np.float32)
+    sess.forward(tokens, gstate, glogits)
+    ostate = omodel.new_state(B)
+    ologits = omodel.forward(tokens, ostate)
+    err = cosine(glogits.numpy(), ologits)
+    assert err >= 0.9995
+    err = rel_err(glogits.numpy(), ologits)
+    assert err <= 4e-3
+    err = rel_err(gstate.wkv.numpy(), ostate[1])
+    assert err <= 1e-3
+    err = rel_err(gstate.shift.numpy().astype(np.float32), ostate[0].astype(np.float32))
+    assert err <= 2e-3
+    sess.close()
+
+
 @pytest.mark.parametrize("fmt,B", [(0, 1), (1, 1), (1, 3)])
 def test_decode_with_row_skipping_ffn_value(gpu, orc, fmt, B):
     """Decode steps of an fp16 or W8 model with the row-skipping ffn.value product (one row by default, up to 12 by
