@@ -145,15 +145,33 @@ def secondary_measurements(hip, model, dims, rng):
         sess.close()
         del state, logits
 
-    # WKV7 op alone: fp16 r,w,k,v,a,b [B,T,C], fp32 state, raw-logit decay, one call
-    Bw, Tw, H = 16, 2048, dims.H
+    # WKV7 op alone at the long-context configuration: fp16 r,w,k,v,a,b [16,16384,4096], fp32 state, raw-logit
+    # decay, one call.  Rows are 4096-token windows of one host-generated sequence (r,k,v ~ N(0,1); decay =
+    # exp(-exp(U(-6,-0.5))) given as its raw logit; kk = k/|k| per head, a = -kk, b = kk * sigmoid(U(-3,3))).
+    Bw, Tw, H, seg = 16, 16384, dims.H, 4096
     C = H * 64
     n = Bw * Tw * C
+    n_win = Bw * (Tw // seg)
+    base_T = seg + 64 * (n_win - 1)
+    g = np.random.default_rng(11)
+    kf = g.standard_normal((base_T, H, 64)).astype(np.float32)
+    kk = kf / np.linalg.norm(kf, axis=-1, keepdims=True)
+    sg = np.exp(g.uniform(-6.0, -0.5, (base_T, C)).astype(np.float32) + np.float32(0.5))
+    host = [g.standard_normal((base_T, C)).astype(np.float16), np.log(sg / (1.0 - sg)).astype(np.float16),
+            kf.reshape(base_T, C).astype(np.float16), g.standard_normal((base_T, C)).astype(np.float16),
+            (-kk).reshape(base_T, C).astype(np.float16),
+            (kk.reshape(base_T, C) / (1.0 + np.exp(-g.uniform(-3.0, 3.0, (base_T, C)).astype(np.float32)))).astype(np.float16)]
+    del kf, kk, sg
     bufs = []
-    for i in range(7):
+    for h in host:
+        src = hip.DeviceArray.from_numpy(h)
         d = hip.DeviceArray((Bw, Tw, C), np.float16)
-        hip.fill_normal_f16(n, 100 + i, 0.0, 0.5, d)
+        for w_i in range(n_win):
+            d.view(w_i * seg * C, (seg, C)).copy_from(src.view(64 * w_i * C, (seg, C)))
+        src.free()
         bufs.append(d)
+    del host
+    bufs.append(hip.DeviceArray((Bw, Tw, C), np.float16))
     wstate = hip.DeviceArray.zeros((Bw, H, 64, 64), np.float32)
     r, w, k, v, a, b, y = bufs
     hip.wkv7(Bw, Tw, C, H, hip.W_RAW_LOGIT, hip.IO_F16, wstate, r, w, k, v, a, b, y)
@@ -168,7 +186,8 @@ def secondary_measurements(hip, model, dims, rng):
     res["wkv7_op"] = {"workload": "B=%d T=%d H=%d N=64, fp16 io, fp32 state, one call (average of 3)" % (Bw, Tw, H),
                       "tok_s": Bw * Tw / (ms * 1e-3), "ms": ms,
                       "fp32_tflops": Bw * Tw * H * 10.0 * 64 * 64 / (ms * 1e-3) / 1e12,
-                      "io_gb_s": n * 7 * 2 / (ms * 1e-3) / 1e9, "us_per_token_step": ms * 1e3 / Tw}
+                      "io_gb_s": n * 7 * 2 / (ms * 1e-3) / 1e9, "us_per_token_step": ms * 1e3 / Tw,
+                      "outputs_finite": bool(np.isfinite(y.view(0, (Tw, C)).numpy().astype(np.float32)).all())}
     for d in bufs:
         d.free()
 

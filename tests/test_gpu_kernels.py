@@ -724,3 +724,58 @@ def test_wkv7_long_chunked_resume_through_host_slab_is_bitwise(gpu):
     assert same
     finite = bool(np.isfinite(y.numpy().astype(np.float32)).all())
     assert finite
+
+
+def test_wkv7_config4_full_size_chunked_resume_is_bitwise(gpu):
+    """Benchmark configuration 4 at its full size: B = 16, T = 16384, H = 64, fp16 r,w,k,v,a,b (2.1 GB each), fp32
+    state.  The rows are windows of one host-generated sequence with the configuration-0 distributions, copied on
+    the device.  The sequence run as 128 chunks of 128 tokens, with the state slab taken to the host and resumed from
+    a fresh device buffer every 4096 tokens, must give the outputs and the final state of the single uninterrupted
+    call bit for bit; the outputs stay finite over the whole length."""
+    hip = gpu
+    B, T, H, chunk = 16, 16384, 64, 128
+    C = H * 64
+    seg = 4096
+    n_win = B * (T // seg)
+    base_T = seg + 64 * (n_win - 1)
+    t = wkv_inputs(1, base_T, H, seed=11, dtype=np.float16)
+    names = ("r", "w_raw", "k", "v", "a", "b")
+    base = [dev(hip, t[n]) for n in names]
+    del t
+    ops = [hip.DeviceArray((B, T, C), np.float16) for _ in names]
+    for b in range(B):
+        for q in range(T // seg):
+            start = 64 * (b * (T // seg) + q)
+            for src, dst in zip(base, ops):
+                dst.view((b * T + q * seg) * C, (seg, C)).copy_from(src.view(start * C, (seg, C)))
+    for d in base:
+        d.free()
+
+    s_full = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y_full = hip.DeviceArray((B, T, C), np.float16)
+    hip.wkv7(B, T, C, H, hip.W_RAW_LOGIT, hip.IO_F16, s_full, *ops, y_full)
+    hip.device_sync()
+
+    state = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y = hip.DeviceArray((B, T, C), np.float16)
+    stage = [hip.DeviceArray((B, chunk, C), np.float16) for _ in names]
+    y_stage = hip.DeviceArray((B, chunk, C), np.float16)
+    for t0 in range(0, T, chunk):
+        if t0 and t0 % seg == 0:                  # checkpoint: slab to the host, resume from a fresh allocation
+            slab = state.numpy()
+            state = hip.DeviceArray.from_numpy(slab)
+        for b in range(B):
+            for src, dst in zip(ops, stage):
+                dst.view(b * chunk * C, (chunk, C)).copy_from(src.view((b * T + t0) * C, (chunk, C)))
+        hip.wkv7(B, chunk, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state, *stage, y_stage)
+        for b in range(B):
+            y.view((b * T + t0) * C, (chunk, C)).copy_from(y_stage.view(b * chunk * C, (chunk, C)))
+    hip.device_sync()
+    for b in range(B):
+        got = y.view(b * T * C, (T, C)).numpy()
+        same = np.array_equal(got.view(np.uint16), y_full.view(b * T * C, (T, C)).numpy().view(np.uint16))
+        assert same, "batch row %d" % b
+        finite = bool(np.isfinite(got.astype(np.float32)).all())
+        assert finite, "batch row %d" % b
+    same = np.array_equal(state.numpy().view(np.uint32), s_full.numpy().view(np.uint32))
+    assert same
