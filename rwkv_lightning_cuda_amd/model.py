@@ -266,8 +266,9 @@ class Session:
         return out
 
     def set_fused_ln(self, on):
-        """Decode steps fold LayerNorm + token shift into the linear launches (bitwise the same; default off)."""
-        hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(1 if on else 0)))
+        """Decode steps fold LayerNorm + token shift into the linear launches (bitwise the same): True always, False
+        never, None (the default of a new session) for one row of at most 2048 channels."""
+        hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(-1 if on is None else 1 if on else 0)))
 
     def set_sparse_ffn(self, max_rows):
         """Decode steps of up to max_rows rows (0..12; True = 1, False = 0) read only the ffn.value rows with a
