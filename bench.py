@@ -17,6 +17,7 @@ whole-job tokens/s plus
                   and the WKV7 op alone on a long sequence.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -121,11 +122,33 @@ def cpu_baseline(dims, fmt_name):
     }
 
 
+def sampled_decode(hip, sess, dims, state, logits, B, first, steps=64):
+    """The decode loop a server runs: forward, then the device sampler (repetition penalties, temperature, top-k,
+    top-p) on the session stream, then the picked token ids back to the host, every step."""
+    penalties = hip.DeviceArray.zeros((B, dims.V), np.float32)
+    probs = hip.DeviceArray((B, dims.V), np.float32)
+    picked = hip.DeviceArray((B,), np.int32)
+    stream = sess.stream
+    lib = hip.load()
+    kw = dict(presence=0.5, frequency=0.1, decay=0.99, temperature=1.0, top_k=50, top_p=0.6, seed=3, stream=stream)
+    tok = np.asarray(first, np.int64).reshape(B, 1)
+    for phase_steps in (4, steps):
+        hip.device_sync()
+        t0 = time.perf_counter()
+        for i in range(phase_steps):
+            sess.forward(tok, state, logits, sync=False)
+            hip.sample(B, dims.V, logits, penalties, probs, picked, step=i, **kw)
+            hip.check(lib.rwkv_hip_stream_sync(ctypes.c_void_p(stream)))
+            tok = picked.numpy().astype(np.int64).reshape(B, 1)
+        dt = time.perf_counter() - t0
+    return {"decode_sampled_bs%d_tok_s" % B: steps * B / dt, "decode_sampled_bs%d_ms_per_step" % B: dt * 1e3 / steps}
+
+
 def secondary_measurements(hip, model, dims, rng):
     """Batch-8, -16 and -64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7 op alone."""
     from rwkv_lightning_cuda_amd.model import Session, State
     res = {}
-    for B in (8, 16, 64):
+    for B in (1, 8, 16, 64):
         sess = Session(model)
         state = State(dims, B)
         logits = hip.DeviceArray((B, dims.V), np.float32)
@@ -142,6 +165,7 @@ def secondary_measurements(hip, model, dims, rng):
         res["decode_bs%d_tok_s" % B] = steps * B / dt
         res["decode_bs%d_ms_per_step" % B] = dt * 1e3 / steps
         res["decode_bs%d_hbm_fraction" % B] = (model.weight_bytes() + state_bytes) / (dt / steps) / 1e9 / HBM_PEAK_GBPS
+        res.update(sampled_decode(hip, sess, dims, state, logits, B, first))
         sess.close()
         del state, logits
 
