@@ -6,9 +6,11 @@
 // {p >= t} still holds at least top_k entries or at least top_p mass; entries equal to t are scaled by
 // `comp` so the kept set has exactly top_k entries / top_p mass (:393-404).
 //
-// gfx950 re-design: one 1024-thread block (16 wavefronts) per row; each thread owns a contiguous slice
-// of the row so the draw is a single inverse-CDF walk with one uniform number; block reductions are
-// wave64 shuffles + one LDS exchange; top_k == 1 (greedy, what top_p == 0 normalises to) skips the
+// gfx950 re-design: one 1024-thread block (16 wavefronts) per row; each thread owns a fixed set of entries -
+// for rows of up to 65536 entries the float4 t, t + 1024, ..., loaded once (coalesced) and kept in registers
+// through the softmax, the bisection and the draw; for larger rows a contiguous slice that stays in `probs` -
+// so the draw is a single inverse-CDF walk with one uniform number over a fixed order of the row; block
+// reductions are wave64 shuffles + one LDS exchange; top_k == 1 (greedy, what top_p == 0 normalises to) skips the
 // bisection.  Randomness is counter-based Philox4x32-10 keyed by (seed; row, step) instead of a
 // per-row cuRAND state seeded from the wall clock (src/rwkv_sampler.cpp:14-19), so a run is reproducible.
 #include <cfloat>
@@ -110,6 +112,36 @@ struct SampleArgs {
   uint64_t seed, step;
 };
 
+// count and mass of one bisection step through one LDS exchange (the same sums, in the same order, as
+// block_sum_u and block_reduce_f one after the other)
+__device__ __forceinline__ void block_count_mass(unsigned& c, float& m, BlockRed& red) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    c += __shfl_xor(c, off, 64);
+    m += __shfl_xor(m, off, 64);
+  }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+    red.u[threadIdx.x >> 6] = c;
+    red.f[threadIdx.x >> 6] = m;
+  }
+  __syncthreads();
+  unsigned rc = 0;
+  float rm = red.f[0];
+#pragma unroll
+  for (int i = 0; i < kSampleWaves; ++i) rc += red.u[i];
+#pragma unroll
+  for (int i = 1; i < kSampleWaves; ++i) rm += red.f[i];
+  c = rc;
+  m = rm;
+}
+
+constexpr int kSampleRegVecs = 16;  // float4 per thread held in registers: rows of up to 65536 entries
+
+// REG: a thread's slice of the row (up to 16 float4) stays in registers from the first load to the draw, so
+// the softmax, the ~30 bisection steps and the tie count touch no memory; `probs` is not written.  Larger
+// rows keep the slice in `probs` (L2) and re-read it in every pass.  Same arithmetic in the same order.
+template <bool REG>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
   __shared__ BlockRed red;
   __shared__ int s_pick;
@@ -124,15 +156,45 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
   const int per = (V4 + kSampleThreads - 1) / kSampleThreads;
   const int i0 = min(t * per, V4);
   const int i1 = min(i0 + per, V4);
+  // REG: thread t owns the float4 t, t + 1024, ... (every load of a wavefront is one contiguous KiB); the draw
+  // walks the kept entries thread by thread, a fixed permutation of the row, which leaves every entry its probability.
+  const int n = REG ? (t < V4 ? min((V4 - t + kSampleThreads - 1) / kSampleThreads, kSampleRegVecs) : 0) : i1 - i0;
   auto fmax_op = [](float x, float y) { return fmaxf(x, y); };
   auto fmin_op = [](float x, float y) { return fminf(x, y); };
   auto fadd_op = [](float x, float y) { return x + y; };
 
+  float4_t vals[REG ? kSampleRegVecs : 1];
+  // f(q, i): q = position in the slice, i = float4 index in the row
+  auto for_each = [&](auto&& f) {
+    if constexpr (REG) {
+#pragma unroll
+      for (int q = 0; q < kSampleRegVecs; ++q)
+        if (q < n) f(q, q * kSampleThreads + t);
+    } else {
+      for (int i = i0; i < i1; ++i) f(0, i);
+    }
+  };
+  auto get = [&](int q, int i) -> float4_t {
+    if constexpr (REG) return vals[q];
+    else return reinterpret_cast<const float4_t*>(probs)[i];
+  };
+  auto put = [&](int q, int i, const float4_t& v) {
+    if constexpr (REG) vals[q] = v;
+    else reinterpret_cast<float4_t*>(probs)[i] = v;
+  };
+
   // 1. penalised, temperature-scaled logits in base-2 units; row maximum and its lowest index
+  if constexpr (REG) {
+#pragma unroll
+    for (int q = 0; q < kSampleRegVecs; ++q)  // all loads of the slice in flight together
+      if (q < n) vals[q] = reinterpret_cast<const float4_t*>(logits)[q * kSampleThreads + t];
+  }
   float maxu = -INFINITY;
   int maxi = 0x7fffffff;
-  for (int i = i0; i < i1; ++i) {
-    float4_t l = reinterpret_cast<const float4_t*>(logits)[i];
+  for_each([&](int q, int i) {
+    float4_t l;
+    if constexpr (REG) l = vals[q];
+    else l = reinterpret_cast<const float4_t*>(logits)[i];
     float4_t p = {0.0f, 0.0f, 0.0f, 0.0f};
     if (pen) p = reinterpret_cast<const float4_t*>(pen)[i];
 #pragma unroll
@@ -143,8 +205,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
         maxi = i * 4 + j;
       }
     }
-    reinterpret_cast<float4_t*>(probs)[i] = l;
-  }
+    put(q, i, l);
+  });
   const float gmax = block_reduce_f(maxu, fmax_op, red.f);
   int pick = -1;
 
@@ -163,22 +225,24 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
   } else {
     // 2.-3. softmax
     float den = 0.0f;
-    for (int i = i0; i < i1; ++i) {
-      const float4_t l = reinterpret_cast<const float4_t*>(probs)[i];
-      den += exp2f(l[0] - gmax) + exp2f(l[1] - gmax) + exp2f(l[2] - gmax) + exp2f(l[3] - gmax);
-    }
+    for_each([&](int q, int i) {
+      const float4_t l = get(q, i);
+      const float4_t e = {exp2f(l[0] - gmax), exp2f(l[1] - gmax), exp2f(l[2] - gmax), exp2f(l[3] - gmax)};
+      den += e[0] + e[1] + e[2] + e[3];
+      if constexpr (REG) put(q, i, e);  // registers keep the exponentials for the division below
+    });
     den = block_reduce_f(den, fadd_op, red.f);
     float pmax = -INFINITY, pmin = INFINITY;
-    for (int i = i0; i < i1; ++i) {
-      float4_t l = reinterpret_cast<const float4_t*>(probs)[i];
+    for_each([&](int q, int i) {
+      float4_t l = get(q, i);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        l[j] = exp2f(l[j] - gmax) / den;
+        l[j] = (REG ? l[j] : exp2f(l[j] - gmax)) / den;
         pmax = fmaxf(pmax, l[j]);
         pmin = fminf(pmin, l[j]);
       }
-      reinterpret_cast<float4_t*>(probs)[i] = l;
-    }
+      put(q, i, l);
+    });
     pmax = block_reduce_f(pmax, fmax_op, red.f);
     pmin = block_reduce_f(pmin, fmin_op, red.f);
 
@@ -191,17 +255,16 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
       const float thr = __uint_as_float(mid);
       unsigned c = 0;
       float m = 0.0f;
-      for (int i = i0; i < i1; ++i) {
-        const float4_t l = reinterpret_cast<const float4_t*>(probs)[i];
+      for_each([&](int q, int i) {
+        const float4_t l = get(q, i);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           if (l[j] >= thr) {
             ++c;
             m += l[j];
           }
-      }
-      c = block_sum_u(c, red.u);
-      m = block_reduce_f(m, fadd_op, red.f);
+      });
+      block_count_mass(c, m, red);
       if (c < static_cast<unsigned>(a.top_k) && m < a.top_p) {
         right = mid;
       } else {
@@ -215,8 +278,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
     // 5. tie compensation
     unsigned eqk = 0, gtk = 0;
     float gtp = 0.0f;
-    for (int i = i0; i < i1; ++i) {
-      const float4_t l = reinterpret_cast<const float4_t*>(probs)[i];
+    for_each([&](int q, int i) {
+      const float4_t l = get(q, i);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (l[j] == thr) ++eqk;
@@ -225,7 +288,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
           gtp += l[j];
         }
       }
-    }
+    });
     const unsigned n_eq = block_sum_u(eqk, red.u);
     const unsigned n_gt = block_sum_u(gtk, red.u);
     const float p_gt = block_reduce_f(gtp, fadd_op, red.f);
@@ -236,7 +299,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
       comp = fmaxf(comp, 0.0f);
     }
 
-    // 6. inverse-CDF draw over the kept set, thread slices in index order
+    // 6. inverse-CDF draw over the kept set, thread by thread
     const float mine = gtp + (thr * eqk) * comp;
     float total;
     const float before = block_exclusive_scan(mine, red.f, &total);
@@ -249,18 +312,18 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
     if (mine > 0.0f && target > before && target <= before + mine) {
       float cum = before;
       int found = -1, last = -1;
-      for (int i = i0; i < i1 && found < 0; ++i) {
-        const float4_t l = reinterpret_cast<const float4_t*>(probs)[i];
+      for_each([&](int q, int i) {
+        const float4_t l = get(q, i);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float w = (l[j] < thr) ? 0.0f : (l[j] == thr ? l[j] * comp : l[j]);
-          if (w > 0.0f) {
+          if (w > 0.0f && found < 0) {
             cum += w;
             last = i * 4 + j;
-            if (found < 0 && cum >= target) found = last;
+            if (cum >= target) found = last;
           }
         }
-      }
+      });
       if (found < 0) found = last;  // rounding inside the slice: its last kept entry
       atomicMax(&s_pick, found);
     }
@@ -269,12 +332,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
     __syncthreads();
     if (fallback && mine > 0.0f) {
       int last = -1;
-      for (int i = i0; i < i1; ++i) {
-        const float4_t l = reinterpret_cast<const float4_t*>(probs)[i];
+      for_each([&](int q, int i) {
+        const float4_t l = get(q, i);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           if (l[j] > thr || (l[j] == thr && comp > 0.0f)) last = i * 4 + j;
-      }
+      });
       atomicMax(&s_pick, last);
     }
     __syncthreads();
@@ -284,7 +347,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
   if (t == 0) a.out[b] = pick;
   // 7. penalty update (sampling.cu:461-470)
   if (pen) {
-    for (int i = i0; i < i1; ++i) {
+    for_each([&](int, int i) {
       float4_t p = reinterpret_cast<float4_t*>(pen)[i];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -292,7 +355,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
         p[j] = fmaf(p[j], a.decay, add);
       }
       reinterpret_cast<float4_t*>(pen)[i] = p;
-    }
+    });
   }
 }
 
@@ -400,7 +463,11 @@ int rwkv_hip_sample(rwkv_stream_t s, int B, int V, const void* logits, void* pen
   a.top_p = static_cast<float>(top_p);
   a.seed = seed;
   a.step = step;
-  hipLaunchKernelGGL(sample_kernel, dim3(B), dim3(kSampleThreads), 0, as_stream(s), a);
+  if (V / 4 <= kSampleRegVecs * kSampleThreads) {
+    hipLaunchKernelGGL(sample_kernel<true>, dim3(B), dim3(kSampleThreads), 0, as_stream(s), a);
+  } else {
+    hipLaunchKernelGGL(sample_kernel<false>, dim3(B), dim3(kSampleThreads), 0, as_stream(s), a);
+  }
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
