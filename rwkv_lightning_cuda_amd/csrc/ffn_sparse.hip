@@ -132,7 +132,7 @@ __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, in
     }
     uint4_t q[kSparseBatch];
 #pragma unroll
-    for (int p = 0; p < kSparseBatch; ++p) q[p] = wlane[static_cast<int64_t>(f0 + row[p]) * row_pieces];
+    for (int p = 0; p < kSparseBatch; ++p) q[p] = __builtin_nontemporal_load(&wlane[static_cast<int64_t>(f0 + row[p]) * row_pieces]);
 #pragma unroll
     for (int p = 0; p < kSparseBatch; p += 2) {
       const half2_t ap = as_half2(coef[p] | (coef[p + 1] << 16));

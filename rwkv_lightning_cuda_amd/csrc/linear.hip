@@ -239,7 +239,10 @@ struct WaveGemv {
       if (k0 < kn) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          bt.w[u][r] = *reinterpret_cast<const uint4_t*>(wbase + r * row_bytes + T::byte_off(k_lo + k0));
+          // streamed once per step: non-temporal, so that the weights do not push the rows that are re-read (LoRA
+          // matrices, state, activations) out of the caches (batch-1 step 2.39 -> 2.34 ms)
+          bt.w[u][r] = __builtin_nontemporal_load(
+              reinterpret_cast<const uint4_t*>(wbase + r * row_bytes + T::byte_off(k_lo + k0)));
           if constexpr (FMT == RWKV_FMT_W4) {
             const int64_t gi = static_cast<int64_t>(row0 + r) * (K >> 7) + ((k_lo + k0) >> 7);
             bt.sc[u][r] = prob.scale[gi];

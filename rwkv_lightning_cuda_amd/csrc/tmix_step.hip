@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
 
   // ---- all global loads up front
   float* srow = p.state + (static_cast<int64_t>(bh) * kHead + i) * kHead + 4 * q;
-  float4_t S = *reinterpret_cast<const float4_t*>(srow);
+  float4_t S = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(srow));
   const LoraRow w2 = lora_row_load(p.w2 + static_cast<int64_t>(c) * p.Rw, p.Rw, q);
   const LoraRow a2 = lora_row_load(p.a2 + static_cast<int64_t>(c) * p.Ra, p.Ra, q);
   const LoraRow g2 = lora_row_load(p.g2 + static_cast<int64_t>(c) * p.Rg, p.Rg, q);
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
   S.y = fmaf(S.y, d4.y, fmaf(sa, b4.y, k4.y * v_use));
   S.z = fmaf(S.z, d4.z, fmaf(sa, b4.z, k4.z * v_use));
   S.w = fmaf(S.w, d4.w, fmaf(sa, b4.w, k4.w * v_use));
-  *reinterpret_cast<float4_t*>(srow) = S;
+  __builtin_nontemporal_store(S, reinterpret_cast<float4_t*>(srow));
   float yy = S.x * r4.x;
   yy = fmaf(S.y, r4.y, yy);
   yy = fmaf(S.z, r4.z, yy);

@@ -115,7 +115,7 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
 
   float4_t S[RPL];
 #pragma unroll
-  for (int i = 0; i < RPL; ++i) S[i] = *reinterpret_cast<const float4_t*>(sblk + i * kHead);
+  for (int i = 0; i < RPL; ++i) S[i] = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(sblk + i * kHead));
 
   const int64_t base = static_cast<int64_t>(bi) * op_bs + h * kHead;
   const int64_t iob = static_cast<int64_t>(bi) * io_bs + h * kHead;
@@ -360,7 +360,7 @@ __global__ __launch_bounds__(1024 / RPL / PARTS) void wkv7_seq_kernel(int T, int
   write_out(t_last, T - t_last, (t_last / kSeqChunk) & 1);
 
 #pragma unroll
-  for (int i = 0; i < RPL; ++i) *reinterpret_cast<float4_t*>(sblk + i * kHead) = S[i];
+  for (int i = 0; i < RPL; ++i) __builtin_nontemporal_store(S[i], reinterpret_cast<float4_t*>(sblk + i * kHead));
 }
 
 // Heads in flight up to which a head is cut into four (two) row ranges of four wavefronts each, one block per
