@@ -33,7 +33,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak, published
 # HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled
 # by what the same counter reads for a 1 GiB device-to-device copy (FETCH_SIZE reads half the bytes copied,
 # WRITE_SIZE all of them); the summary of those runs is kept under profiles/.  Keyed by (preset, format, batch).
-MEASURED_TRAFFIC = {("7.2B", "w8", 1): 2.0 * 24277.7 * 1024 + 1.0 * 46.0 * 1024}
+MEASURED_TRAFFIC = {("7.2B", "w8", 1): 2.0 * 24290.5 * 1024 + 1.0 * 45.9 * 1024}
 
 
 def parse_args():
