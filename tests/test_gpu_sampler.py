@@ -75,6 +75,29 @@ def test_draws_stay_in_kept_set_and_follow_filtered_distribution(gpu, orc, top_k
     assert tv <= 0.5 * np.sqrt(max(kept, 1) / n) + 0.02
 
 
+def test_rows_longer_than_the_register_path_follow_the_filtered_distribution(gpu, orc):
+    """Rows of more than 65536 entries keep their slices in the probs scratch instead of registers: same kept set,
+    same distribution; greedy picks the lowest index among tied maxima."""
+    hip = gpu
+    rng = np.random.default_rng(13)
+    V = 131072
+    logits = (rng.standard_normal(V) * 2.5).astype(np.float32)
+    logits[[7, 70000, 131071]] = logits.max() + 0.25      # a tie that straddles the 65536 boundary
+    kept, probs = orc.sample_filter(logits, None, 0.8, 12, 0.9)
+    draws = _draw(hip, logits, 64, 64, seed=5, temperature=0.8, top_k=12, top_p=0.9).ravel()
+    in_set = bool(np.all(probs[draws] > 0))
+    assert in_set
+    want = probs.astype(np.float64) / probs.sum(dtype=np.float64)
+    freq = np.bincount(draws, minlength=V) / draws.size
+    heavy = np.nonzero(want * draws.size >= 20)[0]
+    assert heavy.size >= 3
+    sigma = np.sqrt(want[heavy] * (1 - want[heavy]) / draws.size)
+    worst = float(np.max(np.abs(freq[heavy] - want[heavy]) / sigma))
+    assert worst <= 5.0
+    greedy = _draw(hip, logits, 2, 2, seed=1, top_k=1).ravel()
+    assert set(greedy.tolist()) == {7}
+
+
 def test_draw_is_a_function_of_seed_row_and_step(gpu):
     hip = gpu
     rng = np.random.default_rng(5)
