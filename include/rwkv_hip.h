@@ -280,9 +280,9 @@ int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
 /* Decode steps on the GEMV path (one or two rows) can fold the two LayerNorm + token-shift kernels of a layer
  * into the prologue of the linear launches that consume them (bitwise the same results).  on > 0: always,
- * 0: never, < 0 (the default): for one row of at most 2048 channels, where two launches fewer per layer are
- * worth more than the extra work inside every GEMV block (0.1B shape: 0.471 -> 0.442 ms per step; at 4096
- * channels or two rows the stand-alone kernels are faster).  No counterpart in the reference. */
+ * 0: never, < 0 (the default): for one row of at most 1024 channels, where two launches fewer per layer are
+ * worth more than the extra work inside every GEMV block (0.1B shape: 0.446 -> 0.423 ms per step; from 2048
+ * channels on, or with two rows, the stand-alone kernels are faster).  No counterpart in the reference. */
 int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on);
 /* debugging/parity tap: device address of one of the session's activation buffers, holding what the last
  * layer of the last rwkv_hip_forward call left there.  Ids in order: x, xx, xr, xw, xk, xv, xa, xg, r, k, v,

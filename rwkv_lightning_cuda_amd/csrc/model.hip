@@ -123,7 +123,7 @@ struct rwkv_hip_session {
   size_t sparse_ws_bytes = 0;
   int sparse_ffn_rows = 1;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
   int fused_ln = -1;          // decode steps fold LayerNorm + token shift into the linear launches: 1 always, 0 never,
-                              // -1 for one row of at most 2048 channels (faster there: 0.1B shape 0.471 -> 0.442 ms)
+                              // -1 for one row of at most 1024 channels (faster there: 0.1B shape 0.446 -> 0.423 ms)
 };
 
 namespace {
@@ -335,7 +335,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   // Decode steps of up to 8 rows fold both LayerNorm + token-shift kernels of a layer into the prologue of the
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key).  The residual-stream tap needs the
   // stand-alone kernels.
-  const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows == 1 && C <= 2048);
+  const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows == 1 && C <= 1024);
   const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace &&
                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
 
