@@ -302,18 +302,21 @@ def main():
                                     # at M = 128 the launches are weight-streaming bound: the same time against HBM
                                     "weights_gb_s": model.weight_bytes() / (total_ms * 1e-3) / 1e9,
                                     "hbm_frac": model.weight_bytes() / (total_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
-            # the same prompt in chunks of 512 (the chunk width is the caller's choice: wider chunks stream the
-            # weights once per 512 tokens), into a scratch state
-            wide = State(dims, B)
-            sess.forward(prompt[:, :min(512, args.prefill)], wide, logits)
-            hip.device_sync()
-            tw = time.perf_counter()
-            for t0 in range(0, args.prefill, 512):
-                sess.forward(prompt[:, t0:t0 + 512], wide, logits, sync=False)
-            hip.device_sync()
-            tw = time.perf_counter() - tw
-            also["prefill_chunk512_tok_s"] = B * args.prefill / tw
-            del wide
+            # the same prompt in chunks of 512 and 2048 (the chunk width is the caller's choice: wider chunks
+            # stream the weights once per chunk), into a scratch state
+            for width in (512, 2048):
+                if B * width > 4096:
+                    continue
+                wide = State(dims, B)
+                sess.forward(prompt[:, :min(width, args.prefill)], wide, logits)
+                hip.device_sync()
+                tw = time.perf_counter()
+                for t0 in range(0, args.prefill, width):
+                    sess.forward(prompt[:, t0:t0 + width], wide, logits, sync=False)
+                hip.device_sync()
+                tw = time.perf_counter() - tw
+                also["prefill_chunk%d_tok_s" % width] = B * args.prefill / tw
+                del wide
     first = rng.integers(0, dims.V, (B,))
 
     if args.warmup > 0:
