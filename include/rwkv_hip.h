@@ -141,8 +141,15 @@ int rwkv_hip_linear_packed(rwkv_stream_t s, int fmt, int M, int N, int K, const 
  * cmix_sparse_pack turns the [C,F] matrix (fp16 values, or the codes of rwkv_hip_quantize_w8) into the [F,C]
  * copy `wt` (same size) that the product reads - the layout the reference keeps ffn.value in
  * (include/rwkv7_fast_v4_common.hpp:313-321); `scale` is the per-output-channel tensor of the codes (unused
- * for fp16).  C % 16 == 0, F % 256 == 0.  workspace: fp32 partial rows, size from cmix_sparse_workspace. */
+ * for fp16).  C % 16 == 0, F % 256 == 0.  workspace: fp32 partial rows, size from cmix_sparse_workspace.
+ * int4 codes (RWKV_FMT_W4, groups of 128 along F; no counterpart in the reference):
+ *   out[c] = f16(sum over groups g of scale[c][g] * sum over f in g with vec[f] != 0 of vec[f] * (q[c][f] - zp[c][g]));
+ * cmix_sparse_pack_w4 writes the codes [F,C/2], then the scales and zero points transposed to [F/128,C], into one
+ * allocation `wt` of cmix_sparse_packed_bytes; the product then ignores its `scale` argument. */
 int rwkv_hip_cmix_sparse_pack(rwkv_stream_t s, int fmt, int C, int F, const void* w, void* wt);
+int rwkv_hip_cmix_sparse_pack_w4(rwkv_stream_t s, int C, int F, const void* q, const void* scale, const void* zp,
+                                 void* wt);
+int rwkv_hip_cmix_sparse_packed_bytes(int fmt, int C, int F, size_t* bytes);
 int rwkv_hip_cmix_sparse_workspace(int rows, int C, int F, size_t* bytes);
 int rwkv_hip_cmix_sparse_down_relu_rows(rwkv_stream_t s, int fmt, int rows, int C, int F, const void* preact,
                                         const void* wt, const void* scale, void* workspace, size_t workspace_bytes,

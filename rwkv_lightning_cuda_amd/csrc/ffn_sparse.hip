@@ -28,11 +28,21 @@ constexpr int kSparseRowsPerBlock = kSparseRowsPerWave * kSparseWaves;  // 256
 constexpr int kSparseBatch = 8;
 
 // columns per lane = values in a 16-byte piece
-constexpr int sparse_lane_cols(int fmt) { return fmt == RWKV_FMT_W8 ? 16 : 8; }
+constexpr int sparse_lane_cols(int fmt) { return fmt == RWKV_FMT_F16 ? 8 : 16; }
 
 bool ffn_sparse_supported(int fmt, int C, int F) {
-  if (fmt != RWKV_FMT_W8 && fmt != RWKV_FMT_F16) return false;
+  if (fmt != RWKV_FMT_W8 && fmt != RWKV_FMT_F16 && fmt != RWKV_FMT_W4) return false;
   return C >= 16 && C % 16 == 0 && F >= kSparseRowsPerBlock && F % kSparseRowsPerBlock == 0;
+}
+
+// Bytes of the transposed copy.  int4: the [F,C/2] codes, then the scales [F/128,C] (fp16), then the zero points
+// [F/128,C] (one byte each) - a wavefront's 32 rows lie in one 128-group, so it needs one scale and one zero point
+// per column.
+size_t ffn_sparse_packed_bytes(int fmt, int C, int F) {
+  const size_t cf = static_cast<size_t>(C) * F;
+  if (fmt == RWKV_FMT_F16) return cf * 2;
+  if (fmt == RWKV_FMT_W8) return cf;
+  return cf / 2 + static_cast<size_t>(F / 128) * C * 3;
 }
 
 size_t ffn_sparse_workspace_bytes(int rows, int C, int F) {
@@ -63,7 +73,8 @@ __global__ __launch_bounds__(256) void ffn_sparse_pack_kernel(int C, int F, cons
 }
 
 int ffn_sparse_pack_launch(hipStream_t st, int fmt, int C, int F, const void* w, void* wt) {
-  RWKV_REQUIRE(ffn_sparse_supported(fmt, C, F), "ffn_sparse_pack: unsupported format %d or shape C=%d F=%d", fmt, C, F);
+  RWKV_REQUIRE(fmt != RWKV_FMT_W4 && ffn_sparse_supported(fmt, C, F),
+               "ffn_sparse_pack: unsupported format %d or shape C=%d F=%d (int4 codes: ffn_sparse_pack_w4)", fmt, C, F);
   RWKV_REQUIRE(w && wt && w != wt, "ffn_sparse_pack: bad pointers");
   const dim3 grid(ceil_div(F, 64), ceil_div(C, 64));
   if (fmt == RWKV_FMT_W8) {
@@ -73,6 +84,59 @@ int ffn_sparse_pack_launch(hipStream_t st, int fmt, int C, int F, const void* w,
     hipLaunchKernelGGL(ffn_sparse_pack_kernel<uint16_t>, grid, dim3(256), 0, st, C, F, static_cast<const uint16_t*>(w),
                        static_cast<uint16_t*>(wt));
   }
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+// int4: q [C,F/2] (even f in the low nibble) -> t [F,C/2] (even c in the low nibble); 64 x 64 tiles of nibbles.
+__global__ __launch_bounds__(256) void ffn_sparse_pack_w4_kernel(int C, int F, const uint8_t* __restrict__ q,
+                                                                 uint8_t* __restrict__ t) {
+  __shared__ uint8_t tile[64][65];
+  const int f0 = blockIdx.x * 64;
+  const int c0 = blockIdx.y * 64;
+  for (int i = threadIdx.x; i < 64 * 32; i += 256) {
+    const int c = i >> 5;
+    const int fb = i & 31;
+    uint8_t v = 0;
+    if (c0 + c < C && f0 + 2 * fb < F) v = q[static_cast<int64_t>(c0 + c) * (F / 2) + f0 / 2 + fb];
+    tile[c][2 * fb] = v & 15;
+    tile[c][2 * fb + 1] = v >> 4;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 32; i += 256) {
+    const int f = i >> 5;
+    const int cb = i & 31;
+    if (c0 + 2 * cb < C && f0 + f < F)
+      t[static_cast<int64_t>(f0 + f) * (C / 2) + c0 / 2 + cb] = tile[2 * cb][f] | (tile[2 * cb + 1][f] << 4);
+  }
+}
+
+// scale / zp [C,F/128] -> [F/128,C]
+__global__ __launch_bounds__(256) void ffn_sparse_pack_w4_groups_kernel(int C, int G, const half_t* __restrict__ scale,
+                                                                        const uint8_t* __restrict__ zp,
+                                                                        half_t* __restrict__ scale_t,
+                                                                        uint8_t* __restrict__ zp_t) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= static_cast<int64_t>(C) * G) return;
+  const int g = static_cast<int>(i / C);
+  const int c = static_cast<int>(i - static_cast<int64_t>(g) * C);
+  scale_t[i] = scale[static_cast<int64_t>(c) * G + g];
+  zp_t[i] = zp[static_cast<int64_t>(c) * G + g];
+}
+
+int ffn_sparse_pack_w4_launch(hipStream_t st, int C, int F, const void* q, const half_t* scale, const uint8_t* zp,
+                              void* wt) {
+  RWKV_REQUIRE(ffn_sparse_supported(RWKV_FMT_W4, C, F), "ffn_sparse_pack: unsupported shape C=%d F=%d", C, F);
+  RWKV_REQUIRE(q && scale && zp && wt && q != wt, "ffn_sparse_pack: bad pointers");
+  uint8_t* codes = static_cast<uint8_t*>(wt);
+  const int G = F / 128;
+  half_t* scale_t = reinterpret_cast<half_t*>(codes + static_cast<size_t>(C) * F / 2);
+  uint8_t* zp_t = reinterpret_cast<uint8_t*>(scale_t + static_cast<size_t>(G) * C);
+  hipLaunchKernelGGL(ffn_sparse_pack_w4_kernel, dim3(ceil_div(F, 64), ceil_div(C, 64)), dim3(256), 0, st, C, F,
+                     static_cast<const uint8_t*>(q), codes);
+  RWKV_LAUNCH_CHECK();
+  hipLaunchKernelGGL(ffn_sparse_pack_w4_groups_kernel, dim3(static_cast<unsigned>((static_cast<int64_t>(C) * G + 255) / 256)),
+                     dim3(256), 0, st, C, G, scale, zp, scale_t, zp_t);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
@@ -174,6 +238,124 @@ __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_kernel(int C, in
   }
 }
 
+// int4 codes: the same walk with 8-byte pieces (16 columns per lane, 1024 per block).  The two rows of a
+// v_dot2_f32_f16 are paired nibble by nibble: even and odd nibbles of each dword are masked into bytes, v_perm_b32
+// puts row A's byte under exponent 0x64 in the low half and row B's in the high half, one packed subtract of
+// 1024 gives the exact codes.  sum_f a_f (q_fc - zp_c) = sum_f a_f q_fc - zp_c sum_f a_f: the zero point and the
+// scale of the wavefront's 128-group are applied once, after the walk.
+__global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_w4_kernel(int C, int F, int activated,
+                                                                          const half_t* __restrict__ in,
+                                                                          const uint8_t* __restrict__ blob,
+                                                                          float* __restrict__ partial) {
+  constexpr int LC = 16;
+  constexpr int kCols = 64 * LC;
+  __shared__ __align__(16) float red[kSparseWaves][kCols];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int f0 = blockIdx.x * kSparseRowsPerBlock + wave * kSparseRowsPerWave;
+  const int c0 = blockIdx.y * kCols;
+  const bool col_ok = c0 + LC * lane < C;
+  const int cl = c0 + (col_ok ? LC * lane : 0);  // this lane's first column
+  const int row_pieces = C / LC;                 // 8-byte pieces per row
+  const uint2_t* wlane = reinterpret_cast<const uint2_t*>(blob) + cl / LC;
+  const int G = F / 128;
+  const half_t* scale_t = reinterpret_cast<const half_t*>(blob + static_cast<size_t>(C) * F / 2);
+  const uint8_t* zp_t = reinterpret_cast<const uint8_t*>(scale_t + static_cast<size_t>(G) * C);
+  const int64_t gat = static_cast<int64_t>(f0 / 128) * C + cl;
+  const half8_t sc0 = *reinterpret_cast<const half8_t*>(scale_t + gat);
+  const half8_t sc1 = *reinterpret_cast<const half8_t*>(scale_t + gat + 8);
+  const uint4_t zq = *reinterpret_cast<const uint4_t*>(zp_t + gat);
+  in += static_cast<int64_t>(blockIdx.z) * F;
+  partial += static_cast<int64_t>(blockIdx.z) * gridDim.x * C;
+
+  float a = 0.0f;
+  if (lane < kSparseRowsPerWave) {
+    a = h2f(in[f0 + lane]);
+    if (!activated) {
+      a = fmaxf(round_h(a), 0.0f);
+      a = round_h(a * a);
+    }
+  }
+  const half_t ah = f2h(a);
+  const uint32_t abits = __builtin_bit_cast(uint16_t, ah);
+  uint64_t mask = __ballot((abits << 17) != 0u);
+
+  float acc[LC];
+#pragma unroll
+  for (int i = 0; i < LC; ++i) acc[i] = 0.0f;
+  float asum = 0.0f;
+  const half2_t bias = {static_cast<half_t>(1024.0f), static_cast<half_t>(1024.0f)};
+
+  while (mask != 0) {
+    int row[kSparseBatch];
+    uint32_t coef[kSparseBatch];
+    const int first = __builtin_ctzll(mask);
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p) {
+      if (mask != 0) {
+        row[p] = __builtin_ctzll(mask);
+        mask &= mask - 1;
+        coef[p] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(abits), row[p]));
+      } else {
+        row[p] = first;
+        coef[p] = 0u;
+      }
+    }
+    uint2_t q[kSparseBatch];
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p)
+      q[p] = __builtin_nontemporal_load(&wlane[static_cast<int64_t>(f0 + row[p]) * row_pieces]);
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; p += 2) {
+      const half2_t ap = as_half2(coef[p] | (coef[p + 1] << 16));
+      asum += h2f(ap[0]) + h2f(ap[1]);
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        const uint32_t lo = q[p][d];
+        const uint32_t hi = q[p + 1][d];
+        const uint32_t ea = lo & 0x0f0f0f0fu, oa = (lo >> 4) & 0x0f0f0f0fu;
+        const uint32_t eb = hi & 0x0f0f0f0fu, ob = (hi >> 4) & 0x0f0f0f0fu;
+        // nibble n of the dword is column 8 d + n: byte n / 2 of the even (n even) or odd word
+        const half2_t w0 = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c040c00u) | 0x64006400u) - bias;
+        const half2_t w1 = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c040c00u) | 0x64006400u) - bias;
+        const half2_t w2 = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c050c01u) | 0x64006400u) - bias;
+        const half2_t w3 = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c050c01u) | 0x64006400u) - bias;
+        const half2_t w4 = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c060c02u) | 0x64006400u) - bias;
+        const half2_t w5 = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c060c02u) | 0x64006400u) - bias;
+        const half2_t w6 = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c070c03u) | 0x64006400u) - bias;
+        const half2_t w7 = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c070c03u) | 0x64006400u) - bias;
+        acc[8 * d + 0] = __builtin_amdgcn_fdot2(ap, w0, acc[8 * d + 0], false);
+        acc[8 * d + 1] = __builtin_amdgcn_fdot2(ap, w1, acc[8 * d + 1], false);
+        acc[8 * d + 2] = __builtin_amdgcn_fdot2(ap, w2, acc[8 * d + 2], false);
+        acc[8 * d + 3] = __builtin_amdgcn_fdot2(ap, w3, acc[8 * d + 3], false);
+        acc[8 * d + 4] = __builtin_amdgcn_fdot2(ap, w4, acc[8 * d + 4], false);
+        acc[8 * d + 5] = __builtin_amdgcn_fdot2(ap, w5, acc[8 * d + 5], false);
+        acc[8 * d + 6] = __builtin_amdgcn_fdot2(ap, w6, acc[8 * d + 6], false);
+        acc[8 * d + 7] = __builtin_amdgcn_fdot2(ap, w7, acc[8 * d + 7], false);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < LC; ++i) {
+    const float zpf = static_cast<float>((zq[i >> 2] >> (8 * (i & 3))) & 0xffu);
+    const float scf = h2f(i < 8 ? sc0[i] : sc1[i - 8]);
+    acc[i] = (acc[i] - zpf * asum) * scf;
+  }
+#pragma unroll
+  for (int i = 0; i < LC / 4; ++i)
+    *reinterpret_cast<float4_t*>(&red[wave][LC * lane + 4 * i]) =
+        float4_t{acc[4 * i], acc[4 * i + 1], acc[4 * i + 2], acc[4 * i + 3]};
+  __syncthreads();
+  if (threadIdx.x < kCols / 4) {
+    const int c = 4 * threadIdx.x;
+    float4_t sum = *reinterpret_cast<const float4_t*>(&red[0][c]);
+#pragma unroll
+    for (int w = 1; w < kSparseWaves; ++w) sum = sum + *reinterpret_cast<const float4_t*>(&red[w][c]);
+    if (c0 + c < C) *reinterpret_cast<float4_t*>(partial + static_cast<int64_t>(blockIdx.x) * C + c0 + c) = sum;
+  }
+}
+
 // ---- kernel 2: out[c] = f16(scale[c] * sum of the partial rows); block 0 also does the optional row copy --------
 // grid = (ceil(C/64), tokens), block = 256 = 16 groups of partial rows x 16 column quads.  Group g sums rows g, g+16, ... (its
 // loads are independent, so they are all in flight together), the 16 group sums meet in LDS in group order.
@@ -223,7 +405,10 @@ int ffn_sparse_launch(hipStream_t st, int fmt, int rows, int C, int F, int activ
   }
   const int n_partial = F / kSparseRowsPerBlock;
   const dim3 grid(n_partial, ceil_div(C, 64 * sparse_lane_cols(fmt)), rows);
-  if (fmt == RWKV_FMT_W8) {
+  if (fmt == RWKV_FMT_W4) {
+    hipLaunchKernelGGL(ffn_sparse_w4_kernel, grid, dim3(64 * kSparseWaves), 0, st, C, F, activated, in,
+                       static_cast<const uint8_t*>(wt), static_cast<float*>(workspace));
+  } else if (fmt == RWKV_FMT_W8) {
     hipLaunchKernelGGL(ffn_sparse_kernel<RWKV_FMT_W8>, grid, dim3(64 * kSparseWaves), 0, st, C, F, activated, in,
                        static_cast<const uint4_t*>(wt), static_cast<float*>(workspace));
   } else {
@@ -245,6 +430,20 @@ extern "C" {
 
 int rwkv_hip_cmix_sparse_pack(rwkv_stream_t s, int fmt, int C, int F, const void* w, void* wt) {
   return ffn_sparse_pack_launch(as_stream(s), fmt, C, F, w, wt);
+}
+
+int rwkv_hip_cmix_sparse_pack_w4(rwkv_stream_t s, int C, int F, const void* q, const void* scale, const void* zp,
+                                 void* wt) {
+  return ffn_sparse_pack_w4_launch(as_stream(s), C, F, q, static_cast<const half_t*>(scale),
+                                   static_cast<const uint8_t*>(zp), wt);
+}
+
+int rwkv_hip_cmix_sparse_packed_bytes(int fmt, int C, int F, size_t* bytes) {
+  RWKV_REQUIRE(bytes, "cmix_sparse_packed_bytes: NULL argument");
+  RWKV_REQUIRE(ffn_sparse_supported(fmt, C, F), "cmix_sparse_packed_bytes: unsupported format %d or shape C=%d F=%d", fmt, C,
+               F);
+  *bytes = ffn_sparse_packed_bytes(fmt, C, F);
+  return RWKV_OK;
 }
 
 int rwkv_hip_cmix_sparse_workspace(int rows, int C, int F, size_t* bytes) {

@@ -25,7 +25,7 @@ struct Matrix {
   const half_t* scale = nullptr;
   const uint8_t* zp = nullptr;
   void* packed = nullptr;  // owned: the same codes in the MFMA-native order, for calls with >= 16 rows
-  void* sparse_t = nullptr;  // owned, ffn.value with int8 codes or fp16 only: the [F,C] copy for the one-token row-skipping product
+  void* sparse_t = nullptr;  // owned, ffn.value only: the [F,C] copy for the one-token row-skipping product
 };
 
 struct Layer {
@@ -780,8 +780,9 @@ int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, con
   }
   if (id == RWKV_M_FFN_VALUE && ffn_sparse_supported(fmt, N, K)) {
     // third copy: transposed, for decode steps of one sequence
-    RWKV_HIP_TRY(hipMalloc(&mat.sparse_t, static_cast<size_t>(N) * K * (fmt == RWKV_FMT_F16 ? 2 : 1)));
-    const int rc = ffn_sparse_pack_launch(nullptr, fmt, N, K, data, mat.sparse_t);
+    RWKV_HIP_TRY(hipMalloc(&mat.sparse_t, ffn_sparse_packed_bytes(fmt, N, K)));
+    const int rc = fmt == RWKV_FMT_W4 ? ffn_sparse_pack_w4_launch(nullptr, N, K, data, mat.scale, mat.zp, mat.sparse_t)
+                                      : ffn_sparse_pack_launch(nullptr, fmt, N, K, data, mat.sparse_t);
     if (rc != RWKV_OK) {
       (void)hipFree(mat.sparse_t);
       if (mat.packed) (void)hipFree(mat.packed);

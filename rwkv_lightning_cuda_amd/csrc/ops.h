@@ -179,7 +179,10 @@ struct LoraOutMultiArgs {
 int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a);
 
 // ---- ffn_sparse.hip: one-token ffn.value product that skips the rows with a zero activation ---------------
-bool ffn_sparse_supported(int fmt, int C, int F);  // int8 codes or fp16
+bool ffn_sparse_supported(int fmt, int C, int F);  // fp16, int8 or int4 codes
+size_t ffn_sparse_packed_bytes(int fmt, int C, int F);  // size of the transposed copy
+// int4: codes [C,F/2] + scale / zp [C,F/128] -> codes [F,C/2], then scale and zp [F/128,C], in one allocation
+int ffn_sparse_pack_w4_launch(hipStream_t st, int C, int F, const void* q, const half_t* scale, const uint8_t* zp, void* wt);
 constexpr int kSparseMaxRows = 12;  // the reference's largest row count for this path (default_cmix_nofc_max_rows)
 size_t ffn_sparse_workspace_bytes(int rows, int C, int F);
 // [C,F] -> [F,C]; int8 codes are stored offset by 128

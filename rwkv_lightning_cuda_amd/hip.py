@@ -36,7 +36,8 @@ EXPORTS = [
     "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_bf16_to_f16", "rwkv_hip_bf16_to_f16_transpose",
     "rwkv_hip_emb_ln0_bf16_to_f16", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",
     "rwkv_hip_pack_weights", "rwkv_hip_linear_packed_workspace", "rwkv_hip_linear_packed", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
-    "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
+    "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_pack_w4", "rwkv_hip_cmix_sparse_packed_bytes",
+    "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
     "rwkv_hip_cmix_sparse_down_relu_rows",
     "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln",
     "rwkv_hip_layer_norm", "rwkv_hip_add_layer_norm", "rwkv_hip_add_last_layer_norm", "rwkv_hip_token_shift_mix",
@@ -256,6 +257,16 @@ def lora_in(M, C, R, x, w1, h, stream=None):
 
 def cmix_sparse_pack(fmt, C, F, w, wt, stream=None):
     check(load().rwkv_hip_cmix_sparse_pack(_p(stream), _i(fmt), _i(C), _i(F), _p(w), _p(wt)))
+
+
+def cmix_sparse_pack_w4(C, F, q, scale, zp, wt, stream=None):
+    check(load().rwkv_hip_cmix_sparse_pack_w4(_p(stream), _i(C), _i(F), _p(q), _p(scale), _p(zp), _p(wt)))
+
+
+def cmix_sparse_packed_bytes(fmt, C, F):
+    n = ctypes.c_size_t(0)
+    check(load().rwkv_hip_cmix_sparse_packed_bytes(_i(fmt), _i(C), _i(F), ctypes.byref(n)))
+    return n.value
 
 
 def cmix_sparse_workspace(C, F, rows=1):

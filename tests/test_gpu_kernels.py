@@ -448,7 +448,27 @@ def test_lora_out_keeps_the_activated_hidden_in_fp32(gpu, rows, C, R):
         assert off <= 0.01, "act %d: %.4f of the outputs are not the correctly rounded value" % (act, off)
 
 
-@pytest.mark.parametrize("fmt_name", ["w8", "f16"])
+def _sparse_w4_pack(hip, orc, w):
+    """Quantise to int4, pack for the row-skipping product and check the packed bytes: codes [F,C/2] (even c in the
+    low nibble), then scales [F/128,C] fp16, then zero points [F/128,C]."""
+    C, F = w.shape
+    q, s, z = orc.quantize_w4(w)
+    wt = hip.DeviceArray((hip.cmix_sparse_packed_bytes(hip.FMT_W4, C, F),), np.uint8)
+    hip.cmix_sparse_pack_w4(C, F, dev(hip, q), dev(hip, s), dev(hip, z), wt)
+    hip.device_sync()
+    nib = np.empty((C, F), np.uint8)
+    nib[:, 0::2] = q & 15
+    nib[:, 1::2] = q >> 4
+    nt = np.ascontiguousarray(nib.T)
+    codes_t = (nt[:, 0::2] | (nt[:, 1::2] << 4)).astype(np.uint8)
+    want = np.concatenate([codes_t.ravel(), np.ascontiguousarray(s.reshape(C, F // 128).T).view(np.uint8).ravel(),
+                           np.ascontiguousarray(z.reshape(C, F // 128).T).ravel()])
+    same = np.array_equal(wt.numpy(), want)
+    assert same
+    return q, s, z, wt
+
+
+@pytest.mark.parametrize("fmt_name", ["w8", "f16", "w4"])
 @pytest.mark.parametrize("C,F", [(768, 3072), (2560, 10240), (4096, 16384)])
 def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F, fmt_name):
     """ffn.value of one token over the transposed copy, skipping rows with a zero activation: against the
@@ -457,22 +477,28 @@ def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F, fmt_n
     hip = gpu
     rng = np.random.default_rng(C + F)
     w = (rng.standard_normal((C, F)) * 0.02).astype(np.float16)
-    if fmt_name == "w8":
-        fmt = hip.FMT_W8
-        q, s = orc.quantize_w8(w)
-        qd, sd = dev(hip, q), dev(hip, s)
-        wt = hip.DeviceArray((F, C), np.uint8)
-        want_t = (q.T.astype(np.int16) + 128).astype(np.uint8)
+    z, zd = None, None
+    if fmt_name == "w4":
+        fmt = hip.FMT_W4
+        q, s, z, wt = _sparse_w4_pack(hip, orc, w)
+        qd, sd, zd = dev(hip, q), dev(hip, s), dev(hip, z)
     else:
-        fmt = hip.FMT_F16
-        q, s = w, None
-        qd, sd = dev(hip, w), None
-        wt = hip.DeviceArray((F, C), np.float16)
-        want_t = np.ascontiguousarray(w.T)
-    hip.cmix_sparse_pack(fmt, C, F, qd, wt)
-    hip.device_sync()
-    same = np.array_equal(wt.numpy().view(np.uint8), want_t.view(np.uint8))
-    assert same
+        if fmt_name == "w8":
+            fmt = hip.FMT_W8
+            q, s = orc.quantize_w8(w)
+            qd, sd = dev(hip, q), dev(hip, s)
+            wt = hip.DeviceArray((F, C), np.uint8)
+            want_t = (q.T.astype(np.int16) + 128).astype(np.uint8)
+        else:
+            fmt = hip.FMT_F16
+            q, s = w, None
+            qd, sd = dev(hip, w), None
+            wt = hip.DeviceArray((F, C), np.float16)
+            want_t = np.ascontiguousarray(w.T)
+        hip.cmix_sparse_pack(fmt, C, F, qd, wt)
+        hip.device_sync()
+        same = np.array_equal(wt.numpy().view(np.uint8), want_t.view(np.uint8))
+        assert same
     ws = hip.DeviceArray.zeros((hip.cmix_sparse_workspace(C, F),), np.uint8)
 
     base = rng.standard_normal(F).astype(np.float16)
@@ -486,7 +512,7 @@ def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F, fmt_n
     }
     for name, pre in patterns.items():
         act = orc.relu_square(pre.reshape(1, F))
-        want = orc.gemv(fmt, act, q, s)
+        want = orc.gemv(fmt, act, q, s, z)
         out = hip.DeviceArray((1, C), np.float16)
         hip.cmix_sparse_down_relu_one(fmt, C, F, dev(hip, pre), wt, sd, ws, out)
         hip.device_sync()
@@ -497,7 +523,7 @@ def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F, fmt_n
             err = rel_err(got.astype(np.float32), want.astype(np.float32))
             assert err <= F16_TOL, name
         dense = hip.DeviceArray((1, C), np.float16)
-        hip.linear(fmt, 1, C, F, dev(hip, act), qd, sd, None, dense)
+        hip.linear(fmt, 1, C, F, dev(hip, act), qd, sd, zd, dense)
         out2 = hip.DeviceArray((1, C), np.float16)
         hip.cmix_sparse_down_relu_one(fmt, C, F, dev(hip, pre), wt, sd, ws, out2)
         hip.device_sync()
@@ -508,7 +534,7 @@ def test_cmix_sparse_down_matches_dense_product_and_oracle(gpu, orc, C, F, fmt_n
         assert same, name
 
 
-@pytest.mark.parametrize("fmt_name", ["w8", "f16"])
+@pytest.mark.parametrize("fmt_name", ["w8", "f16", "w4"])
 def test_cmix_sparse_down_rows_matches_the_one_row_product(gpu, orc, fmt_name):
     """Several tokens per call: each row of the output is bitwise what the one-row call gives for that token, and
     matches the oracle's dense product."""
@@ -516,7 +542,12 @@ def test_cmix_sparse_down_rows_matches_the_one_row_product(gpu, orc, fmt_name):
     C, F, rows = 768, 3072, 5
     rng = np.random.default_rng(17)
     w = (rng.standard_normal((C, F)) * 0.02).astype(np.float16)
-    if fmt_name == "w8":
+    z = None
+    if fmt_name == "w4":
+        fmt = hip.FMT_W4
+        q, s, z, wt = _sparse_w4_pack(hip, orc, w)
+        sd = None
+    elif fmt_name == "w8":
         fmt = hip.FMT_W8
         q, s = orc.quantize_w8(w)
         sd = dev(hip, s)
@@ -525,7 +556,8 @@ def test_cmix_sparse_down_rows_matches_the_one_row_product(gpu, orc, fmt_name):
         fmt = hip.FMT_F16
         q, s, sd = w, None, None
         wt = hip.DeviceArray((F, C), np.float16)
-    hip.cmix_sparse_pack(fmt, C, F, dev(hip, q), wt)
+    if fmt_name != "w4":
+        hip.cmix_sparse_pack(fmt, C, F, dev(hip, q), wt)
     pre = rng.standard_normal((rows, F)).astype(np.float16)
     pre[2] = -np.abs(pre[2])  # a token with no active row at all
     ws = hip.DeviceArray.zeros((hip.cmix_sparse_workspace(C, F, rows),), np.uint8)
@@ -533,7 +565,7 @@ def test_cmix_sparse_down_rows_matches_the_one_row_product(gpu, orc, fmt_name):
     hip.cmix_sparse_down_relu_rows(fmt, rows, C, F, dev(hip, pre), wt, sd, ws, out)
     hip.device_sync()
     got = out.numpy()
-    want = orc.gemv(fmt, orc.relu_square(pre), q, s)
+    want = orc.gemv(fmt, orc.relu_square(pre), q, s, z)
     err = rel_err(got.astype(np.float32), want.astype(np.float32))
     assert err <= F16_TOL
     assert not got[2].any()

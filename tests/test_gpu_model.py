@@ -107,9 +107,9 @@ def test_many_row_prefill_chunk_on_the_wide_gemm_tile(gpu, orc, fmt):
     sess.close()
 
 
-@pytest.mark.parametrize("fmt,B", [(0, 1), (1, 1), (1, 3)])
+@pytest.mark.parametrize("fmt,B", [(0, 1), (1, 1), (1, 3), (2, 1), (2, 2)])
 def test_decode_with_row_skipping_ffn_value(gpu, orc, fmt, B):
-    """Decode steps of an fp16 or W8 model with the row-skipping ffn.value product (one row by default, up to 12 by
+    """Decode steps of an fp16, W8 or W4 model with the row-skipping ffn.value product (one row by default, up to 12 by
     session option; eager and graph replay): the steps match the oracle, stay within an fp16 ulp of the dense
     product's logits, and the activations really are sparse (else the test would not exercise the skip)."""
     from rwkv_lightning_cuda_amd.model import Session, State
