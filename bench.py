@@ -331,7 +331,7 @@ def main():
 
     # one-sequence steps over int8 or fp16 weights skip the ffn.value rows with a zero activation (the reference's default
     # for rows == 1, include/rwkv7_fast_v4_common.hpp:198-211); the dense product is timed beside it below
-    sparse_value = B == 1 and args.fmt in ("w8", "f16") and dims.F % 256 == 0 and dims.C % 16 == 0
+    sparse_value = B == 1 and dims.F % 256 == 0 and dims.C % 16 == 0
     if sparse_value and not args.no_also:
         sess.set_sparse_ffn(0)
         sess.decode_greedy(first, min(args.warmup, 8) or 1, state, logits)
