@@ -12,8 +12,9 @@
 // two fp16 terms, hi = f16(a) and lo = f16(a - hi): hi + lo carries 22 bits of a, both products with the fp16
 // weight are exact in fp32, and the result differs from an fp32 dot only by summation order.  Without an
 // activation the hidden is fp16 already and the lo term is skipped.  One launch takes up to four problems
-// (w, a, g, v of a layer): grid = (C/128, M/32, problems), block = 4 wavefronts x 32 output channels, the
-// 32 x R slice of act(h) staged in LDS once per block.
+// (w, a, g, v of a layer): grid = (C/128, M/32, problems), block = 2 groups of 4 wavefronts x 32 output channels
+// (the groups take alternate 16-wide steps of the rank and add up through LDS), the 32 x R slice of act(h)
+// staged in LDS once per block.
 #include "ops.h"
 
 namespace rwkv {
@@ -23,7 +24,8 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 constexpr int kLoraMaxR = 512;
 constexpr int kLoraRows = 32;   // rows per block: one MFMA tile
 constexpr int kLoraCols = 128;  // output channels per block: 32 per wavefront
-constexpr int kLoraThreads = 2 * kLoraCols;
+constexpr int kLoraKG = 2;       // wavefront groups that split the rank between them (even / odd 16-wide steps)
+constexpr int kLoraThreads = 2 * kLoraCols * kLoraKG;
 constexpr int kLoraStage = (kLoraRows * (kLoraMaxR / 8 + 1) + kLoraThreads - 1) / kLoraThreads;  // pieces per thread
 
 // Every lane first requests its whole weight row (up to 32 pieces of 8), the block turns its 32 x R slice of the
@@ -40,7 +42,8 @@ __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs
   const int ld = R + 8;
   const int m0 = blockIdx.y * kLoraRows;
   const int mn = min(kLoraRows, a.M - m0);
-  const int wave = threadIdx.x >> 6;
+  const int wave = (threadIdx.x >> 6) & 3;
+  const int kg = threadIdx.x >> 8;  // this wavefront's share of the rank: steps kg, kg + 2, ...
   const int lane = threadIdx.x & 63;
   const int j = lane & 31;
   const int h = lane >> 5;
@@ -50,15 +53,15 @@ __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs
   const half_t* wrow = p.w2 + static_cast<int64_t>(col_ok ? c : 0) * R;
 
   // this lane's W2 values, all requested before the activation work: k = 16*kk + 8h .. +8 of output channel c
-  half8_t w[kLoraMaxR / 16];
+  half8_t w[kLoraMaxR / 16 / kLoraKG];
 #pragma unroll
-  for (int kk = 0; kk < kLoraMaxR / 16; ++kk) {
-    const int k = kk * 16 + h * 8;
+  for (int i = 0; i < kLoraMaxR / 16 / kLoraKG; ++i) {
+    const int k = (i * kLoraKG + kg) * 16 + h * 8;
     if (k < R) {
-      w[kk] = *reinterpret_cast<const half8_t*>(wrow + k);
+      w[i] = *reinterpret_cast<const half8_t*>(wrow + k);
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) w[kk][e] = static_cast<half_t>(0.0f);
+      for (int e = 0; e < 8; ++e) w[i][e] = static_cast<half_t>(0.0f);
     }
   }
 
@@ -103,16 +106,30 @@ __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
 #pragma unroll
-  for (int kk = 0; kk < kLoraMaxR / 16; ++kk) {
-    const int k = kk * 16;
+  for (int i = 0; i < kLoraMaxR / 16 / kLoraKG; ++i) {
+    const int k = (i * kLoraKG + kg) * 16;
     if (k < R) {
       const half8_t ah = *reinterpret_cast<const half8_t*>(&hi_s[j * ld + k + h * 8]);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, w[kk], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, w[i], acc, 0, 0, 0);
       if (split) {
         const half8_t al = *reinterpret_cast<const half8_t*>(&lo_s[j * ld + k + h * 8]);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, w[kk], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, w[i], acc, 0, 0, 0);
       }
     }
+  }
+  // the second group's sums go through LDS (over the lo tile, which nobody reads any more) to the first
+  __syncthreads();
+  float* xch = reinterpret_cast<float*>(lo_s) + (wave * 64 + lane) * 16;
+  if (kg == 1) {
+#pragma unroll
+    for (int v = 0; v < 16; v += 4) *reinterpret_cast<float4_t*>(xch + v) = float4_t{acc[v], acc[v + 1], acc[v + 2], acc[v + 3]};
+  }
+  __syncthreads();
+  if (kg == 1) return;
+#pragma unroll
+  for (int v = 0; v < 16; v += 4) {
+    const float4_t o = *reinterpret_cast<const float4_t*>(xch + v);
+    acc[v] += o[0]; acc[v + 1] += o[1]; acc[v + 2] += o[2]; acc[v + 3] += o[3];
   }
 
   if (!col_ok) return;
