@@ -245,6 +245,12 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
     s->sparse_ws_bytes = bytes;
   }
   if (static_cast<int>(rows) > s->tokens_cap) {
+    // captured decode graphs read their tokens from the old buffer (embedding gather, token feedback)
+    for (auto& g : s->graphs) {
+      if (g.exec) (void)hipGraphExecDestroy(g.exec);
+      if (g.graph) (void)hipGraphDestroy(g.graph);
+    }
+    s->graphs.clear();
     RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
     if (s->tokens_dev) RWKV_HIP_TRY(hipFree(s->tokens_dev));
     if (s->tokens_pinned) RWKV_HIP_TRY(hipHostFree(s->tokens_pinned));

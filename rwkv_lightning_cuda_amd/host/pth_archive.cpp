@@ -213,6 +213,12 @@ Result<PthArchive> PthArchive::open(const std::string& path, bool chunk_load) {
     if (e.data_offset > ar.file_size_ || e.compressed_size > ar.file_size_ - e.data_offset) {
       return Status::error("entry data is out of file bounds: " + e.name);
     }
+    // a stored member occupies exactly its uncompressed size: a directory that claims more would let a read
+    // run past the member (and past the file)
+    if (e.is_stored() && e.uncompressed_size != e.compressed_size) {
+      return Status::error("stored entry sizes disagree (compressed " + std::to_string(e.compressed_size) +
+                           ", uncompressed " + std::to_string(e.uncompressed_size) + "): " + e.name);
+    }
   }
   return ar;
 }
@@ -235,6 +241,11 @@ Status PthArchive::read_stored_entry_range(const PthEntry& entry, std::uint64_t 
   }
   if (size == 0) return Status::ok();
   if (destination == nullptr) return Status::error("null destination for entry: " + entry.name);
+  // the entry may not come from this archive's own directory: check it against the file again
+  // (src/pth_archive.cpp:511 does the same)
+  if (entry.data_offset > file_size_ || entry.uncompressed_size > file_size_ - entry.data_offset) {
+    return Status::error("entry data is out of file bounds: " + entry.name);
+  }
   const std::uint64_t from = entry.data_offset + entry_offset;
   if (!chunk_load_) {
     std::memcpy(destination, bytes_.data() + from, size);
@@ -246,6 +257,9 @@ Status PthArchive::read_stored_entry_range(const PthEntry& entry, std::uint64_t 
 }
 
 Result<std::vector<std::uint8_t>> PthArchive::read_stored_entry(const PthEntry& entry) const {
+  if (entry.is_stored() && (entry.data_offset > file_size_ || entry.uncompressed_size > file_size_ - entry.data_offset)) {
+    return Status::error("entry data is out of file bounds: " + entry.name);  // before anything is allocated
+  }
   std::vector<std::uint8_t> out(static_cast<std::size_t>(entry.is_stored() ? entry.uncompressed_size : 0));
   Status s = read_stored_entry_range(entry, 0, out.data(), out.size());
   if (!s.ok_status()) return s;
@@ -256,6 +270,9 @@ Result<std::vector<std::uint8_t>> PthArchive::read_stored_entry(const PthEntry& 
 Result<PthEntryView> PthArchive::stored_entry_view(const PthEntry& entry) const {
   if (chunk_load_) return Status::error("entry views need the whole file in memory (chunk_load is on): " + entry.name);
   if (!entry.is_stored()) return Status::error("entry is compressed: " + entry.name);
+  if (entry.data_offset > file_size_ || entry.uncompressed_size > file_size_ - entry.data_offset) {
+    return Status::error("entry data is out of file bounds: " + entry.name);  // src/pth_archive.cpp:578
+  }
   PthEntryView view;
   view.data = bytes_.data() + entry.data_offset;
   view.size = entry.uncompressed_size;

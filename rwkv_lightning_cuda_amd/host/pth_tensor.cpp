@@ -8,6 +8,7 @@
 #include "pth_tensor.hpp"
 
 #include <algorithm>
+#include <cstdint>
 #include <cmath>
 #include <cstring>
 #include <map>
@@ -218,6 +219,7 @@ private:
     if (f[1]->text != "torch.BFloat16Storage") {
       throw PickleError("unsupported storage dtype; this reader only supports torch.BFloat16Storage, got: " + f[1]->text);
     }
+    if (f[4]->num < 0) throw PickleError("negative storage element count");
     auto st = make(Obj::kStorage);
     st->text = f[2]->text;
     st->count = static_cast<std::uint64_t>(f[4]->num);
@@ -252,6 +254,18 @@ private:
         throw PickleError("unsupported _rebuild_tensor_v2 arguments");
       }
       if (t->tensor.shape.size() != t->tensor.stride.size()) throw PickleError("tensor shape / stride rank mismatch");
+      if (a[1]->num < 0) throw PickleError("negative tensor storage offset");
+      {
+        // dimensions are non-negative and their product fits 63 bits: every later size computation is then exact
+        std::uint64_t count = 1;
+        for (std::int64_t d : t->tensor.shape) {
+          if (d < 0) throw PickleError("negative tensor dimension");
+          if (d != 0 && count > (static_cast<std::uint64_t>(1) << 62) / static_cast<std::uint64_t>(d)) {
+            throw PickleError("tensor element count overflows");
+          }
+          count *= static_cast<std::uint64_t>(d);
+        }
+      }
       t->tensor.dtype = TensorDType::kBFloat16;
       t->tensor.storage_key = a[0]->text;
       t->tensor.storage_size = a[0]->count;
@@ -289,10 +303,13 @@ std::string top_folder(const PthArchive& archive) {
   return {};
 }
 
+// Product of the dimensions; 0 for a negative dimension, saturates instead of wrapping (records from the pickle
+// machine are already range-checked, hand-made ones may not be).
 std::uint64_t element_count(const std::vector<std::int64_t>& shape) {
   std::uint64_t n = 1;
   for (std::int64_t d : shape) {
     if (d < 0) return 0;
+    if (d != 0 && n > UINT64_MAX / static_cast<std::uint64_t>(d)) return UINT64_MAX;
     n *= static_cast<std::uint64_t>(d);
   }
   return n;
@@ -473,13 +490,17 @@ Result<TensorData> load_bf16_tensor_select(const PthArchive& archive, const Tens
   TensorData out;
   out.name = record.name;
   out.shape = record.shape;
-  const std::size_t n = static_cast<std::size_t>(element_count(record.shape));
+  // nothing is reserved before the element count has been checked against the storage: a state dict's tensors are
+  // views of their storage without repeated elements, so a count beyond the storage is a damaged record
+  const std::uint64_t n64 = element_count(record.shape);
+  if (n64 > record.storage_size || record.storage_offset > record.storage_size ||
+      (row_major(record.shape, record.stride) && n64 > record.storage_size - record.storage_offset)) {
+    return Status::error("tensor data range exceeds storage: " + record.name);
+  }
+  const std::size_t n = static_cast<std::size_t>(n64);
   if (need_bf16) out.values_bf16.reserve(n);
   if (need_f16) out.values_f16.reserve(n);
   if (need_float) out.values.reserve(n);
-  if (row_major(record.shape, record.stride) && record.storage_offset + n > record.storage_size) {
-    return Status::error("tensor data range exceeds storage: " + record.name);
-  }
   const bool inside = walk(record, [&](std::uint64_t at) {
     const std::uint16_t b = bits_at(storage, at);
     if (need_bf16) out.values_bf16.push_back(b);

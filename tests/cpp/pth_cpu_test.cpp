@@ -167,6 +167,40 @@ HOST_TEST(damaged_and_unsupported_archives) {
   CHECK(!PthArchive::open(path2, true).ok());
   std::remove(path.c_str());
   std::remove(path2.c_str());
+  // a stored member whose directory entry claims more bytes than the member holds: refused at open (a read of
+  // the claimed size would run past the member and past the file), in both modes
+  {
+    std::vector<Member> two{{"m/data.pkl", {1, 2, 3, 4}}, {"m/data/0", {9, 8, 7, 6, 5}}};
+    std::vector<std::uint8_t> zz = zip_bytes(two, false);
+    std::size_t dir = 0;
+    for (std::size_t i = 0; i + 4 <= zz.size(); ++i) {
+      if (zz[i] == 0x50 && zz[i + 1] == 0x4b && zz[i + 2] == 0x01 && zz[i + 3] == 0x02) { dir = i; break; }
+    }
+    CHECK(dir != 0);
+    const std::uint32_t claimed = 1u << 30;
+    for (int b = 0; b < 4; ++b) zz[dir + 24 + b] = static_cast<std::uint8_t>(claimed >> (8 * b));
+    const std::string bad = write_temp("oversize", zz);
+    for (bool lazy : {false, true}) {
+      auto opened = PthArchive::open(bad, lazy);
+      CHECK(!opened.ok());
+      CHECK(opened.status().message().find("stored entry sizes disagree") != std::string::npos);
+    }
+    std::remove(bad.c_str());
+    // and an entry record that does not come from the archive's own directory is checked against the file again
+    const std::string good = write_temp("oversize_good", zip_bytes(two, false));
+    for (bool lazy : {false, true}) {
+      auto opened = PthArchive::open(good, lazy);
+      CHECK(opened.ok());
+      PthEntry forged = *opened.value().find_entry("m/data/0");
+      forged.uncompressed_size = 1u << 20;
+      forged.compressed_size = 1u << 20;
+      std::vector<std::uint8_t> buf(64);
+      CHECK(!opened.value().read_stored_entry_range(forged, 0, buf.data(), buf.size()).ok_status());
+      CHECK(!opened.value().read_stored_entry(forged).ok());
+      CHECK(!opened.value().stored_entry_view(forged).ok());
+    }
+    std::remove(good.c_str());
+  }
   // a pickle that is not a tensor state dict
   std::vector<Member> odd{{"m/data.pkl", {0x80, 2, ']', '.'}}};
   const std::string path3 = write_temp("odd", zip_bytes(odd, false));

@@ -36,10 +36,42 @@ def test_wkv7_f32_matches_oracle(gpu, orc, B, T, H, mode):
     hip.device_sync()
     err = rel_err(y.numpy(), y_ref)
     assert err <= WKV_TOL
+    err = elem_err(y.numpy(), y_ref)          # per element, not only against the largest output
+    assert err <= WKV_TOL
     err = rel_err(state.numpy(), s_ref)
     assert err <= WKV_TOL
     err = elem_err(state.numpy(), s_ref)
     assert err <= WKV_TOL
+
+
+def test_wkv7_drift_over_16384_tokens_against_the_fp32_oracle(gpu, orc):
+    """The long-context configuration's length against the oracle (B = 1, H = 2, T = 16384, fp16 operands with the
+    configuration-0 distributions, fp32 state): the state after 16384 sequential updates within 1e-4 of the
+    oracle's, relative to its scale and per element, and the outputs of the last 128 tokens within the fp16 bar -
+    the two sides differ only in summation order and in the last bits of the decay map, and the decay keeps
+    those differences from accumulating."""
+    hip = gpu
+    B, T, H = 1, 16384, 2
+    C = H * 64
+    inp = wkv_inputs(B, T, H, seed=16384, dtype=np.float16)
+    names = ["r", "w_raw", "k", "v", "a", "b"]
+    s_ref = np.zeros((B, H, 64, 64), np.float32)
+    y_ref = orc.wkv7(s_ref, *[inp[n] for n in names], H, 0)
+    d = {n: dev(hip, inp[n]) for n in names}
+    state = hip.DeviceArray.zeros((B, H, 64, 64), np.float32)
+    y = hip.DeviceArray((B, T, C), np.float16)
+    hip.wkv7(B, T, C, H, hip.W_RAW_LOGIT, hip.IO_F16, state, *[d[n] for n in names], y)
+    hip.device_sync()
+    s_rel = rel_err(state.numpy(), s_ref)
+    s_elem = elem_err(state.numpy(), s_ref)
+    y_last = rel_err(y.numpy()[:, -128:].astype(np.float32), y_ref[:, -128:].astype(np.float32))
+    y_all = rel_err(y.numpy().astype(np.float32), y_ref.astype(np.float32))
+    print("wkv7 T=16384: state max-rel %.2e, per element %.2e; y last 128 tokens %.2e, all tokens %.2e"
+          % (s_rel, s_elem, y_last, y_all))
+    assert s_rel <= WKV_TOL
+    assert s_elem <= WKV_TOL
+    assert y_last <= F16_TOL
+    assert y_all <= F16_TOL
 
 
 def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):

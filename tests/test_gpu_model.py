@@ -22,6 +22,35 @@ def small_dims():
     return ModelDims(L=3, C=256, H=4, F=1024, V=2048, Rw=32, Ra=32, Rg=64, Rv=16)
 
 
+_CFG3 = {}
+
+
+def cfg3_pair(gpu, orc, fmt):
+    """Benchmark configuration 3 at full width (C 4096, H 64, F 16384, LoRA ranks 128/128/480/96), two layers and a
+    reduced vocabulary; the host weights and the models of both sides are built once per format and shared by the
+    tests of this module (generating the fp16 weights takes longer than any of the tests)."""
+    import os
+    from rwkv_lightning_cuda_amd.model import PRESETS, HipModel, ModelDims, synth_weights
+    big = PRESETS["7.2B"]
+    dims = ModelDims(L=2, C=big.C, H=big.H, F=big.F, V=8192, Rw=big.Rw, Ra=big.Ra, Rg=big.Rg, Rv=big.Rv)
+    if "weights" not in _CFG3:
+        _CFG3["weights"] = synth_weights(dims, 77)
+    if fmt not in _CFG3:
+        orc.set_threads(min(16, os.cpu_count() or 1))  # the oracle's results do not depend on the thread count
+        _CFG3[fmt] = (orc.Model(dims, _CFG3["weights"], fmt), HipModel.from_host_weights(dims, _CFG3["weights"], fmt))
+    orc.set_threads(min(16, os.cpu_count() or 1))
+    return (dims,) + _CFG3[fmt]
+
+
+def tie_or_fail(ologits_row, want, got, what):
+    """A token that differs from the oracle's is accepted only as a tie: logits are fp16-rounded values and a
+    random-init head is nearly flat at the top, so the oracle's own best two can sit one or two fp16 ulps apart and
+    either side may then order them differently.  Anything further apart fails."""
+    gap = float(ologits_row[want] - ologits_row[got])
+    ulp = float(np.spacing(np.float16(abs(ologits_row[want]))))
+    assert gap <= 2 * ulp, "%s: token %d instead of %d, oracle gap %.5f (fp16 ulp %.5f)" % (what, got, want, gap, ulp)
+
+
 def build_pair(gpu, orc, dims, fmt, seed):
     from rwkv_lightning_cuda_amd.model import HipModel, synth_weights
     weights = synth_weights(dims, seed)
@@ -317,6 +346,7 @@ def test_config1_0p1b_prefill_512_then_128_greedy_steps(gpu, orc):
             assert gap <= 2 * ulp, "step %d: token %d instead of %d, oracle gap %.5f (ulp %.5f)" % (i, got, want, gap, ulp)
             ties += 1
         tok = np.array([[want]], np.int64)
+    print("config 1: %d tie-breaks (oracle's best two within 2 fp16 ulps) in %d greedy steps" % (ties, steps))
     assert ties <= 3, "%d tie-breaks in %d steps" % (ties, steps)
     orc.set_threads(1)
     cos = cosine(glogits.numpy(), ologits)
@@ -385,16 +415,10 @@ def test_config3_7p2b_width_two_layers_quantised(gpu, orc, fmt_name):
     reduced vocabulary, W8A16 and W4A16 quantised from the same fp16 weights on both sides: one prefill call of
     2 x 16 tokens (streaming MFMA GEMM, row-tiled time-mix kernels) and decode steps at batch 2 (GEMV, fused
     time-mix kernel), per-layer residual streams and logits against the oracle."""
-    import os
-    from rwkv_lightning_cuda_amd.model import PRESETS, HipModel, ModelDims, Session, State, synth_weights
+    from rwkv_lightning_cuda_amd.model import Session, State
     hip = gpu
-    big = PRESETS["7.2B"]
-    dims = ModelDims(L=2, C=big.C, H=big.H, F=big.F, V=8192, Rw=big.Rw, Ra=big.Ra, Rg=big.Rg, Rv=big.Rv)
     fmt = {"w8": hip.FMT_W8, "w4": hip.FMT_W4}[fmt_name]
-    weights = synth_weights(dims, 77)
-    orc.set_threads(min(16, os.cpu_count() or 1))
-    omodel = orc.Model(dims, weights, fmt)
-    gmodel = HipModel.from_host_weights(dims, weights, fmt)
+    dims, omodel, gmodel = cfg3_pair(gpu, orc, fmt)
     rng = np.random.default_rng(6)
     B, T = 2, 16
     tokens = rng.integers(0, dims.V, (B, T))
@@ -437,6 +461,161 @@ def test_config3_7p2b_width_two_layers_quantised(gpu, orc, fmt_name):
     # the state integrates the first tokens' perturbation (above): 5e-3 of its scale
     err = rel_err(gstate.wkv.numpy(), ostate[1])
     assert err <= 5e-3
+    sess.close()
+
+
+def test_config3_7p2b_width_w8_batch1_chunk128_prefill_then_256_greedy_steps(gpu, orc):
+    """Benchmark configuration 3 at its own batch-1 sizes (full width, two layers, reduced vocabulary, W8A16): one
+    128-token prefill chunk (the 128-row streaming-GEMM tile, the row-range-split WKV sequence kernels), then 256
+    greedy steps through the device-side loop (GEMV launches, single-launch time-mix core, row-skipping ffn.value,
+    graph replay).  The token stream must be the oracle's; a differing token is accepted only where the oracle's
+    own best two are within two fp16 ulps (counted and reported; the GPU is then re-run with the oracle's tokens
+    forced up to that step), anything else fails."""
+    from rwkv_lightning_cuda_amd.model import Session, State
+    hip = gpu
+    dims, omodel, gmodel = cfg3_pair(gpu, orc, hip.FMT_W8)
+    rng = np.random.default_rng(31)
+    prompt = rng.integers(0, dims.V, (1, 128))
+    steps = 256
+
+    ostate = omodel.new_state(1)
+    ologits = omodel.forward(prompt, ostate)
+    after_prompt = ologits.copy()
+    first = int(np.argmax(ologits[0]))
+    want = np.zeros(steps, np.int64)
+    orows = np.zeros((steps, dims.V), np.float32)
+    tok = first
+    for i in range(steps):
+        ologits = omodel.forward(np.array([[tok]], np.int64), ostate)
+        orows[i] = ologits[0]
+        want[i] = tok = int(np.argmax(ologits[0]))
+
+    sess = Session(gmodel)
+    glogits = hip.DeviceArray((1, dims.V), np.float32)
+
+    def gpu_stream(forced):
+        """Fresh state, the prompt, `forced` steps fed with the oracle's tokens, the rest free-running on the device.
+        Returns the tokens picked at steps forced .. steps-1 and the state."""
+        st = State(dims, 1)
+        sess.forward(prompt, st, glogits)
+        if forced == 0:
+            cos = cosine(glogits.numpy(), after_prompt)
+            assert cos >= 0.9995
+            assert int(np.argmax(glogits.numpy()[0])) == first
+        feed = [first] + want[:forced].tolist()   # feed[i] is the input of step i
+        for i in range(forced):
+            sess.forward(np.array([[feed[i]]], np.int64), st, glogits)
+        got = sess.decode_greedy(np.array([feed[forced]]), steps - forced, st, glogits)
+        return got[:, 0], st
+
+    ties = 0
+    forced = 0
+    while True:
+        got, gstate = gpu_stream(forced)
+        diff = np.nonzero(got != want[forced:])[0]
+        if diff.size == 0:
+            break
+        i = forced + int(diff[0])
+        tie_or_fail(orows[i], int(want[i]), int(got[diff[0]]), "step %d" % i)
+        ties += 1
+        assert ties <= 3, "more than 3 tie-breaks in %d steps" % steps
+        forced = i + 1   # the step is redone with the oracle's tokens up to and including this one
+    print("config 3 batch 1: %d tie-breaks (oracle's best two within 2 fp16 ulps) in %d greedy steps" % (ties, steps))
+    cos = cosine(glogits.numpy(), orows[-1])
+    assert cos >= 0.9995
+    act = sess.debug_buffer("act", (1, dims.F))
+    frac = float(np.mean(act == 0))
+    assert 0.2 <= frac <= 0.8, frac   # the row-skipping product really skipped rows
+    err = rel_err(gstate.wkv.numpy(), ostate[1])
+    assert err <= 5e-3
+    assert gstate.elapsed.numpy().tolist() == [128 + steps]
+    orc.set_threads(1)
+    sess.close()
+
+
+@pytest.mark.parametrize("fmt_name,B", [("w8", 16), ("w8", 64), ("w4", 16), ("w4", 64)])
+def test_config3_7p2b_width_batched_decode(gpu, orc, fmt_name, B):
+    """Benchmark configuration 3 at batch 16 and 64 (full width, two layers, reduced vocabulary; W8A16 and W4A16):
+    per-sequence state from a short random prefill, then decode steps on the streaming-GEMM path with the LoRA
+    rank-outs on the matrix core and the fused time-mix pass over 64 heads per sequence: every row's logits against
+    the oracle (cosine >= 0.9995, same top-1 except for ties of the oracle's best two within two fp16 ulps)."""
+    from rwkv_lightning_cuda_amd.model import Session, State
+    hip = gpu
+    fmt = {"w8": hip.FMT_W8, "w4": hip.FMT_W4}[fmt_name]
+    dims, omodel, gmodel = cfg3_pair(gpu, orc, fmt)
+    rng = np.random.default_rng(100 + B)
+    P = 16 if B == 16 else 8
+    steps = 3 if B == 16 else 2
+    prompt = rng.integers(0, dims.V, (B, P))
+    sess = Session(gmodel)
+    gstate = State(dims, B)
+    glogits = hip.DeviceArray((B, dims.V), np.float32)
+    ostate = omodel.new_state(B)
+    sess.forward(prompt, gstate, glogits)
+    ologits = omodel.forward(prompt, ostate)
+    ties = 0
+    for step in range(steps + 1):
+        g = glogits.numpy()
+        for b in range(B):
+            cos = cosine(g[b], ologits[b])
+            assert cos >= 0.9995, "step %d row %d" % (step, b)
+            w_, g_ = int(np.argmax(ologits[b])), int(np.argmax(g[b]))
+            if w_ != g_:
+                tie_or_fail(ologits[b], w_, g_, "step %d row %d" % (step, b))
+                ties += 1
+        err = rel_err(g, ologits)
+        assert err <= 4e-3
+        if step == steps:
+            break
+        nxt = np.argmax(ologits, axis=1).reshape(B, 1)
+        sess.forward(nxt, gstate, glogits)
+        ologits = omodel.forward(nxt, ostate)
+    print("config 3 %s batch %d: %d top-1 ties over %d rows x %d logit rows" % (fmt_name, B, ties, B, steps + 1))
+    assert ties <= max(2, B // 8)
+    err = rel_err(gstate.wkv.numpy(), ostate[1])
+    assert err <= 5e-3
+    err = rel_err(gstate.shift.numpy().astype(np.float32), ostate[0].astype(np.float32))
+    assert err <= 4e-3
+    assert gstate.elapsed.numpy().tolist() == [P + steps] * B
+    orc.set_threads(1)
+    sess.close()
+
+
+def test_config3_7p2b_width_w4_batch1_greedy_steps(gpu, orc):
+    """W4A16 at batch 1 and full width: the int4 GEMV and the int4 row-skipping ffn.value inside the graph, 48 greedy
+    steps after a 32-token prefill, token stream against the oracle (ties as above)."""
+    from rwkv_lightning_cuda_amd.model import Session, State
+    hip = gpu
+    dims, omodel, gmodel = cfg3_pair(gpu, orc, hip.FMT_W4)
+    rng = np.random.default_rng(77)
+    prompt = rng.integers(0, dims.V, (1, 32))
+    steps = 48
+    sess = Session(gmodel)
+    gstate = State(dims, 1)
+    glogits = hip.DeviceArray((1, dims.V), np.float32)
+    ostate = omodel.new_state(1)
+    sess.forward(prompt, gstate, glogits)
+    ologits = omodel.forward(prompt, ostate)
+    cos = cosine(glogits.numpy(), ologits)
+    assert cos >= 0.9995
+    tok = int(np.argmax(ologits[0]))
+    ties = 0
+    for i in range(steps):
+        feed = np.array([[tok]], np.int64)
+        sess.forward(feed, gstate, glogits)
+        ologits = omodel.forward(feed, ostate)
+        want, got = int(np.argmax(ologits[0])), int(np.argmax(glogits.numpy()[0]))
+        if got != want:
+            tie_or_fail(ologits[0], want, got, "step %d" % i)
+            ties += 1
+        tok = want
+    print("config 3 w4 batch 1: %d tie-breaks in %d greedy steps" % (ties, steps))
+    assert ties <= 2
+    cos = cosine(glogits.numpy(), ologits)
+    assert cos >= 0.9995
+    err = rel_err(gstate.wkv.numpy(), ostate[1])
+    assert err <= 5e-3
+    orc.set_threads(1)
     sess.close()
 
 
