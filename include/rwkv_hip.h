@@ -156,6 +156,17 @@ int rwkv_hip_cmix_sparse_down_relu_rows(rwkv_stream_t s, int fmt, int rows, int 
                                         void* out);
 int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int fmt, int C, int F, const void* preact, const void* wt,
                                        const void* scale, void* workspace, size_t workspace_bytes, void* out);
+/* The same product as rwkv_hip_cmix_sparse_down_relu_rows (same kernels, bitwise the same result) for callers
+ * that cannot allocate or bring a workspace: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  No counterpart in the reference.  The fp32 partial rows live in a 16 MiB array that is part
+ * of the library's device image (one copy per GPU, held until the process ends); the call allocates and frees
+ * nothing.  rows * (F / 256) * C * 4 bytes must fit in it (7.2B shape: all 12 rows), else RWKV_E_INVALID.  Every
+ * call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls
+ * on one stream are ordered.  Nothing in the array needs clearing between calls (every partial row that is read
+ * has been written by the same call).  The first call on a device looks up the array's device address
+ * (hipGetSymbolAddress), so make it outside a stream capture. */
+int rwkv_hip_cmix_sparse_down_relu_rows_static(rwkv_stream_t s, int fmt, int rows, int C, int F, const void* preact,
+                                               const void* wt, const void* scale, void* out);
 
 /* ---- LoRA pairs.  Replaces rwkv7_v3a_linear_wag(v)_rank_in_f16_launch,
  * rwkv7_v3a_linear_wag(v)_rank_out_f16_launch, rwkv7_v3a_linear_t_f16_launch,

@@ -18,9 +18,17 @@
 // values of the two rows (int8: bytes under exponent 0x64, then one packed subtract gives the exact codes).  The eight wavefronts' sums meet in LDS in wavefront
 // order and the block writes one fp32 partial row.  Kernel 2 sums the F/256 partial rows in a fixed order,
 // applies the scale and rounds to fp16.
+#include <mutex>
+
 #include "ops.h"
 
 namespace rwkv {
+
+// Partial rows of the entry point that allocates nothing (rwkv_hip_cmix_sparse_down_relu_rows_static): a fixed
+// array in the library's device image, one copy per GPU, held until the process ends.  In host code this name
+// is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+constexpr size_t kStaticScratchBytes = static_cast<size_t>(16) << 20;
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
 
 constexpr int kSparseRowsPerWave = 32;
 constexpr int kSparseWaves = 8;
@@ -459,6 +467,40 @@ int rwkv_hip_cmix_sparse_down_relu_rows(rwkv_stream_t s, int fmt, int rows, int 
                                         void* out) {
   return ffn_sparse_launch(as_stream(s), fmt, rows, C, F, 0, static_cast<const half_t*>(preact), wt,
                            static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr);
+}
+
+// Device address of this GPU's copy of `scratch`, looked up once per device (with that device current).
+static int static_scratch_address(float** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static float* address[kMaxDevices] = {nullptr};
+  int dev = 0;
+  RWKV_HIP_TRY(hipGetDevice(&dev));
+  RWKV_REQUIRE(dev >= 0 && dev < kMaxDevices, "cmix_sparse_static: device index %d out of range", dev);
+  std::lock_guard<std::mutex> guard(lock);
+  if (address[dev] == nullptr) {
+    float* p = nullptr;
+    RWKV_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)));
+    RWKV_REQUIRE(p != nullptr, "cmix_sparse_static: no device address for the scratch array");
+    address[dev] = p;
+  }
+  *out = address[dev];
+  return RWKV_OK;
+}
+
+int rwkv_hip_cmix_sparse_down_relu_rows_static(rwkv_stream_t s, int fmt, int rows, int C, int F, const void* preact,
+                                               const void* wt, const void* scale, void* out) {
+  RWKV_REQUIRE(ffn_sparse_supported(fmt, C, F), "cmix_sparse_static: unsupported format %d or shape C=%d F=%d", fmt, C, F);
+  RWKV_REQUIRE(rows >= 1 && rows <= kSparseMaxRows, "cmix_sparse_static: %d rows (1..%d)", rows, kSparseMaxRows);
+  const size_t need = ffn_sparse_workspace_bytes(rows, C, F);
+  RWKV_REQUIRE(need <= kStaticScratchBytes,
+               "cmix_sparse_static: rows=%d C=%d F=%d needs %zu bytes of partial rows, the built-in scratch holds %zu", rows,
+               C, F, need, kStaticScratchBytes);
+  float* ws = nullptr;
+  const int rc = static_scratch_address(&ws);
+  if (rc != RWKV_OK) return rc;
+  return ffn_sparse_launch(as_stream(s), fmt, rows, C, F, 0, static_cast<const half_t*>(preact), wt,
+                           static_cast<const half_t*>(scale), ws, kStaticScratchBytes, static_cast<half_t*>(out), nullptr);
 }
 
 int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int fmt, int C, int F, const void* preact, const void* wt,

@@ -38,7 +38,7 @@ EXPORTS = [
     "rwkv_hip_pack_weights", "rwkv_hip_linear_packed_workspace", "rwkv_hip_linear_packed", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
     "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_pack_w4", "rwkv_hip_cmix_sparse_packed_bytes",
     "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
-    "rwkv_hip_cmix_sparse_down_relu_rows",
+    "rwkv_hip_cmix_sparse_down_relu_rows", "rwkv_hip_cmix_sparse_down_relu_rows_static",
     "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln",
     "rwkv_hip_layer_norm", "rwkv_hip_add_layer_norm", "rwkv_hip_add_last_layer_norm", "rwkv_hip_token_shift_mix",
     "rwkv_hip_add_layer_norm_cmix_mix", "rwkv_hip_add_layer_norm_tmix_mix6", "rwkv_hip_kk_a_gate",
@@ -283,6 +283,12 @@ def cmix_sparse_down_relu_one(fmt, C, F, preact, wt, scale, workspace, out, stre
 def cmix_sparse_down_relu_rows(fmt, rows, C, F, preact, wt, scale, workspace, out, stream=None):
     check(load().rwkv_hip_cmix_sparse_down_relu_rows(_p(stream), _i(fmt), _i(rows), _i(C), _i(F), _p(preact), _p(wt),
                                                      _p(scale), _p(workspace), ctypes.c_size_t(workspace.nbytes), _p(out)))
+
+
+def cmix_sparse_down_relu_rows_static(fmt, rows, C, F, preact, wt, scale, out, stream=None):
+    """The product above with the partial rows in the library's built-in scratch array: allocates nothing."""
+    check(load().rwkv_hip_cmix_sparse_down_relu_rows_static(_p(stream), _i(fmt), _i(rows), _i(C), _i(F), _p(preact),
+                                                            _p(wt), _p(scale), _p(out)))
 
 
 def lora_out(M, C, R, act, h, w2, out, bias=None, vres=0, v=None, v_first=None, stream=None):
