@@ -32,8 +32,30 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak, published
 # HBM bytes per launch of the GEMV kernel from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (two runs), each scaled
 # by what the same counter reads for a 1 GiB device-to-device copy (FETCH_SIZE reads half the bytes copied,
-# WRITE_SIZE all of them); the summary of those runs is kept under profiles/.  Keyed by (preset, format, batch).
-MEASURED_TRAFFIC = {("7.2B", "w8", 1): 2.0 * 24290.5 * 1024 + 1.0 * 45.9 * 1024}
+# WRITE_SIZE all of them).  Keyed by (preset, format, batch); each record names the summary under profiles/ it was
+# taken from and the SHA-256 of the kernel source it was measured on: when csrc/linear.hip no longer matches, the
+# figure is stale and `traffic` is reported as null until the counters are collected again.
+MEASURED_TRAFFIC = {
+    ("7.2B", "w8", 1): {
+        "bytes_per_launch": None,
+        "profile": "profiles/linear_gemv_row1_decode_7p2b_w8_bs1_pmc_traffic.md",
+        "kernel_source": "rwkv_lightning_cuda_amd/csrc/linear.hip",
+        "kernel_source_sha256": None,
+    },
+}
+
+
+def measured_traffic(key):
+    """(bytes per launch or None, record) - None when there is no record or the kernel source has changed since."""
+    import hashlib
+    rec = MEASURED_TRAFFIC.get(key)
+    if rec is None or rec["bytes_per_launch"] is None:
+        return None, rec
+    with open(os.path.join(ROOT, rec["kernel_source"]), "rb") as f:
+        sha = hashlib.sha256(f.read()).hexdigest()
+    if sha != rec["kernel_source_sha256"]:
+        return None, dict(rec, stale=True)
+    return rec["bytes_per_launch"], rec
 
 
 def parse_args():
@@ -87,38 +109,48 @@ def gemv_bytes_per_step(dims, fmt, sparse_value):
 
 def cpu_baseline(dims, fmt_name):
     """Times the CPU oracle on one decode step of 1- and 2-layer slices of the same shape (full width, full
-    vocabulary) and extrapolates linearly in the layer count to the full depth."""
+    vocabulary) and extrapolates linearly in the layer count to the full depth: with all host threads (the headline
+    `value`) and with one thread."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle
     from rwkv_lightning_cuda_amd.model import ModelDims, synth_weights
     threads = min(os.cpu_count() or 1, 16)
-    oracle.set_threads(threads)
     fmt = {"f16": 0, "w8": 1, "w4": 2}[fmt_name]
-    times = {}
     d2 = ModelDims(L=2, C=dims.C, H=dims.H, F=dims.F, V=dims.V, Rw=dims.Rw, Ra=dims.Ra, Rg=dims.Rg, Rv=dims.Rv)
     weights = synth_weights(d2, seed=7)
+    models = {}
     for layers in (1, 2):
         d = ModelDims(L=layers, C=dims.C, H=dims.H, F=dims.F, V=dims.V, Rw=dims.Rw, Ra=dims.Ra, Rg=dims.Rg, Rv=dims.Rv)
-        om = oracle.Model(d, dict(weights, layers=weights["layers"][:layers]), fmt)
-        st = om.new_state(1)
-        tok = np.array([[17]], np.int64)
-        om.forward(tok, st)  # touch everything once
-        reps = 3
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            om.forward(tok, st)
-        times[layers] = (time.perf_counter() - t0) / reps
-        del om
-    per_layer = max(times[2] - times[1], 1e-9)
-    fixed = max(times[1] - per_layer, 0.0)
-    step_s = fixed + per_layer * dims.L
+        models[layers] = oracle.Model(d, dict(weights, layers=weights["layers"][:layers]), fmt)
+    tok = np.array([[17]], np.int64)
+
+    def step_seconds(n_threads, reps):
+        oracle.set_threads(n_threads)
+        times = {}
+        for layers, om in models.items():
+            st = om.new_state(1)
+            om.forward(tok, st)  # touch everything once
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                om.forward(tok, st)
+            times[layers] = (time.perf_counter() - t0) / reps
+        per_layer = max(times[2] - times[1], 1e-9)
+        fixed = max(times[1] - per_layer, 0.0)
+        return fixed + per_layer * dims.L, per_layer, fixed
+
+    step_n, per_layer_n, fixed_n = step_seconds(threads, 3)
+    step_1, per_layer_1, fixed_1 = step_seconds(1, 1)
+    oracle.set_threads(1)
     return {
-        "value": 1.0 / step_s,
+        "value": 1.0 / step_n,
         "unit": "tok/s",
         "cores": threads,
         "kind": "port",
         "sample": "one batch-1 decode step of 1- and 2-layer slices at full width/vocab (%s), "
-                  "extrapolated linearly to %d layers: %.3f s/layer + %.3f s fixed" % (fmt_name, dims.L, per_layer, fixed),
+                  "extrapolated linearly to %d layers: %.3f s/layer + %.3f s fixed with %d threads; "
+                  "%.3f s/layer + %.3f s fixed with 1 thread" % (fmt_name, dims.L, per_layer_n, fixed_n, threads,
+                                                                per_layer_1, fixed_1),
+        "value_1_thread": 1.0 / step_1,
     }
 
 
@@ -237,6 +269,66 @@ def secondary_measurements(hip, model, dims, rng):
     return res
 
 
+def other_configs(hip, rng):
+    """Benchmark configurations 1 and 2 on the same GPU: the 0.1B shape with fp16 weights (512-token prompt in chunks
+    of 128, then 128 greedy steps at batch 1) and the 1.5B shape W8A16 (256-token prefill per sequence, then decode at
+    batch 1, 8 and 64)."""
+    from rwkv_lightning_cuda_amd.model import PRESETS, HipModel, Session, State
+    res = {}
+    dims = PRESETS["0.1B"]
+    model = HipModel.random_on_device(dims, hip.FMT_F16, seed=2)
+    sess = Session(model)
+    lg = hip.DeviceArray((1, dims.V), np.float32)
+    prompt = rng.integers(0, dims.V, (1, 512))
+    warm = State(dims, 1)
+    sess.forward(prompt[:, :128], warm, lg)
+    st = State(dims, 1)
+    hip.device_sync()
+    t0 = time.perf_counter()
+    for c0 in range(0, 512, 128):
+        sess.forward(prompt[:, c0:c0 + 128], st, lg, sync=False)
+    hip.device_sync()
+    res["cfg1_0p1b_f16_prefill512_tok_s"] = 512 / (time.perf_counter() - t0)
+    first = rng.integers(0, dims.V, (1,))
+    sess.decode_greedy(first, 8, st, lg)
+    hip.device_sync()
+    t0 = time.perf_counter()
+    sess.decode_greedy(first, 128, st, lg)
+    hip.device_sync()
+    dt = time.perf_counter() - t0
+    res["cfg1_0p1b_f16_decode_bs1_tok_s"] = 128 / dt
+    res["cfg1_0p1b_f16_decode_bs1_ms_per_step"] = dt * 1e3 / 128
+    sess.close()
+    model.close()
+    del model, st, warm
+
+    dims = PRESETS["1.5B"]
+    model = HipModel.random_on_device(dims, hip.FMT_W8, seed=3)
+    wbytes = model.weight_bytes()
+    for B in (1, 8, 64):
+        sess = Session(model)
+        st = State(dims, B)
+        lg = hip.DeviceArray((B, dims.V), np.float32)
+        prompt = rng.integers(0, dims.V, (B, 256))
+        for c0 in range(0, 256, 128):
+            sess.forward(prompt[:, c0:c0 + 128], st, lg, sync=False)
+        first = rng.integers(0, dims.V, (B,))
+        sess.decode_greedy(first, 8, st, lg)
+        hip.device_sync()
+        t0 = time.perf_counter()
+        sess.decode_greedy(first, 64, st, lg)
+        hip.device_sync()
+        dt = time.perf_counter() - t0
+        sbytes = B * (2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2)
+        res["cfg2_1p5b_w8_decode_bs%d_tok_s" % B] = 64 * B / dt
+        res["cfg2_1p5b_w8_decode_bs%d_ms_per_step" % B] = dt * 1e3 / 64
+        res["cfg2_1p5b_w8_decode_bs%d_hbm_fraction" % B] = (wbytes + sbytes) / (dt / 64) / 1e9 / HBM_PEAK_GBPS
+        sess.close()
+        del st, lg
+    model.close()
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -346,6 +438,11 @@ def main():
 
     weight_bytes = model.weight_bytes()
     state_bytes = B * (2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2)
+    # bytes the timed step really moved: the row-skipping ffn.value reads only the rows with a non-zero activation
+    # (fraction measured on the last layer's activations of the last step)
+    skipped = also.get("ffn_value_rows_skipped_fraction_last_layer", 0.0) if sparse_value else 0.0
+    value_code_bytes = dims.L * dims.C * dims.F * {"f16": 2.0, "w8": 1.0, "w4": 0.5}[args.fmt]
+    moved_bytes = weight_bytes + state_bytes - skipped * value_code_bytes
     out = {
         "metric": "decode tok/s @%s W%sA16 bs%d" % (args.preset, {"f16": "16", "w8": "8", "w4": "4"}[args.fmt], B),
         "value": value,
@@ -366,7 +463,11 @@ def main():
                    "hip_graph": not args.no_graph, "sparse_ffn_value": sparse_value,
                    "weight_bytes_per_step": weight_bytes,
                    "state_bytes_per_step": state_bytes,
+                   # dense convention: every weight byte counted once per step, whether the step read it or not
                    "step_hbm_fraction": (weight_bytes + state_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                   # the bytes the step really moved (rows of ffn.value with a zero activation are not read)
+                   "bytes_moved_per_step": moved_bytes,
+                   "bytes_moved_fraction": moved_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                    "distinct_tokens": int(len(np.unique(toks)))},
     }
 
@@ -390,13 +491,15 @@ def main():
         bytes_per_launch = gemv_bytes / per_step
         avg_ms = total_ms / launches
         achieved = bytes_per_launch / (avg_ms * 1e-3) / 1e9
-        traffic = MEASURED_TRAFFIC.get((args.preset, args.fmt, B))
+        traffic, traffic_rec = measured_traffic((args.preset, args.fmt, B))
         out["roofline"] = {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-            "kernel": "linear_gemv_kernel (weight-streaming GEMV: r/k/v + LoRA rank-ins, output, ffn.key%s, lm_head)"
-                      % ("" if sparse_value else ", ffn.value"),
+            "kernel": "linear_gemv_row1_kernel (weight-streaming GEMV: r/k/v + LoRA rank-ins with the LayerNorm prologue, "
+                      "output, ffn.key with the LayerNorm prologue%s, lm_head)" % ("" if sparse_value else ", ffn.value"),
             "bytes_per_launch": bytes_per_launch, "avg_launch_us": avg_ms * 1e3, "launches_per_step": per_step,
+            "traffic_source": (traffic_rec or {}).get("profile"),
+            "traffic_stale": bool((traffic_rec or {}).get("stale", False)),
         }
 
     if not args.no_also:
@@ -422,6 +525,11 @@ def main():
         also["decode_w4_bs1_hbm_fraction"] = (m4.weight_bytes() + sb4) / (t4 / 64) / 1e9 / HBM_PEAK_GBPS
         s4.close()
         del m4
+    if not args.no_also and args.preset == "7.2B":
+        also.update(other_configs(hip, rng))
+        # what a launch that waits for its predecessor costs on this box: a captured graph of 260 near-empty launches
+        also["launch_chain_us_per_link_graph"] = hip.measure_launch_chain(260, 256, 256, True, 20)
+        also["launch_chain_us_per_link_direct"] = hip.measure_launch_chain(260, 256, 256, False, 20)
     if also:
         out["also"] = also
     if not args.no_cpu_baseline:

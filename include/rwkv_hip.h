@@ -68,6 +68,13 @@ int rwkv_hip_event_destroy(void* ev);
 int rwkv_hip_event_record(void* ev, rwkv_stream_t s);
 int rwkv_hip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms);
 
+/* Measurement aid (no counterpart in the reference): the cost of a launch that has to wait for its predecessor.
+ * Runs a chain of `links` launches of a kernel that does next to nothing (every block reads a counter, one thread
+ * writes it back incremented) with `blocks` x `threads` each, on a stream of its own, `reps` times after one warm
+ * run - as direct launches or as one captured graph per run - and returns the microseconds per link.  A decode step
+ * at batch 1 is such a chain (8 launches per layer); this is the part of its time that no kernel can remove. */
+int rwkv_hip_measure_launch_chain(int links, int blocks, int threads, int use_graph, int reps, float* us_per_link);
+
 /* ---- WKV7 time-mix recurrence.  Replaces rwkv7_wkv_fp32io16_launch
  * (cuda/rwkv7_fast_v4_kernels.cuh:49-52, cuda/rwkv7_wkv_fp32_v2.cu:237-294).
  * state f32 [B,H,64,64] in/out; r,w,k,v,a,b,y [B,T,C], C == H*64.
@@ -297,10 +304,12 @@ int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double
  * non-zero with random-init weights, far fewer with trained ones.  0 selects the dense product. */
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
 /* Decode steps on the GEMV path (one or two rows) can fold the two LayerNorm + token-shift kernels of a layer
- * into the prologue of the linear launches that consume them (bitwise the same results).  on > 0: always,
- * 0: never, < 0 (the default): for one row of at most 1024 channels, where two launches fewer per layer are
- * worth more than the extra work inside every GEMV block (0.1B shape: 0.446 -> 0.423 ms per step; from 2048
- * channels on, or with two rows, the stand-alone kernels are faster).  No counterpart in the reference. */
+ * into the prologue of the linear launches that consume them.  on > 0: always, 0: never, < 0 (the default): for
+ * one row of at most 4096 channels.  One row goes through a kernel that requests whole weight rows up front and
+ * normalises while they are in flight (two launches fewer per layer: 7.2B shape 2.04 -> 1.92 ms per step, 0.1B
+ * shape 0.413 -> 0.373; same formulas and rounding points as the stand-alone kernels, sums associated differently);
+ * two rows through a prologue that is bitwise the stand-alone kernels but slower than them from 2048 channels
+ * on.  No counterpart in the reference (its fused decode kernels are cuda/rwkv7_v3a_ops.cu:1637-1798). */
 int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on);
 /* debugging/parity tap: device address of one of the session's activation buffers, holding what the last
  * layer of the last rwkv_hip_forward call left there.  Ids in order: x, xx, xr, xw, xk, xv, xa, xg, r, k, v,

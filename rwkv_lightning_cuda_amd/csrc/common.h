@@ -105,6 +105,45 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// x + (x of the lane that the DPP control CTRL pairs this lane with)
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false);
+  return x + __builtin_bit_cast(float, moved);
+}
+// Sum over the 16 lanes of a DPP row.  Every exchange is between two lanes that hold each other's operands,
+// so all 16 lanes end with the bitwise same value.
+__device__ __forceinline__ float row16_sum(float x) {
+  x = dpp_add<0xB1>(x);   // quad_perm [1,0,3,2]
+  x = dpp_add<0x4E>(x);   // quad_perm [2,3,0,1]
+  x = dpp_add<0x141>(x);  // row_half_mirror: quad 0 <-> 1, 2 <-> 3
+  x = dpp_add<0x140>(x);  // row_mirror: quads (0,1) <-> (3,2)
+  return x;
+}
+// Sum over the 64 lanes of a wave without index registers (DPP inside the four rows, then the four row sums through
+// scalar registers); the result is wave-uniform.  For kernels that are short of vector registers.
+__device__ __forceinline__ float wave_sum_uniform(float v) {
+  const int r = __builtin_bit_cast(int, row16_sum(v));
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 0));
+  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 16));
+  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 32));
+  const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(r, 48));
+  return (a + b) + (c + d);
+}
+// `scratch` (NW floats of LDS) must not be in use by an earlier call that some wave may still be reading: give
+// consecutive calls their own scratch.
+template <int NW>
+__device__ __forceinline__ float block_sum_uniform(float v, float* scratch) {
+  v = wave_sum_uniform(v);
+  if constexpr (NW == 1) return v;
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) t += scratch[i];
+  return t;
+}
+
 // Block-wide sum for blocks of NW waves; `scratch` holds NW floats of LDS.  All threads get the sum.
 template <int NW>
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

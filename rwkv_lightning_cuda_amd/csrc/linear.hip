@@ -31,6 +31,7 @@ struct LinearArgs {
   int out_f32;
   LnPrologue ln;
   RowCopy copy;
+  int weights_first_mask;  // one-row launches with a prologue: blocks with (index & mask) == 0 request their weights first
 };
 
 // One row of the LayerNorm + lerp prologue into xs (K fp16 values).  Same two-pass statistics, explicit FMAs and
@@ -423,6 +424,327 @@ static int launch_one(hipStream_t st, LinearArgs& args) {
   return RWKV_OK;
 }
 
+// ---- one row (M == 1): whole weight rows in flight ---------------------------------------------------------------
+// A decode step of one sequence is a chain of dependent launches, each of which moves 17-67 MB: what a launch costs
+// beyond its bytes is the trip to memory at its start.  Here a wavefront requests ALL the 16-byte vectors of its rows
+// (R = 2 rows of int8 / int4 codes, one row of fp16) before it does anything else - K <= 4096 int8 codes are 4
+// vectors per lane and row, so the whole matrix is requested by the first instructions of the launch - and the block
+// builds its copy of x in LDS while those requests are in flight.  With the LayerNorm prologue (LN) that copy is
+// LayerNorm(x + residual) + token-shift lerp computed by the block itself (same formulas and rounding points as
+// ln_fused_kernel, fused_ops.hip; four values per thread, so the sums associate differently and the last bits
+// may differ from that kernel's): the stand-alone LayerNorm launch and its kernel boundary disappear behind this
+// launch's first trip to memory.  Every block of the launch must be resident at once for that (a block that starts
+// later pays the prologue in the open): 64 registers per thread, 32 of them weight vectors in flight.
+// Accumulation order per lane is that of linear_gemv_kernel (steps in order, then the same butterfly): same bits.
+
+template <int FMT, int KCAP>
+struct Row1Cfg {
+  static constexpr int kRows = FMT == RWKV_FMT_F16 ? 1 : 2;
+  static constexpr int kSteps = KCAP / FmtTraits<FMT>::kStep > 0 ? KCAP / FmtTraits<FMT>::kStep : 1;
+};
+
+// LayerNorm(x + res) (or of a gathered table row) + lerp against the previous token's LN output into xs[0..K), by
+// the NT threads of the block, four values each; block 0 also stores the residual sum and the LN output.
+// In two parts, because a wavefront's loads complete in the order they were issued: everything the prologue reads
+// from memory is requested BEFORE the weight vectors (ln_row1_request), so that the arithmetic (ln_row1_finish, no
+// memory reads) can run while the weights are still on their way - a read issued after them would wait for them.
+struct LnRow1 {
+  half4_t xv, rv, wv, bv, pv, mv;
+};
+
+__device__ __forceinline__ LnRow1 ln_row1_request(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
+  const int c = threadIdx.x * 4;
+  const int cc = c < K ? c : 0;
+  const int64_t xsrc = ln.mode == 2 ? ln.tokens[0] * static_cast<int64_t>(K) : 0;
+  LnRow1 q;
+  q.xv = *reinterpret_cast<const half4_t*>(ln.x + xsrc + cc);
+  // unconditional (without a residual the row is read twice): a conditional read would wait for the first one
+  q.rv = *reinterpret_cast<const half4_t*>(ln.mode == 1 ? ln.res + cc : ln.x + xsrc + cc);
+  q.wv = *reinterpret_cast<const half4_t*>(ln.w + cc);
+  q.bv = *reinterpret_cast<const half4_t*>(ln.b + cc);
+  q.pv = *reinterpret_cast<const half4_t*>(ln.shift + cc);
+  q.mv = *reinterpret_cast<const half4_t*>(mu + cc);
+  return q;
+}
+
+// stash: NT * 4 floats (the row sum) followed by 4 x NT * 4 fp16 values (LN weight, bias, previous LN output, lerp
+// coefficients).  Everything that arrived from memory goes to LDS at once and is read back piece by piece (each
+// thread only what it wrote, so no barrier): while the weight vectors are in flight their 32 registers are all
+// but the block's whole budget, and a block that does not fit next to the others starts late.
+template <int NT>
+__device__ __forceinline__ void ln_row1_finish(const LnRow1& q, const LnPrologue& ln, int K, half_t* xs, float* stash,
+                                               float* red, bool store) {
+  const int c = threadIdx.x * 4;
+  const bool in = c < K;
+  float* vbuf = stash + c;
+  half_t* hbuf = reinterpret_cast<half_t*>(stash + NT * 4) + c;
+  float sum = 0.0f;
+  {
+    float4_t v;
+    if (ln.mode == 1) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = h2f(q.xv[e]) + h2f(q.rv[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = h2f(q.xv[e]);
+    }
+    if (in) sum = (v[0] + v[1]) + (v[2] + v[3]);
+    *reinterpret_cast<float4_t*>(vbuf) = v;
+    *reinterpret_cast<half4_t*>(hbuf) = q.wv;
+    *reinterpret_cast<half4_t*>(hbuf + NT * 4) = q.bv;
+    *reinterpret_cast<half4_t*>(hbuf + NT * 8) = q.pv;
+    *reinterpret_cast<half4_t*>(hbuf + NT * 12) = q.mv;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  sum = block_sum_uniform<NT / 64>(sum, red);
+  const float mean = sum / static_cast<float>(K);
+  float sv = 0.0f;
+  if (in) {
+    const float4_t v = *reinterpret_cast<const float4_t*>(vbuf);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float d = v[e] - mean;
+      sv = fmaf(d, d, sv);
+    }
+  }
+  sv = block_sum_uniform<NT / 64>(sv, red + NT / 64);
+  const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
+  half4_t ov = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+  if (in) {
+    const float4_t v = *reinterpret_cast<const float4_t*>(vbuf);
+    const half4_t wv = *reinterpret_cast<const half4_t*>(hbuf);
+    const half4_t bv = *reinterpret_cast<const half4_t*>(hbuf + NT * 4);
+    const half4_t pv = *reinterpret_cast<const half4_t*>(hbuf + NT * 8);
+    const half4_t mv = *reinterpret_cast<const half4_t*>(hbuf + NT * 12);
+    half4_t yv;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      yv[e] = f2h(fmaf((v[e] - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
+      const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
+      ov[e] = f2h(fmaf(h2f(pv[e]) - yf, h2f(mv[e]), yf));
+    }
+    if (store) {
+      *reinterpret_cast<half4_t*>(ln.ln_out + c) = yv;
+      if (ln.x_out) {
+        half4_t xo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xo[e] = f2h(v[e]);
+        *reinterpret_cast<half4_t*>(ln.x_out + c) = xo;
+      }
+    }
+  }
+  *reinterpret_cast<half4_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
+}
+
+template <int FMT, int NT, bool LN>
+__device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const LinearProblem& prob, int blk, half_t* xs,
+                                                float* red) {
+  using T = FmtTraits<FMT>;
+  constexpr int KCAP = LN ? NT * 4 : NT * 8;  // values of x the block stages: one slice per thread
+  using Cfg = Row1Cfg<FMT, KCAP>;
+  constexpr int R = Cfg::kRows;
+  constexpr int S = Cfg::kSteps;
+  constexpr int NW = NT / 64;
+  const int K = args.K;
+  const int N = prob.N;
+  // wavefront-uniform values in scalar registers: row addresses then cost no vector registers
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int lane = threadIdx.x & 63;
+  const int row0 = (blk * NW + wave) * R;
+  const bool active = row0 < N;
+  const int64_t row_bytes = T::byte_off(K);
+  const unsigned char* wbase = static_cast<const unsigned char*>(prob.w) + static_cast<int64_t>(active ? row0 : 0) * row_bytes;
+
+  LnRow1 lnq = {};
+  uint4_t xq = {0u, 0u, 0u, 0u};
+  // Which comes first, the prologue or the weight requests?  A wavefront stalls on its weight requests until the
+  // memory pipeline has room for them - late in a 67 MB launch that takes microseconds (measured with timestamps:
+  // the last wavefronts get their requests out 11 us after the launch began) - and it cannot run the prologue while
+  // it is stalled.  So only some blocks request their weights first (they keep memory busy from the start); the
+  // others run the prologue first, in the shadow of those requests, and then queue theirs.
+  bool ln_first = false;
+  if constexpr (LN) {
+    ln_first = (static_cast<int>(blockIdx.x) & args.weights_first_mask) != 0;
+    lnq = ln_row1_request(args.ln, prob.mu, K);
+    if (ln_first) ln_row1_finish<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0);
+  } else {
+    if (static_cast<int>(threadIdx.x) * 8 < K) xq = *reinterpret_cast<const uint4_t*>(prob.x + threadIdx.x * 8);
+  }
+  // the int8 rows' output scales too: read at the end they would cost every wavefront one more trip to memory
+  half_t row_scale[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    row_scale[r] = static_cast<half_t>(1.0f);
+    if constexpr (FMT == RWKV_FMT_W8) row_scale[r] = prob.scale[active ? row0 + r : r];
+  }
+  // the compiler must not move these reads behind the weight reads below (loads complete in issue order)
+  __builtin_amdgcn_sched_barrier(0);
+
+  // every weight vector of the wavefront's rows, requested up front.  No load sits under a branch: a lane past the
+  // end of the row re-reads the row's last vector (and multiplies it by the zeros that pad x).
+  uint4_t w[S][R];
+  half_t sc[S][R];
+  uint8_t zp[S][R];
+#pragma unroll
+  for (int st = 0; st < S; ++st) {
+    const int k0 = st * T::kStep + lane * T::kElems;
+    const int kc = k0 < K ? k0 : K - T::kElems;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      w[st][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wbase + r * row_bytes + T::byte_off(kc)));
+      if constexpr (FMT == RWKV_FMT_W4) {
+        const int64_t gi = static_cast<int64_t>(active ? row0 + r : r) * (K >> 7) + (kc >> 7);
+        sc[st][r] = prob.scale[gi];
+        zp[st][r] = prob.zp[gi];
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // x in LDS: one slice per thread, zeros beyond K
+  if constexpr (LN) {
+    if (!ln_first) ln_row1_finish<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0);
+  } else {
+    *reinterpret_cast<uint4_t*>(xs + threadIdx.x * 8) = xq;
+  }
+  __syncthreads();
+  if (!active) return;
+
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll
+  for (int st = 0; st < S; ++st) {
+    const int k0 = st * T::kStep + lane * T::kElems;
+    if (st * T::kStep < K && k0 + T::kElems <= KCAP) {  // (the second test only where a step is wider than KCAP)
+      constexpr int XV = T::kElems / 2;
+      half2_t xv[XV];
+#pragma unroll
+      for (int q = 0; q < XV / 4; ++q) {
+        const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + k0 + q * 8);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
+      }
+      if constexpr (FMT == RWKV_FMT_W4) {
+        half2_t xp[XV];
+        WeightVec<FMT>::pair_x(xv, xp);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const half_t zf = static_cast<half_t>(1024.0f + static_cast<float>(zp[st][r]));
+          const half2_t zb = {zf, zf};
+          const float part = WeightVec<FMT>::dot(w[st][r], xp, zb, 0.0f);
+          acc[r] = fmaf(part, h2f(sc[st][r]), acc[r]);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = WeightVec<FMT>::dot(w[st][r], xv, acc[r]);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = row0 + r;
+      float v = round_h(acc[r] * h2f(row_scale[r]));
+      if (args.epilogue == RWKV_EPI_RELU_SQUARE) {
+        v = fmaxf(v, 0.0f);
+        v = round_h(v * v);
+      }
+      if (args.out_f32) {
+        static_cast<float*>(prob.y)[n] = v;
+      } else {
+        static_cast<half_t*>(prob.y)[n] = f2h(v);
+      }
+    }
+  }
+}
+
+// grid = blocks over all problems; a block of NT threads covers NT/64 * (1 or 2) rows; dynamic LDS = x (NT * 4 fp16
+// values with the prologue, NT * 8 without).  DF is the format of the launch's quantised problems; fp16 problems
+// (the LoRA rank-ins) may ride along.
+template <int NT, bool LN, int DF>
+__global__ __launch_bounds__(NT) void linear_gemv_row1_kernel(LinearArgs args) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  __shared__ float red[2 * (NT / 64)];
+  half_t* xs = reinterpret_cast<half_t*>(lds_raw);
+  if (blockIdx.x == 0 && args.copy.n > 0) {
+    for (int i = threadIdx.x * 8; i < args.copy.n; i += NT * 8)
+      *reinterpret_cast<uint4_t*>(args.copy.dst + i) = *reinterpret_cast<const uint4_t*>(args.copy.src + i);
+  }
+  int pi = 0;
+  int first = 0;
+  for (int i = 0; i < args.n_problems - 1; ++i) {
+    if (static_cast<int>(blockIdx.x) >= args.block_end[i]) {
+      pi = i + 1;
+      first = args.block_end[i];
+    }
+  }
+  const LinearProblem prob = args.p[pi];
+  const int blk = blockIdx.x - first;
+  if (DF != RWKV_FMT_F16 && prob.fmt == DF) {  // uniform per block
+    gemv_row1_block<DF, NT, LN>(args, prob, blk, xs, red);
+  } else {
+    gemv_row1_block<RWKV_FMT_F16, NT, LN>(args, prob, blk, xs, red);
+  }
+}
+
+// The quantised format of the launch (fp16 if none), or -1 if the launch mixes int8 and int4 problems or a row is
+// longer than a wavefront holds in registers (K > 4096).
+static int row1_format(const LinearArgs& args) {
+  if (args.K > 4096) return -1;
+  int df = RWKV_FMT_F16;
+  for (int i = 0; i < args.n_problems; ++i) {
+    const int fmt = args.p[i].fmt;
+    if (fmt == RWKV_FMT_F16) continue;
+    if (df != RWKV_FMT_F16 && df != fmt) return -1;
+    df = fmt;
+  }
+  return df;
+}
+
+template <int NT, bool LN, int DF>
+static int launch_row1(hipStream_t st, LinearArgs& args) {
+  int total = 0;
+  for (int i = 0; i < args.n_problems; ++i) {
+    const int rows_per_block = (NT / 64) * (args.p[i].fmt == RWKV_FMT_F16 ? 1 : 2);
+    total += ceil_div(args.p[i].N, rows_per_block);
+    args.block_end[i] = total;
+  }
+  args.KT = LN ? NT * 4 : NT * 8;
+  // every fourth block requests its weights before the prologue; with int4 codes none (measured, 7.2B shape, ms per
+  // step: int8 1.940 all / 1.917 every fourth / 1.923 none; int4 1.892 / 1.814 / 1.778)
+  args.weights_first_mask = DF == RWKV_FMT_W4 ? -1 : 3;
+  // x; with the prologue also its stash: the fp32 row sum and four fp16 vectors
+  const size_t lds = static_cast<size_t>(args.KT) * (LN ? 2 + 4 + 4 * 2 : 2);
+  hipLaunchKernelGGL((linear_gemv_row1_kernel<NT, LN, DF>), dim3(total), dim3(NT), lds, st, args);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+template <int NT, bool LN>
+static int launch_row1_fmt(hipStream_t st, LinearArgs& args, int df) {
+  switch (df) {
+    case RWKV_FMT_W8: return launch_row1<NT, LN, RWKV_FMT_W8>(st, args);
+    case RWKV_FMT_W4: return launch_row1<NT, LN, RWKV_FMT_W4>(st, args);
+    default: return launch_row1<NT, LN, RWKV_FMT_F16>(st, args);
+  }
+}
+
+// Block size by row length: one slice of x per thread (4 values with the prologue, 8 without).
+static int launch_row1_any(hipStream_t st, LinearArgs& args, int df) {
+  const int K = args.K;
+  if (args.ln.mode != 0) {
+    if (K <= 1024) return launch_row1_fmt<256, true>(st, args, df);
+    if (K <= 2048) return launch_row1_fmt<512, true>(st, args, df);
+    return launch_row1_fmt<1024, true>(st, args, df);
+  }
+  if (K <= 2048) return launch_row1_fmt<256, false>(st, args, df);
+  return launch_row1_fmt<512, false>(st, args, df);
+}
+
+
 // Batched small-M linear: n_problems problems sharing M (<= 8), K, epilogue and output type.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
                    int out_f32, const LnPrologue* ln, const RowCopy* copy) {
@@ -465,6 +787,10 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
   if (copy && copy->n > 0) {
     RWKV_REQUIRE(copy->src && copy->dst && copy->n % 8 == 0, "linear: bad row copy");
     args.copy = *copy;
+  }
+  if (M == 1) {
+    const int df = row1_format(args);
+    if (df >= 0) return launch_row1_any(st, args, df);
   }
   switch (M) {
     case 1: return launch_one<1, 2, 1>(st, args);

@@ -123,7 +123,8 @@ struct rwkv_hip_session {
   size_t sparse_ws_bytes = 0;
   int sparse_ffn_rows = 1;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
   int fused_ln = -1;          // decode steps fold LayerNorm + token shift into the linear launches: 1 always, 0 never,
-                              // -1 for one row of at most 1024 channels (faster there: 0.1B shape 0.446 -> 0.423 ms)
+                              // -1 for one row of at most 4096 channels (the row-resident GEMV hides the prologue
+                              // behind its weight requests: 7.2B shape 2.04 -> 1.92 ms per step, 0.1B 0.413 -> 0.373)
 };
 
 namespace {
@@ -338,10 +339,10 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   // row-tiled kernels of the prefill path (LoRA rank-outs on the matrix core) are faster (measured: 4.2 -> 4.0 ms
   // per step at 16 rows, 5.5 -> 4.6 ms at 32).
   const bool fused_tmix = step && rows <= 8;
-  // Decode steps of up to 8 rows fold both LayerNorm + token-shift kernels of a layer into the prologue of the
-  // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key).  The residual-stream tap needs the
-  // stand-alone kernels.
-  const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows == 1 && C <= 1024);
+  // Decode steps on the GEMV path can fold both LayerNorm + token-shift kernels of a layer into the prologue of the
+  // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key): by default for one row of up to 4096
+  // channels.  The residual-stream tap needs the stand-alone kernels.
+  const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows == 1 && C <= 4096);
   const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace &&
                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
 
@@ -832,6 +833,7 @@ int rwkv_hip_session_create(rwkv_hip_session** out, const rwkv_hip_model* m) {
     return RWKV_E_NOMEM;
   }
   s->model = m;
+
   const hipError_t err = hipStreamCreateWithFlags(&s->stream, hipStreamNonBlocking);
   if (err != hipSuccess) {
     set_error("hipStreamCreateWithFlags failed: %s", hipGetErrorString(err));

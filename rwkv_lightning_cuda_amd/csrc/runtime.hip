@@ -19,9 +19,84 @@ void set_error(const char* fmt, ...) {
 
 using namespace rwkv;
 
+namespace {
+
+// One link of a chain of dependent launches: every block reads the counter the previous launch left, one thread
+// writes it back incremented.  Next to no work: what a chain of these costs per link is the cost of a launch that
+// has to wait for its predecessor.
+__global__ void chain_link_kernel(unsigned* counter) {
+  const unsigned seen = *counter;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *counter = seen + 1;
+}
+
+}  // namespace
+
 extern "C" {
 
 const char* rwkv_hip_last_error(void) { return g_error; }
+
+int rwkv_hip_measure_launch_chain(int links, int blocks, int threads, int use_graph, int reps, float* us_per_link) {
+  RWKV_REQUIRE(us_per_link != nullptr, "us_per_link is NULL");
+  RWKV_REQUIRE(links >= 1 && links <= 4096 && blocks >= 1 && blocks <= 65536 && threads >= 1 && threads <= 1024 && reps >= 1 &&
+                   reps <= 1000,
+               "measure_launch_chain: argument out of range");
+  hipStream_t st = nullptr;
+  unsigned* counter = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  int rc = RWKV_OK;
+  auto fail = [&](hipError_t err, const char* what) {
+    if (err != hipSuccess && rc == RWKV_OK) {
+      set_error("measure_launch_chain: %s failed: %s", what, hipGetErrorString(err));
+      rc = RWKV_E_RUNTIME;
+    }
+    return err != hipSuccess;
+  };
+  auto chain = [&] {
+    for (int i = 0; i < links; ++i) hipLaunchKernelGGL(chain_link_kernel, dim3(blocks), dim3(threads), 0, st, counter);
+  };
+  do {
+    if (fail(hipStreamCreateWithFlags(&st, hipStreamNonBlocking), "stream create")) break;
+    if (fail(hipMalloc(reinterpret_cast<void**>(&counter), 256), "malloc")) break;
+    if (fail(hipMemsetAsync(counter, 0, 256, st), "memset")) break;
+    if (fail(hipEventCreate(&e0), "event create") || fail(hipEventCreate(&e1), "event create")) break;
+    if (use_graph) {
+      if (fail(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal), "begin capture")) break;
+      chain();
+      if (fail(hipStreamEndCapture(st, &graph), "end capture")) break;
+      if (fail(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "graph instantiate")) break;
+    }
+    auto run = [&] {
+      if (use_graph) (void)hipGraphLaunch(exec, st);
+      else chain();
+    };
+    run();  // warm
+    if (fail(hipStreamSynchronize(st), "sync")) break;
+    if (fail(hipEventRecord(e0, st), "event record")) break;
+    for (int r = 0; r < reps; ++r) run();
+    if (fail(hipEventRecord(e1, st), "event record")) break;
+    if (fail(hipStreamSynchronize(st), "sync")) break;
+    if (fail(hipGetLastError(), "launch")) break;
+    float ms = 0.0f;
+    if (fail(hipEventElapsedTime(&ms, e0, e1), "elapsed")) break;
+    unsigned count = 0;
+    if (fail(hipMemcpy(&count, counter, sizeof(count), hipMemcpyDeviceToHost), "copy back")) break;
+    if (count != static_cast<unsigned>(links) * (reps + 1)) {
+      set_error("measure_launch_chain: the chain counted %u links instead of %u", count, static_cast<unsigned>(links) * (reps + 1));
+      rc = RWKV_E_RUNTIME;
+      break;
+    }
+    *us_per_link = ms * 1e3f / (static_cast<float>(reps) * links);
+  } while (false);
+  if (exec) (void)hipGraphExecDestroy(exec);
+  if (graph) (void)hipGraphDestroy(graph);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (counter) (void)hipFree(counter);
+  if (st) (void)hipStreamDestroy(st);
+  return rc;
+}
 
 int rwkv_hip_device_count(int* count) {
   RWKV_REQUIRE(count != nullptr, "count is NULL");

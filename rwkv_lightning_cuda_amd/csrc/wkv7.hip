@@ -35,21 +35,6 @@ __device__ __forceinline__ float decay_from_logit(float w) {
 // idle (RPL = 1 up to 64 heads, 2 up to 128); RPL = 4 reads each operand least often.
 constexpr int kSeqChunk = 8;
 
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float x) {
-  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false);
-  return x + __builtin_bit_cast(float, moved);
-}
-// Sum over the 16 lanes of a DPP row.  Every exchange is between two lanes that hold each other's operands,
-// so all 16 lanes end with the bitwise same value.
-__device__ __forceinline__ float row16_sum(float x) {
-  x = dpp_add<0xB1>(x);   // quad_perm [1,0,3,2]
-  x = dpp_add<0x4E>(x);   // quad_perm [2,3,0,1]
-  x = dpp_add<0x141>(x);  // row_half_mirror: quad 0 <-> 1, 2 <-> 3
-  x = dpp_add<0x140>(x);  // row_mirror: quads (0,1) <-> (3,2)
-  return x;
-}
-
 // Where the five operand vectors of a token come from (SRC):
 //   kSrcFp32  - fp32 tensors r, d, k, a, b (decay applied), `op_bs` elements between batch rows, staged with 16-byte
 //               loads: what kk_a_gate_kernel writes for the model's stand-alone path;

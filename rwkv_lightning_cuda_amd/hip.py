@@ -32,7 +32,7 @@ EXPORTS = [
     "rwkv_hip_memcpy_h2d_async", "rwkv_hip_memcpy_d2h_async", "rwkv_hip_memcpy_d2d_async", "rwkv_hip_memset",
     "rwkv_hip_mem_info", "rwkv_hip_stream_create", "rwkv_hip_stream_destroy", "rwkv_hip_stream_sync",
     "rwkv_hip_device_sync", "rwkv_hip_event_create", "rwkv_hip_event_destroy", "rwkv_hip_event_record",
-    "rwkv_hip_event_elapsed_ms", "rwkv_hip_wkv7", "rwkv_hip_quantize_w8", "rwkv_hip_dequant_w8",
+    "rwkv_hip_event_elapsed_ms", "rwkv_hip_measure_launch_chain", "rwkv_hip_wkv7", "rwkv_hip_quantize_w8", "rwkv_hip_dequant_w8",
     "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_bf16_to_f16", "rwkv_hip_bf16_to_f16_transpose",
     "rwkv_hip_emb_ln0_bf16_to_f16", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",
     "rwkv_hip_pack_weights", "rwkv_hip_linear_packed_workspace", "rwkv_hip_linear_packed", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
@@ -283,6 +283,14 @@ def cmix_sparse_down_relu_one(fmt, C, F, preact, wt, scale, workspace, out, stre
 def cmix_sparse_down_relu_rows(fmt, rows, C, F, preact, wt, scale, workspace, out, stream=None):
     check(load().rwkv_hip_cmix_sparse_down_relu_rows(_p(stream), _i(fmt), _i(rows), _i(C), _i(F), _p(preact), _p(wt),
                                                      _p(scale), _p(workspace), ctypes.c_size_t(workspace.nbytes), _p(out)))
+
+
+def measure_launch_chain(links, blocks=1, threads=64, use_graph=True, reps=20):
+    """Microseconds per link of a chain of dependent launches of a near-empty kernel."""
+    us = ctypes.c_float(0)
+    check(load().rwkv_hip_measure_launch_chain(_i(links), _i(blocks), _i(threads), _i(1 if use_graph else 0), _i(reps),
+                                               ctypes.byref(us)))
+    return us.value
 
 
 def cmix_sparse_down_relu_rows_static(fmt, rows, C, F, preact, wt, scale, out, stream=None):

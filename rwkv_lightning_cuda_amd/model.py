@@ -267,7 +267,7 @@ class Session:
 
     def set_fused_ln(self, on):
         """Decode steps fold LayerNorm + token shift into the linear launches (bitwise the same): True always, False
-        never, None (the default of a new session) for one row of at most 1024 channels."""
+        never, None (the default of a new session) for one row of at most 4096 channels."""
         hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(-1 if on is None else 1 if on else 0)))
 
     def set_sparse_ffn(self, max_rows):
