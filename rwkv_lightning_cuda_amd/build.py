@@ -32,6 +32,26 @@ HIP_FLAGS = [
 ]
 
 
+# Kernels whose design depends on how many wavefronts fit a SIMD (mangled-name fragment -> required waves per SIMD):
+# the compiler's resource report is checked at build time, so that a change that costs a few registers fails the
+# build instead of silently halving the occupancy.  The one-row GEMV with the LayerNorm prologue needs two
+# 1024-thread blocks per CU (all blocks of a launch resident at once), i.e. at most 64 registers.
+REQUIRED_OCCUPANCY = {"linear_gemv_row1_kernelILi1024ELb1": 8}
+
+
+def _check_occupancy(src, stderr_text):
+    name = None
+    for line in stderr_text.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+        elif "Occupancy [waves/SIMD]:" in line and name:
+            got = int(line.split("Occupancy [waves/SIMD]:")[1].split()[0])
+            for frag, need in REQUIRED_OCCUPANCY.items():
+                if frag in name and got < need:
+                    raise RuntimeError("%s: kernel %s fits %d wavefronts per SIMD, its design needs %d "
+                                       "(register count went up)" % (src, name, got, need))
+
+
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -48,11 +68,13 @@ def _compile(src, force):
     if (not force and os.path.exists(obj)
             and os.path.getmtime(obj) > max(os.path.getmtime(spath), _headers_mtime())):
         return obj, ""
-    cmd = [HIPCC] + HIP_FLAGS + ["-c", spath, "-o", obj]
+    cmd = [HIPCC] + HIP_FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", spath, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
-    log = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
+    log = "\n".join(l for l in proc.stderr.splitlines()
+                    if "packed-fp32-ops" not in l and "kernel-resource-usage" not in l)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    _check_occupancy(src, proc.stderr)
     return obj, log
 
 

@@ -31,7 +31,6 @@ struct LinearArgs {
   int out_f32;
   LnPrologue ln;
   RowCopy copy;
-  int weights_first_mask;  // one-row launches with a prologue: blocks with (index & mask) == 0 request their weights first
 };
 
 // One row of the LayerNorm + lerp prologue into xs (K fp16 values).  Same two-pass statistics, explicit FMAs and
@@ -426,17 +425,15 @@ static int launch_one(hipStream_t st, LinearArgs& args) {
 
 // ---- one row (M == 1): whole weight rows in flight ---------------------------------------------------------------
 // A decode step of one sequence is a chain of dependent launches, each of which moves 17-67 MB: what a launch costs
-// beyond its bytes is the trip to memory at its start.  Here a wavefront requests ALL the 16-byte vectors of its rows
-// (R = 2 rows of int8 / int4 codes, one row of fp16) before it does anything else - K <= 4096 int8 codes are 4
-// vectors per lane and row, so the whole matrix is requested by the first instructions of the launch - and the block
-// builds its copy of x in LDS while those requests are in flight.  With the LayerNorm prologue (LN) that copy is
-// LayerNorm(x + residual) + token-shift lerp computed by the block itself (same formulas and rounding points as
-// ln_fused_kernel, fused_ops.hip; four values per thread, so the sums associate differently and the last bits
-// may differ from that kernel's): the stand-alone LayerNorm launch and its kernel boundary disappear behind this
-// launch's first trip to memory.  Every block of the launch must be resident at once for that (a block that starts
-// later pays the prologue in the open): 64 registers per thread, 32 of them weight vectors in flight.
+// beyond its bytes is the trip to memory at its start and the one at its end.  Here a wavefront requests ALL the
+// 16-byte vectors of its rows (R = 2 rows of int8 / int4 codes, one row of fp16) in one go - K <= 4096 int8 codes
+// are 4 vectors per lane and row - so every byte of the matrix is requested by the first instructions of its block
+// and nothing is requested late.  With the LayerNorm prologue (LN) the block first computes its own copy of
+// LayerNorm(x + residual) + token-shift lerp into LDS (same formulas and rounding points as ln_fused_kernel,
+// fused_ops.hip; four values per thread, so the sums associate differently and the last bits may differ from
+// that kernel's): the stand-alone LayerNorm launch and its kernel boundary disappear.  Every block of the launch
+// is resident at once (two 1024-thread blocks per CU: at most 64 registers per thread, checked at build time).
 // Accumulation order per lane is that of linear_gemv_kernel (steps in order, then the same butterfly): same bits.
-
 template <int FMT, int KCAP>
 struct Row1Cfg {
   static constexpr int kRows = FMT == RWKV_FMT_F16 ? 1 : 2;
@@ -445,9 +442,8 @@ struct Row1Cfg {
 
 // LayerNorm(x + res) (or of a gathered table row) + lerp against the previous token's LN output into xs[0..K), by
 // the NT threads of the block, four values each; block 0 also stores the residual sum and the LN output.
-// In two parts, because a wavefront's loads complete in the order they were issued: everything the prologue reads
-// from memory is requested BEFORE the weight vectors (ln_row1_request), so that the arithmetic (ln_row1_finish, no
-// memory reads) can run while the weights are still on their way - a read issued after them would wait for them.
+// In two parts: everything the prologue reads from memory is requested at once (ln_row1_request, six reads in
+// flight together), the arithmetic (ln_row1_finish) reads no memory.
 struct LnRow1 {
   half4_t xv, rv, wv, bv, pv, mv;
 };
@@ -469,8 +465,8 @@ __device__ __forceinline__ LnRow1 ln_row1_request(const LnPrologue& ln, const ha
 
 // stash: NT * 4 floats (the row sum) followed by 4 x NT * 4 fp16 values (LN weight, bias, previous LN output, lerp
 // coefficients).  Everything that arrived from memory goes to LDS at once and is read back piece by piece (each
-// thread only what it wrote, so no barrier): while the weight vectors are in flight their 32 registers are all
-// but the block's whole budget, and a block that does not fit next to the others starts late.
+// thread only what it wrote, so no barrier), which keeps the prologue's registers few: the 32 registers of the
+// weight vectors are all but the block's whole budget.
 template <int NT>
 __device__ __forceinline__ void ln_row1_finish(const LnRow1& q, const LnPrologue& ln, int K, half_t* xs, float* stash,
                                                float* red, bool store) {
@@ -536,9 +532,15 @@ __device__ __forceinline__ void ln_row1_finish(const LnRow1& q, const LnPrologue
   *reinterpret_cast<half4_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
 }
 
+// One block.  With the prologue, it runs BEFORE the weight requests: a wavefront stalls on its weight requests until
+// the memory pipeline has room for them - late in a 67 MB launch that takes microseconds (timestamps: the last
+// wavefronts get their requests out 11 us after the launch began) - and it cannot run the prologue while it is
+// stalled, so a prologue behind the requests ends up at the tail of the launch.  Measured at the 7.2B shape, ms per
+// step, prologue first / weights first / weights first in every second block: int8 1.924 / 1.947 / 1.915, int4
+// 1.773 / 1.825 / 1.793; the mixed orders need both code paths and 62-66 registers, so it is prologue first for all.
 template <int FMT, int NT, bool LN>
 __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const LinearProblem& prob, int blk, half_t* xs,
-                                                float* red) {
+                                               float* red) {
   using T = FmtTraits<FMT>;
   constexpr int KCAP = LN ? NT * 4 : NT * 8;  // values of x the block stages: one slice per thread
   using Cfg = Row1Cfg<FMT, KCAP>;
@@ -557,16 +559,8 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
 
   LnRow1 lnq = {};
   uint4_t xq = {0u, 0u, 0u, 0u};
-  // Which comes first, the prologue or the weight requests?  A wavefront stalls on its weight requests until the
-  // memory pipeline has room for them - late in a 67 MB launch that takes microseconds (measured with timestamps:
-  // the last wavefronts get their requests out 11 us after the launch began) - and it cannot run the prologue while
-  // it is stalled.  So only some blocks request their weights first (they keep memory busy from the start); the
-  // others run the prologue first, in the shadow of those requests, and then queue theirs.
-  bool ln_first = false;
   if constexpr (LN) {
-    ln_first = (static_cast<int>(blockIdx.x) & args.weights_first_mask) != 0;
     lnq = ln_row1_request(args.ln, prob.mu, K);
-    if (ln_first) ln_row1_finish<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0);
   } else {
     if (static_cast<int>(threadIdx.x) * 8 < K) xq = *reinterpret_cast<const uint4_t*>(prob.x + threadIdx.x * 8);
   }
@@ -580,13 +574,12 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   // the compiler must not move these reads behind the weight reads below (loads complete in issue order)
   __builtin_amdgcn_sched_barrier(0);
 
-  // every weight vector of the wavefront's rows, requested up front.  No load sits under a branch: a lane past the
-  // end of the row re-reads the row's last vector (and multiplies it by the zeros that pad x).
+  // No load sits under a branch: a lane past the end of the row re-reads the row's last vector (and multiplies it
+  // by the zeros that pad x).
   uint4_t w[S][R];
   half_t sc[S][R];
   uint8_t zp[S][R];
-#pragma unroll
-  for (int st = 0; st < S; ++st) {
+  auto request = [&](int st) {
     const int k0 = st * T::kStep + lane * T::kElems;
     const int kc = k0 < K ? k0 : K - T::kElems;
 #pragma unroll
@@ -598,15 +591,17 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
         zp[st][r] = prob.zp[gi];
       }
     }
-  }
-  __builtin_amdgcn_sched_barrier(0);
-
+  };
   // x in LDS: one slice per thread, zeros beyond K
   if constexpr (LN) {
-    if (!ln_first) ln_row1_finish<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0);
+    ln_row1_finish<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0);
   } else {
     *reinterpret_cast<uint4_t*>(xs + threadIdx.x * 8) = xq;
   }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int st = 0; st < S; ++st) request(st);
+  __builtin_amdgcn_sched_barrier(0);
   __syncthreads();
   if (!active) return;
 
@@ -713,9 +708,6 @@ static int launch_row1(hipStream_t st, LinearArgs& args) {
     args.block_end[i] = total;
   }
   args.KT = LN ? NT * 4 : NT * 8;
-  // every fourth block requests its weights before the prologue; with int4 codes none (measured, 7.2B shape, ms per
-  // step: int8 1.940 all / 1.917 every fourth / 1.923 none; int4 1.892 / 1.814 / 1.778)
-  args.weights_first_mask = DF == RWKV_FMT_W4 ? -1 : 3;
   // x; with the prologue also its stash: the fp32 row sum and four fp16 vectors
   const size_t lds = static_cast<size_t>(args.KT) * (LN ? 2 + 4 + 4 * 2 : 2);
   hipLaunchKernelGGL((linear_gemv_row1_kernel<NT, LN, DF>), dim3(total), dim3(NT), lds, st, args);
