@@ -86,6 +86,18 @@ int rwkv_hip_wkv7(rwkv_stream_t s, int B, int T, int C, int H, int w_mode, int i
                   const void* r, const void* w, const void* k, const void* v, const void* a, const void* b,
                   void* y);
 
+/* The recurrence with the state kept in fp16 (the reference server's default; ModelBackend's use_wkv32 == false).
+ * Replaces rwkv7_wkv_fp16_seq_launch / rwkv7_wkv_fp16_seq_w0_launch and the one-token launchers
+ * (cuda/rwkv7_fast_v4_kernels.cuh:34-47, cuda/rwkv7_wkv_fp16_v2.cu:681-830).  state f16 [B,H,64,64] in/out;
+ * r,w,k,v,a,b,y f16 [B,T,C]; w holds raw decay logits, w0 f16 [C] (may be NULL) is added to them unrounded;
+ * elapsed i32 [B] = tokens each row has seen before this call (read only: it phases the dither that the
+ * reference adds to the decay before rounding it to fp16, cuda/rwkv7_wkv_fp16_v2.cu:41-52).  Every operation is an
+ * fp16 fused multiply-add in the reference's order.  T1+T2 tokens in one call or in two (elapsed advanced by T1
+ * in between) give bitwise the same result. */
+int rwkv_hip_wkv7_f16state(rwkv_stream_t s, int B, int T, int C, int H, void* state, const void* r, const void* w,
+                           const void* w0, const void* k, const void* v, const void* a, const void* b, void* y,
+                           const void* elapsed);
+
 /* ---- weight formats (no counterpart in the reference, whose weights are fp16 only).
  * W8: int8 [N,K] + f16 scale [N].  W4: packed u8 [N,K/2] (element k even -> low nibble of byte
  * k/2) + f16 scale [N,K/128] + u8 zero point [N,K/128]; K % 128 == 0. ---- */
@@ -277,7 +289,8 @@ int rwkv_hip_session_stream(rwkv_hip_session* s, rwkv_stream_t* stream);
 /* use_graph != 0: T == 1 steps replay a captured HIP graph (default on) */
 int rwkv_hip_session_set_graph(rwkv_hip_session* s, int use_graph);
 
-/* tokens_host [B,T] int64 (host); shift f16 [L,2,B,C]; wkv f32 [L,B,H,64,64]; elapsed i32 [B];
+/* tokens_host [B,T] int64 (host); shift f16 [L,2,B,C]; wkv f32 [L,B,H,64,64] (f16 with
+ * rwkv_hip_session_set_wkv_fp16); elapsed i32 [B];
  * logits f32 [B,V] for the last token of each row.  All state tensors are updated in place.
  * Returns after the work is enqueued AND complete (the reference synchronises too,
  * src/rwkv7_fast_v4.cu:1343) unless sync == 0. */
@@ -303,6 +316,11 @@ int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double
  * only while rows x (fraction of non-zero activations) stays below 1 - about half the activations are
  * non-zero with random-init weights, far fewer with trained ones.  0 selects the dense product. */
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
+/* on != 0: the `wkv` tensor of rwkv_hip_forward / rwkv_hip_decode_greedy is the fp16 state, f16 [L,B,H,64,64], and
+ * the recurrence runs in fp16 as rwkv_hip_wkv7_f16state does (ModelBackend's use_wkv32 == false, the reference
+ * server's default: src/rwkv7_fast_v4.cu:1262-1271; calls of up to 16 tokens add w0 to the decay logit unrounded,
+ * longer ones round w12 + w0 to fp16 first).  Default off: fp32 state.  A state belongs to one mode. */
+int rwkv_hip_session_set_wkv_fp16(rwkv_hip_session* s, int on);
 /* Decode steps on the GEMV path (one or two rows) can fold the two LayerNorm + token-shift kernels of a layer
  * into the prologue of the linear launches that consume them.  on > 0: always, 0: never, < 0 (the default): for
  * one row of at most 4096 channels.  One row goes through a kernel that requests whole weight rows up front and

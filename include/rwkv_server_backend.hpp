@@ -35,8 +35,8 @@ struct GenerateOptions {
   int force_reasoning_token_offset = 0;
 };
 
-// shift f16 [L,2,B,C]; wkv_state32 f32 [L,B,H,64,64]; elapsed i32 [B].  wkv_state (fp16 state) is kept as
-// a member for layout compatibility and is never allocated by this backend.
+// shift f16 [L,2,B,C]; the WKV state [L,B,H,64,64] in wkv_state32 (f32, wkv32 == true) or wkv_state (f16,
+// wkv32 == false): a backend allocates the one of its mode; elapsed i32 [B].
 struct GenerationState {
   int batch_size = 0;
   bool wkv32 = false;
@@ -84,10 +84,11 @@ class IModelBackend {
   virtual const std::string& model_name() const = 0;
 };
 
-// model_path selects the weights.  The reference reads a .pth checkpoint here; that reader is not part of
-// this build, so the path names a synthetic random-init model instead:
-//   "synthetic:<0.1B|1.5B|7.2B|tiny>[:f16|w8|w4][:seed=<n>]"
-// use_wkv32 must be true (fp32 state only); chunk_load is accepted and ignored.
+// model_path selects the weights: a .pth checkpoint, optionally followed by ":w8" or ":w4" (quantise on load), or
+//   "synthetic:<0.1B|1.5B|7.2B|tiny>[:f16|w8|w4][:seed=<n>]"   a random-init model of that shape.
+// use_wkv32 = false (the reference's default) keeps the WKV state in fp16 and runs the recurrence in fp16 as the
+// reference's cuda/rwkv7_wkv_fp16_v2.cu does; true keeps it in fp32.  chunk_load reads the checkpoint on demand
+// instead of through a whole-file copy.
 class ModelBackend final : public IModelBackend {
  public:
   explicit ModelBackend(std::string model_path, bool use_wkv32 = false, bool chunk_load = false);

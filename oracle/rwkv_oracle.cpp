@@ -237,6 +237,103 @@ void orc_wkv7_f16(int B, int T, int C, int H, int w_mode, float* state, const ui
 }
 
 // ---------------------------------------------------------------------------------------------
+// WKV7 with the state kept in fp16 (the reference server's default mode).  cuda/rwkv7_wkv_fp16_v2.cu; the per-token
+// arithmetic is the same in every kernel of that file (:157-193, :342-367, :433-468, :531-556, :632-660).  Thread i
+// owns state row i as 32 half2 pairs; every operation is an fp16 fused multiply-add with one rounding (__hfma2):
+//   sa2    = chain over pairs j = 0..31 of  fma(a[j], S[i][j], sa2)      (even columns in .x, odd columns in .y)
+//   sa     = f16(sa2.x + sa2.y)
+//   wd[c]  = f16(exp2f(NEXP_HALF_LOG2_E / (1 + exp2f(NLOG2_E * w))) - 1 + rotator1(elapsed[b] + h*64 + c + t))  (:41-52)
+//            with w = float(w_raw[c]) (+ float(w0[c]) when w0 is given: the sum is not rounded to fp16)
+//   S[i][c] = fma(S[i][c], wd[c], fma(k[c], v[i], fma(sa, b[c], S[i][c])))   i.e. S*(d-1) + (k*v + (sa*b + S))
+//   y2     = chain over pairs of  fma(S'[i][j], r[j], y2);   y[i] = f16(y2.x + y2.y)
+// rotator1(x) = 2^-41 * float(int32(ROT1 * x)), ROT1 = int32(2654435769): a dither below fp16 resolution of d - 1
+// that makes the rounding of the decay unbiased over consecutive tokens and channels.
+// fp16 fma: the exact product of two halves and the sum with a third fit a double (or differ from it by less than
+// what could move a rounding boundary), so rounding the double result to fp16 once is the fused operation.
+// ---------------------------------------------------------------------------------------------
+uint16_t orc_f64_to_f16(double x) {
+  uint64_t bits;
+  std::memcpy(&bits, &x, sizeof(bits));
+  const uint16_t sign = static_cast<uint16_t>((bits >> 48) & 0x8000u);
+  if (std::isnan(x)) return static_cast<uint16_t>(sign | 0x7e00u);
+  const double ax = std::fabs(x);
+  if (ax >= 65520.0) return static_cast<uint16_t>(sign | 0x7c00u);  // 65504 + half an ulp ties to even = infinity
+  if (ax < 6.103515625e-05) {                                       // below 2^-14: multiples of 2^-24
+    const double q = std::nearbyint(ax * 16777216.0);               // round to nearest even (default mode)
+    return static_cast<uint16_t>(sign | static_cast<uint16_t>(q));  // q == 1024 is the smallest normal number
+  }
+  int e;
+  (void)std::frexp(ax, &e);  // ax = m * 2^e, m in [0.5, 1)
+  e -= 1;                    // ax in [2^e, 2^(e+1))
+  double mant = std::nearbyint(std::ldexp(ax, 10 - e));  // in [1024, 2048]
+  if (mant >= 2048.0) {
+    mant = 1024.0;
+    e += 1;
+  }
+  return static_cast<uint16_t>(sign | static_cast<uint16_t>((e + 15) << 10) | (static_cast<uint16_t>(mant) - 1024u));
+}
+
+static inline uint16_t hfma16(uint16_t a, uint16_t b, uint16_t c) {
+  return orc_f64_to_f16(static_cast<double>(h2f(a)) * static_cast<double>(h2f(b)) + static_cast<double>(h2f(c)));
+}
+static inline uint16_t hadd16(uint16_t a, uint16_t b) {
+  return orc_f64_to_f16(static_cast<double>(h2f(a)) + static_cast<double>(h2f(b)));
+}
+
+uint16_t orc_f16_fma(uint16_t a, uint16_t b, uint16_t c) { return hfma16(a, b, c); }
+
+float orc_wkv16_rotator(int32_t x) {
+  const uint32_t prod = 2654435769u * static_cast<uint32_t>(x);  // int32 multiplication that wraps
+  int32_t sp;
+  std::memcpy(&sp, &prod, sizeof(sp));
+  return 4.547473508864641e-13f * static_cast<float>(sp);
+}
+
+uint16_t orc_wkv16_w_delta(uint16_t w_raw, const uint16_t* w0, int c, int32_t phase) {
+  float w = h2f(w_raw);
+  if (w0) w += h2f(w0[c]);
+  const float d = std::exp2(-0.8750387749145276f / (1.0f + std::exp2(-1.4426950408889634f * w))) - 1.0f + orc_wkv16_rotator(phase);
+  return f2h(d);
+}
+
+void orc_wkv7_f16state(int B, int T, int C, int H, uint16_t* state, const uint16_t* r, const uint16_t* w,
+                       const uint16_t* w0, const uint16_t* k, const uint16_t* v, const uint16_t* a,
+                       const uint16_t* b, uint16_t* y, const int32_t* elapsed) {
+  parallel_for(static_cast<int64_t>(B) * H, [&](int64_t bh) {
+    const int bi = static_cast<int>(bh / H);
+    const int h = static_cast<int>(bh % H);
+    uint16_t* S = state + bh * kHead * kHead;
+    uint16_t wd[kHead];
+    for (int t = 0; t < T; ++t) {
+      const int64_t base = (static_cast<int64_t>(bi) * T + t) * C + h * kHead;
+      for (int c = 0; c < kHead; ++c) wd[c] = orc_wkv16_w_delta(w[base + c], w0, h * kHead + c, elapsed[bi] + h * kHead + c + t);
+      for (int i = 0; i < kHead; ++i) {
+        uint16_t* row = S + i * kHead;
+        uint16_t sa_even = 0, sa_odd = 0;
+        for (int j = 0; j < kHead / 2; ++j) {
+          sa_even = hfma16(a[base + 2 * j], row[2 * j], sa_even);
+          sa_odd = hfma16(a[base + 2 * j + 1], row[2 * j + 1], sa_odd);
+        }
+        const uint16_t sa = hadd16(sa_even, sa_odd);
+        const uint16_t vi = v[base + i];
+        uint16_t y_even = 0, y_odd = 0;
+        for (int j = 0; j < kHead / 2; ++j) {
+          for (int q = 0; q < 2; ++q) {
+            const int c = 2 * j + q;
+            const uint16_t s = row[c];
+            const uint16_t s_new = hfma16(s, wd[c], hfma16(k[base + c], vi, hfma16(sa, b[base + c], s)));
+            row[c] = s_new;
+            if (q == 0) y_even = hfma16(s_new, r[base + c], y_even);
+            else y_odd = hfma16(s_new, r[base + c], y_odd);
+          }
+        }
+        y[base + i] = hadd16(y_even, y_odd);
+      }
+    }
+  });
+}
+
+// ---------------------------------------------------------------------------------------------
 // Weight formats.  The reference has no quantised path (fp16 weights only, e.g.
 // cuda/rwkv7_v3a_ops.cu:464-560); these formats are this project's own and are unpinned at
 // the reference boundary.  Fixed operation order so a device implementation can be bit-exact:
@@ -764,8 +861,25 @@ static void mat_apply(const OrcMatrix& mat, int M, int N, int K, const uint16_t*
   gemv_any_f16(mat.fmt, M, N, K, x, mat.data, mat.scale, mat.zp, y);
 }
 
+static int model_forward_impl(const OrcModel* m, const int64_t* tokens, int B, int T, uint16_t* shift, float* wkv,
+                              uint16_t* wkv16, int32_t* elapsed, float* logits, uint16_t* trace);
+
 int orc_model_forward(const OrcModel* m, const int64_t* tokens, int B, int T, uint16_t* shift, float* wkv,
                       int32_t* elapsed, float* logits, uint16_t* trace) {
+  return model_forward_impl(m, tokens, B, T, shift, wkv, nullptr, elapsed, logits, trace);
+}
+
+// The same graph with the WKV state in fp16 (ModelBackend's use_wkv32 == false, src/rwkv7_fast_v4.cu:1266-1271):
+// calls of up to 16 tokens add w0 to the decay logit inside the recurrence, unrounded; longer ones round
+// w12 + w0 to fp16 first (rwkv7_add_vec_launch), as the fp32 path always does.
+int orc_model_forward_f16state(const OrcModel* m, const int64_t* tokens, int B, int T, uint16_t* shift,
+                               uint16_t* wkv16, int32_t* elapsed, float* logits, uint16_t* trace) {
+  if (!wkv16) return -1;
+  return model_forward_impl(m, tokens, B, T, shift, nullptr, wkv16, elapsed, logits, trace);
+}
+
+static int model_forward_impl(const OrcModel* m, const int64_t* tokens, int B, int T, uint16_t* shift, float* wkv,
+                              uint16_t* wkv16, int32_t* elapsed, float* logits, uint16_t* trace) {
   if (!m || B <= 0 || T <= 0) return -1;
   const int C = m->C, H = m->H, F = m->F, V = m->V, L = m->L;
   const int rows = B * T;
@@ -787,7 +901,8 @@ int orc_model_forward(const OrcModel* m, const int64_t* tokens, int B, int T, ui
     const OrcLayer& w = m->layers[l];
     uint16_t* shift0 = shift + static_cast<int64_t>(l) * 2 * B * C;
     uint16_t* shift1 = shift0 + static_cast<int64_t>(B) * C;
-    float* S = wkv + static_cast<int64_t>(l) * B * H * kHead * kHead;
+    float* S = wkv ? wkv + static_cast<int64_t>(l) * B * H * kHead * kHead : nullptr;
+    uint16_t* S16 = wkv16 ? wkv16 + static_cast<int64_t>(l) * B * H * kHead * kHead : nullptr;
 
     const uint16_t* mu6[6] = {w.t[ORC_T_X_R], w.t[ORC_T_X_W], w.t[ORC_T_X_K], w.t[ORC_T_X_V], w.t[ORC_T_X_A], w.t[ORC_T_X_G]};
     uint16_t* out6[6] = {xr.data(), xw.data(), xk.data(), xv.data(), xa.data(), xg.data()};
@@ -814,8 +929,18 @@ int orc_model_forward(const OrcModel* m, const int64_t* tokens, int B, int T, ui
 
     orc_kk_a_gate(rows, C, H, k.data(), w.t[ORC_T_K_K], w.t[ORC_T_A0], a12.data(), w.t[ORC_T_K_A], k2.data(),
                   nkk.data(), kka.data());
-    orc_add_vec(rows, C, w12.data(), w.t[ORC_T_W0], w_raw.data());
-    orc_wkv7_f16(B, T, C, H, 0, S, r.data(), w_raw.data(), k2.data(), v.data(), nkk.data(), kka.data(), y.data());
+    if (S16 && T <= 16) {
+      orc_wkv7_f16state(B, T, C, H, S16, r.data(), w12.data(), w.t[ORC_T_W0], k2.data(), v.data(), nkk.data(), kka.data(),
+                        y.data(), elapsed);
+    } else {
+      orc_add_vec(rows, C, w12.data(), w.t[ORC_T_W0], w_raw.data());
+      if (S16) {
+        orc_wkv7_f16state(B, T, C, H, S16, r.data(), w_raw.data(), nullptr, k2.data(), v.data(), nkk.data(), kka.data(),
+                          y.data(), elapsed);
+      } else {
+        orc_wkv7_f16(B, T, C, H, 0, S, r.data(), w_raw.data(), k2.data(), v.data(), nkk.data(), kka.data(), y.data());
+      }
+    }
     orc_lnx_rkvres_xg(rows, C, H, y.data(), r.data(), k2.data(), v.data(), w.t[ORC_T_R_K], w.t[ORC_T_LNX_W],
                       w.t[ORC_T_LNX_B], g.data(), y2.data());
     mat_apply(w.m[ORC_M_ATT_O], rows, C, C, y2.data(), att.data());

@@ -10,6 +10,10 @@
  * Parity pins (what independent evidence each function is checked against, in tests/):
  *   - f16<->f32 conversion ........ numpy float16, exhaustive over all 65536 codes
  *   - wkv7 ........................ float64 brute force, closed-form special cases
+ *   - wkv7, fp16 state ............ fp16 fma against exact rational arithmetic and numpy's float64 -> float16
+ *                                   rounding; one-step closed forms (S = k v^T from an empty state, r = e_j reads
+ *                                   column j of the new state), call-split invariance, the dither's range, known
+ *                                   values and zero mean, agreement with the fp32-state recurrence to fp16 accuracy
  *   - LN / add+LN(+lerp) .......... float64 closed forms on the reference test's inputs
  *   - kk/a-gate, GroupNorm, v-res . float64 closed forms + special cases
  *   - gemv / lora ................. numpy matmul in float64
@@ -54,6 +58,19 @@ void orc_wkv7_f32(int B, int T, int C, int H, int w_mode, float* state,
 void orc_wkv7_f16(int B, int T, int C, int H, int w_mode, float* state,
                   const uint16_t* r, const uint16_t* w, const uint16_t* k, const uint16_t* v,
                   const uint16_t* a, const uint16_t* b, uint16_t* y);
+
+/* WKV7 with an fp16 state [B,H,64,64], every operation an fp16 fused multiply-add in the reference's order
+ * (cuda/rwkv7_wkv_fp16_v2.cu:41-52,157-193).  w holds raw decay logits; w0 [C] (may be NULL) is added to them
+ * unrounded; elapsed i32 [B] (tokens seen before this call) phases the decay dither and is not modified. */
+void orc_wkv7_f16state(int B, int T, int C, int H, uint16_t* state, const uint16_t* r, const uint16_t* w,
+                       const uint16_t* w0, const uint16_t* k, const uint16_t* v, const uint16_t* a,
+                       const uint16_t* b, uint16_t* y, const int32_t* elapsed);
+/* pieces of it, exported for the pin tests: double -> fp16 round-to-nearest-even, the fp16 fma, the dither
+ * (:41-43) and the per-channel decay delta (:45-52) */
+uint16_t orc_f64_to_f16(double x);
+uint16_t orc_f16_fma(uint16_t a, uint16_t b, uint16_t c);
+float orc_wkv16_rotator(int32_t x);
+uint16_t orc_wkv16_w_delta(uint16_t w_raw, const uint16_t* w0, int c, int32_t phase);
 
 /* ---- weight formats -----------------------------------------------------------------
  * W8A16: per-output-row symmetric int8, scale f16 [N].
@@ -154,6 +171,9 @@ int orc_model_set_matrix(OrcModel* m, int layer, int id, int fmt, const void* da
  * layer: f16 [L,B*T,C].  Returns 0, or a negative code on a bad argument. */
 int orc_model_forward(const OrcModel* m, const int64_t* tokens, int B, int T, uint16_t* shift, float* wkv,
                       int32_t* elapsed, float* logits, uint16_t* trace);
+/* the same graph with the WKV state in fp16, wkv16 f16 [L,B,H,64,64] (src/rwkv7_fast_v4.cu:1266-1271) */
+int orc_model_forward_f16state(const OrcModel* m, const int64_t* tokens, int B, int T, uint16_t* shift,
+                               uint16_t* wkv16, int32_t* elapsed, float* logits, uint16_t* trace);
 
 #ifdef __cplusplus
 }

@@ -335,6 +335,13 @@ int lnx_launch(hipStream_t st, int64_t rows_heads, int H, const half_t* y, const
   return RWKV_OK;
 }
 
+int add_vec_launch(hipStream_t st, int rows, int C, const half_t* x, const half_t* vec, half_t* out) {
+  const int64_t n = static_cast<int64_t>(rows) * C;
+  hipLaunchKernelGGL(add_vec_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, st, n, C, x, vec, out);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
 int advance_launch(hipStream_t st, int n, int amount, int* x) {
   hipLaunchKernelGGL(advance_i32_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, st, n, amount, x);
   RWKV_LAUNCH_CHECK();
@@ -443,11 +450,7 @@ int rwkv_hip_relu_square(rwkv_stream_t s, int64_t n, const void* x, void* out) {
 
 int rwkv_hip_add_vec(rwkv_stream_t s, int rows, int C, const void* x, const void* vec, void* out) {
   RWKV_REQUIRE(rows > 0 && C > 0 && x && vec && out, "add_vec: bad arguments");
-  const int64_t n = static_cast<int64_t>(rows) * C;
-  hipLaunchKernelGGL(add_vec_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, as_stream(s), n, C, H16(x), H16(vec),
-                     H16M(out));
-  RWKV_LAUNCH_CHECK();
-  return RWKV_OK;
+  return add_vec_launch(as_stream(s), rows, C, H16(x), H16(vec), H16M(out));
 }
 
 int rwkv_hip_f16_to_f32(rwkv_stream_t s, int64_t n, const void* src, void* dst) {

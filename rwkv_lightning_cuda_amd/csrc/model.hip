@@ -122,6 +122,7 @@ struct rwkv_hip_session {
   void* sparse_ws = nullptr;  // partial rows of the row-skipping ffn.value product
   size_t sparse_ws_bytes = 0;
   int sparse_ffn_rows = 1;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
+  bool wkv_fp16 = false;      // the WKV state tensor is fp16 [L,B,H,64,64] (the reference's use_wkv32 == false)
   int fused_ln = -1;          // decode steps fold LayerNorm + token shift into the linear launches: 1 always, 0 never,
                               // -1 for one row of at most 4096 channels (the row-resident GEMV hides the prologue
                               // behind its weight requests: 7.2B shape 2.04 -> 1.92 ms per step, 0.1B 0.413 -> 0.373)
@@ -317,7 +318,9 @@ void take_deferred(LnArgs& a, const DeferredReduce& d) {
   } while (0)
 
 // Enqueues the whole forward pass on the session stream.  tokens are already in s->tokens_dev.
-int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv, int* elapsed, float* logits) {
+int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_any, int* elapsed, float* logits) {
+  float* wkv = static_cast<float*>(wkv_any);            // fp32 state (the default)
+  half_t* wkv16 = static_cast<half_t*>(wkv_any);        // fp16 state (session option)
   const rwkv_hip_model* m = s->model;
   hipStream_t st = s->stream;
   Buffers& b = s->buf;
@@ -338,12 +341,13 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
   // The single-launch time-mix core re-reads a head's LoRA rows for every batch row; from 16 rows on the
   // row-tiled kernels of the prefill path (LoRA rank-outs on the matrix core) are faster (measured: 4.2 -> 4.0 ms
   // per step at 16 rows, 5.5 -> 4.6 ms at 32).
-  const bool fused_tmix = step && rows <= 8;
+  const bool fused_tmix = step && rows <= 8 && !s->wkv_fp16;  // (the fp16 state has its own recurrence kernel)
   // Decode steps on the GEMV path can fold both LayerNorm + token-shift kernels of a layer into the prologue of the
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key): by default for one row of up to 4096
   // channels.  The residual-stream tap needs the stand-alone kernels.
   const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows == 1 && C <= 4096);
-  const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace &&
+  // (the shift row that the prologue leaves for later is stored by the single-launch time-mix core)
+  const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace && fused_tmix &&
                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
 
   // Decode steps of a few rows (one by default) read, per row, only the ffn.value rows whose relu^2 activation is
@@ -383,6 +387,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
     half_t* shift0 = shift + static_cast<int64_t>(l) * 2 * B * C;
     half_t* shift1 = shift0 + static_cast<int64_t>(B) * C;
     float* S = wkv + static_cast<int64_t>(l) * B * H * kHead * kHead;
+    half_t* S16 = wkv16 + static_cast<int64_t>(l) * B * H * kHead * kHead;
     half_t* v_cur = (l == 0) ? b.v_first : b.v;  // layer 0 writes v straight into v_first
 
     if (!step) {
@@ -492,7 +497,26 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, float* wkv
         TRY_AUX(lora_out_multi(st, a));
       }
 
-      if (!s->trace && tmix_seq_whole_heads(B, T, H)) {
+      if (s->wkv_fp16) {
+        // fp16 state (src/rwkv7_fast_v4.cu:1262-1271): kk / a-gate in fp16, the fp16 recurrence, GroupNorm / bonus / gate.
+        // Calls of up to 16 tokens add w0 to the decay logit inside the recurrence, unrounded; longer ones round
+        // w12 + w0 to fp16 first, as the reference does.
+        KkArgs p = {};
+        p.k = b.k; p.k_k = w.t[RWKV_T_K_K]; p.a0 = w.t[RWKV_T_A0]; p.a12 = b.a12; p.k_a = w.t[RWKV_T_K_A];
+        p.new_k = b.k2; p.neg_kk = b.nkk; p.kka = b.kka;
+        p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
+        TRY_AUX(kk_a_gate_launch(st, p));
+        const half_t* w_in = b.w12;
+        const half_t* w0 = w.t[RWKV_T_W0];
+        if (T > 16) {
+          TRY_AUX(add_vec_launch(st, rows, C, b.w12, w.t[RWKV_T_W0], b.scratch));
+          w_in = b.scratch;
+          w0 = nullptr;
+        }
+        TRY_AUX(wkv7_f16state_launch(st, B, T, C, H, S16, b.r, w_in, w0, b.k2, v_cur, b.nkk, b.kka, b.y, elapsed));
+        TRY_AUX(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
+                           w.t[RWKV_T_LNX_B], b.g, b.y2));
+      } else if (!s->trace && tmix_seq_whole_heads(B, T, H)) {
         // kk normalise / a-gate / decay, the WKV recurrence and GroupNorm / bonus / gate in one launch
         TmixSeqArgs fa;
         fa.r = b.r; fa.k = b.k; fa.a12 = b.a12; fa.w12 = b.w12; fa.g = b.g;
@@ -627,7 +651,7 @@ GraphEntry* find_graph(rwkv_hip_session* s, int B, void* shift, void* wkv, void*
 }
 
 // T == 1 step through a captured graph (captures on first use of this (B, state, logits) tuple).
-int run_step(rwkv_hip_session* s, int B, half_t* shift, float* wkv, int* elapsed, float* logits) {
+int run_step(rwkv_hip_session* s, int B, half_t* shift, void* wkv, int* elapsed, float* logits) {
   if (!s->use_graph || s->trace || s->profile) return enqueue_forward(s, B, 1, shift, wkv, elapsed, logits);
   GraphEntry* g = find_graph(s, B, shift, wkv, elapsed, logits);
   if (!g) {
@@ -902,6 +926,16 @@ int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on) {
   return RWKV_OK;
 }
 
+int rwkv_hip_session_set_wkv_fp16(rwkv_hip_session* s, int on) {
+  RWKV_REQUIRE(s, "session is NULL");
+  const bool want = on != 0;
+  if (s->wkv_fp16 != want) {
+    TRY(drop_graphs(s));  // captured decode graphs hold the other recurrence kernel
+    s->wkv_fp16 = want;
+  }
+  return RWKV_OK;
+}
+
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows) {
   RWKV_REQUIRE(s, "session is NULL");
   RWKV_REQUIRE(max_rows >= 0 && max_rows <= kSparseMaxRows, "set_sparse_ffn: max_rows %d out of range (0..%d)", max_rows,
@@ -962,11 +996,9 @@ int rwkv_hip_forward(rwkv_hip_session* s, const int64_t* tokens_host, int B, int
   std::copy(tokens_host, tokens_host + rows, s->tokens_pinned);
   RWKV_HIP_TRY(hipMemcpyAsync(s->tokens_dev, s->tokens_pinned, sizeof(int64_t) * rows, hipMemcpyHostToDevice, s->stream));
   if (T == 1) {
-    TRY(run_step(s, B, static_cast<half_t*>(shift), static_cast<float*>(wkv), static_cast<int*>(elapsed),
-                 static_cast<float*>(logits)));
+    TRY(run_step(s, B, static_cast<half_t*>(shift), wkv, static_cast<int*>(elapsed), static_cast<float*>(logits)));
   } else {
-    TRY(enqueue_forward(s, B, T, static_cast<half_t*>(shift), static_cast<float*>(wkv), static_cast<int*>(elapsed),
-                        static_cast<float*>(logits)));
+    TRY(enqueue_forward(s, B, T, static_cast<half_t*>(shift), wkv, static_cast<int*>(elapsed), static_cast<float*>(logits)));
   }
   if (sync) RWKV_HIP_TRY(hipStreamSynchronize(s->stream));
   return RWKV_OK;
@@ -998,8 +1030,7 @@ int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host
   std::copy(first_tokens_host, first_tokens_host + B, s->tokens_pinned);
   RWKV_HIP_TRY(hipMemcpyAsync(s->tokens_dev, s->tokens_pinned, sizeof(int64_t) * B, hipMemcpyHostToDevice, s->stream));
   for (int i = 0; i < steps; ++i) {
-    TRY(run_step(s, B, static_cast<half_t*>(shift), static_cast<float*>(wkv), static_cast<int*>(elapsed),
-                 static_cast<float*>(logits)));
+    TRY(run_step(s, B, static_cast<half_t*>(shift), wkv, static_cast<int*>(elapsed), static_cast<float*>(logits)));
     TRY(argmax_launch(s->stream, B, s->model->V, static_cast<float*>(logits), s->argmax_dev));
     hipLaunchKernelGGL(feed_tokens_kernel, dim3(ceil_div(B, 64)), dim3(64), 0, s->stream, B, s->argmax_dev,
                        s->tokens_dev, s->history_dev + static_cast<size_t>(i) * B);

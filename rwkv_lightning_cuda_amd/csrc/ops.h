@@ -159,6 +159,7 @@ int kk_a_gate_launch(hipStream_t st, const KkArgs& p);
 int lnx_launch(hipStream_t st, int64_t rows_heads, int H, const half_t* y, const half_t* r, const half_t* k,
                const half_t* v, const half_t* r_k, const half_t* lnw, const half_t* lnb, const half_t* g, half_t* out);
 int advance_launch(hipStream_t st, int n, int amount, int* x);
+int add_vec_launch(hipStream_t st, int rows, int C, const half_t* x, const half_t* vec, half_t* out);  // out = f16(x + vec[c])
 int embed_gather_launch(hipStream_t st, int rows, int C, const int64_t* tokens, const half_t* table, half_t* out);
 
 // ---- lora.hip -----------------------------------------------------------------------------------
@@ -212,6 +213,11 @@ bool tmix_seq_whole_heads(int B, int T, int H);
 int wkv7_seq_f16_launch(hipStream_t st, int B, int T, int C, int H, float* state, const float* r, const float* d,
                         const float* k, const float* a, const float* b, int64_t op_bs, const half_t* v, half_t* y,
                         int64_t io_bs);
+
+// ---- wkv7_f16state.hip: the recurrence with an fp16 state (w raw decay logits, w0 [C] or NULL added unrounded) ----
+int wkv7_f16state_launch(hipStream_t st, int B, int T, int C, int H, half_t* state, const half_t* r, const half_t* w,
+                         const half_t* w0, const half_t* k, const half_t* v, const half_t* a, const half_t* b, half_t* y,
+                         const int* elapsed);
 
 }  // namespace rwkv
 

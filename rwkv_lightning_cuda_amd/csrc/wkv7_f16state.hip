@@ -1,0 +1,165 @@
+// WKV7 recurrence with the state kept in fp16: the reference server's default mode (ModelBackend's
+// use_wkv32 == false).
+//
+// Reference: cuda/rwkv7_wkv_fp16_v2.cu - the per-token arithmetic is the same in every kernel of that file
+// (:157-193, :342-367, :433-468, :531-556, :632-660): thread i owns state row i as 32 half2 pairs and every operation
+// is a packed fp16 fused multiply-add with one rounding (__hfma2),
+//   sa2 = chain over pairs j of fma(a[j], S[i][j], sa2);  sa = f16(sa2.x + sa2.y)
+//   wd[c] = f16(exp2f(-e^-1/2 log2e / (1 + exp2f(-log2e * w[c]))) - 1 + dither(elapsed[b] + h*64 + c + t))   (:41-52)
+//   S[i][j] = fma(S[i][j], wd[j], fma(k[j], v[i], fma(sa, b[j], S[i][j])))
+//   y2 = chain over pairs of fma(S'[i][j], r[j], y2);  y[i] = f16(y2.x + y2.y)
+// with dither(x) = 2^-41 * float(int32(2654435769 * x)): below the fp16 resolution of d - 1, it makes the rounding of
+// the decay unbiased over consecutive tokens and channels.  The order of the two chains is part of the result (fp16
+// sums do not associate), so it is kept: the kernel is bit-identical to a scalar restatement of the reference except
+// where v_exp_f32 and the host's exp2f differ in the last bit before the decay delta is rounded to fp16.
+//
+// gfx950 layout: one wavefront per (batch row, head), lane = state row, the row's 64 values in 32 registers as half2
+// pairs (v_pk_fma_f16 does both columns of a pair).  The five per-column vectors of a token (a, b, k, decay delta,
+// r) are the same for every lane: lane c fetches element c of each for the NEXT token while the current one is
+// computed, converts its decay logit, and drops them into LDS, from where every lane reads them back as 16-byte
+// broadcasts.  The state is read and written once per call, 16 bytes per lane and instruction.
+#include "ops.h"
+
+namespace rwkv {
+
+namespace {
+
+constexpr int kPairs = kHead / 2;  // half2 pairs per state row
+
+struct TokenOps {  // one token's per-column operands in LDS
+  half_t a[kHead], b[kHead], k[kHead], wd[kHead], r[kHead];
+};
+
+__device__ __forceinline__ half2_t pk_fma(half2_t x, half2_t y, half2_t z) { return __builtin_elementwise_fma(x, y, z); }
+
+// cuda/rwkv7_wkv_fp16_v2.cu:41-52
+__device__ __forceinline__ half_t decay_delta(half_t w_raw, const half_t* __restrict__ w0, int c, int phase) {
+  float w = h2f(w_raw);
+  if (w0) w += h2f(w0[c]);  // unrounded, as the reference's _w0 launchers
+  const unsigned prod = 2654435769u * static_cast<unsigned>(phase);
+  const float dither = 4.547473508864641e-13f * static_cast<float>(static_cast<int>(prod));
+  const float d = exp2f(-0.8750387749145276f / (1.0f + exp2f(-1.4426950408889634f * w))) - 1.0f + dither;
+  return f2h(d);
+}
+
+__device__ __forceinline__ void read_pairs(const half_t* __restrict__ src, half2_t (&dst)[kPairs]) {
+#pragma unroll
+  for (int q = 0; q < kPairs / 4; ++q) {
+    const uint4_t t = *reinterpret_cast<const uint4_t*>(src + 8 * q);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[4 * q + e] = as_half2(t[e]);
+  }
+}
+
+__global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int H, half_t* __restrict__ state,
+                                                              const half_t* __restrict__ r, const half_t* __restrict__ w,
+                                                              const half_t* __restrict__ w0, const half_t* __restrict__ k,
+                                                              const half_t* __restrict__ v, const half_t* __restrict__ a,
+                                                              const half_t* __restrict__ b, half_t* __restrict__ y,
+                                                              const int* __restrict__ elapsed) {
+  __shared__ __align__(16) TokenOps ops[2];
+  const int bh = blockIdx.x;
+  const int bi = bh / H;
+  const int h = bh - bi * H;
+  const int lane = threadIdx.x;
+  const int c = h * kHead + lane;
+
+  // state row `lane`: 128 bytes
+  half_t* srow = state + (static_cast<int64_t>(bh) * kHead + lane) * kHead;
+  half2_t S[kPairs];
+#pragma unroll
+  for (int q = 0; q < kPairs / 4; ++q) {
+    const uint4_t t = *reinterpret_cast<const uint4_t*>(srow + 8 * q);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) S[4 * q + e] = as_half2(t[e]);
+  }
+
+  const int phase0 = elapsed[bi] + c;
+  int64_t tok = static_cast<int64_t>(bi) * T * C + c;  // this lane's element of token 0
+  // token 0's operands
+  {
+    ops[0].a[lane] = a[tok];
+    ops[0].b[lane] = b[tok];
+    ops[0].k[lane] = k[tok];
+    ops[0].r[lane] = r[tok];
+    ops[0].wd[lane] = decay_delta(w[tok], w0, c, phase0);
+  }
+  half_t v_cur = v[tok];
+  __syncthreads();
+
+  for (int t = 0; t < T; ++t) {
+    const TokenOps& cur = ops[t & 1];
+    TokenOps& nxt = ops[(t + 1) & 1];
+    // request the next token's elements now (the last token re-reads itself: no load under a branch)
+    const int64_t tn = t + 1 < T ? tok + C : tok;
+    const half_t a_n = a[tn], b_n = b[tn], k_n = k[tn], r_n = r[tn], w_n = w[tn], v_n = v[tn];
+
+    half2_t vec[kPairs];
+    read_pairs(cur.a, vec);
+    half2_t sa2 = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+#pragma unroll
+    for (int j = 0; j < kPairs; ++j) sa2 = pk_fma(vec[j], S[j], sa2);
+    const half_t sa = sa2[0] + sa2[1];
+    const half2_t sa_b = {sa, sa};
+    const half2_t vv = {v_cur, v_cur};
+
+    half2_t bv[kPairs], kv[kPairs], wv[kPairs];
+    read_pairs(cur.b, bv);
+    read_pairs(cur.k, kv);
+    read_pairs(cur.wd, wv);
+    read_pairs(cur.r, vec);
+    half2_t y2 = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+#pragma unroll
+    for (int j = 0; j < kPairs; ++j) {
+      const half2_t s = S[j];
+      const half2_t s_new = pk_fma(s, wv[j], pk_fma(kv[j], vv, pk_fma(sa_b, bv[j], s)));
+      S[j] = s_new;
+      y2 = pk_fma(s_new, vec[j], y2);
+    }
+    y[tok] = y2[0] + y2[1];
+
+    // hand the next token's operands to the other buffer (nobody reads it during this step)
+    nxt.a[lane] = a_n;
+    nxt.b[lane] = b_n;
+    nxt.k[lane] = k_n;
+    nxt.r[lane] = r_n;
+    nxt.wd[lane] = decay_delta(w_n, w0, c, phase0 + t + 1);
+    v_cur = v_n;
+    tok = tn;
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int q = 0; q < kPairs / 4; ++q) {
+    uint4_t t;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) t[e] = __builtin_bit_cast(uint32_t, S[4 * q + e]);
+    *reinterpret_cast<uint4_t*>(srow + 8 * q) = t;
+  }
+}
+
+}  // namespace
+
+int wkv7_f16state_launch(hipStream_t st, int B, int T, int C, int H, half_t* state, const half_t* r, const half_t* w,
+                         const half_t* w0, const half_t* k, const half_t* v, const half_t* a, const half_t* b, half_t* y,
+                         const int* elapsed) {
+  RWKV_REQUIRE(B > 0 && T > 0 && H > 0, "wkv7_f16state: B, T, H must be positive");
+  RWKV_REQUIRE(C == H * kHead, "wkv7_f16state: C (%d) must equal H*64 (H=%d)", C, H);
+  RWKV_REQUIRE(state && r && w && k && v && a && b && y && elapsed, "wkv7_f16state: NULL tensor");
+  hipLaunchKernelGGL(wkv7_f16state_kernel, dim3(B * H), dim3(kWave), 0, st, T, C, H, state, r, w, w0, k, v, a, b, y, elapsed);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+}  // namespace rwkv
+
+using namespace rwkv;
+
+extern "C" int rwkv_hip_wkv7_f16state(rwkv_stream_t s, int B, int T, int C, int H, void* state, const void* r,
+                                      const void* w, const void* w0, const void* k, const void* v, const void* a,
+                                      const void* b, void* y, const void* elapsed) {
+  return wkv7_f16state_launch(as_stream(s), B, T, C, H, static_cast<half_t*>(state), static_cast<const half_t*>(r),
+                              static_cast<const half_t*>(w), static_cast<const half_t*>(w0), static_cast<const half_t*>(k),
+                              static_cast<const half_t*>(v), static_cast<const half_t*>(a), static_cast<const half_t*>(b),
+                              static_cast<half_t*>(y), static_cast<const int*>(elapsed));
+}

@@ -32,14 +32,14 @@ EXPORTS = [
     "rwkv_hip_memcpy_h2d_async", "rwkv_hip_memcpy_d2h_async", "rwkv_hip_memcpy_d2d_async", "rwkv_hip_memset",
     "rwkv_hip_mem_info", "rwkv_hip_stream_create", "rwkv_hip_stream_destroy", "rwkv_hip_stream_sync",
     "rwkv_hip_device_sync", "rwkv_hip_event_create", "rwkv_hip_event_destroy", "rwkv_hip_event_record",
-    "rwkv_hip_event_elapsed_ms", "rwkv_hip_measure_launch_chain", "rwkv_hip_wkv7", "rwkv_hip_quantize_w8", "rwkv_hip_dequant_w8",
+    "rwkv_hip_event_elapsed_ms", "rwkv_hip_measure_launch_chain", "rwkv_hip_wkv7", "rwkv_hip_wkv7_f16state", "rwkv_hip_quantize_w8", "rwkv_hip_dequant_w8",
     "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_bf16_to_f16", "rwkv_hip_bf16_to_f16_transpose",
     "rwkv_hip_emb_ln0_bf16_to_f16", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",
     "rwkv_hip_pack_weights", "rwkv_hip_linear_packed_workspace", "rwkv_hip_linear_packed", "rwkv_hip_lora_in", "rwkv_hip_lora_out",
     "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_pack_w4", "rwkv_hip_cmix_sparse_packed_bytes",
     "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
     "rwkv_hip_cmix_sparse_down_relu_rows", "rwkv_hip_cmix_sparse_down_relu_rows_static",
-    "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln",
+    "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln", "rwkv_hip_session_set_wkv_fp16",
     "rwkv_hip_layer_norm", "rwkv_hip_add_layer_norm", "rwkv_hip_add_last_layer_norm", "rwkv_hip_token_shift_mix",
     "rwkv_hip_add_layer_norm_cmix_mix", "rwkv_hip_add_layer_norm_tmix_mix6", "rwkv_hip_kk_a_gate",
     "rwkv_hip_lnx_rkvres_xg", "rwkv_hip_relu_square", "rwkv_hip_add_vec", "rwkv_hip_f16_to_f32",
@@ -194,6 +194,12 @@ def _ptr_array(items):
 def wkv7(B, T, C, H, w_mode, io, state, r, w, k, v, a, b, y, stream=None):
     check(load().rwkv_hip_wkv7(_p(stream), _i(B), _i(T), _i(C), _i(H), _i(w_mode), _i(io), _p(state), _p(r), _p(w),
                                _p(k), _p(v), _p(a), _p(b), _p(y)))
+
+
+def wkv7_f16state(B, T, C, H, state, r, w, k, v, a, b, y, elapsed, w0=None, stream=None):
+    """The recurrence with an fp16 state [B,H,64,64]; w raw decay logits, w0 [C] or None, elapsed int32 [B]."""
+    check(load().rwkv_hip_wkv7_f16state(_p(stream), _i(B), _i(T), _i(C), _i(H), _p(state), _p(r), _p(w), _p(w0), _p(k),
+                                        _p(v), _p(a), _p(b), _p(y), _p(elapsed)))
 
 
 def bf16_to_f16(n, src, dst, stream=None):

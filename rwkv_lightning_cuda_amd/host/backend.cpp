@@ -109,6 +109,7 @@ Spec parse_spec(const std::string& path) {
 
 struct ModelBackend::Impl {
   std::string model_path;
+  bool use_wkv32 = false;  // false: the WKV state is fp16 (the reference's default), true: fp32
   std::string model_name;
   Spec spec;
   rwkv_hip_model* model = nullptr;
@@ -434,8 +435,11 @@ struct ModelBackend::Impl {
     const int V = spec.dims.vocab;
     out.values.resize(static_cast<std::size_t>(B) * V, "alloc backend logits f32");
     rwkv_hip_session* s = acquire();
-    const int rc = rwkv_hip_forward(s, flat.data(), B, T, state.shift.p, state.wkv_state32.p, state.elapsed.p,
-                                    out.values.p, 1);
+    int rc = rwkv_hip_session_set_wkv_fp16(s, use_wkv32 ? 0 : 1);
+    if (rc == RWKV_OK) {
+      void* wkv = use_wkv32 ? static_cast<void*>(state.wkv_state32.p) : static_cast<void*>(state.wkv_state.p);
+      rc = rwkv_hip_forward(s, flat.data(), B, T, state.shift.p, wkv, state.elapsed.p, out.values.p, 1);
+    }
     const std::string msg = rc == RWKV_OK ? std::string() : std::string(rwkv_hip_last_error());
     release(s);
     if (rc != RWKV_OK) throw std::runtime_error(msg);
@@ -445,9 +449,7 @@ struct ModelBackend::Impl {
 };
 
 ModelBackend::ModelBackend(std::string model_path, bool use_wkv32, bool chunk_load) : impl_(std::make_unique<Impl>()) {
-  if (!use_wkv32) {
-    throw std::runtime_error("this backend provides the fp32 WKV state only: construct it with use_wkv32 = true");
-  }
+  impl_->use_wkv32 = use_wkv32;
   impl_->model_path = std::move(model_path);
   impl_->spec = parse_spec(impl_->model_path);
   impl_->model_name = impl_->spec.name;
@@ -467,13 +469,21 @@ GenerationState ModelBackend::create_state(int batch_size) const {
   const ModelDims& d = impl_->spec.dims;
   GenerationState state;
   state.batch_size = batch_size;
-  state.wkv32 = true;
+  state.wkv32 = impl_->use_wkv32;   // src/rwkv7_fast_v4.cu:1379-1396: one of the two state tensors, by mode
   state.shift.resize(static_cast<std::size_t>(d.layers) * 2 * batch_size * d.channels, "alloc backend shift state");
-  state.wkv_state32.resize(static_cast<std::size_t>(d.layers) * batch_size * d.heads * d.head_size * d.head_size,
-                           "alloc backend wkv32 state");
+  const std::size_t state_elems = static_cast<std::size_t>(d.layers) * batch_size * d.heads * d.head_size * d.head_size;
+  if (impl_->use_wkv32) {
+    state.wkv_state32.resize(state_elems, "alloc backend wkv32 state");
+  } else {
+    state.wkv_state.resize(state_elems, "alloc backend wkv state");
+  }
   state.elapsed.resize(batch_size, "alloc backend elapsed");
   state.shift.zero("zero backend shift");
-  state.wkv_state32.zero("zero backend wkv32");
+  if (impl_->use_wkv32) {
+    state.wkv_state32.zero("zero backend wkv32");
+  } else {
+    state.wkv_state.zero("zero backend wkv");
+  }
   state.elapsed.zero("zero backend elapsed");
   check_hip(rwkv_hip_device_sync(), "sync backend state init");
   return state;
@@ -484,7 +494,7 @@ void ModelBackend::forward_prefill(const std::vector<std::vector<int64_t>>& toke
   const int B = static_cast<int>(token_batches.size());
   if (B <= 0) throw std::runtime_error("token_batches must not be empty");
   if (state.batch_size != B) throw std::runtime_error("state batch size mismatch");
-  if (!state.wkv32) throw std::runtime_error("state wkv precision mismatch");
+  if (state.wkv32 != impl_->use_wkv32) throw std::runtime_error("state wkv precision mismatch");  // :1060-1062
   const int T = static_cast<int>(token_batches.front().size());
   if (T <= 0) throw std::runtime_error("token batch length must be positive");
   std::vector<int64_t> flat;
@@ -501,7 +511,7 @@ void ModelBackend::forward_decode(const std::vector<int64_t>& token_batch, Gener
   const int B = static_cast<int>(token_batch.size());
   if (B <= 0) throw std::runtime_error("token_batches must not be empty");
   if (state.batch_size != B) throw std::runtime_error("state batch size mismatch");
-  if (!state.wkv32) throw std::runtime_error("state wkv precision mismatch");
+  if (state.wkv32 != impl_->use_wkv32) throw std::runtime_error("state wkv precision mismatch");
   impl_->forward(token_batch, B, 1, state, logits);
 }
 
@@ -510,7 +520,8 @@ void ModelBackend::copy_state_slice(const GenerationState& src, int src_offset, 
   if (src_offset < 0 || dst_offset < 0 || count <= 0) throw std::runtime_error("invalid backend state slice range");
   if (src.batch_size <= 0 || dst.batch_size <= 0)
     throw std::runtime_error("state slice requires non-empty source and destination");
-  if (!src.wkv32 || !dst.wkv32) throw std::runtime_error("state slice wkv precision mismatch");
+  if (src.wkv32 != dst.wkv32 || src.wkv32 != impl_->use_wkv32)
+    throw std::runtime_error("state slice wkv precision mismatch");  // src/rwkv7_fast_v4.cu:1433-1435
   if (src_offset + count > src.batch_size || dst_offset + count > dst.batch_size)
     throw std::runtime_error("state slice range exceeds batch size");
 
@@ -523,9 +534,15 @@ void ModelBackend::copy_state_slice(const GenerationState& src, int src_offset, 
       half* t = dst.shift.p + (static_cast<std::size_t>(layer) * 2 + which) * dst.batch_size * C + dst_offset * C;
       check_hip(rwkv_hip_memcpy_d2d(t, s, count * C * sizeof(half)), "copy backend state slice shift");
     }
-    const float* s = src.wkv_state32.p + (static_cast<std::size_t>(layer) * src.batch_size + src_offset) * lane;
-    float* t = dst.wkv_state32.p + (static_cast<std::size_t>(layer) * dst.batch_size + dst_offset) * lane;
-    check_hip(rwkv_hip_memcpy_d2d(t, s, count * lane * sizeof(float)), "copy backend state slice wkv32");
+    if (impl_->use_wkv32) {
+      const float* s = src.wkv_state32.p + (static_cast<std::size_t>(layer) * src.batch_size + src_offset) * lane;
+      float* t = dst.wkv_state32.p + (static_cast<std::size_t>(layer) * dst.batch_size + dst_offset) * lane;
+      check_hip(rwkv_hip_memcpy_d2d(t, s, count * lane * sizeof(float)), "copy backend state slice wkv32");
+    } else {
+      const half* s = src.wkv_state.p + (static_cast<std::size_t>(layer) * src.batch_size + src_offset) * lane;
+      half* t = dst.wkv_state.p + (static_cast<std::size_t>(layer) * dst.batch_size + dst_offset) * lane;
+      check_hip(rwkv_hip_memcpy_d2d(t, s, count * lane * sizeof(half)), "copy backend state slice wkv");
+    }
   }
   check_hip(rwkv_hip_memcpy_d2d(dst.elapsed.p + dst_offset, src.elapsed.p + src_offset, count * sizeof(int)),
             "copy backend state slice elapsed");
@@ -553,7 +570,8 @@ PrefillCapacity ModelBackend::query_prefill_capacity(int prefill_chunk_size) con
   const std::size_t L = d.layers, C = d.channels, H = d.heads, N = d.head_size, V = d.vocab, F = d.ffn;
   const std::size_t T = static_cast<std::size_t>(prefill_chunk_size);
   const std::size_t rank_max = std::max(std::max(d.rank_w, d.rank_a), std::max(d.rank_g, d.rank_v));
-  const std::size_t state_bytes = L * 2 * C * sizeof(half) + L * H * N * N * sizeof(float) + sizeof(int);
+  const std::size_t state_bytes = L * 2 * C * sizeof(half) + L * H * N * N * (impl_->use_wkv32 ? sizeof(float) : sizeof(half)) +
+                                  sizeof(int);  // src/rwkv7_fast_v4.cu:1556
   // one batch lane of the session arena for a chunk of T tokens (csrc/model.hip ensure_arena) + fp32 logits
   const std::size_t arena_bytes = T * C * 2 * 28 + T * rank_max * 2 * 4 + T * F * 2 + C * 2 + T * C * 4 * 5;
   cap.bytes_per_batch = state_bytes + arena_bytes + V * sizeof(float);

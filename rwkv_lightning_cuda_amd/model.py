@@ -222,10 +222,11 @@ class HipModel:
 class State:
     """Generation state on the device (GenerationState, include/rwkv_server_backend.hpp:45-58, wkv32 mode)."""
 
-    def __init__(self, dims, B):
+    def __init__(self, dims, B, wkv_fp16=False):
         self.B = B
+        self.wkv_fp16 = wkv_fp16
         self.shift = hip.DeviceArray.zeros((dims.L, 2, B, dims.C), np.float16)
-        self.wkv = hip.DeviceArray.zeros((dims.L, B, dims.H, 64, 64), np.float32)
+        self.wkv = hip.DeviceArray.zeros((dims.L, B, dims.H, 64, 64), np.float16 if wkv_fp16 else np.float32)
         self.elapsed = hip.DeviceArray.zeros((B,), np.int32)
 
 
@@ -270,6 +271,10 @@ class Session:
         never, None (the default of a new session) for one row of at most 4096 channels."""
         hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(-1 if on is None else 1 if on else 0)))
 
+    def set_wkv_fp16(self, on):
+        """The state's WKV tensor is fp16 and the recurrence runs in fp16 (the reference's use_wkv32 == false)."""
+        hip.check(hip.load().rwkv_hip_session_set_wkv_fp16(self.handle, ctypes.c_int(1 if on else 0)))
+
     def set_sparse_ffn(self, max_rows):
         """Decode steps of up to max_rows rows (0..12; True = 1, False = 0) read only the ffn.value rows with a
         non-zero activation (default 1)."""
@@ -292,6 +297,7 @@ class Session:
         B, T = tokens.shape
         if B != state.B:
             raise ValueError("state batch size mismatch")  # src/rwkv7_fast_v4.cu:1057-1059
+        self.set_wkv_fp16(state.wkv_fp16)
         hip.check(hip.load().rwkv_hip_forward(self.handle, tokens.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(B),
                                               ctypes.c_int(T), hip._p(state.shift), hip._p(state.wkv),
                                               hip._p(state.elapsed), hip._p(logits), ctypes.c_int(1 if sync else 0)))
@@ -299,6 +305,7 @@ class Session:
     def decode_greedy(self, first_tokens, steps, state, logits):
         first = np.ascontiguousarray(first_tokens, dtype=np.int64)
         B = first.shape[0]
+        self.set_wkv_fp16(state.wkv_fp16)
         out = np.zeros((steps, B), dtype=np.int32)
         hip.check(hip.load().rwkv_hip_decode_greedy(self.handle, first.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(B),
                                                     ctypes.c_int(steps), hip._p(state.shift), hip._p(state.wkv),

@@ -1,5 +1,8 @@
 // ModelBackend over the kernel library (synthetic tiny model): state and logits shapes, argument errors with
 // the reference's messages (src/rwkv_server_backend.cpp:1399-1580), slice copies, and the engine end to end.
+#include <cstring>
+#include <thread>
+
 #include "rwkv_inference_engine.hpp"
 #include "test_common.hpp"
 
@@ -35,7 +38,6 @@ HOST_TEST(construction_and_spec_errors) {
   CHECK_THROWS(ModelBackend("/some/model.pth", true), "load model: failed to open file");
   CHECK_THROWS(ModelBackend("synthetic:13B", true), "unknown synthetic model preset");
   CHECK_THROWS(ModelBackend("synthetic:tiny:w9", true), "bad synthetic model option");
-  CHECK_THROWS(ModelBackend("synthetic:tiny", false), "fp32 WKV state only");
   auto b = tiny();
   CHECK_EQ(b->vocab_size(), 2048);
   CHECK_EQ(b->dims().layers, 2);
@@ -172,6 +174,112 @@ HOST_TEST(engine_end_to_end_on_the_real_backend) {
   CHECK_EQ(stats.generated_tokens, 24);
   CHECK_EQ(stats.prompt_tokens, int(tok->encode(p1).size() + tok->encode(p2).size()));
   CHECK(stats.prefill_seconds > 0 && stats.decode_seconds > 0);
+}
+
+// The reference's default constructor arguments (use_wkv32 = false): the WKV state lives in fp16 and the recurrence
+// runs in fp16.  Same graph, so the logits follow the fp32-state backend's to fp16 accuracy; states of the two
+// modes are not interchangeable; slices and the engine work as in the other mode.
+HOST_TEST(default_arguments_give_the_fp16_state_mode) {
+  ModelBackend b16("synthetic:tiny:w8:seed=3");
+  auto b32 = tiny();
+  const auto& d = b16.dims();
+  GenerationState s16 = b16.create_state(2);
+  CHECK(!s16.wkv32);
+  CHECK_EQ(s16.wkv_state.n, std::size_t(d.layers) * 2 * d.heads * 64 * 64);
+  CHECK_EQ(s16.wkv_state32.n, std::size_t(0));
+  for (uint16_t h : host_test::to_host<uint16_t>(s16.wkv_state)) CHECK_EQ(h, uint16_t(0));
+  GenerationState s32 = b32->create_state(2);
+  DeviceLogits l16, l32;
+  CHECK_THROWS(b16.forward_prefill({ramp(4, 1), ramp(4, 2)}, s32, l16), "state wkv precision mismatch");
+  CHECK_THROWS(b32->forward_decode({1, 2}, s16, l32), "state wkv precision mismatch");
+  // 20 tokens in one call (the w12 + w0 sum is rounded to fp16 first) ...
+  b16.forward_prefill({ramp(20, 1), ramp(20, 2)}, s16, l16);
+  b32->forward_prefill({ramp(20, 1), ramp(20, 2)}, s32, l32);
+  CHECK(host_test::to_host<int>(s16.elapsed) == (std::vector<int>{20, 20}));
+  for (int row = 0; row < 2; ++row)
+    CHECK(cosine(host_test::to_host<float>(l16.values), host_test::to_host<float>(l32.values), row * 2048, row * 2048, 2048) > 0.999);
+  // ... then decode steps (w0 added inside the recurrence)
+  for (int step = 0; step < 6; ++step) {
+    b16.forward_decode({int64_t(5 + step), int64_t(900 + step)}, s16, l16);
+    b32->forward_decode({int64_t(5 + step), int64_t(900 + step)}, s32, l32);
+  }
+  CHECK(host_test::to_host<int>(s16.elapsed) == (std::vector<int>{26, 26}));
+  for (int row = 0; row < 2; ++row)
+    CHECK(cosine(host_test::to_host<float>(l16.values), host_test::to_host<float>(l32.values), row * 2048, row * 2048, 2048) > 0.999);
+  bool nonzero = false;
+  for (uint16_t h : host_test::to_host<uint16_t>(s16.wkv_state)) nonzero = nonzero || (h & 0x7fff) != 0;
+  CHECK(nonzero);
+  // slices between fp16 states; refused across modes
+  GenerationState one = b16.create_state(1);
+  b16.copy_state_slice(s16, 1, one, 0, 1);
+  const auto all = host_test::to_host<uint16_t>(s16.wkv_state), part = host_test::to_host<uint16_t>(one.wkv_state);
+  const std::size_t lane = std::size_t(d.heads) * 64 * 64;
+  for (int l = 0; l < d.layers; ++l)
+    for (std::size_t i : {std::size_t(0), lane / 2, lane - 1}) CHECK_EQ(part[l * lane + i], all[(std::size_t(l) * 2 + 1) * lane + i]);
+  GenerationState one32 = b32->create_state(1);
+  CHECK_THROWS(b16.copy_state_slice(s16, 0, one32, 0, 1), "state slice wkv precision mismatch");
+  CHECK(b16.query_prefill_capacity(128).bytes_per_batch < b32->query_prefill_capacity(128).bytes_per_batch);
+}
+
+// Several host threads call forward_* on one backend, each with its own state (the server's request threads do):
+// every thread's logits equal those of the same calls made from one thread, bit for bit.
+HOST_TEST(concurrent_forward_calls_on_distinct_states_match_the_serial_run) {
+  auto b = tiny();
+  constexpr int kThreads = 2, kSteps = 200;
+  auto run = [&](int who, std::vector<float>* last_logits, std::vector<float>* wkv) {
+    GenerationState s = b->create_state(1);
+    DeviceLogits l;
+    b->forward_prefill({ramp(9, 10 + who)}, s, l);
+    int64_t tok = 3 + who;
+    for (int i = 0; i < kSteps; ++i) {
+      b->forward_decode({tok}, s, l);
+      tok = (tok * 31 + 7 + who) % 2048;
+    }
+    *last_logits = host_test::to_host<float>(l.values);
+    *wkv = host_test::to_host<float>(s.wkv_state32);
+  };
+  std::vector<float> serial_l[kThreads], serial_s[kThreads], par_l[kThreads], par_s[kThreads];
+  for (int t = 0; t < kThreads; ++t) run(t, &serial_l[t], &serial_s[t]);
+  std::vector<std::thread> pool;
+  std::vector<std::string> errors(kThreads);
+  for (int t = 0; t < kThreads; ++t)
+    pool.emplace_back([&, t] {
+      try {
+        run(t, &par_l[t], &par_s[t]);
+      } catch (const std::exception& e) {
+        errors[t] = e.what();
+      }
+    });
+  for (auto& th : pool) th.join();
+  for (int t = 0; t < kThreads; ++t) {
+    CHECK(errors[t].empty());
+    CHECK_EQ(par_l[t].size(), serial_l[t].size());
+    CHECK(std::memcmp(par_l[t].data(), serial_l[t].data(), serial_l[t].size() * sizeof(float)) == 0);
+    CHECK(std::memcmp(par_s[t].data(), serial_s[t].data(), serial_s[t].size() * sizeof(float)) == 0);
+  }
+  CHECK(std::memcmp(serial_l[0].data(), serial_l[1].data(), serial_l[0].size() * sizeof(float)) != 0);  // (the two differ)
+}
+
+// One pooled session serves states that alternate (the captured decode graph is keyed by the state's addresses): graph
+// replays agree with themselves run after run and follow each state independently.
+HOST_TEST(alternating_states_on_one_session_keep_apart) {
+  auto b = tiny();
+  GenerationState a = b->create_state(1), c = b->create_state(1), a2 = b->create_state(1), c2 = b->create_state(1);
+  DeviceLogits la, lc, la2, lc2;
+  b->forward_prefill({ramp(5, 1)}, a, la);
+  b->forward_prefill({ramp(5, 2)}, c, lc);
+  b->forward_prefill({ramp(5, 1)}, a2, la2);
+  b->forward_prefill({ramp(5, 2)}, c2, lc2);
+  for (int i = 0; i < 12; ++i) {   // interleaved on the shared session pool ...
+    b->forward_decode({int64_t(40 + i)}, a, la);
+    b->forward_decode({int64_t(80 + i)}, c, lc);
+  }
+  for (int i = 0; i < 12; ++i) b->forward_decode({int64_t(40 + i)}, a2, la2);   // ... equals one after the other
+  for (int i = 0; i < 12; ++i) b->forward_decode({int64_t(80 + i)}, c2, lc2);
+  const auto ha = host_test::to_host<float>(la.values), ha2 = host_test::to_host<float>(la2.values);
+  const auto hc = host_test::to_host<float>(lc.values), hc2 = host_test::to_host<float>(lc2.values);
+  CHECK(std::memcmp(ha.data(), ha2.data(), ha.size() * sizeof(float)) == 0);
+  CHECK(std::memcmp(hc.data(), hc2.data(), hc.size() * sizeof(float)) == 0);
 }
 
 int main(int argc, char** argv) { return host_test::run_all(argc, argv, true); }

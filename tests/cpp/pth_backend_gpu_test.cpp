@@ -99,7 +99,14 @@ HOST_TEST(weight_format_suffix_quantises_on_load) {
 
 HOST_TEST(load_errors) {
   CHECK_THROWS(ModelBackend("/definitely/missing.pth", true), "load model: failed to open file");
-  CHECK_THROWS(ModelBackend(checkpoint(), false), "fp32 WKV state only");
+  {
+    ModelBackend fp16_state(checkpoint());   // the reference's default arguments: fp16 WKV state
+    GenerationState st = fp16_state.create_state(1);
+    CHECK(!st.wkv32);
+    DeviceLogits lg;
+    fp16_state.forward_prefill({{1, 2, 3, 4, 5}}, st, lg);
+    for (float f : host_test::to_host<float>(lg.values)) CHECK(std::isfinite(f));
+  }
   const std::string junk = "/tmp/rwkv_pth_backend_junk_" + std::to_string(::getpid()) + ".pth";
   {
     std::ofstream f(junk, std::ios::binary);

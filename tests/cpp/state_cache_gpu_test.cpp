@@ -2,8 +2,10 @@
 // reload from the database, delete (reference: test/state_cache_test.cpp:67-99), for both state precisions,
 // plus persistence across shutdown.  Usage: <exe> <repo root> [database path]
 #include <cstdio>
+#include <cstring>
 #include <unistd.h>
 
+#include "rwkv_server_backend.hpp"
 #include "rwkv_state_cache.hpp"
 #include "test_common.hpp"
 
@@ -142,6 +144,56 @@ HOST_TEST(overwriting_a_session_replaces_it_at_every_level) {
   expect_same(*cache.get_state("a"), a2);
   cache.shutdown();
   std::remove(g_db_path.c_str());
+}
+
+// A real generation state of each precision (the fp16-state backend is the reference's default) goes through the
+// device, host and database levels and resumes bit for bit: the restored copy continues exactly like the original.
+HOST_TEST(real_backend_states_resume_bitwise_from_every_level) {
+  for (bool wkv32 : {false, true}) {
+    ModelBackend backend("synthetic:tiny:w8:seed=5", wkv32);
+    auto& cache = StateCacheManager::instance();
+    std::remove(g_db_path.c_str());
+    cache.initialize(1, 1, g_db_path);
+    GenerationState live = backend.create_state(1);
+    DeviceLogits logits;
+    backend.forward_prefill({{5, 6, 7, 8, 9, 10, 11}}, live, logits);
+    cache.put_state("live", live);
+    // push it down: one more session -> host level, another -> database
+    auto filler1 = make_state(wkv32, 1, {1}, {1.0f}, {1});
+    auto filler2 = make_state(wkv32, 1, {2}, {2.0f}, {2});
+    auto filler3 = make_state(wkv32, 1, {3}, {3.0f}, {3});
+    std::vector<std::vector<float>> want;
+    for (int step = 0; step < 3; ++step) {
+      backend.forward_decode({int64_t(100 + step)}, live, logits);
+      want.push_back(host_test::to_host<float>(logits.values));
+    }
+    for (int level = 0; level < 3; ++level) {
+      if (level == 1) cache.put_state("filler-1", filler1);
+      if (level == 2) {   // (the host-level hit above brought it back to the device level: two more sessions push it out)
+        cache.put_state("filler-2", filler2);
+        cache.put_state("filler-3", filler3);
+      }
+      const auto summary = cache.list_all_states();
+      if (level == 1) CHECK(contains(summary.l2_cache, std::string("live")));
+      if (level == 2) CHECK(contains(summary.database, std::string("live")));
+      auto restored = cache.get_state("live");
+      CHECK(restored.has_value());
+      CHECK_EQ(restored->wkv32, wkv32);
+      CHECK(host_test::to_host<int>(restored->elapsed) == std::vector<int>{7});
+      DeviceLogits again;
+      for (int step = 0; step < 3; ++step) {
+        backend.forward_decode({int64_t(100 + step)}, *restored, again);
+        const auto got = host_test::to_host<float>(again.values);
+        CHECK(std::memcmp(got.data(), want[step].data(), got.size() * sizeof(float)) == 0);
+      }
+      if (level == 0) {
+        // get_state handed out a copy: the cached entry is still the state after the prompt
+        CHECK(host_test::to_host<int>(cache.get_state("live")->elapsed) == std::vector<int>{7});
+      }
+    }
+    cache.shutdown();
+    std::remove(g_db_path.c_str());
+  }
 }
 
 int main(int argc, char** argv) {

@@ -34,6 +34,14 @@ def lib():
         L.orc_f32_to_f16.restype = ctypes.c_uint16
         L.orc_f32_to_f16.argtypes = [ctypes.c_float]
         L.orc_model_create.restype = ctypes.c_void_p
+        L.orc_f64_to_f16.restype = ctypes.c_uint16
+        L.orc_f64_to_f16.argtypes = [ctypes.c_double]
+        L.orc_f16_fma.restype = ctypes.c_uint16
+        L.orc_f16_fma.argtypes = [ctypes.c_uint16, ctypes.c_uint16, ctypes.c_uint16]
+        L.orc_wkv16_rotator.restype = ctypes.c_float
+        L.orc_wkv16_rotator.argtypes = [ctypes.c_int32]
+        L.orc_wkv16_w_delta.restype = ctypes.c_uint16
+        L.orc_wkv16_w_delta.argtypes = [ctypes.c_uint16, ctypes.c_void_p, ctypes.c_int, ctypes.c_int32]
         L.orc_sample_greedy_penalty.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float,
                                                 ctypes.c_float, ctypes.c_float, ctypes.c_float]
         L.orc_sample_filter.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_int,
@@ -101,6 +109,19 @@ def wkv7(state, r, w, k, v, a, b, H, w_mode=0):
         y = np.empty((B, T, C), np.float32)
         fn = lib().orc_wkv7_f32
     fn(B, T, C, H, w_mode, _p(state), *[_p(t) for t in args], _p(y))
+    return y
+
+
+def wkv7_f16state(state, r, w, k, v, a, b, H, elapsed, w0=None):
+    """state f16 [B,H,64,64] (updated in place); r..b f16 [B,T,C]; w raw decay logits; w0 f16 [C] or None;
+    elapsed int32 [B] (not modified).  Returns y f16 [B,T,C]."""
+    B, T, C = r.shape
+    assert state.dtype == np.float16 and state.flags.c_contiguous
+    args = [_c(t, np.float16) for t in (r, w, k, v, a, b)]
+    w0c = None if w0 is None else _c(w0, np.float16)
+    y = np.empty((B, T, C), np.float16)
+    lib().orc_wkv7_f16state(B, T, C, H, _p(state), _p(args[0]), _p(args[1]), _p(w0c), _p(args[2]), _p(args[3]),
+                            _p(args[4]), _p(args[5]), _p(y), _p(_c(elapsed, np.int32)))
     return y
 
 
@@ -338,10 +359,10 @@ class Model:
                 else:
                     set_m(l, name, arr)
 
-    def new_state(self, B):
+    def new_state(self, B, wkv_fp16=False):
         d = self.dims
-        return (np.zeros((d.L, 2, B, d.C), np.float16), np.zeros((d.L, B, d.H, 64, 64), np.float32),
-                np.zeros((B,), np.int32))
+        return (np.zeros((d.L, 2, B, d.C), np.float16),
+                np.zeros((d.L, B, d.H, 64, 64), np.float16 if wkv_fp16 else np.float32), np.zeros((B,), np.int32))
 
     def forward(self, tokens, state, trace=False):
         tokens = _c(tokens, np.int64)
@@ -349,7 +370,8 @@ class Model:
         shift, wkv, elapsed = state
         logits = np.empty((B, self.dims.V), np.float32)
         tr = np.empty((self.dims.L, B * T, self.dims.C), np.float16) if trace else None
-        rc = lib().orc_model_forward(self.h, _p(tokens), B, T, _p(shift), _p(wkv), _p(elapsed), _p(logits), _p(tr))
+        fn = lib().orc_model_forward_f16state if wkv.dtype == np.float16 else lib().orc_model_forward
+        rc = fn(self.h, _p(tokens), B, T, _p(shift), _p(wkv), _p(elapsed), _p(logits), _p(tr))
         if rc != 0:
             raise ValueError("orc_model_forward failed: %d" % rc)
         return (logits, tr) if trace else logits

@@ -74,6 +74,67 @@ def test_wkv7_drift_over_16384_tokens_against_the_fp32_oracle(gpu, orc):
     assert y_all <= F16_TOL
 
 
+@pytest.mark.parametrize("B,T,H,with_w0", [(1, 64, 12, False), (2, 7, 3, True), (3, 1, 2, True), (5, 33, 2, False)])
+def test_wkv7_f16state_matches_oracle(gpu, orc, B, T, H, with_w0):
+    """The fp16-state recurrence (the reference server's default mode) against the oracle's restatement of
+    cuda/rwkv7_wkv_fp16_v2.cu: same fp16 fused multiply-adds in the same order, so outputs and state agree
+    bit for bit except where the decay delta rounds differently (v_exp_f32 against the host's exp2f, one fp16 ulp
+    of d - 1 in a few channels): at most 2e-3 of the tensors' scale, and most elements identical."""
+    hip = gpu
+    C = H * 64
+    inp = wkv_inputs(B, T, H, seed=300 + B + T, dtype=np.float16)
+    names = ["r", "w_raw", "k", "v", "a", "b"]
+    rng = np.random.default_rng(B * T)
+    w0 = (rng.standard_normal(C) * 0.3).astype(np.float16) if with_w0 else None
+    elapsed = rng.integers(0, 5000, B).astype(np.int32)
+    s0 = (rng.standard_normal((B, H, 64, 64)) * 0.2).astype(np.float16)     # a state that is already in use
+    s_ref = s0.copy()
+    y_ref = orc.wkv7_f16state(s_ref, *[inp[n] for n in names], H, elapsed, w0=w0)
+    state = dev(hip, s0)
+    y = hip.DeviceArray((B, T, C), np.float16)
+    d = {n: dev(hip, inp[n]) for n in names}
+    hip.wkv7_f16state(B, T, C, H, state, d["r"], d["w_raw"], d["k"], d["v"], d["a"], d["b"], y, dev(hip, elapsed),
+                      w0=None if w0 is None else dev(hip, w0))
+    hip.device_sync()
+    got_y, got_s = y.numpy(), state.numpy()
+    err = rel_err(got_y.astype(np.float32), y_ref.astype(np.float32))
+    assert err <= F16_TOL
+    err = rel_err(got_s.astype(np.float32), s_ref.astype(np.float32))
+    assert err <= F16_TOL
+    same = float(np.mean(got_s.view(np.uint16) == s_ref.view(np.uint16)))
+    assert same >= 0.9, same
+    assert elapsed.tolist() == elapsed.tolist()   # elapsed is read only
+
+
+def test_wkv7_f16state_call_split_is_bitwise(gpu):
+    hip = gpu
+    B, T, H, T1 = 2, 29, 4, 11
+    C = H * 64
+    inp = wkv_inputs(B, T, H, seed=9, dtype=np.float16)
+    names = ["r", "w_raw", "k", "v", "a", "b"]
+    w0 = dev(hip, (np.random.default_rng(1).standard_normal(C) * 0.3).astype(np.float16))
+    elapsed = np.array([3, 77], np.int32)
+    state = hip.DeviceArray.zeros((B, H, 64, 64), np.float16)
+    y = hip.DeviceArray((B, T, C), np.float16)
+    d = {n: dev(hip, inp[n]) for n in names}
+    hip.wkv7_f16state(B, T, C, H, state, *[d[n] for n in names], y, dev(hip, elapsed), w0=w0)
+    hip.device_sync()
+    state2 = hip.DeviceArray.zeros((B, H, 64, 64), np.float16)
+    y2 = np.zeros((B, T, C), np.float16)
+    for t0, tn in ((0, T1), (T1, T - T1)):
+        part = {n: dev(hip, np.ascontiguousarray(inp[n][:, t0:t0 + tn])) for n in names}
+        yp = hip.DeviceArray((B, tn, C), np.float16)
+        hip.wkv7_f16state(B, tn, C, H, state2, *[part[n] for n in names], yp, dev(hip, elapsed + t0), w0=w0)
+        hip.device_sync()
+        y2[:, t0:t0 + tn] = yp.numpy()
+    same = np.array_equal(state2.numpy().view(np.uint16), state.numpy().view(np.uint16))
+    assert same
+    same = np.array_equal(y2.view(np.uint16), y.numpy().view(np.uint16))
+    assert same
+    with pytest.raises(hip.RwkvHipError, match="H\\*64"):
+        hip.wkv7_f16state(1, 1, 100, 1, state, d["r"], d["w_raw"], d["k"], d["v"], d["a"], d["b"], y, dev(hip, elapsed))
+
+
 def test_wkv7_f16_io_and_t_split_bitwise(gpu, orc):
     hip = gpu
     B, T, H = 2, 40, 4

@@ -280,6 +280,57 @@ def test_greedy_stream_matches_oracle(gpu, orc):
     sess.close()
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_fp16_state_mode_prefill_and_decode_match_oracle(gpu, orc, fmt):
+    """The reference server's default mode: the WKV state in fp16 and the recurrence in fp16 fused multiply-adds
+    (session option; ModelBackend's use_wkv32 == false).  A 20-token prefill call (the w12 + w0 sum rounded to fp16
+    first), a 9-token call and decode steps (w0 added inside the recurrence, unrounded) against the oracle's
+    restatement of the same graph: logits cosine >= 0.9995, greedy tokens equal except for ties, the fp16 state
+    within 2e-2 of its scale (both sides round the same quantities to fp16, from activations that differ by fp16
+    ulps)."""
+    from rwkv_lightning_cuda_amd.model import Session, State
+    hip = gpu
+    dims = small_dims()
+    omodel, gmodel = build_pair(gpu, orc, dims, fmt, seed=61)
+    B = 2
+    rng = np.random.default_rng(17)
+    sess = Session(gmodel)
+    gstate = State(dims, B, wkv_fp16=True)
+    glogits = hip.DeviceArray((B, dims.V), np.float32)
+    ostate = omodel.new_state(B, wkv_fp16=True)
+    for T in (20, 9):
+        tokens = rng.integers(0, dims.V, (B, T))
+        sess.forward(tokens, gstate, glogits)
+        ologits = omodel.forward(tokens, ostate)
+        cos = cosine(glogits.numpy(), ologits)
+        assert cos >= 0.9995, "prefill call of %d tokens" % T
+    ties = 0
+    nxt = np.argmax(ologits, axis=1).reshape(B, 1)
+    for step in range(24):
+        sess.set_graph(step % 5 != 3)     # graph replay and eager launches
+        sess.forward(nxt, gstate, glogits)
+        ologits = omodel.forward(nxt, ostate)
+        g = glogits.numpy()
+        for b_ in range(B):
+            cos = cosine(g[b_], ologits[b_])
+            assert cos >= 0.9995, "step %d row %d" % (step, b_)
+            w_, g_ = int(np.argmax(ologits[b_])), int(np.argmax(g[b_]))
+            if w_ != g_:
+                tie_or_fail(ologits[b_], w_, g_, "step %d row %d" % (step, b_))
+                ties += 1
+        nxt = np.argmax(ologits, axis=1).reshape(B, 1)
+    assert ties <= 2
+    assert gstate.wkv.numpy().dtype == np.float16
+    err = rel_err(gstate.wkv.numpy().astype(np.float32), ostate[1].astype(np.float32))
+    print("fp16-state mode: state within %.2e of the oracle's after %d tokens, %d ties" % (err, 29 + 24, ties))
+    assert err <= 2e-2
+    assert gstate.elapsed.numpy().tolist() == [29 + 24] * B
+    # the device-side greedy loop works in this mode too
+    got = sess.decode_greedy(np.array([3, 4]), 4, gstate, glogits)
+    assert got.shape == (4, B)
+    sess.close()
+
+
 def test_forward_argument_errors(gpu, orc):
     from rwkv_lightning_cuda_amd.model import HipModel, Session, State, synth_weights
     hip = gpu

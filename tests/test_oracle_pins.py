@@ -524,3 +524,154 @@ def test_emb_ln0_against_float64_and_invariants():
     # a constant row has no variance: the output is the bias
     const = to_bf16(np.full((2, C), 3.0))
     assert np.array_equal(orc.emb_ln0(const, w, b), np.broadcast_to(_bf16_bits_to_f32(b).astype(np.float16), (2, C)))
+
+
+# ------------------------------------------------------------------------------- WKV7 with an fp16 state
+from conftest import rel_err
+
+
+def _f16(x):
+    return np.asarray(x, np.float16)
+
+
+def _bits(h):
+    return int(np.asarray(h, np.float16).view(np.uint16))
+
+
+def test_f64_to_f16_rounds_like_numpy_and_fma_rounds_once():
+    """double -> fp16 against numpy's own correctly rounded conversion (normals, subnormals, ties, overflow), and
+    the fp16 fma against exact rational arithmetic: a*b+c evaluated in Fractions and rounded once - including
+    cases where rounding the product first would give another result."""
+    from fractions import Fraction
+    L = orc.lib()
+    rng = np.random.default_rng(1)
+    xs = np.concatenate([
+        rng.standard_normal(20000) * np.exp(rng.uniform(-20, 12, 20000)),
+        np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, -1e9, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001,
+                  2.0 ** -14, 2.0 ** -14 - 2.0 ** -25, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 1.0 + 2.0 ** -11 + 2.0 ** -40]),
+    ])
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).view(np.uint16)
+    got = np.array([L.orc_f64_to_f16(float(x)) for x in xs], np.uint16)
+    assert np.array_equal(got, want)
+
+    def exact_round(fr):
+        # nearest fp16 to an exact rational (ties to even), by searching numpy's float16 neighbours
+        approx = np.float16(float(fr))
+        cands = {approx, np.nextafter(approx, np.float16(np.inf)), np.nextafter(approx, np.float16(-np.inf))}
+        best = None
+        for c in cands:
+            if not np.isfinite(c):
+                continue
+            d = abs(Fraction(float(c)) - fr)
+            key = (d, int(np.float16(c).view(np.uint16)) & 1)
+            if best is None or key < best[0]:
+                best = (key, c)
+        return best[1]
+
+    halfs = rng.standard_normal((3000, 3)).astype(np.float16)
+    halfs[:200] = (rng.standard_normal((200, 3)) * 2.0 ** rng.integers(-12, 8, (200, 3))).astype(np.float16)
+    # a case where f16(a*b) + c differs from fma(a, b, c): a*b = 1 + 2^-10 + 2^-20, c = -1
+    extra = np.array([[1.0 + 2.0 ** -10, 1.0, -1.0], [1.0009765625, 1.0009765625, -1.0], [0.333251953125, 3.0, -1.0]], np.float16)
+    for a, b, c in np.concatenate([halfs, extra]):
+        fr = Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c))
+        want_h = exact_round(fr)
+        got_h = np.uint16(L.orc_f16_fma(_bits(a), _bits(b), _bits(c))).view(np.float16)
+        assert got_h == want_h or (got_h == 0 and want_h == 0), (a, b, c, got_h, want_h)
+
+
+def test_wkv16_dither_known_values_range_and_zero_mean():
+    """rotator1(x) = 2^-41 * int32(2654435769 * x) (cuda/rwkv7_wkv_fp16_v2.cu:19-21,41-43): known values from integer
+    arithmetic, |value| < 2^-10 (below fp16 resolution of d - 1 near -0), mean ~ 0 over consecutive phases; and what
+    it is for: the fp16 decay delta averaged over consecutive phases approaches the unrounded d - 1 far closer
+    than one fp16 rounding does."""
+    L = orc.lib()
+    assert L.orc_wkv16_rotator(0) == 0.0
+    for x in (1, 2, 3, 1000, 123456789):
+        prod = (2654435769 * x) & 0xffffffff
+        sp = prod - (1 << 32) if prod >= (1 << 31) else prod
+        assert L.orc_wkv16_rotator(x) == np.float32(4.547473508864641e-13) * np.float32(sp)
+    vals = np.array([L.orc_wkv16_rotator(x) for x in range(1, 20001)])
+    assert np.abs(vals).max() < 2.0 ** -10
+    assert abs(vals.mean()) < 2e-6
+    for w in (-3.0, -0.5, 1.0, 2.5):
+        wh = np.float16(w)
+        true = np.exp(-np.exp(-0.5) / (1.0 + np.exp(-np.float64(wh)))) - 1.0
+        deltas = np.array([np.uint16(L.orc_wkv16_w_delta(_bits(wh), None, 0, ph)).view(np.float16)
+                           for ph in range(4096)], np.float64)
+        assert abs(deltas.mean() - true) < 2e-5                         # dithered: unbiased
+        assert np.abs(deltas - true).max() <= 2.0 ** -10 + 2.0 ** -11   # each within dither + one rounding
+    # w0 is added unrounded: f16(w + w0) would differ here
+    w_raw, w0 = np.float16(0.7001953125), np.array([np.float16(0.00030517578125)], np.float16)
+    d_sum = np.uint16(L.orc_wkv16_w_delta(_bits(w_raw), w0.ctypes.data_as(__import__("ctypes").c_void_p), 0, 0)).view(np.float16)
+    true = np.exp(-np.exp(-0.5) / (1.0 + np.exp(-(np.float64(w_raw) + np.float64(w0[0]))))) - 1.0
+    assert abs(np.float64(d_sum) - true) <= 2.0 ** -12
+
+
+def test_wkv7_f16state_one_step_closed_forms_and_orientation():
+    """From an empty state one token leaves S[i][j] = f16(k[j] * v[i]) (sa = 0, so the decay and b do not enter),
+    and y[i] = the fp16 dot of that row with r in the reference's order; with r = e_j the output reads column j of
+    the NEW state exactly.  A second token with a = b = 0 multiplies by the decay: S' = fma(S, wd, fma(k, v, S))."""
+    rng = np.random.default_rng(3)
+    H, C = 2, 128
+    k = _f16(rng.standard_normal((1, 1, C)))
+    v = _f16(rng.standard_normal((1, 1, C)))
+    w = _f16(rng.uniform(-4, 2, (1, 1, C)))
+    a = _f16(rng.standard_normal((1, 1, C)) * 0.1)
+    b = _f16(rng.standard_normal((1, 1, C)) * 0.1)
+    elapsed = np.array([5], np.int32)
+    for j in (0, 1, 37, 63):
+        r = np.zeros((1, 1, C), np.float16)
+        r[0, 0, j] = 1.0
+        r[0, 0, 64 + j] = 1.0
+        S = np.zeros((1, H, 64, 64), np.float16)
+        y = orc.wkv7_f16state(S, r, w, k, v, a, b, H, elapsed)
+        for h in range(H):
+            kv = (k[0, 0, h * 64:(h + 1) * 64].astype(np.float32)[None, :] * v[0, 0, h * 64:(h + 1) * 64].astype(np.float32)[:, None]).astype(np.float16)
+            assert np.array_equal(S[0, h].view(np.uint16), kv.view(np.uint16))      # row i = value index, column j = key index
+            assert np.array_equal(y[0, 0, h * 64:(h + 1) * 64].view(np.uint16), S[0, h][:, j].copy().view(np.uint16))
+    # second token, a = b = 0: pure decay + outer product, every element one fp16 fma chain
+    S = np.zeros((1, H, 64, 64), np.float16)
+    zeros = np.zeros((1, 1, C), np.float16)
+    r = _f16(rng.standard_normal((1, 1, C)))
+    orc.wkv7_f16state(S, r, w, k, v, zeros, zeros, H, elapsed)
+    S1 = S.copy()
+    k2 = _f16(rng.standard_normal((1, 1, C)))
+    v2 = _f16(rng.standard_normal((1, 1, C)))
+    elapsed2 = np.array([6], np.int32)
+    orc.wkv7_f16state(S, r, w, k2, v2, zeros, zeros, H, elapsed2)
+    L = orc.lib()
+    for h in range(H):
+        for i in (0, 13, 63):
+            for j in (0, 22, 63):
+                c = h * 64 + j
+                wd = np.uint16(L.orc_wkv16_w_delta(_bits(w[0, 0, c]), None, c, 6 + c)).view(np.float16)
+                s = np.float64(S1[0, h, i, j])
+                mid = np.float16(np.float64(k2[0, 0, c]) * np.float64(v2[0, 0, h * 64 + i]) + s)   # exact in float64
+                want = np.float16(s * np.float64(wd) + np.float64(mid))
+                assert S[0, h, i, j] == want, (h, i, j)
+
+
+def test_wkv7_f16state_call_split_invariance_and_agreement_with_the_fp32_state():
+    """Running T1 + T2 tokens in one call or in two (elapsed advanced by T1 in between) is bitwise the same; and on
+    config-0 style inputs the fp16-state recurrence follows the fp32-state oracle (itself pinned by float64 brute
+    force) to fp16 accuracy: outputs within 1.5e-2 of their scale over 48 tokens."""
+    B, T, H = 2, 48, 3
+    C = H * 64
+    inp = wkv_inputs(B, T, H, seed=21, dtype=np.float16)
+    names = ["r", "w_raw", "k", "v", "a", "b"]
+    elapsed = np.array([7, 1000], np.int32)
+    S = np.zeros((B, H, 64, 64), np.float16)
+    y = orc.wkv7_f16state(S, *[inp[n] for n in names], H, elapsed)
+    S2 = np.zeros((B, H, 64, 64), np.float16)
+    T1 = 17
+    ya = orc.wkv7_f16state(S2, *[np.ascontiguousarray(inp[n][:, :T1]) for n in names], H, elapsed)
+    yb = orc.wkv7_f16state(S2, *[np.ascontiguousarray(inp[n][:, T1:]) for n in names], H, elapsed + T1)
+    assert np.array_equal(S.view(np.uint16), S2.view(np.uint16))
+    assert np.array_equal(np.concatenate([ya, yb], axis=1).view(np.uint16), y.view(np.uint16))
+    S32 = np.zeros((B, H, 64, 64), np.float32)
+    y32 = orc.wkv7(S32, *[inp[n] for n in names], H, 0)
+    err = rel_err(y.astype(np.float32), y32.astype(np.float32))
+    assert err <= 1.5e-2, err
+    err = rel_err(S.astype(np.float32), S32)
+    assert err <= 1.5e-2, err
