@@ -23,6 +23,13 @@ struct SamplerPenaltyState {
 // (src/rwkv_sampler.cpp:14-19); any other value makes the token stream reproducible.
 SamplerPenaltyState make_sampler_penalties(int vocab_size, int batch_size = 1, std::uint64_t seed = 0);
 
+// Streams: the sampling kernels run on the device's NULL stream and the token ids come back with a blocking copy,
+// so the call returns with the ids on the host.  ModelBackend's forward calls run on per-session non-blocking
+// streams and return only after their stream has drained, so logits handed from a forward call to the sampler on the
+// same thread are complete, and the NULL stream never waits for another thread's forward.  Sampling calls of several
+// threads queue behind one another on the NULL stream (each works on its own SamplerPenaltyState, so the results do
+// not depend on the order); logits written by work still in flight on a stream of the caller's own must be
+// synchronised by the caller first.
 int sample_repetition_temperature_topk_topp(const DeviceLogits& logits, SamplerPenaltyState& penalties,
                                             const GenerateOptions& options);
 

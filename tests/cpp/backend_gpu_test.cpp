@@ -4,6 +4,7 @@
 #include <thread>
 
 #include "rwkv_inference_engine.hpp"
+#include "rwkv_prefill_admission.hpp"
 #include "test_common.hpp"
 
 using namespace rwkv7_server;
@@ -138,6 +139,39 @@ HOST_TEST(prefill_capacity_is_consistent) {
   const auto cap2 = b->query_prefill_capacity(256);
   CHECK(cap2.bytes_per_batch > cap.bytes_per_batch);
   CHECK_THROWS(b->query_prefill_capacity(0), "prefill chunk size must be positive");
+}
+
+// The admission queue over the real backend, bound as the reference's API layer binds it
+// (src/rwkv_api_service.cpp:808-811: the provider asks the backend for the capacity at the engine's chunk size).
+// A permit sized to the batch brackets a prefill; the hard limit is the start-up capacity.
+HOST_TEST(prefill_admission_over_the_backend_capacity) {
+  auto b = tiny();
+  const int chunk = 128;
+  PrefillAdmissionController ctl([b, chunk] { return b->query_prefill_capacity(chunk); });
+  const auto start = ctl.snapshot(false);
+  CHECK(start.hard_max_batch_size >= 64);  // a tiny model on an empty 288 GB device
+  CHECK_EQ(start.hard_max_batch_size, start.dynamic_max_batch_size);
+  CHECK_EQ(start.capacity.bytes_per_batch, b->query_prefill_capacity(chunk).bytes_per_batch);
+  {
+    auto permit = ctl.acquire(8, "/v1/chat/completions");
+    CHECK(permit.has_value());
+    GenerationState s = b->create_state(8);
+    DeviceLogits l;
+    std::vector<std::vector<int64_t>> ids;
+    for (int i = 0; i < 8; ++i) ids.push_back(ramp(16, 5 + i));
+    b->forward_prefill(ids, s, l);
+    CHECK_EQ(l.rows, 8);
+    CHECK_EQ(ctl.snapshot(true).reserved_batch_size, 8);
+  }
+  CHECK_EQ(ctl.snapshot(true).reserved_batch_size, 0);
+  bool threw = false;
+  try {
+    (void)ctl.acquire(start.hard_max_batch_size + 1, "too wide");
+  } catch (const PrefillBatchLimitExceeded& e) {
+    threw = true;
+    CHECK_EQ(e.max_batch_size(), start.hard_max_batch_size);
+  }
+  CHECK(threw);
 }
 
 HOST_TEST(engine_end_to_end_on_the_real_backend) {

@@ -161,3 +161,140 @@ HOST_TEST(engine_argument_errors) {
 }
 
 int main(int argc, char** argv) { return host_test::run_all(argc, argv, false); }
+
+// ---- prefill admission (scenario of the reference's test/prefill_admission_test.cpp, plus ordering and ownership) ----
+#include <atomic>
+#include <chrono>
+#include <future>
+#include <thread>
+
+#include "rwkv_prefill_admission.hpp"
+
+namespace {
+
+struct FakeCapacity {
+  std::atomic<int> lanes{4};
+  std::atomic<int> asked{0};
+  PrefillAdmissionController::CapacityProvider provider() {
+    return [this] {
+      ++asked;
+      PrefillCapacity c;
+      c.max_batch_size = lanes.load();
+      c.bytes_per_batch = 1024;
+      c.free_vram_bytes = 4096;
+      c.total_vram_bytes = 8192;
+      return c;
+    };
+  }
+};
+
+template <class F>
+bool still_waiting(std::future<F>& f, int ms = 250) {
+  return f.wait_for(std::chrono::milliseconds(ms)) == std::future_status::timeout;
+}
+
+}  // namespace
+
+HOST_TEST(admission_waits_for_lanes_and_follows_the_capacity) {
+  FakeCapacity cap;
+  PrefillAdmissionController ctl(cap.provider());
+  auto first = ctl.acquire(3, "first");
+  CHECK(first.has_value() && bool(*first));
+  CHECK_EQ(first->batch_size(), 3);
+  cap.lanes = 3;  // memory got tighter: 3 of 3 lanes are now taken
+  auto waiter = std::async(std::launch::async, [&] { return ctl.acquire(1, "second"); });
+  CHECK(still_waiting(waiter));
+  auto snap = ctl.snapshot(true);
+  CHECK_EQ(snap.hard_max_batch_size, 4);
+  CHECK_EQ(snap.dynamic_max_batch_size, 3);
+  CHECK_EQ(snap.reserved_batch_size, 3);
+  CHECK_EQ(snap.queued_requests, std::size_t(1));
+  CHECK_EQ(snap.capacity.bytes_per_batch, std::size_t(1024));
+  first->release();
+  CHECK(!bool(*first));
+  auto second = waiter.get();
+  CHECK(second.has_value());
+  CHECK_EQ(second->batch_size(), 1);
+  CHECK_EQ(ctl.snapshot(false).reserved_batch_size, 1);
+  second->release();
+  second->release();  // releasing twice gives nothing back twice
+  CHECK_EQ(ctl.snapshot(false).reserved_batch_size, 0);
+  CHECK(cap.asked.load() >= 4);  // constructor, head-of-queue checks, release
+}
+
+HOST_TEST(admission_rejects_what_can_never_fit) {
+  FakeCapacity cap;
+  PrefillAdmissionController ctl(cap.provider());
+  cap.lanes = 16;  // more memory later does not raise the limit fixed at start-up
+  bool threw = false;
+  try {
+    (void)ctl.acquire(5, "wide");
+  } catch (const PrefillBatchLimitExceeded& e) {
+    threw = true;
+    CHECK_EQ(e.request_batch_size(), 5);
+    CHECK_EQ(e.max_batch_size(), 4);
+    CHECK_EQ(std::string(e.what()), std::string("bsz overflow, Max bsz=4"));
+  }
+  CHECK(threw);
+  CHECK_EQ(ctl.snapshot(true).dynamic_max_batch_size, 4);
+  CHECK_EQ(ctl.snapshot(false).queued_requests, std::size_t(0));
+  auto one = ctl.acquire(0, "zero counts as one");
+  CHECK(one.has_value());
+  CHECK_EQ(one->batch_size(), 1);
+  CHECK_THROWS(PrefillAdmissionController(PrefillAdmissionController::CapacityProvider{}), "capacity provider");
+}
+
+HOST_TEST(admission_cancelled_waiter_leaves_the_queue) {
+  FakeCapacity cap;
+  PrefillAdmissionController ctl(cap.provider());
+  auto all = ctl.acquire(4, "all");
+  CHECK(all.has_value());
+  std::atomic<bool> cancel{false};
+  auto waiter = std::async(std::launch::async, [&] { return ctl.acquire(1, "gives up", [&] { return cancel.load(); }); });
+  CHECK(still_waiting(waiter));
+  CHECK_EQ(ctl.snapshot(false).queued_requests, std::size_t(1));
+  cancel = true;
+  auto none = waiter.get();
+  CHECK(!none.has_value());
+  CHECK_EQ(ctl.snapshot(false).queued_requests, std::size_t(0));
+  CHECK_EQ(ctl.snapshot(false).reserved_batch_size, 4);
+}
+
+HOST_TEST(admission_is_first_come_first_served) {
+  FakeCapacity cap;
+  PrefillAdmissionController ctl(cap.provider());
+  auto held = ctl.acquire(2, "held");
+  CHECK(held.has_value());
+  // a 3-lane request queues first; the 1-lane request behind it would fit at once but must not overtake
+  auto wide = std::async(std::launch::async, [&] { return ctl.acquire(3, "wide"); });
+  while (ctl.snapshot(false).queued_requests < 1) std::this_thread::yield();
+  auto narrow = std::async(std::launch::async, [&] { return ctl.acquire(1, "narrow"); });
+  while (ctl.snapshot(false).queued_requests < 2) std::this_thread::yield();
+  CHECK(still_waiting(wide));
+  CHECK(still_waiting(narrow, 50));
+  held->release();
+  auto w = wide.get();
+  CHECK(w.has_value());
+  auto n = narrow.get();  // 3 + 1 fit together once the wide one is in
+  CHECK(n.has_value());
+  CHECK(w->ticket() < n->ticket());
+  CHECK_EQ(ctl.snapshot(false).reserved_batch_size, 4);
+}
+
+HOST_TEST(admission_permit_owns_its_lanes) {
+  FakeCapacity cap;
+  PrefillAdmissionController ctl(cap.provider());
+  {
+    auto p = ctl.acquire(2, "scoped");
+    CHECK(p.has_value());
+    PrefillAdmissionController::Permit moved(std::move(*p));
+    CHECK(!bool(*p) && bool(moved));
+    CHECK_EQ(ctl.snapshot(false).reserved_batch_size, 2);
+    auto q = ctl.acquire(1, "other");
+    CHECK(q.has_value());
+    moved = std::move(*q);  // assignment gives the 2 lanes back and takes over the 1
+    CHECK_EQ(ctl.snapshot(false).reserved_batch_size, 1);
+    CHECK_EQ(moved.batch_size(), 1);
+  }
+  CHECK_EQ(ctl.snapshot(false).reserved_batch_size, 0);  // destructors released the rest
+}

@@ -37,6 +37,7 @@ def test_host_cpu():
     out = _run("host_cpu_test")
     assert "ok   tokenizer_round_trips" in out
     assert "ok   prompt_templates" in out
+    assert "ok   admission_is_first_come_first_served" in out
 
 
 def test_host_library_exports_the_api():
@@ -55,6 +56,8 @@ def test_host_library_exports_the_api():
                    "rwkv7_server::StateCacheManager::put_state(",
                    "rwkv7_server::StateCacheManager::get_state(",
                    "rwkv7_server::StateCacheManager::delete_state_from_any_level(",
+                   "rwkv7_server::PrefillAdmissionController::acquire(",
+                   "rwkv7_server::PrefillAdmissionController::snapshot(",
                    "rwkv7_server::ModelBackend::forward_prefill(",
                    "rwkv7_server::ModelBackend::forward_decode(",
                    "rwkv7_server::ModelBackend::copy_state_slice(",
