@@ -61,6 +61,16 @@ class InferenceEngine {
   const std::string& model_name() const { return model_name_; }
   int prefill_chunk_size() const { return prefill_chunk_size_; }
 
+  // Continuous batching that shrinks (no counterpart in the reference, which keeps every finished row in the
+  // batch and feeds it a stop token until the last row ends, src/rwkv_inference_engine.cpp:497-499).  When on,
+  // batch_generate and batch_generate_stream gather the rows that are still generating into a narrower state
+  // once at most half of the current width is left, so a batch with one long answer does not pay for the
+  // finished ones.  Off by default: the reference's behaviour.  A row's greedy output is the same either way up
+  // to the rounding differences between the kernels of different batch widths; stochastic draws are keyed by
+  // the row's position in the batch, so they change when rows move.
+  void set_shrink_batch(bool on) { shrink_batch_ = on; }
+  bool shrink_batch() const { return shrink_batch_; }
+
  private:
   std::vector<int64_t> encode_prompt(const std::string& prompt) const;
   std::vector<std::vector<int64_t>> encode_prompts_sorted(const std::vector<std::string>& prompts,
@@ -75,6 +85,7 @@ class InferenceEngine {
   std::shared_ptr<TrieTokenizer> tokenizer_;
   std::string model_name_;
   int prefill_chunk_size_ = 128;
+  bool shrink_batch_ = false;
 };
 
 }  // namespace rwkv7_server

@@ -294,6 +294,50 @@ std::string InferenceEngine::generate_one(const std::string& prompt, GenerationS
   return text;
 }
 
+namespace {
+
+// Gathers the slots listed in `keep` (ascending) to the front of a state, a sampler state and a feed vector of
+// width keep.size(); `rows` maps a slot to its prompt.  Runs of neighbouring slots move with one slice copy.
+void gather_live_slots(const IModelBackend& model, const std::vector<int>& keep, GenerationState& state,
+                       SamplerPenaltyState& penalties, std::vector<size_t>& rows, std::vector<int64_t>& feed) {
+  const int width = static_cast<int>(keep.size());
+  GenerationState narrow = model.create_state(width);
+  SamplerPenaltyState narrow_penalties = make_sampler_penalties(penalties.vocab_size, width, penalties.seed);
+  narrow_penalties.step = penalties.step;
+  const std::size_t row_bytes = static_cast<std::size_t>(penalties.vocab_size) * sizeof(float);
+  for (int to = 0; to < width;) {
+    int run = 1;
+    while (to + run < width && keep[to + run] == keep[to] + run) ++run;
+    model.copy_state_slice(state, keep[to], narrow, to, run);
+    rwkv7_fast_v4::check_hip(
+        rwkv_hip_memcpy_d2d(narrow_penalties.penalties.p + static_cast<std::size_t>(to) * penalties.vocab_size,
+                            penalties.penalties.p + static_cast<std::size_t>(keep[to]) * penalties.vocab_size,
+                            run * row_bytes),
+        "gather sampler penalties");
+    to += run;
+  }
+  std::vector<size_t> new_rows(width);
+  std::vector<int64_t> new_feed(width);
+  for (int to = 0; to < width; ++to) {
+    new_rows[to] = rows[keep[to]];
+    new_feed[to] = feed[keep[to]];
+  }
+  state = std::move(narrow);
+  penalties = std::move(narrow_penalties);
+  rows.swap(new_rows);
+  feed.swap(new_feed);
+}
+
+// slots of the current width whose prompt has not finished
+std::vector<int> live_slots(const std::vector<size_t>& rows, const std::vector<char>& finished) {
+  std::vector<int> keep;
+  for (size_t slot = 0; slot < rows.size(); ++slot)
+    if (!finished[rows[slot]]) keep.push_back(static_cast<int>(slot));
+  return keep;
+}
+
+}  // namespace
+
 std::vector<std::string> InferenceEngine::batch_generate(const std::vector<std::string>& prompts,
                                                          const GenerateOptions& options) const {
   if (prompts.empty()) return {};
@@ -309,24 +353,29 @@ std::vector<std::string> InferenceEngine::batch_generate(const std::vector<std::
   const int64_t filler = options.stop_tokens.empty() ? 0 : options.stop_tokens.front();
   SamplerPenaltyState penalties = make_sampler_penalties(model_->vocab_size(), batch);
   std::vector<std::string> text(prompts.size());
-  std::vector<char> finished(prompts.size(), 0);
+  std::vector<char> finished(prompts.size(), 0);  // by prompt (sorted order)
   std::vector<int64_t> feed(prompts.size(), filler);
+  std::vector<size_t> rows(prompts.size());       // slot of the current batch -> prompt
+  std::iota(rows.begin(), rows.end(), size_t(0));
   int active = batch;
 
   for (int step = 0; step < options.max_tokens && active > 0; ++step) {
     const std::vector<int> sampled = sample_rows(logits, penalties, options, step);
-    for (size_t i = 0; i < sampled.size(); ++i) {
-      feed[i] = filler;
+    for (size_t slot = 0; slot < sampled.size(); ++slot) {
+      const size_t i = rows[slot];
+      feed[slot] = filler;
       if (finished[i]) continue;
-      if (is_stop_token(options, sampled[i])) {
+      if (is_stop_token(options, sampled[slot])) {
         finished[i] = 1;
         --active;
         continue;
       }
-      feed[i] = sampled[i];
-      text[i] += tokenizer_->decode(sampled[i]);
+      feed[slot] = sampled[slot];
+      text[i] += tokenizer_->decode(sampled[slot]);
     }
     if (active == 0) break;
+    if (shrink_batch_ && 2 * active <= static_cast<int>(rows.size()))
+      gather_live_slots(*model_, live_slots(rows, finished), state, penalties, rows, feed);
     model_->forward_decode(feed, state, logits);
   }
 
@@ -374,8 +423,10 @@ InferenceEngine::GenerationStats InferenceEngine::batch_generate_stream(
 
   const int64_t filler = options.stop_tokens.empty() ? 0 : options.stop_tokens.front();
   SamplerPenaltyState penalties = make_sampler_penalties(model_->vocab_size(), batch);
-  std::vector<char> finished(prompts.size(), 0);
+  std::vector<char> finished(prompts.size(), 0);  // by prompt (sorted order), as are the streams
   std::vector<int64_t> feed(prompts.size(), filler);
+  std::vector<size_t> rows(prompts.size());       // slot of the current batch -> prompt
+  std::iota(rows.begin(), rows.end(), size_t(0));
   std::vector<TokenStream> streams(prompts.size(), TokenStream(*tokenizer_, chunk_size));
   int active = batch;
   const auto decode_t0 = Clock::now();
@@ -394,10 +445,11 @@ InferenceEngine::GenerationStats InferenceEngine::batch_generate_stream(
       break;
     }
     const std::vector<int> sampled = sample_rows(logits, penalties, options, step);
-    for (size_t i = 0; i < sampled.size(); ++i) {
-      feed[i] = filler;
+    for (size_t slot = 0; slot < sampled.size(); ++slot) {
+      const size_t i = rows[slot];
+      feed[slot] = filler;
       if (finished[i]) continue;
-      if (is_stop_token(options, sampled[i])) {
+      if (is_stop_token(options, sampled[slot])) {
         finished[i] = 1;
         stats.stop_token = true;
         --active;
@@ -405,10 +457,12 @@ InferenceEngine::GenerationStats InferenceEngine::batch_generate_stream(
         continue;
       }
       ++stats.generated_tokens;
-      feed[i] = sampled[i];
-      if (!deliver(i, streams[i].add(sampled[i]))) return stats;
+      feed[slot] = sampled[slot];
+      if (!deliver(i, streams[i].add(sampled[slot]))) return stats;
     }
     if (active == 0) break;
+    if (shrink_batch_ && 2 * active <= static_cast<int>(rows.size()))
+      gather_live_slots(*model_, live_slots(rows, finished), state, penalties, rows, feed);
     model_->forward_decode(feed, state, logits);
   }
 

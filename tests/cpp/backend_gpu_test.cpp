@@ -1,5 +1,6 @@
 // ModelBackend over the kernel library (synthetic tiny model): state and logits shapes, argument errors with
 // the reference's messages (src/rwkv_server_backend.cpp:1399-1580), slice copies, and the engine end to end.
+#include <algorithm>
 #include <cstring>
 #include <thread>
 
@@ -208,6 +209,69 @@ HOST_TEST(engine_end_to_end_on_the_real_backend) {
   CHECK_EQ(stats.generated_tokens, 24);
   CHECK_EQ(stats.prompt_tokens, int(tok->encode(p1).size() + tok->encode(p2).size()));
   CHECK(stats.prefill_seconds > 0 && stats.decode_seconds > 0);
+}
+
+// The shrinking batch on the real backend: two of four prompts stop at their first token, so the engine gathers the
+// other two (not neighbours in the sorted batch) into a batch of two; their greedy texts are those of the run that
+// keeps all four rows.
+HOST_TEST(shrinking_batch_continues_the_gathered_rows) {
+  auto b = tiny();
+  auto tok = std::make_shared<TrieTokenizer>();
+  CHECK_EQ(tok->load(host_test::vocab_path()), kTokenizerSuccess);
+  InferenceEngine engine(b, tok, "tiny", 128);
+  const std::string first = "System: the longest prompt of the four, so it is row 0\n\nUser: hi\n\nAssistant:";
+  const std::string third = "User: hello there\n\nAssistant: the";
+  // greedy token ids of one prompt, decoded alone
+  auto greedy_ids = [&](const std::string& prompt, int steps) {
+    GenerationState s = b->create_state(1);
+    DeviceLogits l;
+    engine.prefill_prompt(prompt, s, l);
+    std::vector<int> ids;
+    for (int i = 0; i < steps; ++i) {
+      const auto row = host_test::to_host<float>(l.values);
+      ids.push_back(int(std::max_element(row.begin(), row.end()) - row.begin()));
+      b->forward_decode({int64_t(ids.back())}, s, l);
+    }
+    return ids;
+  };
+  // a prompt whose first greedy token - the stop token of this test - the two long-running rows never produce
+  std::vector<int> seen = greedy_ids(first, 24);
+  const auto more = greedy_ids(third, 24);
+  seen.insert(seen.end(), more.begin(), more.end());
+  std::string stopper;
+  int stop = -1;
+  for (const char* candidate : {"User: a question that ends at once\n\nAssistant:", "User: 12345\n\nAssistant:", "zzz",
+                                "User: \xE4\xBD\xA0\xE5\xA5\xBD\n\nAssistant:", "Q", "System: stop here"}) {
+    const int t = greedy_ids(candidate, 1).front();
+    if (std::find(seen.begin(), seen.end(), t) == seen.end()) {
+      stopper = candidate;
+      stop = t;
+      break;
+    }
+  }
+  CHECK(stop >= 0);
+  GenerateOptions o;
+  o.max_tokens = 24;
+  o.stop_tokens = {stop};
+  o.top_k = 0;
+  o.top_p = 0.0;
+  o.alpha_presence = 0.0;
+  o.alpha_frequency = 0.0;
+  const std::vector<std::string> prompts{first, stopper, third, stopper};
+  const auto keep = engine.batch_generate(prompts, o);
+  engine.set_shrink_batch(true);
+  const auto shrunk = engine.batch_generate(prompts, o);
+  CHECK_EQ(keep.size(), std::size_t(4));
+  CHECK(keep[1].empty() && keep[3].empty());
+  CHECK(!keep[0].empty() && !keep[2].empty());
+  CHECK(shrunk == keep);
+  std::vector<std::string> streamed(4);
+  const auto stats = engine.batch_generate_stream(prompts, o, 1, [&](int i, const std::string& piece) {
+    streamed[std::size_t(i)] += piece;
+    return true;
+  });
+  CHECK(stats.stop_token);
+  CHECK(streamed[1].empty() && streamed[3].empty());
 }
 
 // The reference's default constructor arguments (use_wkv32 = false): the WKV state lives in fp16 and the recurrence

@@ -182,6 +182,47 @@ HOST_TEST(two_prompt_batch_prefills_width_2_then_1) {
   for (const auto& step : backend->decodes) CHECK_EQ(step.size(), std::size_t(2));
 }
 
+// With set_shrink_batch(true) the rows that are still generating are gathered into a narrower batch once at most
+// half are left; the texts are those of the batch that never shrinks (the reference's behaviour, the default).
+HOST_TEST(batch_shrinks_when_half_of_the_rows_have_finished) {
+  auto tok = tokenizer();
+  const auto answer_ids = tok->encode(kAnswer);
+  const std::vector<int> short_ids(answer_ids.begin(), answer_ids.begin() + 2);
+  const std::string short_text = tok->decode(short_ids);
+  const auto options = greedy_options(int(answer_ids.size()) + 1);
+  // row 0 (the longest prompt) answers kAnswer, every other row stops after two tokens
+  const std::vector<std::string> prompts{kPrompt, kPrompt + "\nlonger than the others", kPrompt + " b", kPrompt + " c"};
+  for (const bool streaming : {false, true}) {
+    for (const bool shrink : {false, true}) {
+      auto backend = answer_backend(answer_ids, "shrink");
+      backend->set_script_for_other_rows(ScriptedBackend::script_for(short_ids, kVocab));
+      InferenceEngine engine(backend, tok, "shrink");
+      CHECK(!engine.shrink_batch());
+      engine.set_shrink_batch(shrink);
+      std::vector<std::string> out(prompts.size());
+      if (streaming) {
+        const auto stats = engine.batch_generate_stream(
+            prompts, options, 1, [&](int i, const std::string& piece) { out[std::size_t(i)] += piece; return true; });
+        CHECK_EQ(stats.generated_tokens, int(answer_ids.size()) + 3 * 2);
+      } else {
+        out = engine.batch_generate(prompts, options);
+      }
+      CHECK_EQ(out[1], kAnswer);  // the caller's index of the longest prompt
+      CHECK_EQ(out[0], short_text);
+      CHECK_EQ(out[2], short_text);
+      CHECK_EQ(out[3], short_text);
+      CHECK_EQ(backend->decodes.size(), answer_ids.size());
+      // steps 0 and 1 feed all four rows; at step 2 three rows stop, and from then on the batch is one row wide
+      // (or stays at four rows fed the stop token)
+      for (std::size_t step = 0; step < backend->decodes.size(); ++step) {
+        const std::size_t expect = (shrink && step >= 2) ? 1 : 4;
+        CHECK_EQ(backend->decodes[step].size(), expect);
+      }
+      if (shrink) CHECK_EQ(backend->decodes.back()[0], int64_t(answer_ids.back()));
+    }
+  }
+}
+
 HOST_TEST(streaming_routes_chunks_to_the_callers_prompt_index) {
   auto tok = tokenizer();
   const auto answer_ids = tok->encode(kAnswer);
