@@ -561,6 +561,20 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   uint4_t xq = {0u, 0u, 0u, 0u};
   if constexpr (LN) {
     lnq = ln_row1_request(args.ln, prob.mu, K);
+  } else if (prob.x_f32 != nullptr) {
+    // x = f16(x_f32 * gate): the products are formed here, one rounding each
+    if (static_cast<int>(threadIdx.x) * 8 < K) {
+      const float4_t f0 = *reinterpret_cast<const float4_t*>(prob.x_f32 + threadIdx.x * 8);
+      const float4_t f1 = *reinterpret_cast<const float4_t*>(prob.x_f32 + threadIdx.x * 8 + 4);
+      const half8_t gq = *reinterpret_cast<const half8_t*>(prob.x_gate + threadIdx.x * 8);
+      half8_t xh;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        xh[e] = f2h(f0[e] * h2f(gq[e]));
+        xh[4 + e] = f2h(f1[e] * h2f(gq[4 + e]));
+      }
+      xq = __builtin_bit_cast(uint4_t, xh);
+    }
   } else {
     if (static_cast<int>(threadIdx.x) * 8 < K) xq = *reinterpret_cast<const uint4_t*>(prob.x + threadIdx.x * 8);
   }
@@ -753,7 +767,7 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
     RWKV_REQUIRE(K > 0 && K % elems == 0, "linear: K (%d) must be a multiple of %d for this weight format", K, elems);
     if (p.fmt == RWKV_FMT_W4) RWKV_REQUIRE(K % 128 == 0, "linear: W4 needs K %% 128 == 0 (K = %d)", K);
     RWKV_REQUIRE(p.N > 0 && p.N % 4 == 0, "linear: N (%d) must be a positive multiple of 4", p.N);
-    RWKV_REQUIRE(p.w && p.y && (p.x || (ln && ln->mode != 0 && p.mu)), "linear: NULL tensor");
+    RWKV_REQUIRE(p.w && p.y && (p.x || p.x_f32 || (ln && ln->mode != 0 && p.mu)), "linear: NULL tensor");
     RWKV_REQUIRE(p.fmt == RWKV_FMT_F16 || p.scale, "linear: quantised weights need a scale tensor");
     RWKV_REQUIRE(p.fmt != RWKV_FMT_W4 || p.zp, "linear: W4 weights need a zero-point tensor");
     args.p[i] = p;
@@ -780,10 +794,17 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
     RWKV_REQUIRE(copy->src && copy->dst && copy->n % 8 == 0, "linear: bad row copy");
     args.copy = *copy;
   }
+  bool gated = false;
+  for (int i = 0; i < n_problems; ++i) {
+    if (problems[i].x_f32 == nullptr) continue;
+    gated = true;
+    RWKV_REQUIRE(problems[i].x_gate != nullptr && K % 8 == 0, "linear: a gated x needs its gate and K %% 8 == 0");
+  }
   if (M == 1) {
     const int df = row1_format(args);
-    if (df >= 0) return launch_row1_any(st, args, df);
+    if (df >= 0 && !(gated && args.ln.mode != 0)) return launch_row1_any(st, args, df);
   }
+  RWKV_REQUIRE(!gated, "linear: x = x_f32 * gate is formed by one-row launches only (M = %d, K = %d)", M, K);
   switch (M) {
     case 1: return launch_one<1, 2, 1>(st, args);
     case 2: return launch_one<2, 2, 1>(st, args);

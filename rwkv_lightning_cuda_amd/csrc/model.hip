@@ -349,6 +349,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   // (the shift row that the prologue leaves for later is stored by the single-launch time-mix core)
   const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace && fused_tmix &&
                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
+  // One row: the gate rank-out of the time-mix core (more than half of its bytes) runs in blocks of its own and the
+  // output projection's launch applies the gate while it stages x.
+  const bool gate_split = fused_tmix && rows == 1 && C <= 4096 && !s->trace;
 
   // Decode steps of a few rows (one by default) read, per row, only the ffn.value rows whose relu^2 activation is
   // non-zero (int8 or fp16 weights).
@@ -479,6 +482,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       if (ln_in_linear) {
         p.shift_src = b.xx; p.shift_dst = shift0;
       }
+      if (gate_split) {  // the g rank-out in blocks of its own; the output projection applies the gate
+        p.y2_pre = b.r32; p.gate_out = b.g;
+      }
       TRY_AUX(tmix_step_launch(st, p));
     } else {
       // LoRA rank-out (+ activation, + v-residual gate)
@@ -543,7 +549,15 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
     // ffn.value sum the split-K partials themselves instead of a reduce launch; att / cm then stay unwritten.
     const bool defer_ok = !s->trace && !ln_in_linear;
     DeferredReduce att_partial;
-    TRY_PROF(apply_matrix(s, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att, defer_ok ? &att_partial : nullptr));
+    if (gate_split) {
+      const Matrix& mo = w.m[RWKV_M_ATT_O];
+      LinearProblem po = {mo.data, mo.scale, mo.zp, nullptr, b.att, C, mo.fmt, nullptr};
+      po.x_f32 = b.r32;
+      po.x_gate = b.g;
+      TRY_PROF(linear_small_m(st, 1, C, 1, &po, RWKV_EPI_NONE, 0));
+    } else {
+      TRY_PROF(apply_matrix(s, w.m[RWKV_M_ATT_O], rows, C, C, b.y2, RWKV_EPI_NONE, 0, b.att, defer_ok ? &att_partial : nullptr));
+    }
 
     // residual add + LN2 + channel-mix token shift
     if (ln_in_linear) {

@@ -17,6 +17,10 @@ struct LinearProblem {
   int N;
   int fmt;           // RWKV_FMT_*
   const half_t* mu;  // with a LayerNorm prologue: this problem's token-shift lerp coefficients [K]
+  // One-row launches without a LayerNorm prologue only: x = f16(x_f32 * x_gate) is formed while the block stages x
+  // (the gate of the time-mix output, whose rank-out runs beside the heads' blocks instead of inside them).
+  const float* x_f32 = nullptr;
+  const half_t* x_gate = nullptr;
 };
 
 // LayerNorm + token-shift prologue of a small-M linear launch (decode steps): every block recomputes, for each
@@ -234,6 +238,11 @@ struct TmixStepArgs {
   half_t* v_first_out;                      // [B,C], written when hv == NULL (layer 0), may be NULL
   float* state;                             // [B,H,64,64], updated in place
   half_t* y2;                               // [B,C] input of the output projection
+  // Split mode (gate_out != NULL): the g rank-out - more than half of the launch's bytes - runs in B*H further
+  // blocks that write the gate to gate_out [B,C]; the heads' blocks write the ungated output in fp32 to y2_pre
+  // [B,C] instead of y2, and the consumer forms f16(y2_pre * gate) (the same product, rounded once).
+  float* y2_pre;
+  half_t* gate_out;
   const half_t* shift_src;                  // [B,C] LN output kept by the r/k/v launch's prologue, or NULL
   half_t* shift_dst;                        // [B,C] time-mix shift row of the state that receives it
 };
