@@ -45,10 +45,24 @@ __global__ __launch_bounds__(NT) void ln_fused_kernel(LnArgs a) {
   for (int i = 0; i < kLnMaxVec; ++i) {
     const int c = (i * kLnThreads + threadIdx.x) * 8;
     if (c < C) {
+      // the parameter vectors first: the sum over split-K partials below waits for its loads, and loads return in
+      // issue order, so anything requested after that loop would cost a second trip to memory
+      wv[i] = *reinterpret_cast<const half8_t*>(a.w + c);
+      bv[i] = *reinterpret_cast<const half8_t*>(a.b + c);
+      if constexpr (kMix) {
+        pv[i] = *reinterpret_cast<const half8_t*>(a.shift + dst + c);
+        // (no branch per coefficient vector: the unused ones re-read the last one, which costs nothing, whereas a
+        // load under a branch is followed by a wait for everything requested so far)
+#pragma unroll
+        for (int s = 0; s < 6; ++s) mv[i][s] = *reinterpret_cast<const half8_t*>(a.mu[s < a.n_mix ? s : a.n_mix - 1] + c);
+      }
       const half8_t xv = *reinterpret_cast<const half8_t*>(a.x + xsrc + c);
+      __builtin_amdgcn_sched_barrier(0);
       half8_t rv = {};
       if constexpr (MODE != kLn && MODE != kLnMix) {
         if (a.res_partial) {
+          // (the scale vector before the partials, for the same reason; without one any valid vector is read)
+          const half8_t sv8 = *reinterpret_cast<const half8_t*>((a.res_scale ? a.res_scale : a.w) + c);
           const float* pp = a.res_partial + src + c;
           float4_t s0 = *reinterpret_cast<const float4_t*>(pp);
           float4_t s1 = *reinterpret_cast<const float4_t*>(pp + 4);
@@ -59,12 +73,7 @@ __global__ __launch_bounds__(NT) void ln_fused_kernel(LnArgs a) {
           }
           float scl[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) scl[e] = 1.0f;
-          if (a.res_scale) {
-            const half8_t sv8 = *reinterpret_cast<const half8_t*>(a.res_scale + c);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) scl[e] = h2f(sv8[e]);
-          }
+          for (int e = 0; e < 8; ++e) scl[e] = a.res_scale ? h2f(sv8[e]) : 1.0f;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             rv[e] = f2h(mul_f32(s0[e], scl[e]));
@@ -73,14 +82,6 @@ __global__ __launch_bounds__(NT) void ln_fused_kernel(LnArgs a) {
         } else {
           rv = *reinterpret_cast<const half8_t*>(a.res + src + c);
         }
-      }
-      wv[i] = *reinterpret_cast<const half8_t*>(a.w + c);
-      bv[i] = *reinterpret_cast<const half8_t*>(a.b + c);
-      if constexpr (kMix) {
-        pv[i] = *reinterpret_cast<const half8_t*>(a.shift + dst + c);
-#pragma unroll
-        for (int s = 0; s < 6; ++s)
-          if (s < a.n_mix) mv[i][s] = *reinterpret_cast<const half8_t*>(a.mu[s] + c);
       }
       if constexpr (MODE == kLn || MODE == kLnMix) {
 #pragma unroll
