@@ -532,6 +532,112 @@ __device__ __forceinline__ void ln_row1_finish(const LnRow1& q, const LnPrologue
   *reinterpret_cast<half4_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
 }
 
+// The same prologue by the first half of the block's wavefronts, eight values per thread, while the second half is
+// already waiting for its weights (gemv_row1_block); the second half passes the two barriers of the block sums.
+struct LnRow1x8 {
+  half8_t xv, rv, wv, bv, pv, mv;
+};
+
+__device__ __forceinline__ LnRow1x8 ln_row1_request8(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
+  const int c = threadIdx.x * 8;
+  const int cc = c < K ? c : 0;
+  const int64_t xsrc = ln.mode == 2 ? ln.tokens[0] * static_cast<int64_t>(K) : 0;
+  LnRow1x8 q;
+  q.xv = *reinterpret_cast<const half8_t*>(ln.x + xsrc + cc);
+  q.rv = *reinterpret_cast<const half8_t*>(ln.mode == 1 ? ln.res + cc : ln.x + xsrc + cc);
+  q.wv = *reinterpret_cast<const half8_t*>(ln.w + cc);
+  q.bv = *reinterpret_cast<const half8_t*>(ln.b + cc);
+  q.pv = *reinterpret_cast<const half8_t*>(ln.shift + cc);
+  q.mv = *reinterpret_cast<const half8_t*>(mu + cc);
+  return q;
+}
+
+// sum over the first NWL wavefronts of the block (the callers); the other wavefronts pass the barrier too
+template <int NWL>
+__device__ __forceinline__ float front_waves_sum(float v, int wave, float* scratch) {
+  v = wave_sum_uniform(v);
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NWL; ++i) t += scratch[i];
+  return t;
+}
+
+// stash: NT * 4 floats (the row sum), then 4 x NT * 4 fp16 values, as in ln_row1_finish
+template <int NT>
+__device__ __forceinline__ void ln_row1_finish8(const LnRow1x8& q, const LnPrologue& ln, int K, half_t* xs, float* stash,
+                                                float* red, bool store, int wave) {
+  constexpr int NWL = NT / 128;  // wavefronts that compute
+  const int c = threadIdx.x * 8;
+  const bool in = c < K;
+  float* vbuf = stash + c;
+  half_t* hbuf = reinterpret_cast<half_t*>(stash + NT * 4) + c;
+  float sum = 0.0f;
+  {
+    float v[8];
+    if (ln.mode == 1) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[e]) + h2f(q.rv[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[e]);
+    }
+    if (in) sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    *reinterpret_cast<float4_t*>(vbuf) = float4_t{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<float4_t*>(vbuf + 4) = float4_t{v[4], v[5], v[6], v[7]};
+    *reinterpret_cast<half8_t*>(hbuf) = q.wv;
+    *reinterpret_cast<half8_t*>(hbuf + NT * 4) = q.bv;
+    *reinterpret_cast<half8_t*>(hbuf + NT * 8) = q.pv;
+    *reinterpret_cast<half8_t*>(hbuf + NT * 12) = q.mv;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  sum = front_waves_sum<NWL>(sum, wave, red);
+  const float mean = sum / static_cast<float>(K);
+  float sv = 0.0f;
+  if (in) {
+    const float4_t v0 = *reinterpret_cast<const float4_t*>(vbuf);
+    const float4_t v1 = *reinterpret_cast<const float4_t*>(vbuf + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float d = v0[e] - mean;
+      sv = fmaf(d, d, sv);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float d = v1[e] - mean;
+      sv = fmaf(d, d, sv);
+    }
+  }
+  sv = front_waves_sum<NWL>(sv, wave, red + NT / 64);
+  const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
+  half8_t ov;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ov[e] = static_cast<half_t>(0.0f);
+  if (in) {
+    const float4_t v0 = *reinterpret_cast<const float4_t*>(vbuf);
+    const float4_t v1 = *reinterpret_cast<const float4_t*>(vbuf + 4);
+    const half8_t wv = *reinterpret_cast<const half8_t*>(hbuf);
+    const half8_t bv = *reinterpret_cast<const half8_t*>(hbuf + NT * 4);
+    const half8_t pv = *reinterpret_cast<const half8_t*>(hbuf + NT * 8);
+    const half8_t mv = *reinterpret_cast<const half8_t*>(hbuf + NT * 12);
+    half8_t yv, xo;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float ve = e < 4 ? v0[e & 3] : v1[e & 3];
+      yv[e] = f2h(fmaf((ve - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
+      const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
+      ov[e] = f2h(fmaf(h2f(pv[e]) - yf, h2f(mv[e]), yf));
+      xo[e] = f2h(ve);
+    }
+    if (store) {
+      *reinterpret_cast<half8_t*>(ln.ln_out + c) = yv;
+      if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + c) = xo;
+    }
+  }
+  *reinterpret_cast<half8_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
+}
+
 // One block.  With the prologue, it runs BEFORE the weight requests: a wavefront stalls on its weight requests until
 // the memory pipeline has room for them - late in a 67 MB launch that takes microseconds (timestamps: the last
 // wavefronts get their requests out 11 us after the launch began) - and it cannot run the prologue while it is
@@ -557,10 +663,12 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   const int64_t row_bytes = T::byte_off(K);
   const unsigned char* wbase = static_cast<const unsigned char*>(prob.w) + static_cast<int64_t>(active ? row0 : 0) * row_bytes;
 
-  LnRow1 lnq = {};
+  // With the prologue: the first half of the wavefronts computes it (eight values per thread) and requests its
+  // weights afterwards; the second half requests its weights at once, so that HBM streams while the prologue runs.
+  const bool ln_wave = LN && wave < NW / 2;
   uint4_t xq = {0u, 0u, 0u, 0u};
   if constexpr (LN) {
-    lnq = ln_row1_request(args.ln, prob.mu, K);
+    // (below, after the row scales)
   } else if (prob.x_f32 != nullptr) {
     // x = f16(x_f32 * gate): the products are formed here, one rounding each
     if (static_cast<int>(threadIdx.x) * 8 < K) {
@@ -608,13 +716,28 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   };
   // x in LDS: one slice per thread, zeros beyond K
   if constexpr (LN) {
-    ln_row1_finish<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0);
+    // two code paths, so that the prologue's operands and the weight vectors never hold registers together; the
+    // second path passes the two barriers of the first one's block sums
+    if (ln_wave) {
+      const LnRow1x8 lnq = ln_row1_request8(args.ln, prob.mu, K);
+      __builtin_amdgcn_sched_barrier(0);
+      ln_row1_finish8<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0, wave);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int st = 0; st < S; ++st) request(st);
+    } else {
+#pragma unroll
+      for (int st = 0; st < S; ++st) request(st);
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      __syncthreads();
+    }
   } else {
     *reinterpret_cast<uint4_t*>(xs + threadIdx.x * 8) = xq;
-  }
-  __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int st = 0; st < S; ++st) request(st);
+    for (int st = 0; st < S; ++st) request(st);
+  }
   __builtin_amdgcn_sched_barrier(0);
   __syncthreads();
   if (!active) return;
