@@ -428,10 +428,10 @@ static int launch_one(hipStream_t st, LinearArgs& args) {
 // beyond its bytes is the trip to memory at its start and the one at its end.  Here a wavefront requests ALL the
 // 16-byte vectors of its rows (R = 2 rows of int8 / int4 codes, one row of fp16) in one go - K <= 4096 int8 codes
 // are 4 vectors per lane and row - so every byte of the matrix is requested by the first instructions of its block
-// and nothing is requested late.  With the LayerNorm prologue (LN) the block first computes its own copy of
+// and nothing is requested late.  With the LayerNorm prologue (LN) the block computes its own copy of
 // LayerNorm(x + residual) + token-shift lerp into LDS (same formulas and rounding points as ln_fused_kernel,
-// fused_ops.hip; four values per thread, so the sums associate differently and the last bits may differ from
-// that kernel's): the stand-alone LayerNorm launch and its kernel boundary disappear.  Every block of the launch
+// fused_ops.hip; eight or sixteen values per thread, so the sums associate differently and the last bits may
+// differ from that kernel's): the stand-alone LayerNorm launch and its kernel boundary disappear.  Every block of the launch
 // is resident at once (two 1024-thread blocks per CU: at most 64 registers per thread, checked at build time).
 // Accumulation order per lane is that of linear_gemv_kernel (steps in order, then the same butterfly): same bits.
 template <int FMT, int KCAP>
@@ -441,114 +441,33 @@ struct Row1Cfg {
 };
 
 // LayerNorm(x + res) (or of a gathered table row) + lerp against the previous token's LN output into xs[0..K), by
-// the NT threads of the block, four values each; block 0 also stores the residual sum and the LN output.
-// In two parts: everything the prologue reads from memory is requested at once (ln_row1_request, six reads in
-// flight together), the arithmetic (ln_row1_finish) reads no memory.
-struct LnRow1 {
-  half4_t xv, rv, wv, bv, pv, mv;
+// the first half (int4 weights: quarter) of the block's wavefronts while the others are already waiting for their
+// weights (gemv_row1_block); block 0 also stores the residual sum and the LN output.  In two parts: everything
+// the prologue reads from memory is requested at once (ln_row1_request8), the arithmetic (ln_row1_finish8) reads
+// no memory.  Everything that arrived goes to LDS at once (stash: NT * 4 floats for the row sum, then 4 x NT * 4
+// fp16 values: LN weight, bias, previous LN output, lerp coefficients) and is read back piece by piece, each
+// thread only what it wrote, so the prologue's registers stay few.
+template <int V8>
+struct LnRow1xV {  // V8 groups of eight values
+  half8_t xv[V8], rv[V8], wv[V8], bv[V8], pv[V8], mv[V8];
 };
 
-__device__ __forceinline__ LnRow1 ln_row1_request(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
-  const int c = threadIdx.x * 4;
-  const int cc = c < K ? c : 0;
+// thread t of the computing wavefronts owns the groups t, t + NTL, ... (NTL computing threads)
+template <int V8, int NTL>
+__device__ __forceinline__ LnRow1xV<V8> ln_row1_request8(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
   const int64_t xsrc = ln.mode == 2 ? ln.tokens[0] * static_cast<int64_t>(K) : 0;
-  LnRow1 q;
-  q.xv = *reinterpret_cast<const half4_t*>(ln.x + xsrc + cc);
-  // unconditional (without a residual the row is read twice): a conditional read would wait for the first one
-  q.rv = *reinterpret_cast<const half4_t*>(ln.mode == 1 ? ln.res + cc : ln.x + xsrc + cc);
-  q.wv = *reinterpret_cast<const half4_t*>(ln.w + cc);
-  q.bv = *reinterpret_cast<const half4_t*>(ln.b + cc);
-  q.pv = *reinterpret_cast<const half4_t*>(ln.shift + cc);
-  q.mv = *reinterpret_cast<const half4_t*>(mu + cc);
-  return q;
-}
-
-// stash: NT * 4 floats (the row sum) followed by 4 x NT * 4 fp16 values (LN weight, bias, previous LN output, lerp
-// coefficients).  Everything that arrived from memory goes to LDS at once and is read back piece by piece (each
-// thread only what it wrote, so no barrier), which keeps the prologue's registers few: the 32 registers of the
-// weight vectors are all but the block's whole budget.
-template <int NT>
-__device__ __forceinline__ void ln_row1_finish(const LnRow1& q, const LnPrologue& ln, int K, half_t* xs, float* stash,
-                                               float* red, bool store) {
-  const int c = threadIdx.x * 4;
-  const bool in = c < K;
-  float* vbuf = stash + c;
-  half_t* hbuf = reinterpret_cast<half_t*>(stash + NT * 4) + c;
-  float sum = 0.0f;
-  {
-    float4_t v;
-    if (ln.mode == 1) {
+  LnRow1xV<V8> q;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = h2f(q.xv[e]) + h2f(q.rv[e]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = h2f(q.xv[e]);
-    }
-    if (in) sum = (v[0] + v[1]) + (v[2] + v[3]);
-    *reinterpret_cast<float4_t*>(vbuf) = v;
-    *reinterpret_cast<half4_t*>(hbuf) = q.wv;
-    *reinterpret_cast<half4_t*>(hbuf + NT * 4) = q.bv;
-    *reinterpret_cast<half4_t*>(hbuf + NT * 8) = q.pv;
-    *reinterpret_cast<half4_t*>(hbuf + NT * 12) = q.mv;
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
+    const int cc = c < K ? c : 0;
+    q.xv[g] = *reinterpret_cast<const half8_t*>(ln.x + xsrc + cc);
+    q.rv[g] = *reinterpret_cast<const half8_t*>(ln.mode == 1 ? ln.res + cc : ln.x + xsrc + cc);
+    q.wv[g] = *reinterpret_cast<const half8_t*>(ln.w + cc);
+    q.bv[g] = *reinterpret_cast<const half8_t*>(ln.b + cc);
+    q.pv[g] = *reinterpret_cast<const half8_t*>(ln.shift + cc);
+    q.mv[g] = *reinterpret_cast<const half8_t*>(mu + cc);
   }
-  __builtin_amdgcn_sched_barrier(0);
-  sum = block_sum_uniform<NT / 64>(sum, red);
-  const float mean = sum / static_cast<float>(K);
-  float sv = 0.0f;
-  if (in) {
-    const float4_t v = *reinterpret_cast<const float4_t*>(vbuf);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float d = v[e] - mean;
-      sv = fmaf(d, d, sv);
-    }
-  }
-  sv = block_sum_uniform<NT / 64>(sv, red + NT / 64);
-  const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
-  half4_t ov = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
-  if (in) {
-    const float4_t v = *reinterpret_cast<const float4_t*>(vbuf);
-    const half4_t wv = *reinterpret_cast<const half4_t*>(hbuf);
-    const half4_t bv = *reinterpret_cast<const half4_t*>(hbuf + NT * 4);
-    const half4_t pv = *reinterpret_cast<const half4_t*>(hbuf + NT * 8);
-    const half4_t mv = *reinterpret_cast<const half4_t*>(hbuf + NT * 12);
-    half4_t yv;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      yv[e] = f2h(fmaf((v[e] - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
-      const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
-      ov[e] = f2h(fmaf(h2f(pv[e]) - yf, h2f(mv[e]), yf));
-    }
-    if (store) {
-      *reinterpret_cast<half4_t*>(ln.ln_out + c) = yv;
-      if (ln.x_out) {
-        half4_t xo;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) xo[e] = f2h(v[e]);
-        *reinterpret_cast<half4_t*>(ln.x_out + c) = xo;
-      }
-    }
-  }
-  *reinterpret_cast<half4_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
-}
-
-// The same prologue by the first half of the block's wavefronts, eight values per thread, while the second half is
-// already waiting for its weights (gemv_row1_block); the second half passes the two barriers of the block sums.
-struct LnRow1x8 {
-  half8_t xv, rv, wv, bv, pv, mv;
-};
-
-__device__ __forceinline__ LnRow1x8 ln_row1_request8(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
-  const int c = threadIdx.x * 8;
-  const int cc = c < K ? c : 0;
-  const int64_t xsrc = ln.mode == 2 ? ln.tokens[0] * static_cast<int64_t>(K) : 0;
-  LnRow1x8 q;
-  q.xv = *reinterpret_cast<const half8_t*>(ln.x + xsrc + cc);
-  q.rv = *reinterpret_cast<const half8_t*>(ln.mode == 1 ? ln.res + cc : ln.x + xsrc + cc);
-  q.wv = *reinterpret_cast<const half8_t*>(ln.w + cc);
-  q.bv = *reinterpret_cast<const half8_t*>(ln.b + cc);
-  q.pv = *reinterpret_cast<const half8_t*>(ln.shift + cc);
-  q.mv = *reinterpret_cast<const half8_t*>(mu + cc);
   return q;
 }
 
@@ -564,86 +483,92 @@ __device__ __forceinline__ float front_waves_sum(float v, int wave, float* scrat
   return t;
 }
 
-// stash: NT * 4 floats (the row sum), then 4 x NT * 4 fp16 values, as in ln_row1_finish
-template <int NT>
-__device__ __forceinline__ void ln_row1_finish8(const LnRow1x8& q, const LnPrologue& ln, int K, half_t* xs, float* stash,
-                                                float* red, bool store, int wave) {
-  constexpr int NWL = NT / 128;  // wavefronts that compute
-  const int c = threadIdx.x * 8;
-  const bool in = c < K;
-  float* vbuf = stash + c;
-  half_t* hbuf = reinterpret_cast<half_t*>(stash + NT * 4) + c;
+template <int NT, int V8, int NTL>
+__device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8>& q, const LnPrologue& ln, int K, half_t* xs,
+                                                float* stash, float* red, bool store, int wave) {
+  constexpr int NWL = NTL / 64;  // wavefronts that compute
+  half_t* hstash = reinterpret_cast<half_t*>(stash + NT * 4);
   float sum = 0.0f;
-  {
+#pragma unroll
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
     float v[8];
     if (ln.mode == 1) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[e]) + h2f(q.rv[e]);
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[g][e]) + h2f(q.rv[g][e]);
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[e]);
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[g][e]);
     }
-    if (in) sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
-    *reinterpret_cast<float4_t*>(vbuf) = float4_t{v[0], v[1], v[2], v[3]};
-    *reinterpret_cast<float4_t*>(vbuf + 4) = float4_t{v[4], v[5], v[6], v[7]};
-    *reinterpret_cast<half8_t*>(hbuf) = q.wv;
-    *reinterpret_cast<half8_t*>(hbuf + NT * 4) = q.bv;
-    *reinterpret_cast<half8_t*>(hbuf + NT * 8) = q.pv;
-    *reinterpret_cast<half8_t*>(hbuf + NT * 12) = q.mv;
+    if (c < K) sum += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    *reinterpret_cast<float4_t*>(stash + c) = float4_t{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<float4_t*>(stash + c + 4) = float4_t{v[4], v[5], v[6], v[7]};
+    *reinterpret_cast<half8_t*>(hstash + c) = q.wv[g];
+    *reinterpret_cast<half8_t*>(hstash + c + NT * 4) = q.bv[g];
+    *reinterpret_cast<half8_t*>(hstash + c + NT * 8) = q.pv[g];
+    *reinterpret_cast<half8_t*>(hstash + c + NT * 12) = q.mv[g];
   }
   __builtin_amdgcn_sched_barrier(0);
   sum = front_waves_sum<NWL>(sum, wave, red);
   const float mean = sum / static_cast<float>(K);
   float sv = 0.0f;
-  if (in) {
-    const float4_t v0 = *reinterpret_cast<const float4_t*>(vbuf);
-    const float4_t v1 = *reinterpret_cast<const float4_t*>(vbuf + 4);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float d = v0[e] - mean;
-      sv = fmaf(d, d, sv);
-    }
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
+    if (c < K) {
+      const float4_t v0 = *reinterpret_cast<const float4_t*>(stash + c);
+      const float4_t v1 = *reinterpret_cast<const float4_t*>(stash + c + 4);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float d = v1[e] - mean;
-      sv = fmaf(d, d, sv);
+      for (int e = 0; e < 4; ++e) {
+        const float d = v0[e] - mean;
+        sv = fmaf(d, d, sv);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float d = v1[e] - mean;
+        sv = fmaf(d, d, sv);
+      }
     }
   }
   sv = front_waves_sum<NWL>(sv, wave, red + NT / 64);
   const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
-  half8_t ov;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) ov[e] = static_cast<half_t>(0.0f);
-  if (in) {
-    const float4_t v0 = *reinterpret_cast<const float4_t*>(vbuf);
-    const float4_t v1 = *reinterpret_cast<const float4_t*>(vbuf + 4);
-    const half8_t wv = *reinterpret_cast<const half8_t*>(hbuf);
-    const half8_t bv = *reinterpret_cast<const half8_t*>(hbuf + NT * 4);
-    const half8_t pv = *reinterpret_cast<const half8_t*>(hbuf + NT * 8);
-    const half8_t mv = *reinterpret_cast<const half8_t*>(hbuf + NT * 12);
-    half8_t yv, xo;
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
+    half8_t ov;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float ve = e < 4 ? v0[e & 3] : v1[e & 3];
-      yv[e] = f2h(fmaf((ve - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
-      const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
-      ov[e] = f2h(fmaf(h2f(pv[e]) - yf, h2f(mv[e]), yf));
-      xo[e] = f2h(ve);
+    for (int e = 0; e < 8; ++e) ov[e] = static_cast<half_t>(0.0f);
+    if (c < K) {
+      const float4_t v0 = *reinterpret_cast<const float4_t*>(stash + c);
+      const float4_t v1 = *reinterpret_cast<const float4_t*>(stash + c + 4);
+      const half8_t wv = *reinterpret_cast<const half8_t*>(hstash + c);
+      const half8_t bv = *reinterpret_cast<const half8_t*>(hstash + c + NT * 4);
+      const half8_t pv = *reinterpret_cast<const half8_t*>(hstash + c + NT * 8);
+      const half8_t mv = *reinterpret_cast<const half8_t*>(hstash + c + NT * 12);
+      half8_t yv, xo;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float ve = e < 4 ? v0[e & 3] : v1[e & 3];
+        yv[e] = f2h(fmaf((ve - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
+        const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
+        ov[e] = f2h(fmaf(h2f(pv[e]) - yf, h2f(mv[e]), yf));
+        xo[e] = f2h(ve);
+      }
+      if (store) {
+        *reinterpret_cast<half8_t*>(ln.ln_out + c) = yv;
+        if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + c) = xo;
+      }
     }
-    if (store) {
-      *reinterpret_cast<half8_t*>(ln.ln_out + c) = yv;
-      if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + c) = xo;
-    }
+    *reinterpret_cast<half8_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
   }
-  *reinterpret_cast<half8_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
 }
 
-// One block.  With the prologue, it runs BEFORE the weight requests: a wavefront stalls on its weight requests until
-// the memory pipeline has room for them - late in a 67 MB launch that takes microseconds (timestamps: the last
-// wavefronts get their requests out 11 us after the launch began) - and it cannot run the prologue while it is
-// stalled, so a prologue behind the requests ends up at the tail of the launch.  Measured at the 7.2B shape, ms per
-// step, prologue first / weights first / weights first in every second block: int8 1.924 / 1.947 / 1.915, int4
-// 1.773 / 1.825 / 1.793; the mixed orders need both code paths and 62-66 registers, so it is prologue first for all.
+// One block.  A wavefront cannot do both at once: it stalls on its weight requests until the memory pipeline has
+// room for them - late in a 67 MB launch that takes microseconds (timestamps: the last wavefronts get their
+// requests out 11 us after the launch began) - and a prologue behind the requests would end up at the tail of the
+// launch, while a prologue before them leaves HBM idle for its 1.5 us.  So the wavefronts share the work: some
+// compute the prologue and request their weights afterwards, the others request theirs at once and meet the first
+// at the barrier (7.2B shape, int8: 1.79 -> 1.72 ms per step against the prologue in every wavefront first).
 template <int FMT, int NT, bool LN>
 __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const LinearProblem& prob, int blk, half_t* xs,
                                                float* red) {
@@ -665,7 +590,11 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
 
   // With the prologue: the first half of the wavefronts computes it (eight values per thread) and requests its
   // weights afterwards; the second half requests its weights at once, so that HBM streams while the prologue runs.
-  const bool ln_wave = LN && wave < NW / 2;
+  // (half of them for int8 and fp16 weights; a quarter for int4, whose wavefronts have three requests per vector
+  // to get out: 7.2B shape, ms per step with a half / a quarter: int8 1.72 / 1.75, int4 1.70 / 1.64)
+  constexpr int NTL = NT / (FMT == RWKV_FMT_W4 ? 4 : 2);  // threads that compute the prologue
+  constexpr int V8 = NT * 4 / (NTL * 8);  // groups of eight values per computing thread
+  const bool ln_wave = LN && wave < NTL / 64;
   uint4_t xq = {0u, 0u, 0u, 0u};
   if constexpr (LN) {
     // (below, after the row scales)
@@ -719,9 +648,9 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
     // two code paths, so that the prologue's operands and the weight vectors never hold registers together; the
     // second path passes the two barriers of the first one's block sums
     if (ln_wave) {
-      const LnRow1x8 lnq = ln_row1_request8(args.ln, prob.mu, K);
+      const LnRow1xV<V8> lnq = ln_row1_request8<V8, NTL>(args.ln, prob.mu, K);
       __builtin_amdgcn_sched_barrier(0);
-      ln_row1_finish8<NT>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0, wave);
+      ln_row1_finish8<NT, V8, NTL>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0, wave);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int st = 0; st < S; ++st) request(st);
