@@ -56,7 +56,20 @@ private:
   std::string path_;
   std::uint64_t file_size_ = 0;
   bool chunk_load_ = false;
-  std::vector<std::uint8_t> bytes_;
+  // the whole file (chunk_load off): allocated without the zero fill a vector would do first, which costs as
+  // much as a third of the read on a multi-gigabyte file
+  struct FileBytes {
+    std::unique_ptr<std::uint8_t[]> p;
+    std::size_t n = 0;
+    void allocate(std::size_t size) {
+      p.reset(new std::uint8_t[size]);
+      n = size;
+    }
+    std::uint8_t* data() { return p.get(); }
+    const std::uint8_t* data() const { return p.get(); }
+    std::size_t size() const { return n; }
+  };
+  FileBytes bytes_;
   std::vector<PthEntry> entries_;
   std::shared_ptr<StreamReader> stream_reader_;
 };

@@ -67,6 +67,11 @@ int rwkv_hip_event_create(void** ev);
 int rwkv_hip_event_destroy(void* ev);
 int rwkv_hip_event_record(void* ev, rwkv_stream_t s);
 int rwkv_hip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms);
+/* ordering between streams and with the host, for pipelines that copy on one stream and compute on another (the
+ * checkpoint loader; the reference pairs copy and compute streams the same way, src/rwkv7_fast_v4.cu:110-181):
+ * the host waits for a recorded event; work enqueued on `s` after the call starts only once the event has happened */
+int rwkv_hip_event_sync(void* ev);
+int rwkv_hip_stream_wait_event(rwkv_stream_t s, void* ev);
 
 /* Measurement aid (no counterpart in the reference): the cost of a launch that has to wait for its predecessor.
  * Runs a chain of `links` launches of a kernel that does next to nothing (every block reads a counter, one thread

@@ -214,6 +214,16 @@ int rwkv_hip_event_record(void* ev, rwkv_stream_t s) {
   RWKV_HIP_TRY(hipEventRecord(reinterpret_cast<hipEvent_t>(ev), as_stream(s)));
   return RWKV_OK;
 }
+int rwkv_hip_event_sync(void* ev) {
+  RWKV_REQUIRE(ev != nullptr, "event is NULL");
+  RWKV_HIP_TRY(hipEventSynchronize(reinterpret_cast<hipEvent_t>(ev)));
+  return RWKV_OK;
+}
+int rwkv_hip_stream_wait_event(rwkv_stream_t s, void* ev) {
+  RWKV_REQUIRE(ev != nullptr, "event is NULL");
+  RWKV_HIP_TRY(hipStreamWaitEvent(as_stream(s), reinterpret_cast<hipEvent_t>(ev), 0));
+  return RWKV_OK;
+}
 int rwkv_hip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms) {
   RWKV_REQUIRE(ms != nullptr, "ms is NULL");
   RWKV_HIP_TRY(hipEventSynchronize(reinterpret_cast<hipEvent_t>(ev_stop)));

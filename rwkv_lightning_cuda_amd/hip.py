@@ -32,6 +32,7 @@ EXPORTS = [
     "rwkv_hip_memcpy_h2d_async", "rwkv_hip_memcpy_d2h_async", "rwkv_hip_memcpy_d2d_async", "rwkv_hip_memset",
     "rwkv_hip_mem_info", "rwkv_hip_stream_create", "rwkv_hip_stream_destroy", "rwkv_hip_stream_sync",
     "rwkv_hip_device_sync", "rwkv_hip_event_create", "rwkv_hip_event_destroy", "rwkv_hip_event_record",
+    "rwkv_hip_event_sync", "rwkv_hip_stream_wait_event",
     "rwkv_hip_event_elapsed_ms", "rwkv_hip_measure_launch_chain", "rwkv_hip_wkv7", "rwkv_hip_wkv7_f16state", "rwkv_hip_quantize_w8", "rwkv_hip_dequant_w8",
     "rwkv_hip_quantize_w4", "rwkv_hip_dequant_w4", "rwkv_hip_bf16_to_f16", "rwkv_hip_bf16_to_f16_transpose",
     "rwkv_hip_emb_ln0_bf16_to_f16", "rwkv_hip_fill_normal_f16", "rwkv_hip_linear",

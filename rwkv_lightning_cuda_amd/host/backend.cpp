@@ -10,11 +10,15 @@
 // exists, device errors throw instead of exiting, and forward passes run through pooled sessions (stream +
 // arena + decode graphs) so concurrent callers do not allocate per call.
 #include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstring>
 #include <cstdlib>
 #include <limits>
 #include <mutex>
 #include <sstream>
 #include <stdexcept>
+#include <thread>
 #include <unordered_map>
 
 #include "pth_tensor.hpp"
@@ -116,15 +120,42 @@ struct ModelBackend::Impl {
   std::vector<DeviceBuffer<std::uint8_t>> storage;  // owns every weight tensor
   std::uint64_t fill_counter = 0;
   std::string archive_folder;       // "<folder>/data.pkl" names the checkpoint's top folder
-  void* pinned = nullptr;           // host staging of the checkpoint loader
-  std::size_t pinned_bytes = 0;
+
+  // Staging of the checkpoint loader (the reference's copy/compute stream pairs with two pinned buffers,
+  // src/rwkv7_fast_v4.cu:110-181,212-290).  A tensor travels in pieces of 64 MiB through two pinned host buffers:
+  // while one piece is on its way to the device (copy stream) the host reads the next piece from the file into
+  // the other buffer.  The pieces land in one of two device buffers for the bf16 patterns, so that the conversion
+  // kernel of one tensor (NULL stream, ordered behind the tensor's last copy through an event) runs while the next
+  // tensor is being read and copied; a device buffer is reused once the event recorded behind its conversion
+  // kernel has happened.
+  static constexpr std::size_t kPieceBytes = std::size_t(64) << 20;
+  struct PinnedPiece {
+    void* host = nullptr;
+    void* copied = nullptr;  // event on the copy stream: the piece has left the buffer
+    bool in_flight = false;
+  };
+  struct StageSlot {
+    DeviceBuffer<std::uint16_t> dev;
+    void* arrived = nullptr;   // event on the copy stream: the device buffer holds the whole tensor
+    void* consumed = nullptr;  // event on the NULL stream: the kernel that read the device buffer has run
+    bool in_use = false;
+  };
+  PinnedPiece piece[2];
+  int piece_next = 0;
+  StageSlot stage[2];
+  int stage_next = 0;
+  rwkv_stream_t copy_stream = nullptr;
+  std::vector<DeviceBuffer<std::uint8_t>> retired;  // fp16 sources of quantised matrices, freed in batches
+  std::size_t retired_bytes = 0;
+  std::uint64_t loaded_bytes = 0;                   // bf16 bytes that went through the staging
+  bool chunk_loading = false;                       // the archive is read on demand (pread) rather than held in memory
 
   mutable std::mutex pool_mutex;
   mutable std::vector<rwkv_hip_session*> idle_sessions;
 
   ~Impl() {
     for (auto* s : idle_sessions) rwkv_hip_session_destroy(s);
-    if (pinned) rwkv_hip_host_free(pinned);
+    release_staging();
     if (model) rwkv_hip_model_destroy(model);
   }
 
@@ -162,23 +193,115 @@ struct ModelBackend::Impl {
       check_hip(rwkv_hip_quantize_w4(nullptr, N, K, w16, q, s, z), "quantize_w4");
       check_hip(rwkv_hip_model_set_matrix(model, layer, id, RWKV_FMT_W4, q, s, z), "set matrix");
     }
-    // the fp16 source is no longer needed once quantised: free it (it is the last storage entry but two/three)
-    check_hip(rwkv_hip_device_sync(), "sync after quantise");
-    for (auto& buf : storage) {
-      if (buf.p == static_cast<std::uint8_t*>(w16)) {
-        buf = DeviceBuffer<std::uint8_t>();
+    // the fp16 source is no longer needed once the quantisation kernel has run: it is set aside and freed with
+    // others of its kind after one device sync per 2 GiB (a sync per matrix would stall the load pipeline)
+    for (auto it = storage.rbegin(); it != storage.rend(); ++it) {
+      if (it->p == static_cast<std::uint8_t*>(w16)) {
+        retired_bytes += it->n;
+        retired.push_back(std::move(*it));
+        *it = DeviceBuffer<std::uint8_t>();
         break;
       }
     }
+    if (retired_bytes > (std::size_t(2) << 30)) free_retired();
+  }
+
+  void free_retired() {
+    if (retired.empty()) return;
+    check_hip(rwkv_hip_device_sync(), "sync before releasing fp16 sources");
+    retired.clear();
+    retired_bytes = 0;
+  }
+
+  void release_staging() {
+    for (PinnedPiece& pc : piece) {
+      if (pc.host) rwkv_hip_host_free(pc.host);
+      if (pc.copied) rwkv_hip_event_destroy(pc.copied);
+      pc = PinnedPiece();
+    }
+    for (StageSlot& slot : stage) {
+      if (slot.arrived) rwkv_hip_event_destroy(slot.arrived);
+      if (slot.consumed) rwkv_hip_event_destroy(slot.consumed);
+      slot = StageSlot();
+    }
+    if (copy_stream) rwkv_hip_stream_destroy(copy_stream);
+    copy_stream = nullptr;
   }
 
   // ---- checkpoint ------------------------------------------------------------------------------------------
   [[noreturn]] static void load_error(const std::string& what) { throw std::runtime_error("load model: " + what); }
 
-  // The tensor's bf16 patterns in logical order on the device (a temporary the caller releases with the sync
-  // after its conversion kernel).
-  DeviceBuffer<std::uint16_t> upload_bf16(const llm_infer::PthArchive& archive, const llm_infer::TensorRecord& rec) {
-    // Row-major tensors (all of a normal checkpoint): the byte range goes from the file into a pinned buffer and
+  // File bytes [offset, offset + bytes) of a stored entry into host memory.  From the whole-file copy large ranges
+  // are copied by four threads (0.14 -> 0.05 s for 2.7 GB); reads from the file itself stay on one thread - four
+  // concurrent preads of one file were slower than one (0.75 s against 0.51 s for the same 2.7 GB out of the page
+  // cache).
+  static void read_range(const llm_infer::PthArchive& archive, const llm_infer::PthEntry& entry, std::uint64_t offset,
+                         void* dst, std::size_t bytes, bool from_memory) {
+    constexpr std::size_t kParallelFrom = std::size_t(16) << 20;
+    constexpr int kReaders = 4;
+    if (bytes < kParallelFrom || !from_memory) {
+      llm_infer::Status rd = archive.read_stored_entry_range(entry, offset, dst, bytes);
+      if (!rd.ok_status()) load_error(rd.message());
+      return;
+    }
+    std::string errors[kReaders];
+    std::vector<std::thread> readers;
+    const std::size_t piece = ((bytes / kReaders) + 4095) & ~std::size_t(4095);
+    for (int i = 0; i < kReaders; ++i) {
+      const std::size_t from = std::min(bytes, piece * i);
+      const std::size_t len = std::min(bytes - from, piece);
+      if (len == 0) continue;
+      readers.emplace_back([&archive, &entry, &errors, i, offset, dst, from, len] {
+        llm_infer::Status rd = archive.read_stored_entry_range(entry, offset + from, static_cast<char*>(dst) + from, len);
+        if (!rd.ok_status()) errors[i] = rd.message();
+      });
+    }
+    for (auto& t : readers) t.join();
+    for (const std::string& e : errors)
+      if (!e.empty()) load_error(e);
+  }
+
+  // The next device staging buffer, free for reuse and with room for `bytes`.
+  StageSlot& take_slot(std::size_t bytes) {
+    if (copy_stream == nullptr) {
+      check_hip(rwkv_hip_stream_create(&copy_stream), "create copy stream");
+      for (PinnedPiece& pc : piece) {
+        check_hip(rwkv_hip_host_alloc(&pc.host, kPieceBytes), "alloc pinned staging");
+        check_hip(rwkv_hip_event_create(&pc.copied), "create staging event");
+      }
+      for (StageSlot& slot : stage) {
+        check_hip(rwkv_hip_event_create(&slot.arrived), "create staging event");
+        check_hip(rwkv_hip_event_create(&slot.consumed), "create staging event");
+      }
+    }
+    StageSlot& slot = stage[stage_next];
+    stage_next ^= 1;
+    if (slot.in_use) check_hip(rwkv_hip_event_sync(slot.consumed), "wait for staging slot");
+    slot.in_use = false;
+    if (bytes > slot.dev.n * 2) {
+      slot.dev = DeviceBuffer<std::uint16_t>();  // (freeing waits for the device: rare, the largest tensors come first)
+      slot.dev.resize((bytes + 1) / 2, "alloc bf16 staging");
+    }
+    return slot;
+  }
+
+  // One piece (at most kPieceBytes) into a pinned buffer by `fill`, then on its way to `dst` on the copy stream.
+  template <class Fill>
+  void send_piece(void* dst, std::size_t bytes, Fill&& fill) {
+    PinnedPiece& pc = piece[piece_next];
+    piece_next ^= 1;
+    if (pc.in_flight) check_hip(rwkv_hip_event_sync(pc.copied), "wait for pinned buffer");
+    fill(pc.host);
+    check_hip(rwkv_hip_memcpy_h2d_async(copy_stream, dst, pc.host, bytes), "copy bf16 weight");
+    check_hip(rwkv_hip_event_record(pc.copied, copy_stream), "record copy event");
+    pc.in_flight = true;
+  }
+
+  // The tensor's bf16 patterns in logical order in a staging slot's device buffer: valid until the slot comes
+  // round again (two uploads later); the caller enqueues the kernel that reads them on the NULL stream and then
+  // calls consumed(slot).  Returns the slot; *count receives the number of elements.
+  StageSlot& upload_bf16(const llm_infer::PthArchive& archive, const llm_infer::TensorRecord& rec, std::size_t* count) {
+    // Row-major tensors (all of a normal checkpoint): the byte range goes from the file into the pinned buffers and
     // from there to the device, no per-element pass on the host.
     std::uint64_t n = 1;
     std::int64_t expect = 1;
@@ -190,31 +313,42 @@ struct ModelBackend::Impl {
       n *= static_cast<std::uint64_t>(rec.shape[i]);
     }
     const llm_infer::PthEntry* entry = dense && n > 0 ? archive.find_entry(archive_folder + "/data/" + rec.storage_key) : nullptr;
+    StageSlot* slot = nullptr;
+    std::size_t bytes = 0;
     if (entry != nullptr && entry->is_stored() && entry->uncompressed_size == rec.storage_size * 2 &&
         rec.storage_offset + n <= rec.storage_size) {
-      const std::size_t bytes = static_cast<std::size_t>(n) * 2;
-      if (bytes > pinned_bytes) {
-        if (pinned) check_hip(rwkv_hip_host_free(pinned), "free pinned staging");
-        pinned = nullptr;
-        pinned_bytes = 0;
-        check_hip(rwkv_hip_host_alloc(&pinned, bytes), "alloc pinned staging");
-        pinned_bytes = bytes;
+      bytes = static_cast<std::size_t>(n) * 2;
+      slot = &take_slot(bytes);
+      for (std::size_t at = 0; at < bytes; at += kPieceBytes) {
+        const std::size_t len = std::min(kPieceBytes, bytes - at);
+        send_piece(reinterpret_cast<char*>(slot->dev.p) + at, len, [&](void* host) {
+          read_range(archive, *entry, rec.storage_offset * 2 + at, host, len, !chunk_loading);
+        });
       }
-      llm_infer::Status rd = archive.read_stored_entry_range(*entry, rec.storage_offset * 2, pinned, bytes);
-      if (!rd.ok_status()) load_error(rd.message());
-      DeviceBuffer<std::uint16_t> dev;
-      dev.resize(static_cast<std::size_t>(n), "alloc bf16 staging");
-      check_hip(rwkv_hip_memcpy_h2d(dev.p, pinned, bytes), "copy bf16 weight");
-      return dev;
+    } else {
+      auto data = llm_infer::load_bf16_tensor_select(archive, rec, true, false, false);
+      if (!data.ok()) load_error(data.status().message());
+      n = data.value().values_bf16.size();
+      bytes = static_cast<std::size_t>(n) * 2;
+      slot = &take_slot(bytes);
+      const char* src = reinterpret_cast<const char*>(data.value().values_bf16.data());
+      for (std::size_t at = 0; at < bytes; at += kPieceBytes) {
+        const std::size_t len = std::min(kPieceBytes, bytes - at);
+        send_piece(reinterpret_cast<char*>(slot->dev.p) + at, len, [&](void* host) { std::memcpy(host, src + at, len); });
+      }
     }
-    auto data = llm_infer::load_bf16_tensor_select(archive, rec, true, false, false);
-    if (!data.ok()) load_error(data.status().message());
-    DeviceBuffer<std::uint16_t> dev;
-    dev.resize(data.value().values_bf16.size(), "alloc bf16 staging");
-    if (dev.n) {
-      check_hip(rwkv_hip_memcpy_h2d(dev.p, data.value().values_bf16.data(), dev.n * sizeof(std::uint16_t)), "copy bf16 weight");
+    if (bytes) {
+      check_hip(rwkv_hip_event_record(slot->arrived, copy_stream), "record copy event");
+      check_hip(rwkv_hip_stream_wait_event(nullptr, slot->arrived), "order conversion behind the copy");
     }
-    return dev;
+    loaded_bytes += bytes;
+    *count = static_cast<std::size_t>(n);
+    return *slot;
+  }
+
+  void consumed(StageSlot& slot) {
+    check_hip(rwkv_hip_event_record(slot.consumed, nullptr), "record staging event");
+    slot.in_use = true;
   }
 
   // fp16 copy of a checkpoint tensor in `storage`: elements as they are, or a [rows,cols] matrix into [cols,rows]
@@ -230,18 +364,22 @@ struct ModelBackend::Impl {
       load_error("tensor " + rec.name + " has shape " + llm_infer::shape_string(rec.shape) + ", expected [" +
                  std::to_string(t_rows) + "," + std::to_string(t_cols) + "]");
     }
-    DeviceBuffer<std::uint16_t> raw = upload_bf16(archive, rec);
     void* out = alloc(elems * sizeof(half), "alloc weight tensor");
+    std::size_t count = 0;
+    StageSlot& raw = upload_bf16(archive, rec, &count);
+    if (count != elems) load_error("tensor " + rec.name + " has " + std::to_string(count) + " stored elements");
     if (t_rows > 0) {
-      check_hip(rwkv_hip_bf16_to_f16_transpose(nullptr, t_rows, t_cols, raw.p, out), "bf16 -> f16 transpose");
+      check_hip(rwkv_hip_bf16_to_f16_transpose(nullptr, t_rows, t_cols, raw.dev.p, out), "bf16 -> f16 transpose");
     } else {
-      check_hip(rwkv_hip_bf16_to_f16(nullptr, static_cast<int64_t>(elems), raw.p, out), "bf16 -> f16");
+      check_hip(rwkv_hip_bf16_to_f16(nullptr, static_cast<int64_t>(elems), raw.dev.p, out), "bf16 -> f16");
     }
-    check_hip(rwkv_hip_device_sync(), "sync weight preprocess");  // raw is released on return
+    consumed(raw);
     return out;
   }
 
   void load_checkpoint(bool chunk_load) {
+    const auto t_start = std::chrono::steady_clock::now();
+    chunk_loading = chunk_load;
     auto opened = llm_infer::PthArchive::open(spec.checkpoint, chunk_load);
     if (!opened.ok()) load_error(opened.status().message());
     const llm_infer::PthArchive& archive = opened.value();
@@ -323,15 +461,24 @@ struct ModelBackend::Impl {
       const llm_infer::TensorRecord& emb = need("emb.weight");
       const llm_infer::TensorRecord& w = need("blocks.0.ln0.weight");
       const llm_infer::TensorRecord& b = need("blocks.0.ln0.bias");
-      DeviceBuffer<std::uint16_t> emb_raw = upload_bf16(archive, emb);
-      DeviceBuffer<std::uint16_t> w_raw = upload_bf16(archive, w);
-      DeviceBuffer<std::uint16_t> b_raw = upload_bf16(archive, b);
-      if (emb_raw.n != static_cast<std::size_t>(d.vocab) * C || w_raw.n != C || b_raw.n != C) {
-        load_error("emb/ln0 shape mismatch for emb+ln0 preprocessing");
-      }
-      void* out = alloc(emb_raw.n * sizeof(half), "alloc emb+ln0");
-      check_hip(rwkv_hip_emb_ln0_bf16_to_f16(nullptr, d.vocab, Ci, emb_raw.p, w_raw.p, b_raw.p, 1e-5f, out), "emb+ln0 preprocess");
-      check_hip(rwkv_hip_device_sync(), "sync emb+ln0 preprocess");
+      // three tensors at once, two staging slots: the two vectors are copied out of their slots first
+      DeviceBuffer<std::uint16_t> wb;
+      wb.resize(2 * C, "alloc ln0 vectors");
+      std::size_t n_w = 0, n_b = 0, n_emb = 0;
+      StageSlot& w_raw = upload_bf16(archive, w, &n_w);
+      if (n_w != C) load_error("emb/ln0 shape mismatch for emb+ln0 preprocessing");
+      check_hip(rwkv_hip_memcpy_d2d_async(nullptr, wb.p, w_raw.dev.p, C * 2), "copy ln0 weight");
+      consumed(w_raw);
+      StageSlot& b_raw = upload_bf16(archive, b, &n_b);
+      if (n_b != C) load_error("emb/ln0 shape mismatch for emb+ln0 preprocessing");
+      check_hip(rwkv_hip_memcpy_d2d_async(nullptr, wb.p + C, b_raw.dev.p, C * 2), "copy ln0 bias");
+      consumed(b_raw);
+      StageSlot& emb_raw = upload_bf16(archive, emb, &n_emb);
+      if (n_emb != static_cast<std::size_t>(d.vocab) * C) load_error("emb/ln0 shape mismatch for emb+ln0 preprocessing");
+      void* out = alloc(n_emb * sizeof(half), "alloc emb+ln0");
+      check_hip(rwkv_hip_emb_ln0_bf16_to_f16(nullptr, d.vocab, Ci, emb_raw.dev.p, wb.p, wb.p + C, 1e-5f, out), "emb+ln0 preprocess");
+      consumed(emb_raw);
+      check_hip(rwkv_hip_device_sync(), "sync emb+ln0 preprocess");  // wb is released here
       check_hip(rwkv_hip_model_set_tensor(model, -1, RWKV_T_EMB_LN0, out), "set tensor");
     }
     vector(-1, RWKV_T_LN_OUT_W, "ln_out.weight");
@@ -371,9 +518,12 @@ struct ModelBackend::Impl {
       matrix(l, RWKV_M_FFN_VALUE, p + "ffn.value.weight", Ci, d.ffn);  // the file's own [C,F] layout
     }
     check_hip(rwkv_hip_device_sync(), "sync model build");
-    if (pinned) check_hip(rwkv_hip_host_free(pinned), "free pinned staging");
-    pinned = nullptr;
-    pinned_bytes = 0;
+    free_retired();
+    release_staging();
+    const double seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_start).count();
+    std::printf("[ModelBackend] %s: %.2f GB of bf16 tensors read, converted%s in %.2f s (%.2f GB/s)\n", model_name.c_str(),
+                loaded_bytes * 1e-9, spec.fmt == RWKV_FMT_F16 ? "" : " and quantised", seconds,
+                seconds > 0 ? loaded_bytes * 1e-9 / seconds : 0.0);
   }
 
   void build() {

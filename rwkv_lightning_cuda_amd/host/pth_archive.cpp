@@ -87,7 +87,7 @@ Result<PthArchive> PthArchive::open(const std::string& path, bool chunk_load) {
   if (ar.file_size_ < kEndRecord) return Status::error("file is too small to be a zip archive");
 
   if (!chunk_load) {
-    ar.bytes_.resize(static_cast<std::size_t>(ar.file_size_));
+    ar.bytes_.allocate(static_cast<std::size_t>(ar.file_size_));
     Status rd = reader->read(0, ar.bytes_.data(), ar.bytes_.size());
     if (!rd.ok_status()) return Status::error(describe("failed to read file", path));
   } else {

@@ -116,7 +116,19 @@ def write_checkpoint(pth_path, manifest_path, sd, with_metadata=True):
     write_manifest(manifest_path, sd)
 
 
+def load_rate_dims(layers=4):
+    """The 7.2B shape cut to a few layers: full-size embedding, head and per-layer tensors (0.43 GB a layer + 1.07 GB),
+    for timing the checkpoint loader - ModelBackend prints the rate it reached."""
+    return dict(L=layers, C=4096, H=64, F=16384, V=65536, Rw=128, Ra=128, Rg=480, Rv=96)
+
+
 def main():
+    if len(sys.argv) > 2 and sys.argv[1] == "--load-rate":
+        # python make_pth_fixture.py --load-rate OUT.pth [LAYERS]: no manifest, no stress entries
+        sd = state_dict(load_rate_dims(int(sys.argv[3]) if len(sys.argv) > 3 else 4), seed=3)
+        torch.save(sd, sys.argv[2])
+        print("wrote %s (%.2f GB)" % (sys.argv[2], os.path.getsize(sys.argv[2]) / 1e9))
+        return
     pth = sys.argv[1] if len(sys.argv) > 1 else os.path.join(HERE, "rwkv7_tiny.pth")
     manifest = sys.argv[2] if len(sys.argv) > 2 else os.path.join(HERE, "rwkv7_tiny.manifest")
     sd = state_dict(tiny_dims())
