@@ -341,7 +341,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   // The single-launch time-mix core re-reads a head's LoRA rows for every batch row; from 16 rows on the
   // row-tiled kernels of the prefill path (LoRA rank-outs on the matrix core) are faster (measured: 4.2 -> 4.0 ms
   // per step at 16 rows, 5.5 -> 4.6 ms at 32).
-  const bool fused_tmix = step && rows <= 8 && !s->wkv_fp16;  // (the fp16 state has its own recurrence kernel)
+  const bool fused_tmix = step && rows <= 8;
   // Decode steps on the GEMV path can fold both LayerNorm + token-shift kernels of a layer into the prologue of the
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key): by default for one row of up to 4096
   // channels.  The residual-stream tap needs the stand-alone kernels.
@@ -478,7 +478,12 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       p.w0 = w.t[RWKV_T_W0]; p.a0 = w.t[RWKV_T_A0]; p.v0 = w.t[RWKV_T_V0]; p.k_k = w.t[RWKV_T_K_K];
       p.k_a = w.t[RWKV_T_K_A]; p.r_k = w.t[RWKV_T_R_K]; p.lnx_w = w.t[RWKV_T_LNX_W]; p.lnx_b = w.t[RWKV_T_LNX_B];
       p.r = b.r; p.k = b.k; p.v = v_cur; p.v_first = b.v_first; p.v_first_out = nullptr;
-      p.state = S; p.y2 = b.y2;
+      p.y2 = b.y2;
+      if (s->wkv_fp16) {
+        p.state16 = S16; p.elapsed = elapsed;
+      } else {
+        p.state = S;
+      }
       if (ln_in_linear) {
         p.shift_src = b.xx; p.shift_dst = shift0;
       }

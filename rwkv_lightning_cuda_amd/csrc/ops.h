@@ -236,7 +236,9 @@ struct TmixStepArgs {
   const half_t *r, *k, *v;                  // projections [B,C]
   const half_t* v_first;                    // [B,C], read when hv != NULL
   half_t* v_first_out;                      // [B,C], written when hv == NULL (layer 0), may be NULL
-  float* state;                             // [B,H,64,64], updated in place
+  float* state;                             // [B,H,64,64], updated in place (fp32-state mode)
+  half_t* state16;                          // fp16-state mode (state == NULL): [B,H,64,64] in fp16 ...
+  const int* elapsed;                       // ... and the tokens each row has seen, [B] (the decay's dither phase)
   half_t* y2;                               // [B,C] input of the output projection
   // Split mode (gate_out != NULL): the g rank-out - more than half of the launch's bytes - runs in B*H further
   // blocks that write the gate to gate_out [B,C]; the heads' blocks write the ungated output in fp32 to y2_pre

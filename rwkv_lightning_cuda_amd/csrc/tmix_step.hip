@@ -24,7 +24,7 @@
 // A block's loads (123 KB at the 7.2B shape, 61 KB of them the g rank-out rows) arrive at the rate one CU can
 // take in, about 50 GB/s, and only B*H CUs are at work.  In split mode the g rank-out therefore runs in B*H
 // further blocks of the same launch, and the gate is applied by the consumer of the output (see TmixStepArgs).
-#include "ops.h"
+#include "wkv7_f16state.h"
 
 namespace rwkv {
 
@@ -97,7 +97,12 @@ __device__ __forceinline__ void hidden_store(float* __restrict__ hs, half_t raw,
   }
 }
 
+// F16: the WKV state is fp16 and the step follows the fp16-state recurrence (wkv7_f16state.h): the first wavefront
+// holds the head's 64 state rows, one per lane, and does the step itself between its per-channel work and the
+// GroupNorm - the other wavefronts are done after the rank-outs, two barriers in all.
+template <bool F16>
 __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p) {
+  __shared__ __align__(16) half_t ops16[5][kHead];  // fp16-state mode: a~, b~, k', decay delta, r
   __shared__ __align__(16) float hs[4][kStepMaxR];  // activated LoRA hidden vectors: w, a, g, v
   __shared__ __align__(16) float lo[4][kHead];      // rank-out results per channel: w12, a12, g, v-gate logit
   __shared__ __align__(16) float vec[6][kHead];     // WKV operands r, d, k', a~, b~ and the mixed v
@@ -133,8 +138,26 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
   }
 
   // ---- all global loads up front
-  float* srow = p.state + (static_cast<int64_t>(bh) * kHead + i) * kHead + 4 * q;
-  float4_t S = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(srow));
+  float* srow = nullptr;
+  float4_t S = {0.0f, 0.0f, 0.0f, 0.0f};
+  half_t* srow16 = nullptr;
+  half2_t S16[kPairs16];
+  int phase = 0;
+  if constexpr (F16) {
+    if (wave == 0) {  // state row `lane` of the head: 128 bytes
+      srow16 = p.state16 + (static_cast<int64_t>(bh) * kHead + lane) * kHead;
+#pragma unroll
+      for (int g = 0; g < kPairs16 / 4; ++g) {
+        const uint4_t t = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(srow16 + 8 * g));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S16[4 * g + e] = as_half2(t[e]);
+      }
+      phase = p.elapsed[bi];
+    }
+  } else {
+    srow = p.state + (static_cast<int64_t>(bh) * kHead + i) * kHead + 4 * q;
+    S = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(srow));
+  }
   LoraRow w2, a2, g2, v2;
   lora_row_load(w2, p.w2 + static_cast<int64_t>(c) * p.Rw, p.Rw, q);
   lora_row_load(a2, p.a2 + static_cast<int64_t>(c) * p.Ra, p.Ra, q);
@@ -200,6 +223,9 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
 
   // ---- per channel, first wavefront: v-residual gate, kk normalise over the head, a-gate, decay
   float v_use = vv, k2 = 0.0f, gch = 0.0f;
+  if constexpr (F16) {
+    if (wave != 0) return;
+  }
   if (wave == 0) {
     const float w12 = lo[0][lane];
     const float a12 = lo[1][lane];
@@ -216,6 +242,39 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
     const float kk = u * inv;
     const float av = sigmoid_f(a0 + a12);
     k2 = round_h(kv * fmaf(av, ka, 1.0f - ka));
+    if constexpr (F16) {
+      // the operands as the fp16 tensors the stand-alone kernels exchange, then the step on this lane's state row
+      ops16[0][lane] = f2h(-kk);
+      ops16[1][lane] = f2h(kk * av);
+      ops16[2][lane] = f2h(k2);
+      ops16[3][lane] = decay_delta16_of(w12 + w0, phase + cl);  // (w12 + w0 unrounded: a single-token call)
+      ops16[4][lane] = f2h(rv);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const half_t y16 = wkv16_row_step(S16, ops16[0], ops16[1], ops16[2], ops16[3], ops16[4], f2h(v_use));
+#pragma unroll
+      for (int g = 0; g < kPairs16 / 4; ++g) {
+        uint4_t t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[e] = __builtin_bit_cast(uint32_t, S16[4 * g + e]);
+        __builtin_nontemporal_store(t, reinterpret_cast<uint4_t*>(srow16 + 8 * g));
+      }
+      const float yy = h2f(y16);
+      const float mean = wave_sum_uniform(yy) * (1.0f / 64.0f);
+      const float rkv = wave_sum_uniform(rv * k2 * rk);
+      const float dlt = yy - mean;
+      const float var = wave_sum_uniform(dlt * dlt) * (1.0f / 64.0f);
+      const float rstd = rsqrtf(var + kLnxEps);
+      if (p.shift_dst) p.shift_dst[row + cl] = shift_h;
+      const float pre = dlt * rstd * lnw + lnb + rkv * v_use;
+      if (split) {
+        p.y2_pre[row + cl] = pre;
+      } else {
+        p.y2[row + cl] = f2h(pre * gch);
+      }
+      return;
+    }
     const float wraw = round_h(w12 + w0);
     vec[0][lane] = rv;
     vec[1][lane] = exp2f(-0.8750387749145276f / (1.0f + exp2f(-1.4426950408889634f * wraw)));
@@ -280,8 +339,14 @@ int tmix_step_launch(hipStream_t st, const TmixStepArgs& p) {
                    p.Ra <= kStepMaxR && p.Rg <= kStepMaxR && p.Rv <= kStepMaxR,
                "tmix_step: LoRA ranks must be multiples of 8, at most %d", kStepMaxR);
   RWKV_REQUIRE((p.gate_out == nullptr) == (p.y2_pre == nullptr), "tmix_step: split mode needs both y2_pre and gate_out");
+  RWKV_REQUIRE((p.state != nullptr) != (p.state16 != nullptr), "tmix_step: exactly one of the fp32 and the fp16 state");
+  RWKV_REQUIRE(p.state16 == nullptr || p.elapsed != nullptr, "tmix_step: the fp16 state needs the elapsed counters");
   const int blocks = p.B * p.H * (p.gate_out ? 2 : 1);
-  hipLaunchKernelGGL(tmix_step_kernel, dim3(blocks), dim3(kStepThreads), 0, st, p);
+  if (p.state16) {
+    hipLaunchKernelGGL(tmix_step_kernel<true>, dim3(blocks), dim3(kStepThreads), 0, st, p);
+  } else {
+    hipLaunchKernelGGL(tmix_step_kernel<false>, dim3(blocks), dim3(kStepThreads), 0, st, p);
+  }
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }

@@ -18,38 +18,17 @@
 // r) are the same for every lane: lane c fetches element c of each for the NEXT token while the current one is
 // computed, converts its decay logit, and drops them into LDS, from where every lane reads them back as 16-byte
 // broadcasts.  The state is read and written once per call, 16 bytes per lane and instruction.
-#include "ops.h"
+#include "wkv7_f16state.h"
 
 namespace rwkv {
 
 namespace {
 
-constexpr int kPairs = kHead / 2;  // half2 pairs per state row
+constexpr int kPairs = kPairs16;
 
 struct TokenOps {  // one token's per-column operands in LDS
   half_t a[kHead], b[kHead], k[kHead], wd[kHead], r[kHead];
 };
-
-__device__ __forceinline__ half2_t pk_fma(half2_t x, half2_t y, half2_t z) { return __builtin_elementwise_fma(x, y, z); }
-
-// cuda/rwkv7_wkv_fp16_v2.cu:41-52
-__device__ __forceinline__ half_t decay_delta(half_t w_raw, const half_t* __restrict__ w0, int c, int phase) {
-  float w = h2f(w_raw);
-  if (w0) w += h2f(w0[c]);  // unrounded, as the reference's _w0 launchers
-  const unsigned prod = 2654435769u * static_cast<unsigned>(phase);
-  const float dither = 4.547473508864641e-13f * static_cast<float>(static_cast<int>(prod));
-  const float d = exp2f(-0.8750387749145276f / (1.0f + exp2f(-1.4426950408889634f * w))) - 1.0f + dither;
-  return f2h(d);
-}
-
-__device__ __forceinline__ void read_pairs(const half_t* __restrict__ src, half2_t (&dst)[kPairs]) {
-#pragma unroll
-  for (int q = 0; q < kPairs / 4; ++q) {
-    const uint4_t t = *reinterpret_cast<const uint4_t*>(src + 8 * q);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) dst[4 * q + e] = as_half2(t[e]);
-  }
-}
 
 __global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int H, half_t* __restrict__ state,
                                                               const half_t* __restrict__ r, const half_t* __restrict__ w,
@@ -82,7 +61,7 @@ __global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int 
     ops[0].b[lane] = b[tok];
     ops[0].k[lane] = k[tok];
     ops[0].r[lane] = r[tok];
-    ops[0].wd[lane] = decay_delta(w[tok], w0, c, phase0);
+    ops[0].wd[lane] = decay_delta16(w[tok], w0, c, phase0);
   }
   half_t v_cur = v[tok];
   __syncthreads();
@@ -94,36 +73,14 @@ __global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int 
     const int64_t tn = t + 1 < T ? tok + C : tok;
     const half_t a_n = a[tn], b_n = b[tn], k_n = k[tn], r_n = r[tn], w_n = w[tn], v_n = v[tn];
 
-    half2_t vec[kPairs];
-    read_pairs(cur.a, vec);
-    half2_t sa2 = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
-#pragma unroll
-    for (int j = 0; j < kPairs; ++j) sa2 = pk_fma(vec[j], S[j], sa2);
-    const half_t sa = sa2[0] + sa2[1];
-    const half2_t sa_b = {sa, sa};
-    const half2_t vv = {v_cur, v_cur};
-
-    half2_t bv[kPairs], kv[kPairs], wv[kPairs];
-    read_pairs(cur.b, bv);
-    read_pairs(cur.k, kv);
-    read_pairs(cur.wd, wv);
-    read_pairs(cur.r, vec);
-    half2_t y2 = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
-#pragma unroll
-    for (int j = 0; j < kPairs; ++j) {
-      const half2_t s = S[j];
-      const half2_t s_new = pk_fma(s, wv[j], pk_fma(kv[j], vv, pk_fma(sa_b, bv[j], s)));
-      S[j] = s_new;
-      y2 = pk_fma(s_new, vec[j], y2);
-    }
-    y[tok] = y2[0] + y2[1];
+    y[tok] = wkv16_row_step(S, cur.a, cur.b, cur.k, cur.wd, cur.r, v_cur);
 
     // hand the next token's operands to the other buffer (nobody reads it during this step)
     nxt.a[lane] = a_n;
     nxt.b[lane] = b_n;
     nxt.k[lane] = k_n;
     nxt.r[lane] = r_n;
-    nxt.wd[lane] = decay_delta(w_n, w0, c, phase0 + t + 1);
+    nxt.wd[lane] = decay_delta16(w_n, w0, c, phase0 + t + 1);
     v_cur = v_n;
     tok = tn;
     __syncthreads();

@@ -280,19 +280,20 @@ def test_greedy_stream_matches_oracle(gpu, orc):
     sess.close()
 
 
+@pytest.mark.parametrize("B", [1, 2])
 @pytest.mark.parametrize("fmt", [0, 1])
-def test_fp16_state_mode_prefill_and_decode_match_oracle(gpu, orc, fmt):
+def test_fp16_state_mode_prefill_and_decode_match_oracle(gpu, orc, fmt, B):
     """The reference server's default mode: the WKV state in fp16 and the recurrence in fp16 fused multiply-adds
     (session option; ModelBackend's use_wkv32 == false).  A 20-token prefill call (the w12 + w0 sum rounded to fp16
     first), a 9-token call and decode steps (w0 added inside the recurrence, unrounded) against the oracle's
     restatement of the same graph: logits cosine >= 0.9995, greedy tokens equal except for ties, the fp16 state
     within 2e-2 of its scale (both sides round the same quantities to fp16, from activations that differ by fp16
-    ulps)."""
+    ulps).  The decode steps run the single-launch time-mix core with the fp16-state step in its first wavefront;
+    at one row also with the gate rank-out in blocks of its own and the LayerNorm prologues."""
     from rwkv_lightning_cuda_amd.model import Session, State
     hip = gpu
     dims = small_dims()
     omodel, gmodel = build_pair(gpu, orc, dims, fmt, seed=61)
-    B = 2
     rng = np.random.default_rng(17)
     sess = Session(gmodel)
     gstate = State(dims, B, wkv_fp16=True)
@@ -326,7 +327,7 @@ def test_fp16_state_mode_prefill_and_decode_match_oracle(gpu, orc, fmt):
     assert err <= 2e-2
     assert gstate.elapsed.numpy().tolist() == [29 + 24] * B
     # the device-side greedy loop works in this mode too
-    got = sess.decode_greedy(np.array([3, 4]), 4, gstate, glogits)
+    got = sess.decode_greedy(np.arange(3, 3 + B), 4, gstate, glogits)
     assert got.shape == (4, B)
     sess.close()
 
