@@ -176,8 +176,10 @@ struct XRegs {
       const int idx = tid + i * T::GT;
       const int r = idx / (KC / 8);
       const int c = (idx % (KC / 8)) * 8;
-      xv[i] = uint4_t{0u, 0u, 0u, 0u};
-      if (m0 + r < g.M) xv[i] = *reinterpret_cast<const uint4_t*>(pr.x + static_cast<int64_t>(m0 + r) * g.K + kc + c);
+      // rows past M repeat the last row (their sums are never stored): a load under a per-lane branch, or merged
+      // with a default value, makes the compiler drain every load in flight at the head of the chunk loop
+      const int row = m0 + r < g.M ? m0 + r : g.M - 1;
+      xv[i] = *reinterpret_cast<const uint4_t*>(pr.x + static_cast<int64_t>(row) * g.K + kc + c);
     }
   }
 
@@ -197,7 +199,10 @@ template <int FMT, int MT, int KC>
 struct WRegs {
   using T = Tile<FMT, MT, KC>;
   uint4_t w[T::NW];
-  float sc[T::QG], zb[T::QG];
+  // int4 group scale and zero point as loaded: converted at their use in multiply().  Converted beside the loads,
+  // they would make every request wait for all the weights in flight.
+  half_t sc[T::QG];
+  uint32_t zb[T::QG];
 
   __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int kc, const uint4_t* wband,
                                           int n) {
@@ -209,8 +214,8 @@ struct WRegs {
       const int64_t q0 = static_cast<int64_t>(n) * (g.K >> 7) + (kc >> 7);
 #pragma unroll
       for (int q = 0; q < T::QG; ++q) {
-        sc[q] = h2f(pr.scale[q0 + q]);
-        zb[q] = 1024.0f + static_cast<float>(pr.zp[q0 + q]);
+        sc[q] = pr.scale[q0 + q];
+        zb[q] = pr.zp[q0 + q];
       }
     }
   }
@@ -222,6 +227,16 @@ struct WRegs {
                                            float16_t (&part)[MT][T::NACC]) const {
     using P = typename T::P;
     constexpr int NK = T::GROUPS * T::STEPS;
+    float scf[T::QG], zbf[T::QG];
+    if constexpr (FMT == RWKV_FMT_W4) {
+#pragma unroll
+      for (int q = 0; q < T::QG; ++q) {
+        uint32_t sr = __builtin_bit_cast(unsigned short, sc[q]), zr = zb[q];
+        asm volatile("" : "+v"(sr), "+v"(zr));  // the conversions stay here, below the requests of this chunk
+        scf[q] = h2f(__builtin_bit_cast(half_t, static_cast<unsigned short>(sr)));
+        zbf[q] = 1024.0f + static_cast<float>(zr);
+      }
+    }
     const half_t* xlane = xs + j * T::XSTRIDE + h * P::KR;
     half8_t a[2][MT];
     auto load_a = [&](int ks, half8_t (&dst)[MT]) {
@@ -245,7 +260,7 @@ struct WRegs {
         b = s == 0 ? expand_w8(piece[0], piece[1]) : expand_w8(piece[2], piece[3]);
       } else {
         const uint4_t piece = w[gi];
-        const half_t zf = static_cast<half_t>(zb[(gi * T::G) >> 7]);
+        const half_t zf = static_cast<half_t>(zbf[(gi * T::G) >> 7]);
         const half2_t bias = {zf, zf};
         b = expand_w4(piece[s], bias);
       }
@@ -261,7 +276,7 @@ struct WRegs {
       }
       if constexpr (FMT == RWKV_FMT_W4) {
         if (s == T::STEPS - 1 && ((gi + 1) * T::G) % 128 == 0) {  // end of a 128-group: fold with its scale
-          const float s128 = sc[(gi * T::G) >> 7];
+          const float s128 = scf[(gi * T::G) >> 7];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -328,6 +343,9 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
 
   // this lane's first piece of the band; consecutive pieces are 64 uint4 apart
   const uint4_t* wband = pr.wp + (static_cast<int64_t>(band) * (g.K / T::G)) * (P::PIECES * 64) + lane;
+  // the column's int8 scale now: read in the epilogue it costs every block a trip to memory (1.2 us per launch)
+  half_t scale_h = static_cast<half_t>(1.0f);
+  if constexpr (FMT == RWKV_FMT_W8) scale_h = pr.scale[n];
 
   constexpr int D = T::DEPTH;
   WRegs<FMT, MT, KC> wr[D];
@@ -340,9 +358,25 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
   xr[0].store_x(tid, xs);
   __syncthreads();
   constexpr int U = (D % 2 == 0) ? D : 2 * D;  // unroll: register sets and LDS tiles are indexed statically
-  for (int c0 = 0; c0 < nchunks; c0 += U) {
+  // Whole rounds of U chunks run as one basic block: with an exit between the chunks the compiler waits for every
+  // load in flight at the head of each round (the weight ring then drains once per round).  The chunks left over
+  // (K slices that are not a multiple of U chunks) take the same steps with the exits.
+  const int whole = nchunks - nchunks % U;
+  int c0 = 0;
+  for (; c0 < whole; c0 += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      xr[u & 1].request(g, pr, tid, m0, kbeg + (c + 2 <= last ? c + 2 : c) * KSTRIDE);
+      wr[(u + D - 1) % D].request(g, pr, kbeg + (c + D - 1 <= last ? c + D - 1 : c) * KSTRIDE, wband, n);
+      wr[u % D].multiply(xs + (u & 1) * T::kTileHalfs, j, h, acc, part);
+      xr[(u + 1) & 1].store_x(tid, xs + ((u + 1) & 1) * T::kTileHalfs);
+      __syncthreads();
+    }
+  }
+  if (c0 < nchunks) {
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u) {
       const int c = c0 + u;
       if (c >= nchunks) break;
       xr[u & 1].request(g, pr, tid, m0, kbeg + (c + 2 <= last ? c + 2 : c) * KSTRIDE);
@@ -380,10 +414,7 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
   }
   const bool partial_out = g.splits > 1;
   if (kg == 0) {
-    float scl = 1.0f;
-    if constexpr (FMT == RWKV_FMT_W8) {
-      if (!partial_out) scl = h2f(pr.scale[n]);
-    }
+    const float scl = partial_out ? 1.0f : h2f(scale_h);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -482,6 +513,12 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
     n[nb] = band * 32 + j;
     wband[nb] = pr.wp + (static_cast<int64_t>(band) * (g.K / T::G)) * (P::PIECES * 64) + lane;
   }
+  half_t scale_h[NB];  // the columns' int8 scales, requested before the main loop (see stream_block)
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    scale_h[nb] = static_cast<half_t>(1.0f);
+    if constexpr (FMT == RWKV_FMT_W8) scale_h[nb] = pr.scale[n[nb]];
+  }
 
   float16_t acc[NB][MT];
 #pragma unroll
@@ -536,9 +573,25 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
   };
 
   constexpr int U = (D % 2 == 0) ? D : 2 * D;
-  for (int c0 = 0; c0 < nchunks; c0 += U) {
+  // whole rounds of U chunks as one basic block, the chunks left over with exits between them (see stream_block)
+  const int whole = nchunks - nchunks % U;
+  int c0 = 0;
+  for (; c0 < whole; c0 += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      xr.request(g, pr, tid, m0, kbeg + (c + 1 <= last ? c + 1 : c) * KC);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        wr[(u + D - 1) % D][nb].request(g, pr, kbeg + (c + D - 1 <= last ? c + D - 1 : c) * KC, wband[nb], n[nb]);
+      multiply(xs + (u & 1) * T::kTileHalfs, wr[u % D]);
+      xr.store_x(tid, xs + ((u + 1) & 1) * T::kTileHalfs);
+      __syncthreads();
+    }
+  }
+  if (c0 < nchunks) {
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u) {
       const int c = c0 + u;
       if (c >= nchunks) break;
       xr.request(g, pr, tid, m0, kbeg + (c + 1 <= last ? c + 1 : c) * KC);
@@ -561,10 +614,7 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     if (nb > 0) __syncthreads();  // the previous half has been read
-    float scl = 1.0f;
-    if constexpr (FMT == RWKV_FMT_W8) {
-      if (!partial_out) scl = h2f(pr.scale[n[nb]]);
-    }
+    const float scl = partial_out ? 1.0f : h2f(scale_h[nb]);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll

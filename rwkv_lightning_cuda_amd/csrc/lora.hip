@@ -12,9 +12,12 @@
 // two fp16 terms, hi = f16(a) and lo = f16(a - hi): hi + lo carries 22 bits of a, both products with the fp16
 // weight are exact in fp32, and the result differs from an fp32 dot only by summation order.  Without an
 // activation the hidden is fp16 already and the lo term is skipped.  One launch takes up to four problems
-// (w, a, g, v of a layer): grid = (C/128, M/32, problems), block = 2 groups of 4 wavefronts x 32 output channels
-// (the groups take alternate 16-wide steps of the rank and add up through LDS), the 32 x R slice of act(h)
-// staged in LDS once per block.
+// (w, a, g, v of a layer): grid = (C/128, row blocks, problems), block = 2 groups of 4 wavefronts x 32 output
+// channels (the groups take alternate 16-wide steps of the rank and add up through LDS), the 32 x R slice of
+// act(h) of a row tile staged in LDS.
+#include <algorithm>
+#include <cstdint>
+
 #include "ops.h"
 
 namespace rwkv {
@@ -28,131 +31,159 @@ constexpr int kLoraKG = 2;       // wavefront groups that split the rank between
 constexpr int kLoraThreads = 2 * kLoraCols * kLoraKG;
 constexpr int kLoraStage = (kLoraRows * (kLoraMaxR / 8 + 1) + kLoraThreads - 1) / kLoraThreads;  // pieces per thread
 
-// Every lane first requests its whole weight row (up to 32 pieces of 8), the block turns its 32 x R slice of the
-// hidden into hi / lo fp16 in LDS while those loads are in flight (one barrier), then each wavefront runs its MFMA
-// steps.  Rows are R + 8 halves apart:
-// for ranks that are multiples of 16 the ds_read_b128 of lane (j, h) at j * (2R + 16) + 16h bytes is
-// conflict-free (other ranks lose some LDS bandwidth), and the zeroed 8-half pad is what the last MFMA step of
-// a rank that is not a multiple of 16 reads.
+// Per row tile: every lane requests its whole weight row (up to 16 pieces of 8; once per block - a block keeps
+// its weights over all its row tiles), its pieces of the 32 x R hidden slice and its piece of the epilogue
+// operands (v, v_first) in one go; the block turns the hidden slice into hi / lo fp16 in LDS (one barrier), each
+// wavefront runs its MFMA steps, both groups lay their 32 x 128 sums out in LDS (over the hi / lo tiles, free by
+// then) and all threads add the two in group order, apply the epilogue and write 16 bytes of a row each.
+//
+// Every load is issued without a per-lane branch around it: addresses past the rank or the last row are clamped to
+// a valid one and the value is dropped afterwards.  (A load under a per-lane branch, or merged with a default
+// value, makes the compiler wait for all loads in flight inside the branch: the trips to memory then run one
+// after the other.)  Conditions that are the same for a whole wavefront cost nothing of the kind.
+//
+// LDS rows are R + 8 halves apart: for ranks that are multiples of 16 the ds_read_b128 of lane (j, h) at
+// j * (2R + 16) + 16h bytes is conflict-free (other ranks lose some LDS bandwidth), and the zeroed 8-half pad is
+// what the last MFMA step of a rank that is not a multiple of 16 reads (its weights are the clamped, finite ones).
+constexpr int kLoraOutLd = kLoraCols + 4;  // fp32 row of the output tile in LDS
+
 __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs a) {
   __shared__ __attribute__((aligned(16))) half_t hi_s[kLoraRows * (kLoraMaxR + 8)];
   __shared__ __attribute__((aligned(16))) half_t lo_s[kLoraRows * (kLoraMaxR + 8)];
+  static_assert(kLoraRows * kLoraOutLd * 4 <= kLoraRows * (kLoraMaxR + 8) * 2, "output tile exceeds the hidden tile");
   const LoraOutProblem& p = a.p[blockIdx.z];
   const int R = p.R;
   const int ld = R + 8;
-  const int m0 = blockIdx.y * kLoraRows;
-  const int mn = min(kLoraRows, a.M - m0);
-  const int wave = (threadIdx.x >> 6) & 3;
-  const int kg = threadIdx.x >> 8;  // this wavefront's share of the rank: steps kg, kg + 2, ...
+  // wavefront-wide values, said so to the compiler: conditions on them become scalar branches
+  const int wave = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3);
+  const int kg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);  // its share of the rank: steps kg, kg + 2, ...
   const int lane = threadIdx.x & 63;
   const int j = lane & 31;
   const int h = lane >> 5;
   const int c = blockIdx.x * kLoraCols + wave * 32 + j;
-  const bool col_ok = c < a.C;
   const bool split = p.act != RWKV_ACT_NONE;
-  const half_t* wrow = p.w2 + static_cast<int64_t>(col_ok ? c : 0) * R;
+  const half_t* wrow = p.w2 + static_cast<int64_t>(c < a.C ? c : a.C - 1) * R;
 
-  // this lane's W2 values, all requested before the activation work: k = 16*kk + 8h .. +8 of output channel c
-  half8_t w[kLoraMaxR / 16 / kLoraKG];
+  // this lane's W2 values: k = 16*step + 8h .. +8 of output channel c
+  constexpr int kSteps = kLoraMaxR / 16 / kLoraKG;
+  half8_t w[kSteps];
 #pragma unroll
-  for (int i = 0; i < kLoraMaxR / 16 / kLoraKG; ++i) {
-    const int k = (i * kLoraKG + kg) * 16 + h * 8;
-    if (k < R) {
-      w[i] = *reinterpret_cast<const half8_t*>(wrow + k);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) w[i][e] = static_cast<half_t>(0.0f);
+  for (int i = 0; i < kSteps; ++i) {
+    const int k0 = (i * kLoraKG + kg) * 16;  // the same for the whole wavefront
+    if (k0 < R) {
+      const int k = k0 + h * 8;
+      w[i] = *reinterpret_cast<const half8_t*>(wrow + (k < R ? k : R - 8));
     }
   }
 
-  // activation of the 32 x R hidden slice, split into hi + lo; R/8 pieces of 8 per row + the zeroed pad.  All of
-  // a thread's pieces are requested before the first is used.
-  const int pieces = (R >> 3) + 1;
-  half8_t hv[kLoraStage];
+  // the epilogue's view of the tile: thread t owns channels 8*(t%16) .. +8 of row t/16
+  const int orow = threadIdx.x >> 4;
+  const int ocol = blockIdx.x * kLoraCols + (threadIdx.x & 15) * 8;
+  const bool ocol_ok = ocol < a.C;
+  // without a bias any readable address does (C values of W2); the values are dropped in the epilogue
+  uint4_t bias_raw = *reinterpret_cast<const uint4_t*>((p.bias ? p.bias : p.w2) + (ocol_ok ? ocol : 0));
+
+  const int pieces = (R >> 3) + 1;  // R/8 pieces of 8 per row + the zeroed pad
+  const int row_tiles = (a.M + kLoraRows - 1) / kLoraRows;
+  for (int rt = blockIdx.y; rt < row_tiles; rt += gridDim.y) {
+    const int m0 = rt * kLoraRows;
+    const int mn = min(kLoraRows, a.M - m0);
+    uint4_t hv[kLoraStage];  // all of them loaded, whatever the rank: a value left undefined costs more than the load
 #pragma unroll
-  for (int i = 0; i < kLoraStage; ++i) {
-    const int idx = threadIdx.x + i * kLoraThreads;
-    const int m = idx / pieces;
-    const int ks = (idx - m * pieces) * 8;
+    for (int i = 0; i < kLoraStage; ++i) {
+      const int idx = threadIdx.x + i * kLoraThreads;
+      const int m = idx / pieces;
+      const int ks = (idx - m * pieces) * 8;
+      hv[i] = *reinterpret_cast<const uint4_t*>(p.h + static_cast<int64_t>(m0 + (m < mn ? m : mn - 1)) * R +
+                                                (ks < R ? ks : R - 8));
+    }
+    const int64_t o = static_cast<int64_t>(m0 + (orow < mn ? orow : mn - 1)) * a.C + (ocol_ok ? ocol : 0);
+    // without the v-residual gate: the output row itself, readable and unused
+    half8_t v8 = *reinterpret_cast<const half8_t*>((p.vres ? p.v : p.out) + o);
+    half8_t vf8 = *reinterpret_cast<const half8_t*>((p.vres ? p.v_first : p.out) + o);
+    __builtin_amdgcn_sched_barrier(0);
+    // keeps the conversion of the bias below the loads above: moved up beside its own load, it would wait for the
+    // weights before the hidden slice is even requested
+    asm volatile("" : "+v"(bias_raw));
+    const half8_t bias8 = __builtin_bit_cast(half8_t, bias_raw);
+
 #pragma unroll
-    for (int e = 0; e < 8; ++e) hv[i][e] = static_cast<half_t>(0.0f);
-    if (m < mn && ks < R) hv[i] = *reinterpret_cast<const half8_t*>(p.h + static_cast<int64_t>(m0 + m) * R + ks);
-  }
+    for (int i = 0; i < kLoraStage; ++i) {
+      if (i * kLoraThreads < kLoraRows * pieces) {
+        const int idx = threadIdx.x + i * kLoraThreads;
+        const int m = idx / pieces;
+        const int ks = (idx - m * pieces) * 8;
+        if (m < kLoraRows) {
+          const bool live = m < mn && ks < R;  // rows past M and the pad hold exact zeros
+          const half8_t raw = __builtin_bit_cast(half8_t, hv[i]);
+          half8_t hi, lo;
 #pragma unroll
-  for (int i = 0; i < kLoraStage; ++i) {
-    const int idx = threadIdx.x + i * kLoraThreads;
-    const int m = idx / pieces;
-    const int ks = (idx - m * pieces) * 8;
-    if (m < kLoraRows) {
-      half8_t hi, lo;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        // rows past M and the pad hold zeros: every activation here maps them to values whose weights are zero
-        // or whose rows are never stored, but the pad must be exactly zero
-        float f = h2f(hv[i][e]);
-        if (p.act == RWKV_ACT_TANH) f = tanh_f(f);
-        if (p.act == RWKV_ACT_SIGMOID) f = sigmoid_f(f);
-        if (ks >= R) f = 0.0f;
-        hi[e] = f2h(f);
-        lo[e] = f2h(f - h2f(hi[e]));
+          for (int e = 0; e < 8; ++e) {
+            float f = h2f(raw[e]);
+            if (p.act == RWKV_ACT_TANH) f = tanh_f(f);
+            if (p.act == RWKV_ACT_SIGMOID) f = sigmoid_f(f);
+            if (!live) f = 0.0f;
+            hi[e] = f2h(f);
+            lo[e] = f2h(f - h2f(hi[e]));
+          }
+          *reinterpret_cast<half8_t*>(&hi_s[m * ld + ks]) = hi;
+          if (split) *reinterpret_cast<half8_t*>(&lo_s[m * ld + ks]) = lo;
+        }
       }
-      *reinterpret_cast<half8_t*>(&hi_s[m * ld + ks]) = hi;
-      if (split) *reinterpret_cast<half8_t*>(&lo_s[m * ld + ks]) = lo;
     }
-  }
-  __syncthreads();
+    __syncthreads();
 
-  float16_t acc;
+    float16_t acc;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kLoraMaxR / 16 / kLoraKG; ++i) {
-    const int k = (i * kLoraKG + kg) * 16;
-    if (k < R) {
-      const half8_t ah = *reinterpret_cast<const half8_t*>(&hi_s[j * ld + k + h * 8]);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, w[i], acc, 0, 0, 0);
-      if (split) {
-        const half8_t al = *reinterpret_cast<const half8_t*>(&lo_s[j * ld + k + h * 8]);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, w[i], acc, 0, 0, 0);
+    for (int i = 0; i < kSteps; ++i) {
+      const int k = (i * kLoraKG + kg) * 16;
+      if (k < R) {
+        const half8_t ah = *reinterpret_cast<const half8_t*>(&hi_s[j * ld + k + h * 8]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, w[i], acc, 0, 0, 0);
+        if (split) {
+          const half8_t al = *reinterpret_cast<const half8_t*>(&lo_s[j * ld + k + h * 8]);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, w[i], acc, 0, 0, 0);
+        }
       }
     }
-  }
-  // the second group's sums go through LDS (over the lo tile, which nobody reads any more) to the first
-  __syncthreads();
-  float* xch = reinterpret_cast<float*>(lo_s) + (wave * 64 + lane) * 16;
-  if (kg == 1) {
+    __syncthreads();  // the hidden tiles are free: group 0 lays its sums over hi_s, group 1 over lo_s
+    // accumulator v of lane (j, h): row 8*(v/4) + 4h + v%4, column wave*32 + j
+    float* tile = reinterpret_cast<float*>(kg == 0 ? hi_s : lo_s);
 #pragma unroll
-    for (int v = 0; v < 16; v += 4) *reinterpret_cast<float4_t*>(xch + v) = float4_t{acc[v], acc[v + 1], acc[v + 2], acc[v + 3]};
-  }
-  __syncthreads();
-  if (kg == 1) return;
-#pragma unroll
-  for (int v = 0; v < 16; v += 4) {
-    const float4_t o = *reinterpret_cast<const float4_t*>(xch + v);
-    acc[v] += o[0]; acc[v + 1] += o[1]; acc[v + 2] += o[2]; acc[v + 3] += o[3];
-  }
+    for (int v = 0; v < 16; ++v) tile[(8 * (v / 4) + 4 * h + (v % 4)) * kLoraOutLd + wave * 32 + j] = acc[v];
+    __syncthreads();
 
-  if (!col_ok) return;
-  const float bias = p.bias ? h2f(p.bias[c]) : 0.0f;
-  // accumulator v of lane (j, h): row 8*(v/4) + 4h + v%4, column j
+    const float* t0 = reinterpret_cast<const float*>(hi_s) + orow * kLoraOutLd + (threadIdx.x & 15) * 8;
+    const float* t1 = reinterpret_cast<const float*>(lo_s) + orow * kLoraOutLd + (threadIdx.x & 15) * 8;
+    float sum[8];
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int m = 8 * (v / 4) + 4 * h + (v % 4);
-    if (m < mn) {
-      const int64_t o = static_cast<int64_t>(m0 + m) * a.C + c;
-      float res;
+    for (int q = 0; q < 2; ++q) {
+      const float4_t s0 = *reinterpret_cast<const float4_t*>(t0 + 4 * q);
+      const float4_t s1 = *reinterpret_cast<const float4_t*>(t1 + 4 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum[4 * q + e] = s0[e] + s1[e];
+    }
+    half8_t res;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float b = p.bias ? h2f(bias8[e]) : 0.0f;
       if (p.vres) {
-        const float vv = h2f(p.v[o]);
-        const float gate = sigmoid_f(bias + acc[v]);
-        res = vv + (h2f(p.v_first[o]) - vv) * gate;
+        const float vv = h2f(v8[e]);
+        const float gate = sigmoid_f(b + sum[e]);
+        res[e] = f2h(vv + (h2f(vf8[e]) - vv) * gate);
       } else {
-        res = acc[v] + bias;
+        res[e] = f2h(sum[e] + b);
       }
-      p.out[o] = f2h(res);
     }
+    if (orow < mn && ocol_ok) *reinterpret_cast<half8_t*>(p.out + o) = res;
+    __syncthreads();  // the tiles are rewritten by the next row tile
   }
 }
 
+// Row tiles per block: one up to 256 rows; beyond that the blocks of a problem walk the row tiles with a stride, so
+// that the weights of a block are requested once for several tiles and the grid stays at a few blocks per CU.
 int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a) {
   RWKV_REQUIRE(a.n >= 1 && a.n <= 4, "lora_out: %d problems (1..4)", a.n);
   RWKV_REQUIRE(a.M > 0 && a.C > 0 && a.C % 32 == 0, "lora_out: C (%d) must be a positive multiple of 32", a.C);
@@ -162,9 +193,14 @@ int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a) {
                  p.R, kLoraMaxR);
     RWKV_REQUIRE(p.h && p.w2 && p.out, "lora_out: NULL tensor");
     RWKV_REQUIRE(!p.vres || (p.v && p.v_first && p.bias), "lora_out: v-residual gate needs v, v_first and v0");
+    RWKV_REQUIRE((reinterpret_cast<uintptr_t>(p.h) | reinterpret_cast<uintptr_t>(p.w2) | reinterpret_cast<uintptr_t>(p.out) |
+                  reinterpret_cast<uintptr_t>(p.bias) | reinterpret_cast<uintptr_t>(p.v) |
+                  reinterpret_cast<uintptr_t>(p.v_first)) % 16 == 0,
+                 "lora_out: tensors must be 16-byte aligned");
   }
-  hipLaunchKernelGGL(lora_out_kernel, dim3(ceil_div(a.C, kLoraCols), ceil_div(a.M, kLoraRows), a.n), dim3(kLoraThreads), 0, st,
-                     a);
+  const int row_tiles = ceil_div(a.M, kLoraRows);
+  const int row_blocks = row_tiles <= 8 ? row_tiles : std::max(8, ceil_div(row_tiles, 8));
+  hipLaunchKernelGGL(lora_out_kernel, dim3(ceil_div(a.C, kLoraCols), row_blocks, a.n), dim3(kLoraThreads), 0, st, a);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }

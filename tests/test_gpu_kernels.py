@@ -512,7 +512,30 @@ def test_kk_gate_groupnorm_lora(gpu, orc):
             assert err <= F16_TOL
 
 
-@pytest.mark.parametrize("rows,C,R", [(1, 96, 8), (33, 256, 136), (70, 768, 480), (128, 4096, 512), (64, 4096, 96)])
+def test_lora_out_blocks_walk_several_row_tiles(gpu, orc):
+    """Beyond 256 rows a block keeps its weights and walks several 32-row tiles; the last tile here is partial.  The
+    v-residual epilogue is checked on the same rows."""
+    hip = gpu
+    rng = np.random.default_rng(77)
+    rows, C, R = 300 + 13, 256, 40
+    h = rng.standard_normal((rows, R)).astype(np.float16)
+    w2 = (rng.standard_normal((C, R)) * 0.1).astype(np.float16)
+    v, v_first = (rng.standard_normal((rows, C)).astype(np.float16) for _ in range(2))
+    v0 = (rng.standard_normal(C) * 0.3).astype(np.float16)
+    o32 = (h.astype(np.float64) @ w2.astype(np.float64).T).astype(np.float32)
+    o = hip.DeviceArray((rows, C), np.float16)
+    hip.lora_out(rows, C, R, hip.ACT_NONE, dev(hip, h), dev(hip, w2), o)
+    og = hip.DeviceArray((rows, C), np.float16)
+    hip.lora_out(rows, C, R, hip.ACT_NONE, dev(hip, h), dev(hip, w2), og, bias=dev(hip, v0), vres=1, v=dev(hip, v),
+                 v_first=dev(hip, v_first))
+    hip.device_sync()
+    assert rel_err(o.numpy().astype(np.float32), o32) <= F16_TOL
+    ref = orc.vres_gate(v, v_first, v0, o32)
+    assert rel_err(og.numpy().astype(np.float32), ref.astype(np.float32)) <= F16_TOL
+
+
+@pytest.mark.parametrize("rows,C,R", [(1, 96, 8), (33, 256, 136), (70, 768, 480), (128, 4096, 512), (64, 4096, 96),
+                                      (700, 384, 136)])
 def test_lora_out_keeps_the_activated_hidden_in_fp32(gpu, rows, C, R):
     """The rank-out product feeds act(h) to the matrix core as an fp16 hi + lo pair.  Against a float64 dot over
     the float32 activation, the fp16 result is the correctly rounded one except at near-ties; with the lo term
