@@ -66,10 +66,28 @@ __global__ __launch_bounds__(NT) void ln_fused_kernel(LnArgs a) {
           const float* pp = a.res_partial + src + c;
           float4_t s0 = *reinterpret_cast<const float4_t*>(pp);
           float4_t s1 = *reinterpret_cast<const float4_t*>(pp + 4);
-#pragma unroll 4
-          for (int sp = 1; sp < a.res_splits; ++sp) {
-            s0 = s0 + *reinterpret_cast<const float4_t*>(pp + sp * a.res_plane);
-            s1 = s1 + *reinterpret_cast<const float4_t*>(pp + sp * a.res_plane + 4);
+          // The other partials four at a time, all requested before the first is added (in split order, as
+          // always); past the last split the last one is read again and left out.  A plain loop over the splits
+          // would wait for each partial before it asks for the next: one trip to memory per split.
+          for (int base = 1; base < a.res_splits; base += 4) {
+            float4_t q0[4], q1[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int sp = base + u < a.res_splits ? base + u : a.res_splits - 1;
+              q0[u] = *reinterpret_cast<const float4_t*>(pp + sp * a.res_plane);
+              q1[u] = *reinterpret_cast<const float4_t*>(pp + sp * a.res_plane + 4);
+            }
+            // (keeps the four requests together: their only uses sit under the conditions below, and the compiler
+            // would move each load down into its condition)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(q0[u]), "+v"(q1[u]));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              if (base + u < a.res_splits) {
+                s0 = s0 + q0[u];
+                s1 = s1 + q1[u];
+              }
+            }
           }
           float scl[8];
 #pragma unroll

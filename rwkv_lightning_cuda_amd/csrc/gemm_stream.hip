@@ -691,21 +691,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs g) {
   const int64_t i = static_cast<int64_t>(blockIdx.x - (pi > 0 ? g.block_end[pi - 1] : 0)) * 256 + threadIdx.x;
   if (i >= plane4) return;
   const float4_t* partial = pr.partial;
+  // the scale first (without one: any readable vector), then the partials four at a time, each group requested
+  // whole before its first member is added, in split order; past the last split the last one is read again and
+  // left out - no load waits for an earlier one
+  const half4_t sv = *reinterpret_cast<const half4_t*>(pr.scale ? pr.scale + (i % pr.N4) * 4
+                                                                : reinterpret_cast<const half_t*>(partial));
   float4_t sum = partial[i];
-  int s = 1;
-  for (; s + 4 <= g.splits; s += 4) {
-    const float4_t p0 = partial[(s + 0) * plane4 + i];
-    const float4_t p1 = partial[(s + 1) * plane4 + i];
-    const float4_t p2 = partial[(s + 2) * plane4 + i];
-    const float4_t p3 = partial[(s + 3) * plane4 + i];
-    sum = (((sum + p0) + p1) + p2) + p3;
+  for (int base = 1; base < g.splits; base += 4) {
+    float4_t q[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) q[u] = partial[(base + u < g.splits ? base + u : g.splits - 1) * plane4 + i];
+    // (keeps the four requests together: the compiler would move each load down into the condition of its use)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(q[u]));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (base + u < g.splits) sum = sum + q[u];
   }
-  for (; s < g.splits; ++s) sum = sum + partial[s * plane4 + i];
   float4_t scl = {1.0f, 1.0f, 1.0f, 1.0f};
-  if (pr.scale) {
-    const half4_t sv = *reinterpret_cast<const half4_t*>(pr.scale + (i % pr.N4) * 4);
-    scl = float4_t{h2f(sv[0]), h2f(sv[1]), h2f(sv[2]), h2f(sv[3])};
-  }
+  if (pr.scale) scl = float4_t{h2f(sv[0]), h2f(sv[1]), h2f(sv[2]), h2f(sv[3])};
   float4_t val;
 #pragma unroll
   for (int c = 0; c < 4; ++c) val[c] = finish_value(mul_f32(sum[c], scl[c]), g.epilogue);
