@@ -170,27 +170,31 @@ struct XRegs {
   using T = Tile<FMT, MT, KC, WG>;
   uint4_t xv[T::XV];
 
+  // vector i of the thread's slice
+  __device__ __forceinline__ void request_one(int i, const StreamArgs& g, const StreamProblem& pr, int tid, int m0, int kc) {
+    const int idx = tid + i * T::GT;
+    const int r = idx / (KC / 8);
+    const int c = (idx % (KC / 8)) * 8;
+    // rows past M repeat the last row (their sums are never stored): a load under a per-lane branch, or merged
+    // with a default value, makes the compiler drain every load in flight at the head of the chunk loop
+    const int row = m0 + r < g.M ? m0 + r : g.M - 1;
+    xv[i] = *reinterpret_cast<const uint4_t*>(pr.x + static_cast<int64_t>(row) * g.K + kc + c);
+  }
+  __device__ __forceinline__ void store_one(int i, int tid, half_t* xs) const {
+    const int idx = tid + i * T::GT;
+    const int r = idx / (KC / 8);
+    const int c = (idx % (KC / 8)) * 8;
+    *reinterpret_cast<uint4_t*>(xs + r * T::XSTRIDE + c) = xv[i];
+  }
+
   __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int tid, int m0, int kc) {
 #pragma unroll
-    for (int i = 0; i < T::XV; ++i) {
-      const int idx = tid + i * T::GT;
-      const int r = idx / (KC / 8);
-      const int c = (idx % (KC / 8)) * 8;
-      // rows past M repeat the last row (their sums are never stored): a load under a per-lane branch, or merged
-      // with a default value, makes the compiler drain every load in flight at the head of the chunk loop
-      const int row = m0 + r < g.M ? m0 + r : g.M - 1;
-      xv[i] = *reinterpret_cast<const uint4_t*>(pr.x + static_cast<int64_t>(row) * g.K + kc + c);
-    }
+    for (int i = 0; i < T::XV; ++i) request_one(i, g, pr, tid, m0, kc);
   }
 
   __device__ __forceinline__ void store_x(int tid, half_t* xs) const {
 #pragma unroll
-    for (int i = 0; i < T::XV; ++i) {
-      const int idx = tid + i * T::GT;
-      const int r = idx / (KC / 8);
-      const int c = (idx % (KC / 8)) * 8;
-      *reinterpret_cast<uint4_t*>(xs + r * T::XSTRIDE + c) = xv[i];
-    }
+    for (int i = 0; i < T::XV; ++i) store_one(i, tid, xs);
   }
 };
 
@@ -203,6 +207,12 @@ struct WRegs {
   // they would make every request wait for all the weights in flight.
   half_t sc[T::QG];
   uint32_t zb[T::QG];
+
+  // piece i of the chunk at kc (fp16 and int8 codes: no group scales)
+  __device__ __forceinline__ void request_piece(int i, int kc, const uint4_t* wband) {
+    using P = typename T::P;
+    w[i] = wband[static_cast<int64_t>(kc / T::G) * (P::PIECES * 64) + i * 64];
+  }
 
   __device__ __forceinline__ void request(const StreamArgs& g, const StreamProblem& pr, int kc, const uint4_t* wband,
                                           int n) {
@@ -484,10 +494,19 @@ __global__ __launch_bounds__(64 * WG * KG) void gemm_stream_kernel(StreamArgs g)
 // (wave w: bands w and w + 4 of the block), so each X fragment feeds two MFMAs and a block reads X from L2 half as
 // often.  One group of four wavefronts, one wavefront per SIMD (128 accumulator registers per lane); int8 and
 // fp16 weights (the int4 path would double the accumulators once more and stays on the narrower tile).
-template <int FMT>
+//
+// ROLL (int8 weights only): the variant that fits two wavefronts per SIMD (at most 256 registers).  Alone on its
+// SIMD a wavefront overlaps nothing - measured per 128-k chunk: 1.18 us of MFMAs, and on top of them, one after the
+// other, 0.2 us for the weight requests, 0.2 for the X requests and stores, 0.18 for the code expansion, 0.1 for
+// the LDS reads - so a second wavefront, whose MFMAs fill those gaps, is worth more than deep prefetch.  The
+// registers come from the weights: one set per band instead of a ring of sets, each piece requested again for the
+// next chunk right after its last use (six MFMA steps ahead), and from X: one set, requested during the first
+// half of a chunk's steps and stored during the second.
+template <int FMT, bool ROLL, int MT>
 __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const StreamProblem& pr, int row_tile, int col_block,
                                                   int split, half_t* xs) {
-  constexpr int MT = 4, KC = 128, NB = 2;
+  static_assert(!ROLL || FMT == RWKV_FMT_W8, "the rolling weight set is laid out for int8 pieces (two MFMA steps each)");
+  constexpr int KC = 128, NB = 2;
   using T = Tile<FMT, MT, KC, 4>;
   using P = typename T::P;
   constexpr int BM = T::BM;
@@ -528,20 +547,97 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[nb][mt][v] = 0.0f;
 
+  constexpr int NK = T::GROUPS * T::STEPS;        // MFMA steps of a chunk
+  if constexpr (ROLL) {
+    WRegs<FMT, MT, KC> w[NB];
+    XRegs<FMT, MT, KC, 4> xq;
+    const int last = nchunks - 1;
+    xq.request(g, pr, tid, m0, kbeg);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) w[nb].request(g, pr, kbeg, wband[nb], n[nb]);
+    xq.store_x(tid, xs);
+    __syncthreads();
+    static_assert(T::XV % (NK / 2) == 0 && T::STEPS == 2 && T::NW == T::GROUPS,
+                  "a whole number of X vectors per MFMA step, two steps per weight piece");
+    constexpr int XPS = T::XV / (NK / 2);  // X vectors requested (first half of the steps) or stored (second half) per step
+    auto chunk = [&](int u, int c) {
+      const half_t* tile = xs + (u & 1) * T::kTileHalfs;
+      half_t* tile_next = xs + ((u + 1) & 1) * T::kTileHalfs;
+      const int knext = kbeg + (c + 1 <= last ? c + 1 : c) * KC;  // past the end: the current chunk again (in cache)
+      const half_t* xlane = tile + j * T::XSTRIDE + h * P::KR;
+      half8_t a[2][MT];
+      auto load_a = [&](int ks, half8_t (&dst)[MT]) {
+        const half_t* xa = xlane + (ks / T::STEPS) * T::G + 8 * (ks % T::STEPS);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) dst[mt] = *reinterpret_cast<const half8_t*>(xa + mt * 32 * T::XSTRIDE);
+      };
+      load_a(0, a[0]);
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) {
+        const int gi = ks / T::STEPS;
+        const int st = ks % T::STEPS;
+        if (ks + 1 < NK) load_a(ks + 1, a[(ks + 1) & 1]);
+#pragma unroll
+        for (int i = 0; i < XPS; ++i) {
+          if (ks < NK / 2) {
+            xq.request_one(XPS * ks + i, g, pr, tid, m0, knext);
+          } else {
+            xq.store_one(XPS * (ks - NK / 2) + i, tid, tile_next);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const uint4_t piece = w[nb].w[gi];
+          const half8_t b = st == 0 ? expand_w8(piece[0], piece[1]) : expand_w8(piece[2], piece[3]);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[nb][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks & 1][mt], b, acc[nb][mt], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (st == T::STEPS - 1) {  // piece gi has been expanded for the last time: the next chunk's takes its place
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) w[nb].request_piece(gi, knext, wband[nb]);
+        }
+      }
+      __syncthreads();
+    };
+    const int whole = nchunks - nchunks % 2;
+    int c0 = 0;
+    for (; c0 < whole; c0 += 2) {
+      chunk(0, c0);
+      chunk(1, c0 + 1);
+    }
+    if (c0 < nchunks) chunk(0, c0);
+  } else {
   constexpr int D = FMT == RWKV_FMT_F16 ? 2 : 3;  // weight register sets per band
+  constexpr int WPS = NB * T::NW / NK;            // weight pieces requested per MFMA step (1 int8, 2 fp16)
+  static_assert(T::XV == NK && NB * T::NW % NK == 0, "one X vector and a whole number of weight pieces per MFMA step");
+  static_assert(MT == 4, "the ring variant is the 128-row tile");
   WRegs<FMT, MT, KC> wr[D][NB];
-  XRegs<FMT, MT, KC, 4> xr;  // one chunk ahead: a chunk is 64 MFMAs per wavefront, longer than a trip to L2
+  XRegs<FMT, MT, KC, 4> xr[2];
   const int last = nchunks - 1;
-  xr.request(g, pr, tid, m0, kbeg);
+  xr[0].request(g, pr, tid, m0, kbeg);
+  xr[1].request(g, pr, tid, m0, kbeg + min(1, last) * KC);
 #pragma unroll
   for (int i = 0; i < D - 1; ++i)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) wr[i][nb].request(g, pr, kbeg + min(i, last) * KC, wband[nb], n[nb]);
-  xr.store_x(tid, xs);
+  xr[0].store_x(tid, xs);
   __syncthreads();
 
-  constexpr int NK = T::GROUPS * T::STEPS;
-  auto multiply = [&](const half_t* tile, const WRegs<FMT, MT, KC> (&w)[NB]) {
+  // Chunk c out of LDS tile u & 1 with the weights of ring set u % D.  A wavefront is alone on its SIMD (its 128
+  // accumulator registers leave no room for a second one), so whatever it issues besides MFMAs leaves the matrix
+  // core idle: the memory work of a chunk is spread over its MFMA steps instead of standing in a block at its
+  // head - each step stores one vector of the next chunk's X (requested during the previous chunk) into the other
+  // tile, requests one vector of the X of the chunk after that into the register set just freed and WPS pieces of
+  // the weights D - 1 chunks ahead.  (Issued in one block, the 16 requests of a chunk took a wavefront 0.5 us of a
+  // 2.2 us chunk: four wavefronts queue for the one address unit of the CU.)
+  auto chunk = [&](int u, int c) {
+    const half_t* tile = xs + (u & 1) * T::kTileHalfs;
+    half_t* tile_next = xs + ((u + 1) & 1) * T::kTileHalfs;
+    const int kx = kbeg + (c + 2 <= last ? c + 2 : c) * KC;
+    const int kw = kbeg + (c + D - 1 <= last ? c + D - 1 : c) * KC;
+    const WRegs<FMT, MT, KC> (&w)[NB] = wr[u % D];
     const half_t* xlane = tile + j * T::XSTRIDE + h * P::KR;
     half8_t a[2][MT];
     auto load_a = [&](int ks, half8_t (&dst)[MT]) {
@@ -555,6 +651,10 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
       const int gi = ks / T::STEPS;
       const int st = ks % T::STEPS;
       if (ks + 1 < NK) load_a(ks + 1, a[(ks + 1) & 1]);
+      xr[(u + 1) & 1].store_one(ks, tid, tile_next);
+      xr[u & 1].request_one(ks, g, pr, tid, m0, kx);
+#pragma unroll
+      for (int q = ks * WPS; q < (ks + 1) * WPS; ++q) wr[(u + D - 1) % D][q / T::NW].request_piece(q % T::NW, kw, wband[q / T::NW]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
@@ -570,6 +670,7 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    __syncthreads();
   };
 
   constexpr int U = (D % 2 == 0) ? D : 2 * D;
@@ -578,31 +679,16 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
   int c0 = 0;
   for (; c0 < whole; c0 += U) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int c = c0 + u;
-      xr.request(g, pr, tid, m0, kbeg + (c + 1 <= last ? c + 1 : c) * KC);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        wr[(u + D - 1) % D][nb].request(g, pr, kbeg + (c + D - 1 <= last ? c + D - 1 : c) * KC, wband[nb], n[nb]);
-      multiply(xs + (u & 1) * T::kTileHalfs, wr[u % D]);
-      xr.store_x(tid, xs + ((u + 1) & 1) * T::kTileHalfs);
-      __syncthreads();
-    }
+    for (int u = 0; u < U; ++u) chunk(u, c0 + u);
   }
   if (c0 < nchunks) {
 #pragma unroll
     for (int u = 0; u < U - 1; ++u) {
-      const int c = c0 + u;
-      if (c >= nchunks) break;
-      xr.request(g, pr, tid, m0, kbeg + (c + 1 <= last ? c + 1 : c) * KC);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        wr[(u + D - 1) % D][nb].request(g, pr, kbeg + (c + D - 1 <= last ? c + D - 1 : c) * KC, wband[nb], n[nb]);
-      multiply(xs + (u & 1) * T::kTileHalfs, wr[u % D]);
-      xr.store_x(tid, xs + ((u + 1) & 1) * T::kTileHalfs);
-      __syncthreads();
+      if (c0 + u >= nchunks) break;
+      chunk(u, c0 + u);
     }
   }
+  }  // !ROLL
 
   // output: one 128-column half of the tile at a time through LDS (the X tiles are free), written in 16/32-byte
   // pieces along the rows
@@ -650,8 +736,11 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
   }
 }
 
-__global__ __launch_bounds__(256) void gemm_stream_wide_kernel(StreamArgs g) {
-  __shared__ __align__(16) half_t xs[2 * 128 * (128 + 8)];
+// MIXED: the problems of the launch may be int8 or fp16 (one wavefront per SIMD); otherwise all are int8 and two
+// blocks share a CU.
+template <bool MIXED, int MT>
+__global__ __launch_bounds__(256, MIXED ? 1 : 2) void gemm_stream_wide_kernel(StreamArgs g) {
+  __shared__ __align__(16) half_t xs[2 * 32 * MT * (128 + 8)];
   const int id = blockIdx.x;
   const int row_tile = (id >> 3) % g.row_tiles;
   const int pair = (id / (8 * g.row_tiles)) * 8 + (id & 7);
@@ -662,10 +751,12 @@ __global__ __launch_bounds__(256) void gemm_stream_wide_kernel(StreamArgs g) {
   while (pi + 1 < g.n_problems && col_all >= g.block_end[pi]) ++pi;
   const int col_block = col_all - (pi > 0 ? g.block_end[pi - 1] : 0);
   const StreamProblem& pr = g.p[pi];
-  if (pr.fmt == RWKV_FMT_W8) {
-    stream_block_wide<RWKV_FMT_W8>(g, pr, row_tile, col_block, split, xs);
+  if constexpr (!MIXED) {
+    stream_block_wide<RWKV_FMT_W8, true, MT>(g, pr, row_tile, col_block, split, xs);
+  } else if (pr.fmt == RWKV_FMT_W8) {
+    stream_block_wide<RWKV_FMT_W8, false, MT>(g, pr, row_tile, col_block, split, xs);
   } else {
-    stream_block_wide<RWKV_FMT_F16>(g, pr, row_tile, col_block, split, xs);
+    stream_block_wide<RWKV_FMT_F16, false, MT>(g, pr, row_tile, col_block, split, xs);
   }
 }
 
@@ -766,6 +857,15 @@ static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns, c
   // split of 64-row tiles for the same number of blocks (128 rows x 4096 x 4096: 19.8 -> 16.6 us; with K = 16384
   // the 64-row tiles win, 35.5 us against 38.1)
   if (M <= 128 && K <= 4096 && ceil_div(M, 64) * cb128 * 2 <= target_blocks()) return StreamConfig{1, 128, 2, 4};
+  // 129..1024 rows, int8 weights only, and K up to 4096 or up to 384 rows: the 64 x 256 tile of two bands per
+  // wavefront that fits three wavefronts per SIMD (us, 64 x 256 / 128 x 256 / 64 x 128 tiles; * = with a K split:
+  // 256 rows x 16384 x 4096 51 / 59* / 64, 384 x 16384 x 4096 74 / 100* / 105, 384 x 4096 x 16384 85* / 96* / 112*,
+  // 768 x 12288 x 4096 115 / 139 / 160, 1024 x 4096 x 4096 47 / 56* / 66; against it 512 x 4096 x 16384
+  // 108* / 102* / 119 and 1024 x 4096 x 16384 193 / 177* / 223).  Launches with fp16 problems among them keep the
+  // tiles below.
+  bool all_w8 = true;
+  for (int i = 0; i < n_problems; ++i) all_w8 = all_w8 && fmts[i] == RWKV_FMT_W8;
+  if (all_w8 && M > 128 && M <= 1024 && (K <= 4096 || M <= 384)) return StreamConfig{2, 128, 1, 4, 2};
   // 129..256 rows against enough column blocks: 128-row tiles give one round of blocks where 64-row tiles give
   // two (256 rows x 16384 x 4096: 62.5 -> 56 us)
   if (M > 128 && M <= 256 && 2 * cb128 >= target_blocks() && 2 * cb128 <= 256) return StreamConfig{4, 128, 1, 4};
@@ -799,7 +899,7 @@ size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const i
   for (int i = 0; i < n_problems; ++i) n_total += Ns[i];
   int fmts[kMaxProblems];
   size_t need = 0;
-  for (int fmt : {RWKV_FMT_W8, RWKV_FMT_W4}) {
+  for (int fmt : {RWKV_FMT_W8, RWKV_FMT_W4, RWKV_FMT_F16}) {  // all int8, some int4, neither (fp16 among them)
     for (int i = 0; i < n_problems && i < kMaxProblems; ++i) fmts[i] = fmt;
     const StreamConfig c = choose_config(M, K, n_problems, Ns, fmts);
     const int splits = choose_splits(c, M, count_col_blocks(c, n_problems, Ns), K);
@@ -865,7 +965,12 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
   const int pairs8 = ceil_div(col_blocks * g.splits, 8) * 8;
   const dim3 grid(g.row_tiles * pairs8);
   const dim3 block(64 * cfg.wg * cfg.kg);
-  if (cfg.nb == 2) hipLaunchKernelGGL(gemm_stream_wide_kernel, grid, block, 0, st, g);
+  bool all_w8 = true;
+  for (int i = 0; i < n_problems; ++i) all_w8 = all_w8 && problems[i].fmt == RWKV_FMT_W8;
+  if (cfg.nb == 2 && cfg.mt == 2) {
+    RWKV_REQUIRE(all_w8, "linear_packed: the 64 x 256 tile takes int8 weights only");
+    hipLaunchKernelGGL((gemm_stream_wide_kernel<false, 2>), grid, block, 0, st, g);
+  } else if (cfg.nb == 2) hipLaunchKernelGGL((gemm_stream_wide_kernel<true, 4>), grid, block, 0, st, g);
   else if (cfg.wg == 2) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 4, 2>), grid, block, 0, st, g);
   else if (cfg.mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 2, 4>), grid, block, 0, st, g);
   else if (cfg.mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 128, 2, 4>), grid, block, 0, st, g);

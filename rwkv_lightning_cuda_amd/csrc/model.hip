@@ -223,6 +223,10 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
     const int qkv_ns[7] = {m->C, m->C, m->C, m->Rw, m->Ra, m->Rg, m->Rv};
     size_t ws = std::max(linear_packed_multi_workspace_bytes(R, m->C, 7, qkv_ns),
                          linear_packed_multi_workspace_bytes(R, m->C, 6, qkv_ns));  // layer 0 has no v rank-in
+    // (the same launch in two parts: the projections, then the rank-ins)
+    ws = std::max(ws, linear_packed_multi_workspace_bytes(R, m->C, 3, qkv_ns));
+    ws = std::max(ws, linear_packed_multi_workspace_bytes(R, m->C, 4, qkv_ns + 3));
+    ws = std::max(ws, linear_packed_multi_workspace_bytes(R, m->C, 3, qkv_ns + 3));
     ws = std::max(ws, linear_packed_workspace_bytes(R, m->C, m->C));
     ws = std::max(ws, linear_packed_workspace_bytes(R, m->F, m->C));
     ws = std::max(ws, linear_packed_workspace_bytes(R, m->C, m->F));
@@ -459,7 +463,16 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
             p[i] = PackedProblem{w.m[mids[i]].packed, w.m[mids[i]].scale, w.m[mids[i]].zp, xs[i], ys[i], C, w.m[mids[i]].fmt};
           for (int i = 0; i < n_lora; ++i)
             p[3 + i] = PackedProblem{w.lora_in_packed[i], nullptr, nullptr, lx[i], lh[i], ranks[i], RWKV_FMT_F16};
-          TRY_PROF(linear_packed_multi(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0, s->gemm_ws, s->gemm_ws_bytes));
+          // From 129 rows on, three int8 projections go without the fp16 rank-ins: a launch of int8 problems only
+          // takes the tile with several wavefronts per SIMD (the rank-ins follow in a launch of their own).
+          bool w8_only = rows > 128;
+          for (int i = 0; i < 3; ++i) w8_only = w8_only && p[i].fmt == RWKV_FMT_W8;
+          if (w8_only) {
+            TRY_PROF(linear_packed_multi(st, rows, C, 3, p, RWKV_EPI_NONE, 0, s->gemm_ws, s->gemm_ws_bytes));
+            TRY_PROF(linear_packed_multi(st, rows, C, n_lora, p + 3, RWKV_EPI_NONE, 0, s->gemm_ws, s->gemm_ws_bytes));
+          } else {
+            TRY_PROF(linear_packed_multi(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0, s->gemm_ws, s->gemm_ws_bytes));
+          }
         } else {
           for (int i = 0; i < 3; ++i) TRY_PROF(apply_matrix(s, w.m[mids[i]], rows, C, C, xs[i], RWKV_EPI_NONE, 0, ys[i]));
           for (int i = 0; i < n_lora; ++i)
