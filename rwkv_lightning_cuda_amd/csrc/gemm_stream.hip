@@ -847,6 +847,8 @@ struct StreamConfig {
   int nb = 1;  // bands per wavefront
   int cols() const { return 32 * wg * nb; }
 };
+bool linear_packed_int8_tile(int M, int K) { return M > 128 && M <= 1024 && (K <= 4096 || M <= 384); }
+
 static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns, const int* fmts) {
   int cb128 = 0;
   for (int i = 0; i < n_problems; ++i) cb128 += ceil_div(Ns[i], 128);
@@ -865,7 +867,7 @@ static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns, c
   // tiles below.
   bool all_w8 = true;
   for (int i = 0; i < n_problems; ++i) all_w8 = all_w8 && fmts[i] == RWKV_FMT_W8;
-  if (all_w8 && M > 128 && M <= 1024 && (K <= 4096 || M <= 384)) return StreamConfig{2, 128, 1, 4, 2};
+  if (all_w8 && linear_packed_int8_tile(M, K)) return StreamConfig{2, 128, 1, 4, 2};
   // 129..256 rows against enough column blocks: 128-row tiles give one round of blocks where 64-row tiles give
   // two (256 rows x 16384 x 4096: 62.5 -> 56 us)
   if (M > 128 && M <= 256 && 2 * cb128 >= target_blocks() && 2 * cb128 <= 256) return StreamConfig{4, 128, 1, 4};

@@ -63,6 +63,11 @@ __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs
   const int c = blockIdx.x * kLoraCols + wave * 32 + j;
   const bool split = p.act != RWKV_ACT_NONE;
   const half_t* wrow = p.w2 + static_cast<int64_t>(c < a.C ? c : a.C - 1) * R;
+  // packed weights: one 1 KiB piece per wavefront and rank step, consecutive lanes 16 bytes apart.  (Out of the
+  // [C,R] matrix the 64 lanes of a request touch 64 different cache lines, and the address unit takes four times
+  // as long over it.)
+  const int steps = (R + 15) >> 4;
+  const half_t* wpk = p.w2p ? p.w2p + (static_cast<int64_t>(blockIdx.x * (kLoraCols / 32) + wave) * steps * 64 + lane) * 8 : nullptr;
 
   // this lane's W2 values: k = 16*step + 8h .. +8 of output channel c
   constexpr int kSteps = kLoraMaxR / 16 / kLoraKG;
@@ -72,7 +77,7 @@ __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs
     const int k0 = (i * kLoraKG + kg) * 16;  // the same for the whole wavefront
     if (k0 < R) {
       const int k = k0 + h * 8;
-      w[i] = *reinterpret_cast<const half8_t*>(wrow + (k < R ? k : R - 8));
+      w[i] = *reinterpret_cast<const half8_t*>(wpk ? wpk + static_cast<int64_t>(i * kLoraKG + kg) * 512 : wrow + (k < R ? k : R - 8));
     }
   }
 
@@ -85,7 +90,7 @@ __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs
 
   const int pieces = (R >> 3) + 1;  // R/8 pieces of 8 per row + the zeroed pad
   const int row_tiles = (a.M + kLoraRows - 1) / kLoraRows;
-  for (int rt = blockIdx.y; rt < row_tiles; rt += gridDim.y) {
+  auto row_tile = [&](int rt, bool more) {
     const int m0 = rt * kLoraRows;
     const int mn = min(kLoraRows, a.M - m0);
     uint4_t hv[kLoraStage];  // all of them loaded, whatever the rank: a value left undefined costs more than the load
@@ -178,12 +183,47 @@ __global__ __launch_bounds__(kLoraThreads) void lora_out_kernel(LoraOutMultiArgs
       }
     }
     if (orow < mn && ocol_ok) *reinterpret_cast<half8_t*>(p.out + o) = res;
-    __syncthreads();  // the tiles are rewritten by the next row tile
+    if (more) __syncthreads();  // the tiles are rewritten by the next row tile
+  };
+  // One tile per block (up to 256 rows) as straight-line code: inside a loop the compiler makes the requests of a
+  // tile wait for the weights, for the sake of registers that the previous trip round the loop has long released.
+  if (static_cast<int>(gridDim.y) >= row_tiles) {
+    row_tile(blockIdx.y, false);
+  } else {
+    for (int rt = blockIdx.y; rt < row_tiles; rt += gridDim.y) row_tile(rt, true);
   }
 }
 
 // Row tiles per block: one up to 256 rows; beyond that the blocks of a problem walk the row tiles with a stride, so
 // that the weights of a block are requested once for several tiles and the grid stays at a few blocks per CU.
+__global__ __launch_bounds__(256) void lora_pack_w2_kernel(int C, int R, const half_t* __restrict__ w2, half_t* __restrict__ packed,
+                                                           int64_t n_pieces) {
+  const int64_t piece = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;  // (band, step, lane)
+  if (piece >= n_pieces) return;
+  const int steps = (R + 15) >> 4;
+  const int lane = static_cast<int>(piece & 63);
+  const int step = static_cast<int>((piece >> 6) % steps);
+  const int band = static_cast<int>((piece >> 6) / steps);
+  const int c = band * 32 + (lane & 31);
+  const int k = step * 16 + (lane >> 5) * 8;
+  half8_t v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = static_cast<half_t>(0.0f);
+  if (c < C && k < R) v = *reinterpret_cast<const half8_t*>(w2 + static_cast<int64_t>(c) * R + k);  // R % 8 == 0
+  *reinterpret_cast<half8_t*>(packed + piece * 8) = v;
+}
+
+size_t lora_pack_w2_halfs(int C, int R) { return static_cast<size_t>(ceil_div(C, 32)) * ((R + 15) >> 4) * 512; }
+
+int lora_pack_w2_launch(hipStream_t st, int C, int R, const half_t* w2, half_t* packed) {
+  RWKV_REQUIRE(C > 0 && R > 0 && R % 8 == 0 && w2 && packed, "lora_pack_w2: bad arguments (C=%d, R=%d)", C, R);
+  const int64_t n_pieces = static_cast<int64_t>(lora_pack_w2_halfs(C, R) / 8);
+  hipLaunchKernelGGL(lora_pack_w2_kernel, dim3(static_cast<unsigned>((n_pieces + 255) / 256)), dim3(256), 0, st, C, R, w2, packed,
+                     n_pieces);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
 int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a) {
   RWKV_REQUIRE(a.n >= 1 && a.n <= 4, "lora_out: %d problems (1..4)", a.n);
   RWKV_REQUIRE(a.M > 0 && a.C > 0 && a.C % 32 == 0, "lora_out: C (%d) must be a positive multiple of 32", a.C);
@@ -195,7 +235,7 @@ int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a) {
     RWKV_REQUIRE(!p.vres || (p.v && p.v_first && p.bias), "lora_out: v-residual gate needs v, v_first and v0");
     RWKV_REQUIRE((reinterpret_cast<uintptr_t>(p.h) | reinterpret_cast<uintptr_t>(p.w2) | reinterpret_cast<uintptr_t>(p.out) |
                   reinterpret_cast<uintptr_t>(p.bias) | reinterpret_cast<uintptr_t>(p.v) |
-                  reinterpret_cast<uintptr_t>(p.v_first)) % 16 == 0,
+                  reinterpret_cast<uintptr_t>(p.v_first) | reinterpret_cast<uintptr_t>(p.w2p)) % 16 == 0,
                  "lora_out: tensors must be 16-byte aligned");
   }
   const int row_tiles = ceil_div(a.M, kLoraRows);

@@ -32,6 +32,7 @@ struct Layer {
   const half_t* t[64] = {nullptr};
   Matrix m[6];
   void* lora_in_packed[4] = {nullptr, nullptr, nullptr, nullptr};  // owned: W1, A1, G1, V1 in the MFMA-native order
+  half_t* lora_out_packed[4] = {nullptr, nullptr, nullptr, nullptr};  // owned: W2, A2, G2, V2 in the rank-out kernel's order
 };
 
 struct rwkv_hip_model {
@@ -50,6 +51,8 @@ struct rwkv_hip_model {
         if (mat.sparse_t) (void)hipFree(mat.sparse_t);
       }
       for (void* q : l.lora_in_packed)
+        if (q) (void)hipFree(q);
+      for (half_t* q : l.lora_out_packed)
         if (q) (void)hipFree(q);
     }
   }
@@ -463,9 +466,9 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
             p[i] = PackedProblem{w.m[mids[i]].packed, w.m[mids[i]].scale, w.m[mids[i]].zp, xs[i], ys[i], C, w.m[mids[i]].fmt};
           for (int i = 0; i < n_lora; ++i)
             p[3 + i] = PackedProblem{w.lora_in_packed[i], nullptr, nullptr, lx[i], lh[i], ranks[i], RWKV_FMT_F16};
-          // From 129 rows on, three int8 projections go without the fp16 rank-ins: a launch of int8 problems only
-          // takes the tile with several wavefronts per SIMD (the rank-ins follow in a launch of their own).
-          bool w8_only = rows > 128;
+          // Where a launch of int8 problems only has a tile of its own (several wavefronts per SIMD), three int8
+          // projections go without the fp16 rank-ins, which follow in a launch of their own.
+          bool w8_only = linear_packed_int8_tile(rows, C);
           for (int i = 0; i < 3; ++i) w8_only = w8_only && p[i].fmt == RWKV_FMT_W8;
           if (w8_only) {
             TRY_PROF(linear_packed_multi(st, rows, C, 3, p, RWKV_EPI_NONE, 0, s->gemm_ws, s->gemm_ws_bytes));
@@ -512,9 +515,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
         a.p[0].h = b.hw; a.p[0].w2 = w.t[RWKV_T_W2]; a.p[0].R = m->Rw; a.p[0].act = RWKV_ACT_TANH; a.p[0].out = b.w12;
         a.p[1].h = b.ha; a.p[1].w2 = w.t[RWKV_T_A2]; a.p[1].R = m->Ra; a.p[1].act = RWKV_ACT_NONE; a.p[1].out = b.a12;
         a.p[2].h = b.hg; a.p[2].w2 = w.t[RWKV_T_G2]; a.p[2].R = m->Rg; a.p[2].act = RWKV_ACT_SIGMOID; a.p[2].out = b.g;
+        for (int i = 0; i < 3; ++i) a.p[i].w2p = w.lora_out_packed[i];
         if (l > 0) {
           LoraOutProblem& pv = a.p[3];
-          pv.h = b.hv; pv.w2 = w.t[RWKV_T_V2]; pv.R = m->Rv; pv.act = RWKV_ACT_NONE; pv.bias = w.t[RWKV_T_V0];
+          pv.h = b.hv; pv.w2 = w.t[RWKV_T_V2]; pv.w2p = w.lora_out_packed[3]; pv.R = m->Rv; pv.act = RWKV_ACT_NONE;
+          pv.bias = w.t[RWKV_T_V0];
           pv.vres = 1; pv.v = b.v; pv.v_first = b.v_first; pv.out = b.xv;  // xv is free after the projections
           v_cur = b.xv;
         }
@@ -797,6 +802,23 @@ int rwkv_hip_model_set_tensor(rwkv_hip_model* m, int layer, int id, const void* 
     if (linear_packed_supported(RWKV_FMT_F16, static_cast<int>(kPackedMinRows), ranks[i], m->C)) {
       RWKV_HIP_TRY(hipMalloc(&slot, static_cast<size_t>(ranks[i]) * m->C * 2));
       const int rc = pack_weights_launch(nullptr, RWKV_FMT_F16, ranks[i], m->C, data, slot);
+      if (rc != RWKV_OK) return rc;
+      RWKV_HIP_TRY(hipStreamSynchronize(nullptr));
+    }
+  }
+  // rank-out matrices [C, R]: a copy in the order the many-row rank-out kernel reads them
+  const int w2_ids[4] = {RWKV_T_W2, RWKV_T_A2, RWKV_T_G2, RWKV_T_V2};
+  for (int i = 0; i < 4; ++i) {
+    if (id != w2_ids[i]) continue;
+    half_t*& slot = m->layers[layer].lora_out_packed[i];
+    if (slot) {
+      RWKV_HIP_TRY(hipDeviceSynchronize());
+      RWKV_HIP_TRY(hipFree(slot));
+      slot = nullptr;
+    }
+    if (ranks[i] > 0 && ranks[i] % 8 == 0) {
+      RWKV_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&slot), lora_pack_w2_halfs(m->C, ranks[i]) * sizeof(half_t)));
+      const int rc = lora_pack_w2_launch(nullptr, m->C, ranks[i], p, slot);
       if (rc != RWKV_OK) return rc;
       RWKV_HIP_TRY(hipStreamSynchronize(nullptr));
     }

@@ -88,6 +88,9 @@ struct PackedProblem {
   int N;
   int fmt;
 };
+// Row counts and K at which a launch of int8 problems only gets a tile of its own (several wavefronts per SIMD):
+// callers with int8 and fp16 problems for one launch do better with two launches there.
+bool linear_packed_int8_tile(int M, int K);
 size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const int* Ns);
 int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const PackedProblem* problems, int epilogue,
                         int out_f32, void* workspace, size_t workspace_bytes, DeferredReduce* defer = nullptr);
@@ -170,6 +173,7 @@ int embed_gather_launch(hipStream_t st, int rows, int C, const int64_t* tokens, 
 struct LoraOutProblem {
   const half_t* h;        // [M,R]
   const half_t* w2;       // [C,R]
+  const half_t* w2p = nullptr;  // the same in the order of lora_pack_w2_launch (optional: coalesced weight reads)
   const half_t* bias;     // [C] or NULL
   const half_t* v;        // [M,C] (vres)
   const half_t* v_first;  // [M,C] (vres)
@@ -182,6 +186,10 @@ struct LoraOutMultiArgs {
 };
 // up to four rank-out products over the same rows in one launch
 int lora_out_multi(hipStream_t st, const LoraOutMultiArgs& a);
+// W2 [C,R] in the order the rank-out kernel's lanes read it: 32-channel bands x 16-wide rank steps x 64 lanes x 8
+// values, lane (j, h) holding rank 16*step + 8*h .. + 8 of channel 32*band + j; zeros past C and R.
+size_t lora_pack_w2_halfs(int C, int R);
+int lora_pack_w2_launch(hipStream_t st, int C, int R, const half_t* w2, half_t* packed);
 
 // ---- ffn_sparse.hip: one-token ffn.value product that skips the rows with a zero activation ---------------
 bool ffn_sparse_supported(int fmt, int C, int F);  // fp16, int8 or int4 codes
