@@ -79,6 +79,13 @@ __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_c
 // The reference is built with --use_fast_math (approximate division, __expf, fast tanhf); these are the
 // gfx950 counterparts: v_rcp_f32 (1 ulp) and v_exp_f32.
 __device__ __forceinline__ float rcp_f(float x) { return __builtin_amdgcn_rcpf(x); }
+// fp32 -> fp16 as a conversion of its own.  The compiler may fold a conversion into the fma that produced the value
+// (v_fma_mixlo_f16: one rounding) or keep the two apart (two roundings), by context; where two kernels, or two
+// chains of one kernel, must give the same bits, both take this.
+__device__ __forceinline__ half_t f2h_apart(float v) {
+  asm volatile("" : "+v"(v));
+  return f2h(v);
+}
 __device__ __forceinline__ float sigmoid_f(float x) { return rcp_f(1.0f + __expf(-x)); }
 // tanh through e^(-2|x|): absolute error of a few 1e-8 (the library tanhf costs some 80 instructions)
 __device__ __forceinline__ float tanh_f(float x) {

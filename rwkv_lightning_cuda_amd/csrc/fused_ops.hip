@@ -173,6 +173,158 @@ __global__ __launch_bounds__(NT) void ln_fused_kernel(LnArgs a) {
   }
 }
 
+// ---- residual add + LayerNorm + token shift over sequences (prefill chunks): one block per row (b, t) ----------
+// The lerps of row t need the LayerNorm output of row t - 1, which another block computes: instead of a launch of
+// its own between the two (the LN rows written and read back, 5 us of launch and ramp), the block normalises the
+// previous row a second time - the same loads, the same arithmetic in the same order, so bitwise the value the
+// previous row's block gets.  At t == 0 the previous output is the shift row of the state.  Blocks of other rows
+// read that shift row while this launch runs, so the new one (the LN output at t == T - 1) goes to shift_next and
+// the caller moves it over afterwards.
+template <int NT>
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* scratch) {  // block_sum's order, two values
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if constexpr (NT / 64 == 1) return;
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+    scratch[wave] = a;
+    scratch[NT / 64 + wave] = b;
+  }
+  __syncthreads();
+  float ta = 0.0f, tb = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NT / 64; ++i) {
+    ta += scratch[i];
+    tb += scratch[NT / 64 + i];
+  }
+  a = ta;
+  b = tb;
+}
+
+template <int NT>
+__global__ __launch_bounds__(NT) void ln_mix_seq_kernel(LnArgs a) {
+  __shared__ float red[2 * (NT / 64)];
+  const int row = blockIdx.x;
+  const int C = a.C;
+  const int bi = row / a.T;
+  const int t = row - bi * a.T;
+  const bool live = static_cast<int>(threadIdx.x) * 8 < C;
+  const int c = live ? threadIdx.x * 8 : 0;  // idle threads repeat slice 0 and store nothing
+  const int64_t o = static_cast<int64_t>(row) * C + c;
+  const int64_t op = t > 0 ? o - C : o;  // the previous row; at t == 0 this row again, unused
+
+  // every load of the kernel up front, none under a per-lane branch
+  const half8_t wv = *reinterpret_cast<const half8_t*>(a.w + c);
+  const half8_t bv = *reinterpret_cast<const half8_t*>(a.b + c);
+  const half8_t sh = *reinterpret_cast<const half8_t*>(a.shift + static_cast<int64_t>(bi) * C + c);
+  half8_t mv[6];
+#pragma unroll
+  for (int s = 0; s < 6; ++s) mv[s] = *reinterpret_cast<const half8_t*>(a.mu[s < a.n_mix ? s : a.n_mix - 1] + c);
+  const half8_t xv = *reinterpret_cast<const half8_t*>(a.x + o);
+  const half8_t xp = *reinterpret_cast<const half8_t*>(a.x + op);
+  half8_t rv, rp;
+  if (a.res_partial) {
+    const half8_t sv8 = *reinterpret_cast<const half8_t*>((a.res_scale ? a.res_scale : a.w) + c);
+    const float* pp = a.res_partial + o;
+    const float* pq = a.res_partial + op;
+    float4_t s0 = *reinterpret_cast<const float4_t*>(pp), s1 = *reinterpret_cast<const float4_t*>(pp + 4);
+    float4_t u0 = *reinterpret_cast<const float4_t*>(pq), u1 = *reinterpret_cast<const float4_t*>(pq + 4);
+    // the other partials four at a time, all requested before the first is added, in split order (ln_fused_kernel)
+    for (int base = 1; base < a.res_splits; base += 4) {
+      float4_t q0[4], q1[4], p0[4], p1[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t sp = (base + u < a.res_splits ? base + u : a.res_splits - 1) * a.res_plane;
+        q0[u] = *reinterpret_cast<const float4_t*>(pp + sp);
+        q1[u] = *reinterpret_cast<const float4_t*>(pp + sp + 4);
+        p0[u] = *reinterpret_cast<const float4_t*>(pq + sp);
+        p1[u] = *reinterpret_cast<const float4_t*>(pq + sp + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(q0[u]), "+v"(q1[u]), "+v"(p0[u]), "+v"(p1[u]));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (base + u < a.res_splits) {
+          s0 = s0 + q0[u]; s1 = s1 + q1[u];
+          u0 = u0 + p0[u]; u1 = u1 + p1[u];
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float sl = a.res_scale ? h2f(sv8[e]) : 1.0f, sh4 = a.res_scale ? h2f(sv8[4 + e]) : 1.0f;
+      rv[e] = f2h(mul_f32(s0[e], sl)); rv[4 + e] = f2h(mul_f32(s1[e], sh4));
+      rp[e] = f2h(mul_f32(u0[e], sl)); rp[4 + e] = f2h(mul_f32(u1[e], sh4));
+    }
+  } else {
+    rv = *reinterpret_cast<const half8_t*>(a.res + o);
+    rp = *reinterpret_cast<const half8_t*>(a.res + op);
+  }
+
+  float v[8], vp[8];
+  float sum = 0.0f, sump = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    v[e] = h2f(xv[e]) + h2f(rv[e]);
+    vp[e] = h2f(xp[e]) + h2f(rp[e]);
+    if (!live) v[e] = vp[e] = 0.0f;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sum += v[e];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sump += vp[e];
+  block_sum2<NT>(sum, sump, red);
+  const float mean = sum / static_cast<float>(C), meanp = sump / static_cast<float>(C);
+  float sv = 0.0f, svp = 0.0f;
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float d = v[e] - mean;
+      sv = fmaf(d, d, sv);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float d = vp[e] - meanp;
+      svp = fmaf(d, d, svp);
+    }
+  }
+  block_sum2<NT>(sv, svp, red);
+  const float rstd = rsqrtf(sv / static_cast<float>(C) + a.eps);
+  const float rstdp = rsqrtf(svp / static_cast<float>(C) + a.eps);
+  if (!live) return;
+
+  half8_t yv, xo;
+  float prev[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    // Both outputs as an fp32 fma rounded to fp16 afterwards (what the LayerNorm kernels store).  Left alone, the
+    // compiler folds the conversion of the one that is not stored into the fma (v_fma_mixlo_f16: one rounding
+    // instead of two), and the previous row's value then differs from what that row's own block gets in one
+    // element of some ten thousand.  The same for the lerps below, against token_shift_mix_kernel.
+    yv[e] = f2h_apart(fmaf((v[e] - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
+    const half_t yp = f2h_apart(fmaf((vp[e] - meanp) * rstdp, h2f(wv[e]), h2f(bv[e])));
+    prev[e] = t > 0 ? h2f(yp) : h2f(sh[e]);
+    xo[e] = f2h(v[e]);
+  }
+  *reinterpret_cast<half8_t*>(a.x_out + o) = xo;
+  // lerps read the fp16-rounded LN output (rwkv7_v3a_ops.cu:1978-1983)
+#pragma unroll
+  for (int s = 0; s < 6; ++s) {
+    if (s < a.n_mix) {
+      half8_t ov;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float yf = h2f(yv[e]);
+        ov[e] = f2h_apart(fmaf(prev[e] - yf, h2f(mv[s][e]), yf));
+      }
+      *reinterpret_cast<half8_t*>(a.out[s] + o) = ov;
+    }
+  }
+  if (a.y) *reinterpret_cast<half8_t*>(a.y + o) = yv;
+  if (t == a.T - 1) *reinterpret_cast<half8_t*>(a.shift_next + static_cast<int64_t>(bi) * C + c) = yv;
+}
+
 static int check_ln_shape(int rows, int C) {
   RWKV_REQUIRE(rows > 0, "layer norm: rows must be positive");
   RWKV_REQUIRE(C > 0 && C % 8 == 0 && C <= kLnMaxThreads * 8,
@@ -196,6 +348,16 @@ static int ln_launch_nt(hipStream_t st, int mode, int rows, const LnArgs& a) {
 
 int ln_launch(hipStream_t st, int mode, int rows, const LnArgs& a) {
   if (int rc = check_ln_shape(rows, a.C)) return rc;
+  if (mode == kAddLnMixSeq) {
+    RWKV_REQUIRE(a.C <= 512 * 8, "layer norm + token shift over a sequence: C (%d) must be at most 4096", a.C);
+    RWKV_REQUIRE(a.T >= 1 && rows % a.T == 0 && a.shift && a.shift_next && a.x_out && a.n_mix >= 1 && a.n_mix <= 6 &&
+                     (a.res || a.res_partial),
+                 "layer norm + token shift over a sequence: bad arguments");
+    if (a.C <= 256 * 8) hipLaunchKernelGGL(ln_mix_seq_kernel<256>, dim3(rows), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(ln_mix_seq_kernel<512>, dim3(rows), dim3(512), 0, st, a);
+    RWKV_LAUNCH_CHECK();
+    return RWKV_OK;
+  }
   if (a.C <= 256 * 8) return ln_launch_nt<256>(st, mode, rows, a);
   if (a.C <= 512 * 8) return ln_launch_nt<512>(st, mode, rows, a);
   return ln_launch_nt<1024>(st, mode, rows, a);

@@ -107,7 +107,15 @@ struct StreamArgs {
   int splits, k_per_split;
   int row_tiles, col_blocks;
   int epilogue, out_f32;
+  RowCopy copy;  // rides on the launch: the first block moves these rows (they are no operand of the product)
 };
+
+__device__ __forceinline__ void ride_along_copy(const RowCopy& cp) {
+  if (blockIdx.x == 0 && cp.n > 0) {
+    for (int i = threadIdx.x * 8; i < cp.n; i += blockDim.x * 8)
+      *reinterpret_cast<uint4_t*>(cp.dst + i) = *reinterpret_cast<const uint4_t*>(cp.src + i);
+  }
+}
 
 __device__ __forceinline__ half8_t make_half8(half2_t a, half2_t b, half2_t c, half2_t d) {
   half8_t r;
@@ -470,6 +478,7 @@ __device__ __forceinline__ void stream_block(const StreamArgs& g, const StreamPr
 template <int MT, int KC, int KG, int WG>
 __global__ __launch_bounds__(64 * WG * KG) void gemm_stream_kernel(StreamArgs g) {
   __shared__ __align__(16) half_t xs[KG * 2 * 32 * MT * (KC + 8)];
+  ride_along_copy(g.copy);
   const int id = blockIdx.x;
   const int row_tile = (id >> 3) % g.row_tiles;
   const int pair = (id / (8 * g.row_tiles)) * 8 + (id & 7);
@@ -741,6 +750,7 @@ __device__ __forceinline__ void stream_block_wide(const StreamArgs& g, const Str
 template <bool MIXED, int MT>
 __global__ __launch_bounds__(256, MIXED ? 1 : 2) void gemm_stream_wide_kernel(StreamArgs g) {
   __shared__ __align__(16) half_t xs[2 * 32 * MT * (128 + 8)];
+  ride_along_copy(g.copy);
   const int id = blockIdx.x;
   const int row_tile = (id >> 3) % g.row_tiles;
   const int pair = (id / (8 * g.row_tiles)) * 8 + (id & 7);
@@ -913,11 +923,15 @@ size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const i
 size_t linear_packed_workspace_bytes(int M, int N, int K) { return linear_packed_multi_workspace_bytes(M, K, 1, &N); }
 
 int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const PackedProblem* problems, int epilogue,
-                        int out_f32, void* workspace, size_t workspace_bytes, DeferredReduce* defer) {
+                        int out_f32, void* workspace, size_t workspace_bytes, DeferredReduce* defer, const RowCopy* copy) {
   RWKV_REQUIRE(n_problems >= 1 && n_problems <= kMaxProblems, "linear_packed: %d problems (1..%d allowed)", n_problems,
                kMaxProblems);
   StreamArgs g;
   ReduceArgs r;
+  if (copy) {
+    RWKV_REQUIRE(copy->n >= 0 && copy->n % 8 == 0 && (copy->n == 0 || (copy->src && copy->dst)), "linear_packed: bad row copy");
+    g.copy = *copy;
+  }
   g.n_problems = r.n_problems = n_problems;
   g.M = r.M = M;
   g.K = K;
@@ -996,9 +1010,9 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
 
 int linear_packed(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* packed, const half_t* scale,
                   const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes,
-                  DeferredReduce* defer) {
+                  DeferredReduce* defer, const RowCopy* copy) {
   const PackedProblem q = {packed, scale, zp, x, y, N, fmt};
-  return linear_packed_multi(st, M, K, 1, &q, epilogue, out_f32, workspace, workspace_bytes, defer);
+  return linear_packed_multi(st, M, K, 1, &q, epilogue, out_f32, workspace, workspace_bytes, defer, copy);
 }
 
 }  // namespace rwkv

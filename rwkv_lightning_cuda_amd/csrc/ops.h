@@ -77,7 +77,7 @@ size_t linear_packed_workspace_bytes(int M, int N, int K);
 // defer (single problem, fp16 output, no epilogue): the consumer sums the partials instead of a reduce launch.
 int linear_packed(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* packed, const half_t* scale,
                   const uint8_t* zp, int epilogue, int out_f32, void* y, void* workspace, size_t workspace_bytes,
-                  DeferredReduce* defer = nullptr);
+                  DeferredReduce* defer = nullptr, const RowCopy* copy = nullptr);
 // Up to kMaxProblems products sharing M and K (own weights, format, x, y each) in one launch (+ one reduce launch).
 struct PackedProblem {
   const void* packed;
@@ -93,7 +93,8 @@ struct PackedProblem {
 bool linear_packed_int8_tile(int M, int K);
 size_t linear_packed_multi_workspace_bytes(int M, int K, int n_problems, const int* Ns);
 int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const PackedProblem* problems, int epilogue,
-                        int out_f32, void* workspace, size_t workspace_bytes, DeferredReduce* defer = nullptr);
+                        int out_f32, void* workspace, size_t workspace_bytes, DeferredReduce* defer = nullptr,
+                        const RowCopy* copy = nullptr);  // copy: rows moved by the launch's first block (n % 8 == 0)
 
 // ---- fused_ops.hip ------------------------------------------------------------------------------
 enum LnMode {
@@ -102,6 +103,8 @@ enum LnMode {
   kAddLastLn = 2,   // rows = B, reads row b*T + T-1; y only
   kAddLnMix = 3,    // kAddLn + n_mix lerps against shift, shift <- LN output (T == 1)
   kLnMix = 4,       // y = LN(x) without residual, then lerps + shift write (embedding row of layer 0)
+  kAddLnMixSeq = 5, // kAddLn over rows [B,T] + n_mix lerps against the previous token's LN output (the shift row at
+                    // t == 0); the LN output of each sequence's last token goes to shift_next, not to shift
 };
 
 struct LnArgs {
@@ -115,6 +118,7 @@ struct LnArgs {
   const half_t* mu[6];
   half_t* out[6];
   const int64_t* tokens;  // kLnMix: if not NULL, x is a [V,C] table indexed by tokens[row]
+  half_t* shift_next;     // kAddLnMixSeq: [B,C], the next shift rows (the caller moves them into shift afterwards)
   int C;
   int T;
   int n_mix;

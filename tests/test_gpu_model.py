@@ -179,9 +179,12 @@ def test_decode_with_row_skipping_ffn_value(gpu, orc, fmt, B):
 
 
 @pytest.mark.parametrize("fmt", [1, 2])
-@pytest.mark.parametrize("B,T", [(2, 16), (20, 21), (36, 11), (40, 1), (12, 1)])
+@pytest.mark.parametrize("B,T", [(2, 16), (12, 21), (20, 21), (36, 11), (40, 1), (12, 1)])
 def test_fused_launches_match_the_standalone_kernels_bitwise(gpu, fmt, B, T):
-    """Two fusions of the row-tiled path are switched off while the residual-stream tap is on.  (1) The LayerNorm
+    """Three fusions of the row-tiled path are switched off while the residual-stream tap is on.  (0) Prefill calls of
+    up to 256 rows run residual add + LayerNorm + token shift as one kernel per LayerNorm, whose blocks normalise the
+    previous row a second time and leave the new shift rows to the next GEMM launch; tapped, the LayerNorm and the
+    token-shift kernel run one after the other.  (1) The LayerNorm
     kernels after the output projection and after ffn.value sum the fp32 split-K partials of the streaming GEMM
     themselves; tapped, the reduce kernel runs instead.  (2) kk normalise / a-gate / decay, the WKV recurrence and
     GroupNorm / bonus / gate run as one launch; tapped, as the three stand-alone kernels.  Same arithmetic in the
