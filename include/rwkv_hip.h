@@ -334,6 +334,15 @@ int rwkv_hip_session_set_wkv_fp16(rwkv_hip_session* s, int on);
  * two rows through a prologue that is bitwise the stand-alone kernels but slower than them from 2048 channels
  * on.  No counterpart in the reference (its fused decode kernels are cuda/rwkv7_v3a_ops.cu:1637-1798). */
 int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on);
+/* Decode steps run everything between the r/k/v projections and the output projection as one launch per layer, one
+ * block per head and 1, 2 or 4 batch rows (the head's LoRA rows are loaded once per block), up to 8 rows and while
+ * that launch is one round of blocks on the chip; larger batches take the row-tiled kernels of the prefill path.  rows
+ * 1, 2 or 4: always the single launch, with that many rows per block where the batch is a multiple of it (else 1);
+ * 0: never; < 0 (the default): by batch size.  1, 2 and 4 give the same bits; the row-tiled kernels add up the
+ * LoRA rank-outs in another order (fp32 sums, then the same fp16 rounding points).  No counterpart in the reference
+ * (its decode step launches the kernels of cuda/rwkv7_v3a_ops.cu:1027-1130 and cuda/rwkv7_fast_ops_fp16.cu:129-237
+ * one after the other). */
+int rwkv_hip_session_set_tmix_rows(rwkv_hip_session* s, int rows);
 /* debugging/parity tap: device address of one of the session's activation buffers, holding what the last
  * layer of the last rwkv_hip_forward call left there.  Ids in order: x, xx, xr, xw, xk, xv, xa, xg, r, k, v,
  * v_first, w12, a12, g, hw, ha, hg, hv, k2, nkk, kka, y, y2, att, x1, ln2, mixed, act, cm (f16), then

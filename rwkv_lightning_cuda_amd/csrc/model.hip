@@ -76,6 +76,9 @@ constexpr size_t kMaxGraphs = 8;
 // shapes, all three weight formats: at 2 rows the GEMV is 5 % faster, from 3 rows on the streaming GEMM wins
 // (8 rows: 6.1 -> 3.6 ms per decode step with int8 codes; the GEMV pays one v_dot2 per row and weight pair).
 constexpr size_t kPackedMinRows = 3;
+// most blocks of a single-launch time-mix core beyond 8 rows (one round on 256 CUs; us per layer at the 7.2B shape,
+// this launch / the row-tiled kernels: 16 rows 14 / 17, 32 rows 25 / 24)
+constexpr int kTmixStepMaxBlocks = 256;
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -126,6 +129,7 @@ struct rwkv_hip_session {
   size_t sparse_ws_bytes = 0;
   int sparse_ffn_rows = 1;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
   bool wkv_fp16 = false;      // the WKV state tensor is fp16 [L,B,H,64,64] (the reference's use_wkv32 == false)
+  int tmix_rows = -1;         // decode steps' single-launch time-mix core: rows per block 1/2/4, 0 never, < 0 by batch
   int fused_ln = -1;          // decode steps fold LayerNorm + token shift into the linear launches: 1 always, 0 never,
                               // -1 for one row of at most 4096 channels (the row-resident GEMV hides the prologue
                               // behind its weight requests: 7.2B shape 2.04 -> 1.92 ms per step, 0.1B 0.413 -> 0.373)
@@ -350,10 +354,20 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
     RWKV_HIP_TRY(hipEventCreate(&pass_begin));
     RWKV_HIP_TRY(hipEventRecord(pass_begin, st));
   }
-  // The single-launch time-mix core re-reads a head's LoRA rows for every batch row; from 16 rows on the
-  // row-tiled kernels of the prefill path (LoRA rank-outs on the matrix core) are faster (measured: 4.2 -> 4.0 ms
-  // per step at 16 rows, 5.5 -> 4.6 ms at 32).
-  const bool fused_tmix = step && rows <= 8;
+  // The single-launch time-mix core loads a head's LoRA rows once per block, for 1, 2 or 4 batch rows.  It is used
+  // up to 8 rows and while the launch is one round of blocks on the chip; beyond that the row-tiled kernels of the
+  // prefill path (LoRA rank-outs on the matrix core, the recurrence at full memory rate) are faster.  The fp16 state and
+  // batches that are no multiple of 2 or 4 keep one row per block.
+  int tmix_rows = 0;
+  if (step) {
+    if (s->tmix_rows > 0) {
+      tmix_rows = (B % s->tmix_rows == 0 && !s->wkv_fp16) ? s->tmix_rows : 1;
+    } else if (s->tmix_rows < 0) {
+      const int rpb = tmix_step_rows_per_block(B, H, s->wkv_fp16);
+      if (rows <= 8 || B * H / rpb <= kTmixStepMaxBlocks) tmix_rows = rpb;
+    }
+  }
+  const bool fused_tmix = tmix_rows > 0;
   // Decode steps on the GEMV path can fold both LayerNorm + token-shift kernels of a layer into the prologue of the
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key): by default for one row of up to 4096
   // channels.  The residual-stream tap needs the stand-alone kernels.
@@ -533,6 +547,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       if (gate_split) {  // the g rank-out in blocks of its own; the output projection applies the gate
         p.y2_pre = b.r32; p.gate_out = b.g;
       }
+      p.rows_per_block = gate_split ? 1 : tmix_rows;
       TRY_AUX(tmix_step_launch(st, p));
     } else {
       // LoRA rank-out (+ activation, + v-residual gate)
@@ -1022,6 +1037,17 @@ int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on) {
   if (s->fused_ln != want) {
     TRY(drop_graphs(s));  // captured decode graphs hold the other kernels
     s->fused_ln = want;
+  }
+  return RWKV_OK;
+}
+
+int rwkv_hip_session_set_tmix_rows(rwkv_hip_session* s, int rows) {
+  RWKV_REQUIRE(s, "session is NULL");
+  RWKV_REQUIRE(rows < 0 || rows == 0 || rows == 1 || rows == 2 || rows == 4, "rows per block: 1, 2 or 4; 0 or < 0");
+  const int want = rows < 0 ? -1 : rows;
+  if (s->tmix_rows != want) {
+    TRY(drop_graphs(s));  // captured decode graphs hold the other kernels
+    s->tmix_rows = want;
   }
   return RWKV_OK;
 }

@@ -239,7 +239,7 @@ int wkv7_f16state_launch(hipStream_t st, int B, int T, int C, int H, half_t* sta
 
 namespace rwkv {
 
-// ---- tmix_step.hip: the whole time-mix core of a decode step, one workgroup per (batch row, head) ----
+// ---- tmix_step.hip: the whole time-mix core of a decode step, one workgroup per head and 1, 2 or 4 batch rows ----
 struct TmixStepArgs {
   int B, H, C, Rw, Ra, Rg, Rv;
   const half_t *hw, *ha, *hg, *hv;          // LoRA hidden vectors [B,R]; hv == NULL on layer 0
@@ -259,7 +259,10 @@ struct TmixStepArgs {
   half_t* gate_out;
   const half_t* shift_src;                  // [B,C] LN output kept by the r/k/v launch's prologue, or NULL
   half_t* shift_dst;                        // [B,C] time-mix shift row of the state that receives it
+  int rows_per_block;                       // batch rows of a head per block: 1, 2 or 4 (dividing B); 0 = chosen here
 };
 int tmix_step_launch(hipStream_t st, const TmixStepArgs& p);
+// the choice that rows_per_block == 0 stands for (one_row_only: split mode or the fp16 state)
+int tmix_step_rows_per_block(int B, int H, bool one_row_only);
 
 }  // namespace rwkv

@@ -40,7 +40,7 @@ EXPORTS = [
     "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_pack_w4", "rwkv_hip_cmix_sparse_packed_bytes",
     "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
     "rwkv_hip_cmix_sparse_down_relu_rows", "rwkv_hip_cmix_sparse_down_relu_rows_static",
-    "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln", "rwkv_hip_session_set_wkv_fp16",
+    "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln", "rwkv_hip_session_set_tmix_rows", "rwkv_hip_session_set_wkv_fp16",
     "rwkv_hip_layer_norm", "rwkv_hip_add_layer_norm", "rwkv_hip_add_last_layer_norm", "rwkv_hip_token_shift_mix",
     "rwkv_hip_add_layer_norm_cmix_mix", "rwkv_hip_add_layer_norm_tmix_mix6", "rwkv_hip_kk_a_gate",
     "rwkv_hip_lnx_rkvres_xg", "rwkv_hip_relu_square", "rwkv_hip_add_vec", "rwkv_hip_f16_to_f32",

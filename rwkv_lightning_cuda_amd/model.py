@@ -271,6 +271,12 @@ class Session:
         never, None (the default of a new session) for one row of at most 4096 channels."""
         hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(-1 if on is None else 1 if on else 0)))
 
+    def set_tmix_rows(self, rows):
+        """Decode steps' single-launch time-mix core: 1, 2 or 4 batch rows per block (always that launch), 0 never
+        (the row-tiled kernels instead), None (the default of a new session) by batch size.  1, 2 and 4 give the same
+        bits."""
+        hip.check(hip.load().rwkv_hip_session_set_tmix_rows(self.handle, ctypes.c_int(-1 if rows is None else int(rows))))
+
     def set_wkv_fp16(self, on):
         """The state's WKV tensor is fp16 and the recurrence runs in fp16 (the reference's use_wkv32 == false)."""
         hip.check(hip.load().rwkv_hip_session_set_wkv_fp16(self.handle, ctypes.c_int(1 if on else 0)))

@@ -720,3 +720,41 @@ def test_decode_step_with_layernorm_folded_into_linear_matches_the_unfused_step(
             assert same, "wkv state differs at step %d" % step
     assert s_fused.elapsed.numpy().tolist() == [9] * B
     sess.close()
+
+
+@pytest.mark.parametrize("B", [4, 8, 16, 12])
+def test_decode_time_mix_core_with_several_batch_rows_per_block(gpu, B):
+    """The single-launch time-mix core of a decode step serves 1, 2 or 4 batch rows of a head per block (the head's
+    LoRA rows loaded once).  Per row the arithmetic is the same in the same order: logits, shift rows and WKV state
+    after five steps are bit-identical for 1, 2 and 4 rows per block and for the default choice (a batch of 12 takes
+    4, of 4 one).  Against the row-tiled kernels (LoRA rank-outs on the matrix core, sums in another order) they
+    agree to fp16 rounding: logits and shift rows within 2e-3 of their scale, WKV state within 1e-3."""
+    from rwkv_lightning_cuda_amd.model import HipModel, ModelDims, Session, State, synth_weights
+    hip = gpu
+    dims = ModelDims(L=2, C=512, H=8, F=2048, V=1024, Rw=32, Ra=32, Rg=64, Rv=32)
+    gmodel = HipModel.from_host_weights(dims, synth_weights(dims, 4), hip.FMT_W8)
+    rng = np.random.default_rng(B)
+    tokens = rng.integers(0, dims.V, (B, 5))
+    sess = Session(gmodel)
+    sess.set_graph(False)
+    outs = {}
+    for setting in (0, 1, 2, 4, None):
+        st = State(dims, B)
+        lg = hip.DeviceArray((B, dims.V), np.float32)
+        sess.set_tmix_rows(setting)
+        for t in range(tokens.shape[1]):
+            sess.forward(tokens[:, t:t + 1], st, lg)
+        outs[setting] = (lg.numpy().copy(), st.shift.numpy().copy(), st.wkv.numpy().copy())
+    sess.set_tmix_rows(None)
+    for setting in (2, 4, None):
+        for name, a, b in zip(("logits", "shift", "wkv"), outs[1], outs[setting]):
+            same = np.array_equal(a.view(np.uint8), b.view(np.uint8))
+            assert same, "%s differ between 1 and %s rows per block" % (name, setting)
+    assert np.isfinite(outs[1][0]).all() and np.abs(outs[1][0]).max() > 0
+    err = rel_err(outs[1][0], outs[0][0])
+    assert err <= 2e-3
+    err = rel_err(outs[1][1].astype(np.float32), outs[0][1].astype(np.float32))
+    assert err <= 2e-3
+    err = rel_err(outs[1][2], outs[0][2])
+    assert err <= 1e-3
+    sess.close()
