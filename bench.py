@@ -201,6 +201,27 @@ def secondary_measurements(hip, model, dims, rng):
         sess.close()
         del state, logits
 
+    # The same decode with the WKV state kept in fp16 (the reference server's default, use_wkv32 == false): half the
+    # state bytes per step.  Reported beside the fp32-state figures above, never instead of them.
+    for B in (16, 64):
+        sess = Session(model)
+        sess.set_wkv_fp16(True)
+        state = State(dims, B, wkv_fp16=True)
+        logits = hip.DeviceArray((B, dims.V), np.float32)
+        sess.forward(rng.integers(0, dims.V, (B, 128)), state, logits)
+        first = rng.integers(0, dims.V, (B,))
+        sess.decode_greedy(first, 8, state, logits)
+        hip.device_sync()
+        t0 = time.perf_counter()
+        steps = 64
+        sess.decode_greedy(first, steps, state, logits)
+        hip.device_sync()
+        dt = time.perf_counter() - t0
+        res["decode_fp16_state_bs%d_tok_s" % B] = steps * B / dt
+        res["decode_fp16_state_bs%d_ms_per_step" % B] = dt * 1e3 / steps
+        sess.close()
+        del state, logits
+
     # WKV7 op alone at the long-context configuration: fp16 r,w,k,v,a,b [16,16384,4096], fp32 state, raw-logit
     # decay, one call.  Rows are 4096-token windows of one host-generated sequence (r,k,v ~ N(0,1); decay =
     # exp(-exp(U(-6,-0.5))) given as its raw logit; kk = k/|k| per head, a = -kk, b = kk * sigmoid(U(-3,3))).

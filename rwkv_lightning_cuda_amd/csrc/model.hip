@@ -572,6 +572,15 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
         // fp16 state (src/rwkv7_fast_v4.cu:1262-1271): kk / a-gate in fp16, the fp16 recurrence, GroupNorm / bonus / gate.
         // Calls of up to 16 tokens add w0 to the decay logit inside the recurrence, unrounded; longer ones round
         // w12 + w0 to fp16 first, as the reference does.
+        if (step && !s->trace) {
+          // a decode step: the three in one launch (same bits), the state moved in coalesced 1 KB requests
+          Tmix16RowsArgs f = {};
+          f.rows_heads = static_cast<int64_t>(rows) * H; f.H = H; f.state = S16; f.elapsed = elapsed;
+          f.r = b.r; f.k = b.k; f.v = v_cur; f.w12 = b.w12; f.a12 = b.a12; f.g = b.g;
+          f.k_k = w.t[RWKV_T_K_K]; f.a0 = w.t[RWKV_T_A0]; f.k_a = w.t[RWKV_T_K_A]; f.w0 = w.t[RWKV_T_W0];
+          f.r_k = w.t[RWKV_T_R_K]; f.lnx_w = w.t[RWKV_T_LNX_W]; f.lnx_b = w.t[RWKV_T_LNX_B]; f.y2 = b.y2;
+          TRY_AUX(tmix16_rows_launch(st, f));
+        } else {
         KkArgs p = {};
         p.k = b.k; p.k_k = w.t[RWKV_T_K_K]; p.a0 = w.t[RWKV_T_A0]; p.a12 = b.a12; p.k_a = w.t[RWKV_T_K_A];
         p.new_k = b.k2; p.neg_kk = b.nkk; p.kka = b.kka;
@@ -587,6 +596,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
         TRY_AUX(wkv7_f16state_launch(st, B, T, C, H, S16, b.r, w_in, w0, b.k2, v_cur, b.nkk, b.kka, b.y, elapsed));
         TRY_AUX(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
                            w.t[RWKV_T_LNX_B], b.g, b.y2));
+        }
       } else if (!s->trace && tmix_seq_whole_heads(B, T, H)) {
         // kk normalise / a-gate / decay, the WKV recurrence and GroupNorm / bonus / gate in one launch
         TmixSeqArgs fa;

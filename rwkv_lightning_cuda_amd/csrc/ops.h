@@ -235,6 +235,19 @@ int wkv7_f16state_launch(hipStream_t st, int B, int T, int C, int H, half_t* sta
                          const half_t* w0, const half_t* k, const half_t* v, const half_t* a, const half_t* b, half_t* y,
                          const int* elapsed);
 
+// One decode token per batch row with the fp16 state: kk normalise / a-gate, decay delta, the step, GroupNorm / bonus
+// / gate in one launch (bitwise kk_a_gate + wkv7_f16state with T = 1 + lnx_rkvres_xg one after the other).
+struct Tmix16RowsArgs {
+  int64_t rows_heads;  // B * H
+  int H;
+  half_t* state;       // [B,H,64,64] fp16, updated in place
+  const int* elapsed;  // [B]
+  const half_t *r, *k, *v, *w12, *a12, *g;  // [B,C]; v after the residual gate, w12 / a12 / g the LoRA rank-outs
+  const half_t *k_k, *a0, *k_a, *w0, *r_k, *lnx_w, *lnx_b;  // [C]
+  half_t* y2;          // [B,C] input of the output projection
+};
+int tmix16_rows_launch(hipStream_t st, const Tmix16RowsArgs& p);
+
 }  // namespace rwkv
 
 namespace rwkv {

@@ -95,7 +95,104 @@ __global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int 
   }
 }
 
+// ---- one token per batch row (a decode step of many rows): kk normalise / a-gate, the decay delta, the step and
+// GroupNorm / bonus / gate in one launch, one wavefront per (batch row, head), four per block.  The arithmetic is that
+// of kk_a_gate_kernel, wkv7_f16state_kernel (T = 1, w0 added inside) and lnx_rkvres_xg_kernel (fused_ops.hip) in
+// the same order, so the result is bitwise theirs.  What differs is how the state moves: here a wavefront reads
+// its head's 8 KB as eight coalesced 1 KB requests (the stand-alone kernel's lanes read one 128-byte row each, 64
+// lines per request), turns them into one row per lane through a padded LDS tile, and stores the new state the same
+// way back; only the wavefront itself synchronises.
+constexpr int kTileLd = kHead + 8;  // halfs per tile row: 144 bytes, so that the lanes' 16-byte row reads spread over the banks
+
+__global__ __launch_bounds__(256) void tmix16_rows_kernel(Tmix16RowsArgs p) {
+  __shared__ __align__(16) half_t tile[4][kHead * kTileLd];
+  __shared__ __align__(16) half_t ops[4][5][kHead];  // a~, b~, k', decay delta, r
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int lane = threadIdx.x & 63;
+  const int64_t rh = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+  if (rh >= p.rows_heads) return;  // (the whole wavefront; nothing below waits for another wavefront)
+  const int bi = static_cast<int>(rh / p.H);
+  const int h = static_cast<int>(rh - static_cast<int64_t>(bi) * p.H);
+  const int c = h * kHead + lane;
+  const int64_t idx = rh * kHead + lane;
+
+  // ---- every load first
+  half_t* sbase = p.state + rh * (kHead * kHead);
+  uint4_t st[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    st[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(sbase + i * 512 + lane * 8));
+  const half_t k_h = p.k[idx], r_h = p.r[idx], v_h = p.v[idx], w12_h = p.w12[idx], a12_h = p.a12[idx], g_h = p.g[idx];
+  const half_t kk_h = p.k_k[c], a0_h = p.a0[c], ka_h = p.k_a[c], w0_h = p.w0[c], rk_h = p.r_k[c], lnw_h = p.lnx_w[c],
+               lnb_h = p.lnx_b[c];
+  const int phase = p.elapsed[bi] + c;
+  __builtin_amdgcn_sched_barrier(0);
+
+  half_t* tl = tile[wave];
+  const int trow = lane >> 3, tcol = (lane & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4_t*>(tl + (i * 8 + trow) * kTileLd + tcol) = st[i];
+
+  // ---- kk normalise, a-gate, decay delta (kk_a_gate_kernel; decay_delta16 with w0 added unrounded)
+  const float kv = h2f(k_h);
+  const float u = kv * h2f(kk_h);
+  const float total = wave_sum(u * u);
+  const float inv = 1.0f / fmaxf(sqrtf(total), kKkEps);
+  const float kk = u * inv;
+  const float av = sigmoid_f(h2f(a0_h) + h2f(a12_h));
+  const float ka = h2f(ka_h);
+  const half_t nk = f2h(kv * fmaf(av, ka, 1.0f - ka));
+  ops[wave][0][lane] = f2h(-kk);
+  ops[wave][1][lane] = f2h(kk * av);
+  ops[wave][2][lane] = nk;
+  ops[wave][3][lane] = decay_delta16_of(h2f(w12_h) + h2f(w0_h), phase);
+  ops[wave][4][lane] = r_h;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // ---- the step on this lane's state row
+  half2_t S[kPairs];
+  read_pairs16(tl + lane * kTileLd, S);
+  const half_t y16 = wkv16_row_step(S, ops[wave][0], ops[wave][1], ops[wave][2], ops[wave][3], ops[wave][4], v_h);
+#pragma unroll
+  for (int q = 0; q < kPairs / 4; ++q) {
+    uint4_t t;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) t[e] = __builtin_bit_cast(uint32_t, S[4 * q + e]);
+    *reinterpret_cast<uint4_t*>(tl + lane * kTileLd + 8 * q) = t;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const uint4_t t = *reinterpret_cast<const uint4_t*>(tl + (i * 8 + trow) * kTileLd + tcol);
+    __builtin_nontemporal_store(t, reinterpret_cast<uint4_t*>(sbase + i * 512 + lane * 8));
+  }
+
+  // ---- GroupNorm over the head, bonus, gate (lnx_rkvres_xg_kernel)
+  const float yv = h2f(y16);
+  const float mean = wave_sum(yv) * (1.0f / 64.0f);
+  const float d = yv - mean;
+  const float var = wave_sum(d * d) * (1.0f / 64.0f);
+  const float rstd = rsqrtf(var + kLnxEps);
+  const float rkv = wave_sum(h2f(r_h) * h2f(nk) * h2f(rk_h));
+  const float o = (d * rstd * h2f(lnw_h) + h2f(lnb_h) + rkv * h2f(v_h)) * h2f(g_h);
+  p.y2[idx] = f2h(o);
+}
+
 }  // namespace
+
+int tmix16_rows_launch(hipStream_t st, const Tmix16RowsArgs& p) {
+  RWKV_REQUIRE(p.rows_heads > 0 && p.H > 0, "tmix16_rows: bad shape");
+  RWKV_REQUIRE(p.state && p.elapsed && p.r && p.k && p.v && p.w12 && p.a12 && p.g && p.k_k && p.a0 && p.k_a && p.w0 &&
+                   p.r_k && p.lnx_w && p.lnx_b && p.y2,
+               "tmix16_rows: NULL tensor");
+  hipLaunchKernelGGL(tmix16_rows_kernel, dim3(static_cast<unsigned>(ceil_div(p.rows_heads, 4))), dim3(256), 0, st, p);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
 
 int wkv7_f16state_launch(hipStream_t st, int B, int T, int C, int H, half_t* state, const half_t* r, const half_t* w,
                          const half_t* w0, const half_t* k, const half_t* v, const half_t* a, const half_t* b, half_t* y,

@@ -758,3 +758,38 @@ def test_decode_time_mix_core_with_several_batch_rows_per_block(gpu, B):
     err = rel_err(outs[1][2], outs[0][2])
     assert err <= 1e-3
     sess.close()
+
+
+@pytest.mark.parametrize("fmt", [1, 2])
+@pytest.mark.parametrize("B", [12, 40])
+def test_fp16_state_decode_step_of_many_rows_matches_the_standalone_kernels_bitwise(gpu, fmt, B):
+    """With the fp16 WKV state a decode step of more than 8 rows runs kk normalise / a-gate, the recurrence step and
+    GroupNorm / bonus / gate as one launch that moves the state in coalesced requests through an LDS tile; with the
+    residual-stream tap on, the three stand-alone kernels run instead.  Same arithmetic in the same order: logits,
+    shift rows and the fp16 state after a 3-token prefill and four steps are bit-identical."""
+    from rwkv_lightning_cuda_amd.model import HipModel, ModelDims, Session, State, synth_weights
+    hip = gpu
+    dims = ModelDims(L=2, C=512, H=8, F=2048, V=1024, Rw=32, Ra=32, Rg=64, Rv=32)
+    gmodel = HipModel.from_host_weights(dims, synth_weights(dims, 4), fmt)
+    rng = np.random.default_rng(B)
+    tokens = rng.integers(0, dims.V, (B, 7))
+    sess = Session(gmodel)
+    sess.set_graph(False)
+    sess.set_wkv_fp16(True)
+    outs = []
+    for tapped in (False, True):
+        st = State(dims, B, wkv_fp16=True)
+        lg = hip.DeviceArray((B, dims.V), np.float32)
+        trace = hip.DeviceArray((dims.L, B, dims.C), np.float16)
+        sess.forward(tokens[:, :3], st, lg)
+        for t in range(3, tokens.shape[1]):
+            sess.set_trace(trace if tapped else None)
+            sess.forward(tokens[:, t:t + 1], st, lg)
+            sess.set_trace(None)
+        outs.append((lg.numpy().copy(), st.shift.numpy().copy(), st.wkv.numpy().copy()))
+    for name, a, b in zip(("logits", "shift", "wkv"), outs[0], outs[1]):
+        same = np.array_equal(a.view(np.uint8), b.view(np.uint8))
+        assert same, name
+    assert np.isfinite(outs[0][0]).all() and np.abs(outs[0][0]).max() > 0
+    assert np.abs(outs[0][2].astype(np.float32)).max() > 0
+    sess.close()
