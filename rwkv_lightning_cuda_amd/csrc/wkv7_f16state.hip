@@ -25,9 +25,11 @@ namespace rwkv {
 namespace {
 
 constexpr int kPairs = kPairs16;
+constexpr int kAhead = 4;  // tokens whose operands are in flight
 
 struct TokenOps {  // one token's per-column operands in LDS
   half_t a[kHead], b[kHead], k[kHead], wd[kHead], r[kHead];
+  half_t v[kHead];  // per state row, not per column: parked here between its arrival and its step
 };
 
 __global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int H, half_t* __restrict__ state,
@@ -54,36 +56,63 @@ __global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int 
   }
 
   const int phase0 = elapsed[bi] + c;
-  int64_t tok = static_cast<int64_t>(bi) * T * C + c;  // this lane's element of token 0
+  // w0 once, not under a branch inside every step (adding 0.0f changes no decay)
+  const float w0f = w0 ? h2f(w0[c]) : 0.0f;
+  const int64_t tok0 = static_cast<int64_t>(bi) * T * C + c;  // this lane's element of token 0
   // token 0's operands
   {
-    ops[0].a[lane] = a[tok];
-    ops[0].b[lane] = b[tok];
-    ops[0].k[lane] = k[tok];
-    ops[0].r[lane] = r[tok];
-    ops[0].wd[lane] = decay_delta16(w[tok], w0, c, phase0);
+    ops[0].a[lane] = a[tok0];
+    ops[0].b[lane] = b[tok0];
+    ops[0].k[lane] = k[tok0];
+    ops[0].r[lane] = r[tok0];
+    ops[0].wd[lane] = decay_delta16_of(h2f(w[tok0]) + w0f, phase0);
   }
-  half_t v_cur = v[tok];
+  ops[0].v[lane] = v[tok0];
+  // The elements of tokens t + 1 .. t + kAhead wait in registers (slot = token mod kAhead): requested one token
+  // ahead only, every step would last a whole trip to memory.  Tokens past the end re-read the last one (no load
+  // under a branch).
+  half_t qa[kAhead], qb[kAhead], qk[kAhead], qr[kAhead], qw[kAhead], qv[kAhead];
+  auto request = [&](int slot, int t) {
+    const int64_t i = tok0 + static_cast<int64_t>(t < T ? t : T - 1) * C;
+    qa[slot] = a[i];
+    qb[slot] = b[i];
+    qk[slot] = k[i];
+    qr[slot] = r[i];
+    qw[slot] = w[i];
+    qv[slot] = v[i];
+  };
+#pragma unroll
+  for (int u = 1; u <= kAhead; ++u) request(u % kAhead, u);
   __syncthreads();
 
-  for (int t = 0; t < T; ++t) {
+  // One token: token t + 1's elements leave their slot for the other buffer first (nobody reads it during this
+  // step), then the slot is requested again for token t + 1 + kAhead - in that order, so that the new request can
+  // take the registers of the old values - and then the state step with the operands in ops[t & 1].
+  auto step = [&](int t, int slot) {
     const TokenOps& cur = ops[t & 1];
     TokenOps& nxt = ops[(t + 1) & 1];
-    // request the next token's elements now (the last token re-reads itself: no load under a branch)
-    const int64_t tn = t + 1 < T ? tok + C : tok;
-    const half_t a_n = a[tn], b_n = b[tn], k_n = k[tn], r_n = r[tn], w_n = w[tn], v_n = v[tn];
-
-    y[tok] = wkv16_row_step(S, cur.a, cur.b, cur.k, cur.wd, cur.r, v_cur);
-
-    // hand the next token's operands to the other buffer (nobody reads it during this step)
-    nxt.a[lane] = a_n;
-    nxt.b[lane] = b_n;
-    nxt.k[lane] = k_n;
-    nxt.r[lane] = r_n;
-    nxt.wd[lane] = decay_delta16(w_n, w0, c, phase0 + t + 1);
-    v_cur = v_n;
-    tok = tn;
+    nxt.a[lane] = qa[slot];
+    nxt.b[lane] = qb[slot];
+    nxt.k[lane] = qk[slot];
+    nxt.r[lane] = qr[slot];
+    nxt.wd[lane] = decay_delta16_of(h2f(qw[slot]) + w0f, phase0 + t + 1);
+    nxt.v[lane] = qv[slot];
+    __builtin_amdgcn_sched_barrier(0);
+    request(slot, t + 1 + kAhead);
+    __builtin_amdgcn_sched_barrier(0);
+    y[tok0 + static_cast<int64_t>(t) * C] = wkv16_row_step(S, cur.a, cur.b, cur.k, cur.wd, cur.r, cur.v[lane]);
     __syncthreads();
+  };
+  // whole rounds of kAhead tokens as straight-line code (a loop with an exit between the steps would wait for every
+  // outstanding request at its head), then the rest
+  int t = 0;
+  for (; t + kAhead <= T; t += kAhead) {
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) step(t + u, (u + 1) % kAhead);
+  }
+#pragma unroll
+  for (int u = 0; u < kAhead - 1; ++u) {
+    if (t + u < T) step(t + u, (u + 1) % kAhead);
   }
 
 #pragma unroll
