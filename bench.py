@@ -75,6 +75,8 @@ def parse_args():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--wkv-fp16", action="store_true", help="keep the WKV state in fp16 (the reference server's default, "
+                    "use_wkv32 == false) in the main measurement; the headline figure is the fp32 state")
     return ap.parse_args()
 
 
@@ -379,13 +381,19 @@ def main():
     sess = Session(model)
     if args.no_graph:
         sess.set_graph(False)
-    state = State(dims, B)
+    if args.wkv_fp16:
+        sess.set_wkv_fp16(True)
+
+    def new_state(b):
+        return State(dims, b, wkv_fp16=args.wkv_fp16)
+
+    state = new_state(B)
     logits = hip.DeviceArray((B, dims.V), np.float32)
     rng = np.random.default_rng(0)
     also = {}
     if args.prefill > 0:
         prompt = rng.integers(0, dims.V, (B, args.prefill))
-        warm = State(dims, B)
+        warm = new_state(B)
         sess.forward(prompt[:, :min(128, args.prefill)], warm, logits)  # sizes the arena, warms the kernels
         del warm
         hip.device_sync()
@@ -398,7 +406,7 @@ def main():
         also["prefill_workload"] = "%d-token prompt x batch %d in chunks of 128 (state carried in HBM)" % (args.prefill, B)
         if not args.no_also and args.prefill >= 128:
             # MFMA fraction of the chunk's GEMM launches: one more chunk, eagerly, GEMM launches bracketed by events
-            scratch = State(dims, B)
+            scratch = new_state(B)
             sess.set_profile(True)
             sess.read_profile()
             sess.forward(prompt[:, :128], scratch, logits, sync=False)
@@ -420,7 +428,7 @@ def main():
             for width in (512, 2048):
                 if B * width > 4096:
                     continue
-                wide = State(dims, B)
+                wide = new_state(B)
                 sess.forward(prompt[:, :min(width, args.prefill)], wide, logits)
                 hip.device_sync()
                 tw = time.perf_counter()
@@ -458,7 +466,7 @@ def main():
         also["ffn_value_rows_skipped_fraction_last_layer"] = float(np.mean(act == 0))
 
     weight_bytes = model.weight_bytes()
-    state_bytes = B * (2 * dims.L * dims.H * 64 * 64 * 4 + 2 * dims.L * 2 * dims.C * 2)
+    state_bytes = B * (2 * dims.L * dims.H * 64 * 64 * (2 if args.wkv_fp16 else 4) + 2 * dims.L * 2 * dims.C * 2)
     # bytes the timed step really moved: the row-skipping ffn.value reads only the rows with a non-zero activation
     # (fraction measured on the last layer's activations of the last step)
     skipped = also.get("ffn_value_rows_skipped_fraction_last_layer", 0.0) if sparse_value else 0.0
@@ -480,7 +488,7 @@ def main():
         "config": {"workload": "RWKV-7 %s-shape greedy decode, batch %d, %d-token prefill, lm_head+argmax on device"
                                % (args.preset, B, args.prefill),
                    "L": dims.L, "C": dims.C, "H": dims.H, "F": dims.F, "V": dims.V,
-                   "weight_format": args.fmt, "arithmetic": "fp16 activations, fp32 accumulate, fp32 WKV state",
+                   "weight_format": args.fmt, "arithmetic": "fp16 activations, fp32 accumulate, %s WKV state" % ("fp16" if args.wkv_fp16 else "fp32"),
                    "hip_graph": not args.no_graph, "sparse_ffn_value": sparse_value,
                    "weight_bytes_per_step": weight_bytes,
                    "state_bytes_per_step": state_bytes,
@@ -497,7 +505,7 @@ def main():
         # stream, each pass bracketed by one pair of HIP events (the kernels' duration does not depend on the
         # data; the small kernels between them are skipped so that no event sits between two launches).  All
         # 7 GB of weights stream from HBM on every pass, exactly as in the timed run.
-        scratch_state = State(dims, B)
+        scratch_state = new_state(B)
         sess.set_profile(2)
         sess.read_profile()
         tok = toks[-1].reshape(B, 1).astype(np.int64)
