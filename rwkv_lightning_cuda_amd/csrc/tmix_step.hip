@@ -1,5 +1,5 @@
-// Decode-step (T == 1) time-mix core, one workgroup per (batch row, head): everything between the r/k/v
-// projections and the output projection in a single launch.
+// Decode-step (T == 1) time-mix core, one workgroup per head and one, two or four batch rows: everything between
+// the r/k/v projections and the output projection in a single launch.
 //
 // Fuses, with the reference's fp16 rounding points kept in registers:
 //   LoRA rank-out x4 (+tanh / sigmoid, v-residual gate) ... cuda/rwkv7_v3a_ops.cu:1027-1130
@@ -14,7 +14,7 @@
 // use (one memory round trip): lane q of channel i loads its 16-byte slice of state row i (the 16 lanes of
 // a row read 256 contiguous bytes) and up to four 8-element chunks (q, q+16, ...) of each of the channel's
 // LoRA rows; the 16 lanes of a channel are one DPP row, so row sums take four DPP adds.  The twelve per-channel
-// scalars (projections, biases, norm weights) are loaded by the first wavefront only, lane = channel: a load
+// scalars (projections, biases, norm weights) are loaded by one wavefront per batch row only, lane = channel: a load
 // instruction costs the CU's address unit the same 16 clocks whether it fetches 2 or 16 bytes per lane, and with
 // every wavefront fetching its own copies the scalars were more than half of the launch's load instructions.
 // That wavefront also does everything that is per channel - kk normalisation, a-gate, decay, v-residual gate,
