@@ -726,8 +726,8 @@ def test_decode_step_with_layernorm_folded_into_linear_matches_the_unfused_step(
 def test_decode_time_mix_core_with_several_batch_rows_per_block(gpu, B):
     """The single-launch time-mix core of a decode step serves 1, 2 or 4 batch rows of a head per block (the head's
     LoRA rows loaded once).  Per row the arithmetic is the same in the same order: logits, shift rows and WKV state
-    after five steps are bit-identical for 1, 2 and 4 rows per block and for the default choice (a batch of 12 takes
-    4, of 4 one).  Against the row-tiled kernels (LoRA rank-outs on the matrix core, sums in another order) they
+    after five steps are bit-identical for 1, 2 and 4 rows per block and for the default choice (one row per block at
+    this model's 8 heads; the 7.2B-width batch tests run the default at 64 heads, where 16 rows take 4).  Against the row-tiled kernels (LoRA rank-outs on the matrix core, sums in another order) they
     agree to fp16 rounding: logits and shift rows within 2e-3 of their scale, WKV state within 1e-3."""
     from rwkv_lightning_cuda_amd.model import HipModel, ModelDims, Session, State, synth_weights
     hip = gpu
