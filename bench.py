@@ -461,7 +461,7 @@ def main():
         sess.decode_greedy(first, min(args.steps, 64), state, logits)
         hip.device_sync()
         also["decode_dense_ffn_value_tok_s"] = min(args.steps, 64) * B / (time.perf_counter() - td)
-        sess.set_sparse_ffn(1)
+        sess.set_sparse_ffn(2)
         act = sess.debug_buffer("act", (B, dims.F))
         also["ffn_value_rows_skipped_fraction_last_layer"] = float(np.mean(act == 0))
 

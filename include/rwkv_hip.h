@@ -317,9 +317,10 @@ int rwkv_hip_session_set_profile(rwkv_hip_session* s, int mode);
 int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double* total_ms);
 /* Decode steps of up to max_rows rows (0..12) use the row-skipping ffn.value product when the matrix is fp16 or
  * int8 codes (CmixMode::NoFcOne / NoFcRows2 of the reference, include/rwkv7_fast_v4_common.hpp:198-211, whose
- * default is 12 rows at C = 4096).  Default 1: every extra row re-reads its share of the matrix, which pays
+ * default is 12 rows at C = 4096).  Default 2: every extra row re-reads its share of the matrix, which pays
  * only while rows x (fraction of non-zero activations) stays below 1 - about half the activations are
- * non-zero with random-init weights, far fewer with trained ones.  0 selects the dense product. */
+ * non-zero with random-init weights (7.2B shape, two rows: 2.73 -> 2.60 ms per step; from three rows on the
+ * matrix-core product is faster), far fewer with trained ones.  0 selects the dense product. */
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
 /* on != 0: the `wkv` tensor of rwkv_hip_forward / rwkv_hip_decode_greedy is the fp16 state, f16 [L,B,H,64,64], and
  * the recurrence runs in fp16 as rwkv_hip_wkv7_f16state does (ModelBackend's use_wkv32 == false, the reference

@@ -127,7 +127,7 @@ struct rwkv_hip_session {
   size_t gemm_ws_bytes = 0;
   void* sparse_ws = nullptr;  // partial rows of the row-skipping ffn.value product
   size_t sparse_ws_bytes = 0;
-  int sparse_ffn_rows = 1;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
+  int sparse_ffn_rows = 2;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
   bool wkv_fp16 = false;      // the WKV state tensor is fp16 [L,B,H,64,64] (the reference's use_wkv32 == false)
   int tmix_rows = -1;         // decode steps' single-launch time-mix core: rows per block 1/2/4, 0 never, < 0 by batch
   int fused_ln = -1;          // decode steps fold LayerNorm + token shift into the linear launches: 1 always, 0 never,

@@ -283,7 +283,7 @@ class Session:
 
     def set_sparse_ffn(self, max_rows):
         """Decode steps of up to max_rows rows (0..12; True = 1, False = 0) read only the ffn.value rows with a
-        non-zero activation (default 1)."""
+        non-zero activation (default 2)."""
         hip.check(hip.load().rwkv_hip_session_set_sparse_ffn(self.handle, ctypes.c_int(int(max_rows))))
 
     def set_profile(self, mode):
