@@ -72,10 +72,13 @@ struct GraphEntry {
 };
 
 constexpr size_t kMaxGraphs = 8;
-// Calls with at least this many rows stream the packed copy through MFMA.  Measured crossover on the 7.2B
-// shapes, all three weight formats: at 2 rows the GEMV is 5 % faster, from 3 rows on the streaming GEMM wins
-// (8 rows: 6.1 -> 3.6 ms per decode step with int8 codes; the GEMV pays one v_dot2 per row and weight pair).
-constexpr size_t kPackedMinRows = 3;
+// Calls with at least this many rows stream the packed copy through MFMA; below, the weight-streaming GEMV.  The
+// crossover moves with the width (decode ms per step, GEMV / streaming GEMM: C = 4096, int8: 2 rows 2.62 / -, 3 rows
+// 3.08 / 2.79, 8 rows 5.52 / 2.83 - the GEMV pays one v_dot2 per row and weight pair; C = 2048, int8: 3 rows 1.27 /
+// 1.38, 4 rows 1.38 / 1.38, 5 rows 1.74 / 1.39; C = 768, fp16: 3 rows 0.46 / 0.62, 4 rows 0.50 / 0.62, 5 rows 0.63 /
+// 0.63): the narrower the matrices, the more of a GEMM launch is fixed cost.
+constexpr int kPackedMinRows = 3;  // the smallest crossover: what gets a packed copy at all
+inline int packed_min_rows(int C) { return C >= 4096 ? 3 : (C >= 2048 ? 4 : 5); }
 // most blocks of a single-launch time-mix core beyond 8 rows (one round on 256 CUs; us per layer at the 7.2B shape,
 // this launch / the row-tiled kernels: 16 rows 14 / 17, 32 rows 25 / 24)
 constexpr int kTmixStepMaxBlocks = 256;
@@ -227,7 +230,7 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
     s->arena_B = B;
     s->arena_T = T;
   }
-  if (rows >= kPackedMinRows) {
+  if (rows >= static_cast<size_t>(packed_min_rows(m->C))) {
     const int R = static_cast<int>(rows);
     const int qkv_ns[7] = {m->C, m->C, m->C, m->Rw, m->Ra, m->Rg, m->Rv};
     size_t ws = std::max(linear_packed_multi_workspace_bytes(R, m->C, 7, qkv_ns),
@@ -284,7 +287,7 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
 int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int K, const half_t* x, int epilogue,
                  int out_f32, void* y, DeferredReduce* defer = nullptr, const RowCopy* copy = nullptr) {
   if (defer) *defer = DeferredReduce{};
-  if (M >= kPackedMinRows && mat.packed) {
+  if (M >= packed_min_rows(s->model->C) && mat.packed) {
     return linear_packed(s->stream, mat.fmt, M, N, K, x, mat.packed, mat.scale, mat.zp, epilogue, out_f32, y, s->gemm_ws,
                          s->gemm_ws_bytes, defer, copy);
   }
@@ -348,7 +351,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   bool packable = true;
   for (const Matrix& mat : m->layers[0].m) packable = packable && mat.packed != nullptr;
   for (int i = 0; i < 3; ++i) packable = packable && m->layers[0].lora_in_packed[i] != nullptr;
-  const bool small = rows < static_cast<int>(kPackedMinRows) || (rows <= 8 && !packable);
+  const bool small = rows < packed_min_rows(C) || (rows <= 8 && !packable);
   hipEvent_t pass_begin = nullptr;
   if (s->profile == 2) {
     RWKV_HIP_TRY(hipEventCreate(&pass_begin));
@@ -390,7 +393,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   // launch it saves (prefill of a 4096-token prompt in chunks of 128: 22.6 -> 23.2 k tok/s at batch 1, 54.2 ->
   // 53.4 k at batch 16).  RWKV_SEQ_LN=0 (tuning hook) switches it off.
   static const bool seq_ln_on = !(getenv("RWKV_SEQ_LN") && atoi(getenv("RWKV_SEQ_LN")) == 0);
-  const bool seq_fused = seq_ln_on && !step && !s->trace && C <= 4096 && rows >= static_cast<int>(kPackedMinRows) && rows <= 256;
+  const bool seq_fused = seq_ln_on && !step && !s->trace && C <= 4096 && rows >= packed_min_rows(C) && rows <= 256;
   RowCopy pending;  // shift rows waiting to be moved
   auto flush_pending = [&]() -> int {
     if (pending.n > 0) {
@@ -493,7 +496,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
           TRY_PROF(linear_small_m(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0));
         }
       } else {
-        bool all_packed = rows >= static_cast<int>(kPackedMinRows);
+        bool all_packed = rows >= packed_min_rows(C);
         for (int i = 0; i < 3; ++i) all_packed = all_packed && w.m[mids[i]].packed != nullptr;
         for (int i = 0; i < n_lora; ++i) all_packed = all_packed && w.lora_in_packed[i] != nullptr;
         if (all_packed) {
@@ -870,7 +873,7 @@ int rwkv_hip_model_set_tensor(rwkv_hip_model* m, int layer, int id, const void* 
       RWKV_HIP_TRY(hipFree(slot));
       slot = nullptr;
     }
-    if (linear_packed_supported(RWKV_FMT_F16, static_cast<int>(kPackedMinRows), ranks[i], m->C)) {
+    if (linear_packed_supported(RWKV_FMT_F16, kPackedMinRows, ranks[i], m->C)) {
       RWKV_HIP_TRY(hipMalloc(&slot, static_cast<size_t>(ranks[i]) * m->C * 2));
       const int rc = pack_weights_launch(nullptr, RWKV_FMT_F16, ranks[i], m->C, data, slot);
       if (rc != RWKV_OK) return rc;
@@ -922,7 +925,7 @@ int rwkv_hip_model_set_matrix(rwkv_hip_model* m, int layer, int id, int fmt, con
     slot.packed = nullptr;
     slot.sparse_t = nullptr;
   }
-  if (linear_packed_supported(fmt, static_cast<int>(kPackedMinRows), N, K)) {
+  if (linear_packed_supported(fmt, kPackedMinRows, N, K)) {
     // second copy of the codes in the order the MFMA path streams (batched decode and prefill)
     const size_t bytes = fmt == RWKV_FMT_F16 ? static_cast<size_t>(N) * K * 2
                                              : (fmt == RWKV_FMT_W8 ? static_cast<size_t>(N) * K : static_cast<size_t>(N) * K / 2);
