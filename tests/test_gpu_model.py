@@ -283,8 +283,7 @@ def test_greedy_stream_matches_oracle(gpu, orc):
     sess.close()
 
 
-@pytest.mark.parametrize("B", [1, 2])
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt,B", [(0, 1), (0, 2), (1, 1), (1, 2), (1, 12)])
 def test_fp16_state_mode_prefill_and_decode_match_oracle(gpu, orc, fmt, B):
     """The reference server's default mode: the WKV state in fp16 and the recurrence in fp16 fused multiply-adds
     (session option; ModelBackend's use_wkv32 == false).  A 20-token prefill call (the w12 + w0 sum rounded to fp16
@@ -292,7 +291,8 @@ def test_fp16_state_mode_prefill_and_decode_match_oracle(gpu, orc, fmt, B):
     restatement of the same graph: logits cosine >= 0.9995, greedy tokens equal except for ties, the fp16 state
     within 2e-2 of its scale (both sides round the same quantities to fp16, from activations that differ by fp16
     ulps).  The decode steps run the single-launch time-mix core with the fp16-state step in its first wavefront;
-    at one row also with the gate rank-out in blocks of its own and the LayerNorm prologues."""
+    at one row also with the gate rank-out in blocks of its own and the LayerNorm prologues; at twelve rows the
+    row-tiled rank-outs and the one-launch fp16 step that moves the state through an LDS tile."""
     from rwkv_lightning_cuda_amd.model import Session, State
     hip = gpu
     dims = small_dims()
@@ -416,12 +416,13 @@ def test_config1_0p1b_prefill_512_then_128_greedy_steps(gpu, orc):
     sess.close()
 
 
-@pytest.mark.parametrize("B", [1, 8, 64])
+@pytest.mark.parametrize("B", [1, 8, 16, 32, 64])
 def test_config2_1p5b_width_w8_decode_batches(gpu, orc, B):
     """Benchmark configuration 2 at full width (C 2048, H 32, F 8192, LoRA ranks 96/96/256/64; two layers, reduced
     vocabulary), W8A16 quantised on load: per-sequence state from a random prefill (48 tokens in chunks of 16; 16
-    tokens at batch 64 to bound the oracle's time),
-    then decode steps at batch 1 (GEMV + row-skipping ffn.value), 8 (GEMV, fused time-mix step) and 64
+    tokens from batch 16 on to bound the oracle's time),
+    then decode steps at batch 1 (GEMV + row-skipping ffn.value), 8 (streaming GEMM, single-launch time-mix core
+    with one batch row per block), 16 and 32 (the same core with two and four batch rows per block) and 64
     (streaming MFMA GEMM with split-K partials summed by the LayerNorm kernels, row-tiled time-mix kernels),
     every step's logits against the oracle."""
     import os
