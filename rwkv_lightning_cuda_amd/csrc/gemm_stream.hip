@@ -862,7 +862,16 @@ bool linear_packed_int8_tile(int M, int K) { return M > 128 && M <= 1024 && (K <
 static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns, const int* fmts) {
   int cb128 = 0;
   for (int i = 0; i < n_problems; ++i) cb128 += ceil_div(Ns[i], 128);
-  if (M <= 32 && K % (128 * 4) == 0 && cb128 < target_blocks()) return StreamConfig{1, 128, 4, 2};
+  if (M <= 32 && K % (128 * 4) == 0 && cb128 < target_blocks()) {
+    // Narrow matrices (K up to 2048) whose 64-column blocks would not fill the chip without a K split: 32-column
+    // blocks of one wavefront per K group instead - twice the blocks, half the split or none, and with no split no
+    // reduce launch (us with the reduce, 64- / 32-column blocks, 8 rows: 6656 x 2048 11.1 / 9.4, 8192 x 2048
+    // 11.4 / 9.9, 2048 x 2048 8.6 / 8.4; at K = 4096 the 64-column blocks win, 4096 x 4096 11.5 / 12.2).
+    int cb64 = 0;
+    for (int i = 0; i < n_problems; ++i) cb64 += ceil_div(Ns[i], 64);
+    if (K <= 2048 && cb64 < target_blocks()) return StreamConfig{1, 128, 4, 1};
+    return StreamConfig{1, 128, 4, 2};
+  }
   if (M > 32 && M <= 64 && cb128 >= target_blocks()) return StreamConfig{2, 128, 2, 4};
   if (M <= 64) return StreamConfig{1, 128, 2, 4};
   // 65..128 rows against few column blocks (4096 columns and fewer) and a short K: 32-row tiles need half the K
@@ -987,6 +996,7 @@ int linear_packed_multi(hipStream_t st, int M, int K, int n_problems, const Pack
     RWKV_REQUIRE(all_w8, "linear_packed: the 64 x 256 tile takes int8 weights only");
     hipLaunchKernelGGL((gemm_stream_wide_kernel<false, 2>), grid, block, 0, st, g);
   } else if (cfg.nb == 2) hipLaunchKernelGGL((gemm_stream_wide_kernel<true, 4>), grid, block, 0, st, g);
+  else if (cfg.wg == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 4, 1>), grid, block, 0, st, g);
   else if (cfg.wg == 2) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 4, 2>), grid, block, 0, st, g);
   else if (cfg.mt == 1) hipLaunchKernelGGL((gemm_stream_kernel<1, 128, 2, 4>), grid, block, 0, st, g);
   else if (cfg.mt == 2) hipLaunchKernelGGL((gemm_stream_kernel<2, 128, 2, 4>), grid, block, 0, st, g);
