@@ -857,7 +857,11 @@ struct StreamConfig {
   int nb = 1;  // bands per wavefront
   int cols() const { return 32 * wg * nb; }
 };
-bool linear_packed_int8_tile(int M, int K) { return M > 128 && M <= 1024 && (K <= 4096 || M <= 384); }
+// (narrow matrices, K up to 2048, take it from 257 rows: at 256 rows x 6656 / 8192 x 2048 the 64 x 128 tiles need
+// 19.0 / 19.8 us against 24.5 / 24.9; at 384 rows it is ahead again, 30.2 / 33.4 against 33.9 / 35.1)
+bool linear_packed_int8_tile(int M, int K) {
+  return M > (K <= 2048 ? 256 : 128) && M <= 1024 && (K <= 4096 || M <= 384);
+}
 
 static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns, const int* fmts) {
   int cb128 = 0;
@@ -873,11 +877,19 @@ static StreamConfig choose_config(int M, int K, int n_problems, const int* Ns, c
     return StreamConfig{1, 128, 4, 2};
   }
   if (M > 32 && M <= 64 && cb128 >= target_blocks()) return StreamConfig{2, 128, 2, 4};
+  // 33..64 rows of narrow matrices (K up to 2048): the 64-column blocks again, which here need no K split where the
+  // 128-column blocks do, and X is short (us with the reduce, 128- / 64-column blocks, 64 rows: 6656 x 2048
+  // 14.0 / 11.5, 8192 x 2048 15.5 / 12.1, 2048 x 2048 10.7 / 9.6)
+  if (M > 32 && M <= 64 && K <= 2048 && K % (128 * 4) == 0 && 2 * cb128 < target_blocks()) return StreamConfig{1, 128, 4, 2};
   if (M <= 64) return StreamConfig{1, 128, 2, 4};
   // 65..128 rows against few column blocks (4096 columns and fewer) and a short K: 32-row tiles need half the K
   // split of 64-row tiles for the same number of blocks (128 rows x 4096 x 4096: 19.8 -> 16.6 us; with K = 16384
   // the 64-row tiles win, 35.5 us against 38.1)
-  if (M <= 128 && K <= 4096 && ceil_div(M, 64) * cb128 * 2 <= target_blocks()) return StreamConfig{1, 128, 2, 4};
+  // ... and where the 32-row tiles alone fill the chip and the 64-row tiles do not (128 rows x 6656 x 2048:
+  // 19.5 -> 13.4 us, 8192 x 2048: 21.7 -> 14.0; at 96 rows both would split and the 64-row tiles stay ahead)
+  if (M <= 128 && K <= 4096 && ceil_div(M, 64) * cb128 < target_blocks() &&
+      (ceil_div(M, 64) * cb128 * 2 <= target_blocks() || ceil_div(M, 32) * cb128 >= target_blocks()))
+    return StreamConfig{1, 128, 2, 4};
   // 129..1024 rows, int8 weights only, and K up to 4096 or up to 384 rows: the 64 x 256 tile of two bands per
   // wavefront that fits three wavefronts per SIMD (us, 64 x 256 / 128 x 256 / 64 x 128 tiles; * = with a K split:
   // 256 rows x 16384 x 4096 51 / 59* / 64, 384 x 16384 x 4096 74 / 100* / 105, 384 x 4096 x 16384 85* / 96* / 112*,
