@@ -1,5 +1,5 @@
 // Host-side backend API, signature-compatible with the reference's include/rwkv_server_backend.hpp:15-147,
-// implemented over librwkv_hip.so.  Only the fp32 WKV state mode is provided.
+// implemented over librwkv_hip.so.  Both WKV state precisions are provided: fp16 (the default, use_wkv32 = false) and fp32.
 #pragma once
 
 #include <cstddef>

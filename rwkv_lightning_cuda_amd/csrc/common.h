@@ -13,6 +13,8 @@
 namespace rwkv {
 
 void set_error(const char* fmt, ...);
+// Compute units of the current device (asked once per device; 256 if the query fails).
+int device_cu_count();
 
 inline hipStream_t as_stream(rwkv_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -353,6 +353,10 @@ int ln_launch(hipStream_t st, int mode, int rows, const LnArgs& a) {
     RWKV_REQUIRE(a.T >= 1 && rows % a.T == 0 && a.shift && a.shift_next && a.x_out && a.n_mix >= 1 && a.n_mix <= 6 &&
                      (a.res || a.res_partial),
                  "layer norm + token shift over a sequence: bad arguments");
+    // the block of row t reads x and the residual of row t - 1 again while that row's block stores its outputs:
+    // no output may share memory with an input
+    RWKV_REQUIRE(a.x_out != a.x && a.y != a.x && (a.res == nullptr || (a.x_out != a.res && a.y != a.res)),
+                 "layer norm + token shift over a sequence: outputs must not alias x or the residual");
     if (a.C <= 256 * 8) hipLaunchKernelGGL(ln_mix_seq_kernel<256>, dim3(rows), dim3(256), 0, st, a);
     else hipLaunchKernelGGL(ln_mix_seq_kernel<512>, dim3(rows), dim3(512), 0, st, a);
     RWKV_LAUNCH_CHECK();

@@ -107,12 +107,15 @@ struct StreamArgs {
   int splits, k_per_split;
   int row_tiles, col_blocks;
   int epilogue, out_f32;
-  RowCopy copy;  // rides on the launch: the first block moves these rows (they are no operand of the product)
+  RowCopy copy;  // rides on the launch: its first blocks move these rows (they are no operand of the product)
 };
 
+// shared out between the first blocks of the launch, so that no single block carries it on its critical path
 __device__ __forceinline__ void ride_along_copy(const RowCopy& cp) {
-  if (blockIdx.x == 0 && cp.n > 0) {
-    for (int i = threadIdx.x * 8; i < cp.n; i += blockDim.x * 8)
+  constexpr unsigned kCopyBlocks = 8;
+  const unsigned nb = gridDim.x < kCopyBlocks ? gridDim.x : kCopyBlocks;
+  if (blockIdx.x < nb && blockIdx.y == 0 && blockIdx.z == 0 && cp.n > 0) {
+    for (int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8; i < cp.n; i += nb * blockDim.x * 8)
       *reinterpret_cast<uint4_t*>(cp.dst + i) = *reinterpret_cast<const uint4_t*>(cp.src + i);
   }
 }

@@ -213,7 +213,11 @@ __global__ __launch_bounds__(256) void lora_pack_w2_kernel(int C, int R, const h
   *reinterpret_cast<half8_t*>(packed + piece * 8) = v;
 }
 
-size_t lora_pack_w2_halfs(int C, int R) { return static_cast<size_t>(ceil_div(C, 32)) * ((R + 15) >> 4) * 512; }
+// Whole column blocks of the rank-out kernel (kLoraCols channels = four 32-channel bands): the wavefronts of the
+// last block read their bands without a clamp, so the bands past C exist and hold zeros.
+size_t lora_pack_w2_halfs(int C, int R) {
+  return static_cast<size_t>(ceil_div(C, kLoraCols)) * (kLoraCols / 32) * ((R + 15) >> 4) * 512;
+}
 
 int lora_pack_w2_launch(hipStream_t st, int C, int R, const half_t* w2, half_t* packed) {
   RWKV_REQUIRE(C > 0 && R > 0 && R % 8 == 0 && w2 && packed, "lora_pack_w2: bad arguments (C=%d, R=%d)", C, R);

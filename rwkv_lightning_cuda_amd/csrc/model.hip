@@ -79,9 +79,9 @@ constexpr size_t kMaxGraphs = 8;
 // 0.63): the narrower the matrices, the more of a GEMM launch is fixed cost.
 constexpr int kPackedMinRows = 3;  // the smallest crossover: what gets a packed copy at all
 inline int packed_min_rows(int C) { return C >= 4096 ? 3 : (C >= 2048 ? 4 : 5); }
-// most blocks of a single-launch time-mix core beyond 8 rows (one round on 256 CUs; us per layer at the 7.2B shape,
+// most blocks of a single-launch time-mix core beyond 8 rows (one round on the chip's compute units; us per layer at the 7.2B shape,
 // this launch / the row-tiled kernels: 16 rows 14 / 17, 32 rows 25 / 24)
-constexpr int kTmixStepMaxBlocks = 256;
+inline int tmix_step_max_blocks() { return device_cu_count(); }
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -367,7 +367,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       tmix_rows = (B % s->tmix_rows == 0 && !s->wkv_fp16) ? s->tmix_rows : 1;
     } else if (s->tmix_rows < 0) {
       const int rpb = tmix_step_rows_per_block(B, H, s->wkv_fp16);
-      if (rows <= 8 || B * H / rpb <= kTmixStepMaxBlocks) tmix_rows = rpb;
+      if (rows <= 8 || B * H / rpb <= tmix_step_max_blocks()) tmix_rows = rpb;
     }
   }
   const bool fused_tmix = tmix_rows > 0;

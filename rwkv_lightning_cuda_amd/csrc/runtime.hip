@@ -15,6 +15,25 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+int device_cu_count() {
+  constexpr int kMaxDevices = 64;
+  static int cached[kMaxDevices] = {0};  // racing first calls store the same value
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 }  // namespace rwkv
 
 using namespace rwkv;

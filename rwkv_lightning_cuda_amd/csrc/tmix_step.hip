@@ -380,7 +380,7 @@ __global__ __launch_bounds__(kStepThreads) void tmix_step_kernel(TmixStepArgs p)
 int tmix_step_rows_per_block(int B, int H, bool one_row_only) {
   int rows = 1;
   if (one_row_only) return rows;
-  const int cus = 256;  // MI355X
+  const int cus = device_cu_count();
   while (rows < 4 && B % (rows * 2) == 0 && B * H / rows > cus) rows *= 2;
   return rows;
 }

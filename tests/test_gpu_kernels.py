@@ -93,7 +93,8 @@ def test_wkv7_f16state_matches_oracle(gpu, orc, B, T, H, with_w0):
     state = dev(hip, s0)
     y = hip.DeviceArray((B, T, C), np.float16)
     d = {n: dev(hip, inp[n]) for n in names}
-    hip.wkv7_f16state(B, T, C, H, state, d["r"], d["w_raw"], d["k"], d["v"], d["a"], d["b"], y, dev(hip, elapsed),
+    d_elapsed = dev(hip, elapsed)
+    hip.wkv7_f16state(B, T, C, H, state, d["r"], d["w_raw"], d["k"], d["v"], d["a"], d["b"], y, d_elapsed,
                       w0=None if w0 is None else dev(hip, w0))
     hip.device_sync()
     got_y, got_s = y.numpy(), state.numpy()
@@ -103,7 +104,7 @@ def test_wkv7_f16state_matches_oracle(gpu, orc, B, T, H, with_w0):
     assert err <= F16_TOL
     same = float(np.mean(got_s.view(np.uint16) == s_ref.view(np.uint16)))
     assert same >= 0.9, same
-    assert elapsed.tolist() == elapsed.tolist()   # elapsed is read only
+    assert d_elapsed.numpy().tolist() == elapsed.tolist()   # the kernel only reads elapsed
 
 
 def test_wkv7_f16state_call_split_is_bitwise(gpu):
