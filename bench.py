@@ -75,6 +75,8 @@ def parse_args():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true", help="skip the oracle comparison of the measured configurations "
+                    "(the `parity` objects; about a minute of CPU work outside the timed regions)")
     ap.add_argument("--wkv-fp16", action="store_true", help="keep the WKV state in fp16 (the reference server's default, "
                     "use_wkv32 == false) in the main measurement; the headline figure is the fp32 state")
     return ap.parse_args()
@@ -156,6 +158,45 @@ def cpu_baseline(dims, fmt_name):
     }
 
 
+def parity_legs(hip, fmt_name, with_others):
+    """Oracle comparison of what the benchmark times, outside every timed region: the same layer graph with weights
+    generated on the host, so that the CPU oracle (the checker) and the GPU hold the same model.  Teacher-forced
+    greedy steps (both sides fed the oracle's tokens), every step's logits compared; a differing top-1 counts as a
+    tie when the oracle's own best two are within two fp16 ulps.  Returns (headline parity, {name: parity})."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle
+    from parity import greedy_parity
+    from rwkv_lightning_cuda_amd.model import PRESETS, ModelDims, synth_weights
+    fmts = {"f16": hip.FMT_F16, "w8": hip.FMT_W8, "w4": hip.FMT_W4}
+
+    def sliced(preset, layers):
+        d = PRESETS[preset]
+        return ModelDims(L=layers, C=d.C, H=d.H, F=d.F, V=d.V, Rw=d.Rw, Ra=d.Ra, Rg=d.Rg, Rv=d.Rv)
+
+    def leg(dims, weights, fmt_key, prompt_len, steps, what):
+        prompt = np.random.default_rng(89).integers(0, dims.V, (1, prompt_len))
+        res = greedy_parity(hip, oracle, dims, weights, fmts[fmt_key], prompt, steps, control=True)
+        res["workload"] = "%s, %s weights: %d-token prompt, then %d greedy steps at batch 1, all %d logits of every step " \
+                          "against the CPU oracle" % (what, fmt_key, prompt_len, steps, dims.V)
+        return res
+
+    d8 = sliced("7.2B", 8)
+    w8 = synth_weights(d8, 88)
+    what = "7.2B shape at a quarter of the depth (8 of 32 layers, C 4096, full 65536-row head)"
+    headline = leg(d8, w8, fmt_name, 8, 32, what)
+    others = {}
+    if with_others:
+        if fmt_name == "w8":
+            others["w4_parity"] = leg(d8, w8, "w4", 8, 16, what)
+        del w8
+        d1 = PRESETS["0.1B"]
+        others["cfg1_0p1b_f16_parity"] = leg(d1, synth_weights(d1, 12), "f16", 128, 32, "0.1B shape, all 12 layers")
+        d2 = sliced("1.5B", 8)
+        others["cfg2_1p5b_w8_parity"] = leg(d2, synth_weights(d2, 13), "w8", 8, 16,
+                                            "1.5B shape at a third of the depth (8 of 24 layers, C 2048, full head)")
+    return headline, others
+
+
 def sampled_decode(hip, sess, dims, state, logits, B, first, steps=64):
     """The decode loop a server runs: forward, then the device sampler (repetition penalties, temperature, top-k,
     top-p) on the session stream, then the picked token ids back to the host, every step."""
@@ -179,10 +220,11 @@ def sampled_decode(hip, sess, dims, state, logits, B, first, steps=64):
 
 
 def secondary_measurements(hip, model, dims, rng):
-    """Batch-8, -16 and -64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7 op alone."""
+    """Batch-1, -2, -4, -8, -16 and -64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7
+    op alone."""
     from rwkv_lightning_cuda_amd.model import Session, State
     res = {}
-    for B in (1, 8, 16, 64):
+    for B in (1, 2, 4, 8, 16, 64):
         sess = Session(model)
         state = State(dims, B)
         logits = hip.DeviceArray((B, dims.V), np.float32)
@@ -199,7 +241,8 @@ def secondary_measurements(hip, model, dims, rng):
         res["decode_bs%d_tok_s" % B] = steps * B / dt
         res["decode_bs%d_ms_per_step" % B] = dt * 1e3 / steps
         res["decode_bs%d_hbm_fraction" % B] = (model.weight_bytes() + state_bytes) / (dt / steps) / 1e9 / HBM_PEAK_GBPS
-        res.update(sampled_decode(hip, sess, dims, state, logits, B, first))
+        if B not in (2, 4):
+            res.update(sampled_decode(hip, sess, dims, state, logits, B, first))
         sess.close()
         del state, logits
 
@@ -499,6 +542,10 @@ def main():
                    "bytes_moved_fraction": moved_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                    "distinct_tokens": int(len(np.unique(toks)))},
     }
+    if "decode_dense_ffn_value_tok_s" in also:
+        # like for like: the same dense byte count over the step time with the dense ffn.value product
+        out["config"]["step_hbm_fraction_dense_ffn_value"] = \
+            (weight_bytes + state_bytes) * also["decode_dense_ffn_value_tok_s"] / B / 1e9 / HBM_PEAK_GBPS
 
     if not args.no_roofline:
         # The weight-streaming linear launches of the same steps alone, eagerly and back to back on the session
@@ -559,6 +606,9 @@ def main():
         # what a launch that waits for its predecessor costs on this box: a captured graph of 260 near-empty launches
         also["launch_chain_us_per_link_graph"] = hip.measure_launch_chain(260, 256, 256, True, 20)
         also["launch_chain_us_per_link_direct"] = hip.measure_launch_chain(260, 256, 256, False, 20)
+    if not args.no_parity and args.preset == "7.2B":
+        out["parity"], more = parity_legs(hip, args.fmt, not args.no_also)
+        also.update(more)
     if also:
         out["also"] = also
     if not args.no_cpu_baseline:

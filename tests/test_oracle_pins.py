@@ -481,6 +481,48 @@ def test_chunked_prefill_equals_one_call_in_oracle():
         om.forward(np.array([[dims.V]]), om.new_state(1))
 
 
+def test_fp16_state_model_graph_branches_on_the_call_length():
+    """orc_model_forward_f16state follows the reference's dispatch (src/rwkv7_fast_v4.cu:1266-1271): calls of up to 16
+    tokens hand w12 and w0 to the recurrence apart (added unrounded there), longer calls round f16(w12 + w0) first.
+    Which branch runs depends on the call's length only: splitting a call inside one branch changes no bit, crossing
+    the boundary (17 tokens at once against 16 + 1) changes bits but stays within fp16 noise.  The graph around the
+    recurrence is the fp32-state one (pinned against the numpy restatement above): both follow each other to fp16
+    accuracy."""
+    from rwkv_lightning_cuda_amd.model import synth_weights
+    dims = small_dims()
+    om = orc.Model(dims, synth_weights(dims, seed=23), orc.FMT_F16)
+    rng = np.random.default_rng(24)
+
+    def run(tokens, cuts, fp16=True):
+        st = om.new_state(tokens.shape[0], wkv_fp16=fp16)
+        lo = 0
+        for hi in list(cuts) + [tokens.shape[1]]:
+            logits = om.forward(tokens[:, lo:hi], st)
+            lo = hi
+        return logits, st
+
+    def same_bits(a, b):
+        return all(np.array_equal(x.view(np.uint16) if x.dtype == np.float16 else x,
+                                  y.view(np.uint16) if y.dtype == np.float16 else y) for x, y in zip(a[1], b[1])) \
+            and np.array_equal(a[0], b[0])
+
+    t16 = rng.integers(0, dims.V, (2, 16))
+    assert same_bits(run(t16, []), run(t16, [9]))             # both calls in the short branch
+    t34 = rng.integers(0, dims.V, (2, 34))
+    assert same_bits(run(t34, []), run(t34, [17]))            # both calls in the long branch
+    t17 = rng.integers(0, dims.V, (2, 17))
+    whole, split = run(t17, []), run(t17, [16])               # long branch against short + short
+    assert not np.array_equal(whole[1][1].view(np.uint16), split[1][1].view(np.uint16))
+    assert cosine(whole[0], split[0]) >= 0.9999
+    scale = np.max(np.abs(f64(split[1][1])))
+    assert np.max(np.abs(f64(whole[1][1]) - f64(split[1][1]))) <= 2e-2 * scale
+    assert whole[1][2].tolist() == split[1][2].tolist() == [17, 17]
+    # against the fp32-state graph on the same tokens
+    ref = run(t17, [], fp16=False)
+    assert cosine(whole[0], ref[0]) >= 0.999 and cosine(split[0], ref[0]) >= 0.999
+    assert np.max(np.abs(f64(whole[1][1]) - f64(ref[1][1]))) <= 3e-2 * np.max(np.abs(ref[1][1]))
+
+
 # ------------------------------------------------------------------------------- checkpoint tensors (bf16 -> fp16)
 def _bf16_bits_to_f32(bits):
     return (bits.astype(np.uint32) << 16).view(np.float32)
