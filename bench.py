@@ -75,6 +75,8 @@ def parse_args():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--fused-ln", type=int, default=-1, help="tuning hook: 1 / 0 force LayerNorm inside / outside the linear "
+                    "launches of decode steps (default: by row count)")
     ap.add_argument("--no-parity", action="store_true", help="skip the oracle comparison of the measured configurations "
                     "(the `parity` objects; about a minute of CPU work outside the timed regions)")
     ap.add_argument("--wkv-fp16", action="store_true", help="keep the WKV state in fp16 (the reference server's default, "
@@ -426,6 +428,8 @@ def main():
         sess.set_graph(False)
     if args.wkv_fp16:
         sess.set_wkv_fp16(True)
+    if args.fused_ln >= 0:
+        sess.set_fused_ln(bool(args.fused_ln))
 
     def new_state(b):
         return State(dims, b, wkv_fp16=args.wkv_fp16)
@@ -504,7 +508,7 @@ def main():
         sess.decode_greedy(first, min(args.steps, 64), state, logits)
         hip.device_sync()
         also["decode_dense_ffn_value_tok_s"] = min(args.steps, 64) * B / (time.perf_counter() - td)
-        sess.set_sparse_ffn(2)
+        sess.set_sparse_ffn(4)
         act = sess.debug_buffer("act", (B, dims.F))
         also["ffn_value_rows_skipped_fraction_last_layer"] = float(np.mean(act == 0))
 

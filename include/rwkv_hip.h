@@ -180,6 +180,16 @@ int rwkv_hip_cmix_sparse_down_relu_rows(rwkv_stream_t s, int fmt, int rows, int 
                                         void* out);
 int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int fmt, int C, int F, const void* preact, const void* wt,
                                        const void* scale, void* workspace, size_t workspace_bytes, void* out);
+/* The same product for 2..4 tokens that share one walk over the matrix: every row that is non-zero for any of the
+ * tokens is read once (a token for which it is zero takes it with an exact zero coefficient), where the _rows call
+ * reads it once per token that needs it - the form the reference's rows kernel has
+ * (cmix_sparse_spmv_relu_rows_kernel, cuda/rwkv7_fast_ops_fp16.cu:681-737: one block walks a row tile for all
+ * rows of the batch).  Same arguments and workspace as _rows.  Per token the rows add up in increasing order, but
+ * pair up differently than in the token's own walk, so the result equals _rows up to the last bits of the fp32
+ * sums; it repeats bitwise from call to call. */
+int rwkv_hip_cmix_sparse_down_relu_rows_shared(rwkv_stream_t s, int fmt, int rows, int C, int F, const void* preact,
+                                               const void* wt, const void* scale, void* workspace,
+                                               size_t workspace_bytes, void* out);
 /* The same product as rwkv_hip_cmix_sparse_down_relu_rows (same kernels, bitwise the same result) for callers
  * that cannot allocate or bring a workspace: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  No counterpart in the reference.  The fp32 partial rows live in a 16 MiB array that is part
@@ -315,25 +325,27 @@ int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host
  * and returns the number of linear launches and the summed bracketed time since the last read. */
 int rwkv_hip_session_set_profile(rwkv_hip_session* s, int mode);
 int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double* total_ms);
-/* Decode steps of up to max_rows rows (0..12) use the row-skipping ffn.value product when the matrix is fp16 or
- * int8 codes (CmixMode::NoFcOne / NoFcRows2 of the reference, include/rwkv7_fast_v4_common.hpp:198-211, whose
- * default is 12 rows at C = 4096).  Default 2: every extra row re-reads its share of the matrix, which pays
- * only while rows x (fraction of non-zero activations) stays below 1 - about half the activations are
- * non-zero with random-init weights (7.2B shape, two rows: 2.73 -> 2.60 ms per step; from three rows on the
- * matrix-core product is faster), far fewer with trained ones.  0 selects the dense product. */
+/* Decode steps of up to max_rows rows (0..12) use the row-skipping ffn.value product (CmixMode::NoFcOne / NoFcRows2
+ * of the reference, include/rwkv7_fast_v4_common.hpp:198-211, whose default is 12 rows at C = 4096).  Default 4: two
+ * to four rows share one walk that reads every row that is non-zero for any of them once (with a fraction z of zero
+ * activations per row that is 1 - z^rows of the matrix: at the z = 0.5 of random-init weights about what the dense
+ * product reads, far less with trained weights; 7.2B shape, 2 / 3 / 4 rows: 2.19 / 2.39 / 2.56 ms per step against
+ * 2.61 / 2.79 / 2.82 before).  From five rows on every row walks its own rows, which pays only while rows x (1 - z)
+ * stays below 1.  0 selects the dense product. */
 int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
 /* on != 0: the `wkv` tensor of rwkv_hip_forward / rwkv_hip_decode_greedy is the fp16 state, f16 [L,B,H,64,64], and
  * the recurrence runs in fp16 as rwkv_hip_wkv7_f16state does (ModelBackend's use_wkv32 == false, the reference
  * server's default: src/rwkv7_fast_v4.cu:1262-1271; calls of up to 16 tokens add w0 to the decay logit unrounded,
  * longer ones round w12 + w0 to fp16 first).  Default off: fp32 state.  A state belongs to one mode. */
 int rwkv_hip_session_set_wkv_fp16(rwkv_hip_session* s, int on);
-/* Decode steps on the GEMV path (one or two rows) can fold the two LayerNorm + token-shift kernels of a layer
- * into the prologue of the linear launches that consume them.  on > 0: always, 0: never, < 0 (the default): for
- * one row of at most 4096 channels.  One row goes through a kernel that requests whole weight rows up front and
- * normalises while they are in flight (two launches fewer per layer: 7.2B shape 2.04 -> 1.92 ms per step, 0.1B
- * shape 0.413 -> 0.373; same formulas and rounding points as the stand-alone kernels, sums associated differently);
- * two rows through a prologue that is bitwise the stand-alone kernels but slower than them from 2048 channels
- * on.  No counterpart in the reference (its fused decode kernels are cuda/rwkv7_v3a_ops.cu:1637-1798). */
+/* Decode steps on the GEMV path can fold the two LayerNorm + token-shift kernels of a layer into the prologue of
+ * the linear launches that consume them.  on > 0: always (where the rows fit), 0: never, < 0 (the default): for one
+ * or two rows of at most 4096 channels.  Those go through a kernel that requests whole weight rows up front and
+ * normalises while they are in flight (two launches fewer per layer: 7.2B shape, one row 2.04 -> 1.92 ms per step,
+ * 0.1B shape 0.413 -> 0.373; same formulas and rounding points as the stand-alone kernels, sums associated
+ * differently); more rows, when forced, through a prologue that is bitwise the stand-alone kernels but slower than
+ * them from 2048 channels on.  No counterpart in the reference (its fused decode kernels are
+ * cuda/rwkv7_v3a_ops.cu:1637-1798). */
 int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on);
 /* Decode steps run everything between the r/k/v projections and the output projection as one launch per layer, one
  * block per head and 1, 2 or 4 batch rows (the head's LoRA rows are loaded once per block), up to 8 rows and while

@@ -364,6 +364,242 @@ __global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_w4_kernel(int C,
   }
 }
 
+// ---- kernel 1 for several tokens at once ------------------------------------------------------------------------------
+// TOK tokens share one walk: a wavefront ballots the rows that are non-zero for ANY of its tokens and reads each of
+// them once; a token for which a row is zero takes it with coefficient zero (an exact zero product).  With a
+// fraction z of zero activations per token the walk reads 1 - z^TOK of the matrix once, where one walk per token
+// reads TOK * (1 - z) of it.  Per token the rows still add up in increasing order, but a token's rows pair up
+// differently than in its own walk (a pair is one v_dot2), so the last bits of the fp32 sums can differ from the
+// one-token kernel's; the result repeats bitwise from call to call.
+template <int TOK>
+__device__ __forceinline__ void sparse_union_heads(const half_t* __restrict__ in, int F, int f0, int lane, int activated,
+                                                  uint32_t (&abits)[TOK], uint64_t& mask) {
+  mask = 0;
+#pragma unroll
+  for (int t = 0; t < TOK; ++t) {
+    float a = 0.0f;
+    if (lane < kSparseRowsPerWave) {
+      a = h2f(in[static_cast<int64_t>(t) * F + f0 + lane]);
+      if (!activated) {
+        a = fmaxf(round_h(a), 0.0f);
+        a = round_h(a * a);
+      }
+    }
+    const half_t ah = f2h(a);
+    abits[t] = __builtin_bit_cast(uint16_t, ah);
+    mask |= __ballot((abits[t] << 17) != 0u);  // +0 and -0 both count as zero
+  }
+}
+
+// the wavefronts' sums of one token meet in LDS in wavefront order; the block writes the token's partial row
+template <int LC>
+__device__ __forceinline__ void sparse_block_row(const float (&acc)[LC], float (*red)[64 * LC], int wave, int lane, int C, int c0,
+                                                 float* __restrict__ partial_row) {
+  constexpr int kCols = 64 * LC;
+#pragma unroll
+  for (int i = 0; i < LC / 4; ++i)
+    *reinterpret_cast<float4_t*>(&red[wave][LC * lane + 4 * i]) =
+        float4_t{acc[4 * i], acc[4 * i + 1], acc[4 * i + 2], acc[4 * i + 3]};
+  __syncthreads();
+  if (threadIdx.x < kCols / 4) {
+    const int c = 4 * threadIdx.x;
+    float4_t sum = *reinterpret_cast<const float4_t*>(&red[0][c]);
+#pragma unroll
+    for (int w = 1; w < kSparseWaves; ++w) sum = sum + *reinterpret_cast<const float4_t*>(&red[w][c]);
+    if (c0 + c < C) *reinterpret_cast<float4_t*>(partial_row + c0 + c) = sum;
+  }
+  __syncthreads();  // red is written again for the next token
+}
+
+template <int FMT, int TOK>
+__global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_union_kernel(int C, int F, int activated,
+                                                                             const half_t* __restrict__ in,
+                                                                             const uint4_t* __restrict__ wt,
+                                                                             float* __restrict__ partial) {
+  constexpr int LC = sparse_lane_cols(FMT);
+  constexpr int kCols = 64 * LC;
+  __shared__ __align__(16) float red[kSparseWaves][kCols];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int f0 = blockIdx.x * kSparseRowsPerBlock + wave * kSparseRowsPerWave;
+  const int c0 = blockIdx.y * kCols;
+  const bool col_ok = c0 + LC * lane < C;
+  const int row_pieces = C / LC;
+  const uint4_t* wlane = wt + c0 / LC + (col_ok ? lane : 0);
+
+  uint32_t abits[TOK];
+  uint64_t mask;
+  sparse_union_heads<TOK>(in, F, f0, lane, activated, abits, mask);
+
+  float acc[TOK][LC];
+#pragma unroll
+  for (int t = 0; t < TOK; ++t)
+#pragma unroll
+    for (int i = 0; i < LC; ++i) acc[t][i] = 0.0f;
+  const half2_t bias = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
+
+  while (mask != 0) {
+    int row[kSparseBatch];
+    bool live[kSparseBatch];
+    const int first = __builtin_ctzll(mask);
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p) {
+      live[p] = mask != 0;
+      if (live[p]) {
+        row[p] = __builtin_ctzll(mask);
+        mask &= mask - 1;
+      } else {
+        row[p] = first;  // a row already read, taken with coefficient zero: no load sits under a branch
+      }
+    }
+    uint4_t q[kSparseBatch];
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p) q[p] = __builtin_nontemporal_load(&wlane[static_cast<int64_t>(f0 + row[p]) * row_pieces]);
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; p += 2) {
+      half2_t ap[TOK];
+#pragma unroll
+      for (int t = 0; t < TOK; ++t) {
+        const uint32_t c0b = live[p] ? static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(abits[t]), row[p])) : 0u;
+        const uint32_t c1b = live[p + 1] ? static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(abits[t]), row[p + 1])) : 0u;
+        ap[t] = as_half2(c0b | (c1b << 16));
+      }
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t lo = q[p][d];
+        const uint32_t hi = q[p + 1][d];
+        if constexpr (FMT == RWKV_FMT_W8) {
+          const half2_t w0 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c040c00u) | 0x64006400u) - bias;
+          const half2_t w1 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c050c01u) | 0x64006400u) - bias;
+          const half2_t w2 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c060c02u) | 0x64006400u) - bias;
+          const half2_t w3 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x0c070c03u) | 0x64006400u) - bias;
+#pragma unroll
+          for (int t = 0; t < TOK; ++t) {
+            acc[t][4 * d + 0] = __builtin_amdgcn_fdot2(ap[t], w0, acc[t][4 * d + 0], false);
+            acc[t][4 * d + 1] = __builtin_amdgcn_fdot2(ap[t], w1, acc[t][4 * d + 1], false);
+            acc[t][4 * d + 2] = __builtin_amdgcn_fdot2(ap[t], w2, acc[t][4 * d + 2], false);
+            acc[t][4 * d + 3] = __builtin_amdgcn_fdot2(ap[t], w3, acc[t][4 * d + 3], false);
+          }
+        } else {
+          const half2_t w0 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x05040100u));
+          const half2_t w1 = as_half2(__builtin_amdgcn_perm(hi, lo, 0x07060302u));
+#pragma unroll
+          for (int t = 0; t < TOK; ++t) {
+            acc[t][2 * d + 0] = __builtin_amdgcn_fdot2(ap[t], w0, acc[t][2 * d + 0], false);
+            acc[t][2 * d + 1] = __builtin_amdgcn_fdot2(ap[t], w1, acc[t][2 * d + 1], false);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TOK; ++t)
+    sparse_block_row<LC>(acc[t], red, wave, lane, C, c0,
+                         partial + (static_cast<int64_t>(t) * gridDim.x + blockIdx.x) * C);
+}
+
+// int4 codes, several tokens at once: the walk of ffn_sparse_w4_kernel over the union of the tokens' rows
+template <int TOK>
+__global__ __launch_bounds__(64 * kSparseWaves) void ffn_sparse_w4_union_kernel(int C, int F, int activated,
+                                                                                const half_t* __restrict__ in,
+                                                                                const uint8_t* __restrict__ blob,
+                                                                                float* __restrict__ partial) {
+  constexpr int LC = 16;
+  constexpr int kCols = 64 * LC;
+  __shared__ __align__(16) float red[kSparseWaves][kCols];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int f0 = blockIdx.x * kSparseRowsPerBlock + wave * kSparseRowsPerWave;
+  const int c0 = blockIdx.y * kCols;
+  const bool col_ok = c0 + LC * lane < C;
+  const int cl = c0 + (col_ok ? LC * lane : 0);
+  const int row_pieces = C / LC;
+  const uint2_t* wlane = reinterpret_cast<const uint2_t*>(blob) + cl / LC;
+  const int G = F / 128;
+  const half_t* scale_t = reinterpret_cast<const half_t*>(blob + static_cast<size_t>(C) * F / 2);
+  const uint8_t* zp_t = reinterpret_cast<const uint8_t*>(scale_t + static_cast<size_t>(G) * C);
+  const int64_t gat = static_cast<int64_t>(f0 / 128) * C + cl;
+  const half8_t sc0 = *reinterpret_cast<const half8_t*>(scale_t + gat);
+  const half8_t sc1 = *reinterpret_cast<const half8_t*>(scale_t + gat + 8);
+  const uint4_t zq = *reinterpret_cast<const uint4_t*>(zp_t + gat);
+
+  uint32_t abits[TOK];
+  uint64_t mask;
+  sparse_union_heads<TOK>(in, F, f0, lane, activated, abits, mask);
+
+  float acc[TOK][LC];
+  float asum[TOK];
+#pragma unroll
+  for (int t = 0; t < TOK; ++t) {
+    asum[t] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < LC; ++i) acc[t][i] = 0.0f;
+  }
+  const half2_t bias = {static_cast<half_t>(1024.0f), static_cast<half_t>(1024.0f)};
+
+  while (mask != 0) {
+    int row[kSparseBatch];
+    bool live[kSparseBatch];
+    const int first = __builtin_ctzll(mask);
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p) {
+      live[p] = mask != 0;
+      if (live[p]) {
+        row[p] = __builtin_ctzll(mask);
+        mask &= mask - 1;
+      } else {
+        row[p] = first;
+      }
+    }
+    uint2_t q[kSparseBatch];
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; ++p)
+      q[p] = __builtin_nontemporal_load(&wlane[static_cast<int64_t>(f0 + row[p]) * row_pieces]);
+#pragma unroll
+    for (int p = 0; p < kSparseBatch; p += 2) {
+      half2_t ap[TOK];
+#pragma unroll
+      for (int t = 0; t < TOK; ++t) {
+        const uint32_t c0b = live[p] ? static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(abits[t]), row[p])) : 0u;
+        const uint32_t c1b = live[p + 1] ? static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(abits[t]), row[p + 1])) : 0u;
+        ap[t] = as_half2(c0b | (c1b << 16));
+        asum[t] += h2f(ap[t][0]) + h2f(ap[t][1]);
+      }
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        const uint32_t lo = q[p][d];
+        const uint32_t hi = q[p + 1][d];
+        const uint32_t ea = lo & 0x0f0f0f0fu, oa = (lo >> 4) & 0x0f0f0f0fu;
+        const uint32_t eb = hi & 0x0f0f0f0fu, ob = (hi >> 4) & 0x0f0f0f0fu;
+        half2_t w[8];
+        w[0] = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c040c00u) | 0x64006400u) - bias;
+        w[1] = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c040c00u) | 0x64006400u) - bias;
+        w[2] = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c050c01u) | 0x64006400u) - bias;
+        w[3] = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c050c01u) | 0x64006400u) - bias;
+        w[4] = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c060c02u) | 0x64006400u) - bias;
+        w[5] = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c060c02u) | 0x64006400u) - bias;
+        w[6] = as_half2(__builtin_amdgcn_perm(eb, ea, 0x0c070c03u) | 0x64006400u) - bias;
+        w[7] = as_half2(__builtin_amdgcn_perm(ob, oa, 0x0c070c03u) | 0x64006400u) - bias;
+#pragma unroll
+        for (int t = 0; t < TOK; ++t)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[t][8 * d + i] = __builtin_amdgcn_fdot2(ap[t], w[i], acc[t][8 * d + i], false);
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TOK; ++t) {
+#pragma unroll
+    for (int i = 0; i < LC; ++i) {
+      const float zpf = static_cast<float>((zq[i >> 2] >> (8 * (i & 3))) & 0xffu);
+      const float scf = h2f(i < 8 ? sc0[i] : sc1[i - 8]);
+      acc[t][i] = (acc[t][i] - zpf * asum[t]) * scf;
+    }
+    sparse_block_row<LC>(acc[t], red, wave, lane, C, c0,
+                         partial + (static_cast<int64_t>(t) * gridDim.x + blockIdx.x) * C);
+  }
+}
+
 // ---- kernel 2: out[c] = f16(scale[c] * sum of the partial rows); block 0 also does the optional row copy --------
 // grid = (ceil(C/64), tokens), block = 256 = 16 groups of partial rows x 16 column quads.  Group g sums rows g, g+16, ... (its
 // loads are independent, so they are all in flight together), the 16 group sums meet in LDS in group order.
@@ -399,8 +635,24 @@ __global__ __launch_bounds__(256) void ffn_sparse_finish_kernel(int C, int n_par
   *reinterpret_cast<half4_t*>(out + c) = o;
 }
 
+template <int TOK>
+static void launch_union(hipStream_t st, int fmt, dim3 grid, int C, int F, int activated, const half_t* in, const void* wt,
+                         float* ws) {
+  const dim3 block(64 * kSparseWaves);
+  if (fmt == RWKV_FMT_W4) {
+    hipLaunchKernelGGL((ffn_sparse_w4_union_kernel<TOK>), grid, block, 0, st, C, F, activated, in, static_cast<const uint8_t*>(wt), ws);
+  } else if (fmt == RWKV_FMT_W8) {
+    hipLaunchKernelGGL((ffn_sparse_union_kernel<RWKV_FMT_W8, TOK>), grid, block, 0, st, C, F, activated, in,
+                       static_cast<const uint4_t*>(wt), ws);
+  } else {
+    hipLaunchKernelGGL((ffn_sparse_union_kernel<RWKV_FMT_F16, TOK>), grid, block, 0, st, C, F, activated, in,
+                       static_cast<const uint4_t*>(wt), ws);
+  }
+}
+
 int ffn_sparse_launch(hipStream_t st, int fmt, int rows, int C, int F, int activated, const half_t* in, const void* wt,
-                      const half_t* scale, void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy) {
+                      const half_t* scale, void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy,
+                      bool one_walk) {
   RWKV_REQUIRE(ffn_sparse_supported(fmt, C, F), "ffn_sparse: unsupported format %d or shape C=%d F=%d", fmt, C, F);
   RWKV_REQUIRE(rows >= 1 && rows <= kSparseMaxRows, "ffn_sparse: %d rows (1..%d)", rows, kSparseMaxRows);
   RWKV_REQUIRE(in && wt && out && (fmt != RWKV_FMT_W8 || scale), "ffn_sparse: NULL tensor");
@@ -413,7 +665,14 @@ int ffn_sparse_launch(hipStream_t st, int fmt, int rows, int C, int F, int activ
   }
   const int n_partial = F / kSparseRowsPerBlock;
   const dim3 grid(n_partial, ceil_div(C, 64 * sparse_lane_cols(fmt)), rows);
-  if (fmt == RWKV_FMT_W4) {
+  if (one_walk && rows >= 2 && rows <= kSparseUnionMaxRows) {
+    // the tokens share one walk over the rows that are non-zero for any of them
+    const dim3 g2(grid.x, grid.y, 1);
+    float* ws = static_cast<float*>(workspace);
+    if (rows == 2) launch_union<2>(st, fmt, g2, C, F, activated, in, wt, ws);
+    else if (rows == 3) launch_union<3>(st, fmt, g2, C, F, activated, in, wt, ws);
+    else launch_union<4>(st, fmt, g2, C, F, activated, in, wt, ws);
+  } else if (fmt == RWKV_FMT_W4) {
     hipLaunchKernelGGL(ffn_sparse_w4_kernel, grid, dim3(64 * kSparseWaves), 0, st, C, F, activated, in,
                        static_cast<const uint8_t*>(wt), static_cast<float*>(workspace));
   } else if (fmt == RWKV_FMT_W8) {
@@ -466,7 +725,15 @@ int rwkv_hip_cmix_sparse_down_relu_rows(rwkv_stream_t s, int fmt, int rows, int 
                                         const void* wt, const void* scale, void* workspace, size_t workspace_bytes,
                                         void* out) {
   return ffn_sparse_launch(as_stream(s), fmt, rows, C, F, 0, static_cast<const half_t*>(preact), wt,
-                           static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr);
+                           static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr, false);
+}
+
+int rwkv_hip_cmix_sparse_down_relu_rows_shared(rwkv_stream_t s, int fmt, int rows, int C, int F, const void* preact,
+                                               const void* wt, const void* scale, void* workspace,
+                                               size_t workspace_bytes, void* out) {
+  RWKV_REQUIRE(rows >= 2 && rows <= kSparseUnionMaxRows, "cmix_sparse_shared: %d rows (2..%d)", rows, kSparseUnionMaxRows);
+  return ffn_sparse_launch(as_stream(s), fmt, rows, C, F, 0, static_cast<const half_t*>(preact), wt,
+                           static_cast<const half_t*>(scale), workspace, workspace_bytes, static_cast<half_t*>(out), nullptr, true);
 }
 
 // Device address of this GPU's copy of `scratch`, looked up once per device (with that device current).
@@ -500,7 +767,7 @@ int rwkv_hip_cmix_sparse_down_relu_rows_static(rwkv_stream_t s, int fmt, int row
   const int rc = static_scratch_address(&ws);
   if (rc != RWKV_OK) return rc;
   return ffn_sparse_launch(as_stream(s), fmt, rows, C, F, 0, static_cast<const half_t*>(preact), wt,
-                           static_cast<const half_t*>(scale), ws, kStaticScratchBytes, static_cast<half_t*>(out), nullptr);
+                           static_cast<const half_t*>(scale), ws, kStaticScratchBytes, static_cast<half_t*>(out), nullptr, false);
 }
 
 int rwkv_hip_cmix_sparse_down_relu_one(rwkv_stream_t s, int fmt, int C, int F, const void* preact, const void* wt,

@@ -447,25 +447,32 @@ struct Row1Cfg {
 // no memory.  Everything that arrived goes to LDS at once (stash: NT * 4 floats for the row sum, then 4 x NT * 4
 // fp16 values: LN weight, bias, previous LN output, lerp coefficients) and is read back piece by piece, each
 // thread only what it wrote, so the prologue's registers stay few.
-template <int V8>
-struct LnRow1xV {  // V8 groups of eight values
-  half8_t xv[V8], rv[V8], wv[V8], bv[V8], pv[V8], mv[V8];
+template <int V8, int M>
+struct LnRow1xV {  // V8 groups of eight values, M rows
+  half8_t xv[M][V8], rv[M][V8], pv[M][V8];  // per row: x, the residual, the previous token's LN output
+  half8_t wv[V8], bv[V8], mv[V8];           // shared by the rows: LN weight and bias, lerp coefficients
 };
 
-// thread t of the computing wavefronts owns the groups t, t + NTL, ... (NTL computing threads)
-template <int V8, int NTL>
-__device__ __forceinline__ LnRow1xV<V8> ln_row1_request8(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
-  const int64_t xsrc = ln.mode == 2 ? ln.tokens[0] * static_cast<int64_t>(K) : 0;
-  LnRow1xV<V8> q;
+// thread t of the computing wavefronts owns the groups t, t + NTL, ... (NTL computing threads).  Every row's
+// operands are requested in one go, so that the rows share one trip to memory.
+template <int V8, int NTL, int M>
+__device__ __forceinline__ LnRow1xV<V8, M> ln_row1_request8(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
+  LnRow1xV<V8, M> q;
 #pragma unroll
   for (int g = 0; g < V8; ++g) {
     const int c = (threadIdx.x + g * NTL) * 8;
     const int cc = c < K ? c : 0;
-    q.xv[g] = *reinterpret_cast<const half8_t*>(ln.x + xsrc + cc);
-    q.rv[g] = *reinterpret_cast<const half8_t*>(ln.mode == 1 ? ln.res + cc : ln.x + xsrc + cc);
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const int64_t row = static_cast<int64_t>(m) * K;
+      const int64_t xsrc = ln.mode == 2 ? ln.tokens[m] * static_cast<int64_t>(K) : row;
+      q.xv[m][g] = *reinterpret_cast<const half8_t*>(ln.x + xsrc + cc);
+      q.rv[m][g] = *reinterpret_cast<const half8_t*>(ln.mode == 1 ? ln.res + row + cc : ln.x + xsrc + cc);
+    }
     q.wv[g] = *reinterpret_cast<const half8_t*>(ln.w + cc);
     q.bv[g] = *reinterpret_cast<const half8_t*>(ln.b + cc);
-    q.pv[g] = *reinterpret_cast<const half8_t*>(ln.shift + cc);
+#pragma unroll
+    for (int m = 0; m < M; ++m) q.pv[m][g] = *reinterpret_cast<const half8_t*>(ln.shift + static_cast<int64_t>(m) * K + cc);
     q.mv[g] = *reinterpret_cast<const half8_t*>(mu + cc);
   }
   return q;
@@ -483,9 +490,10 @@ __device__ __forceinline__ float front_waves_sum(float v, int wave, float* scrat
   return t;
 }
 
-template <int NT, int V8, int NTL>
-__device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8>& q, const LnPrologue& ln, int K, half_t* xs,
+template <int NT, int V8, int NTL, int M>
+__device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8, M>& q, const LnPrologue& ln, int K, int m, half_t* xs,
                                                 float* stash, float* red, bool store, int wave) {
+  const int64_t row = static_cast<int64_t>(m) * K;
   constexpr int NWL = NTL / 64;  // wavefronts that compute
   half_t* hstash = reinterpret_cast<half_t*>(stash + NT * 4);
   float sum = 0.0f;
@@ -495,17 +503,17 @@ __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8>& q, const LnP
     float v[8];
     if (ln.mode == 1) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[g][e]) + h2f(q.rv[g][e]);
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[m][g][e]) + h2f(q.rv[m][g][e]);
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[g][e]);
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[m][g][e]);
     }
     if (c < K) sum += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
     *reinterpret_cast<float4_t*>(stash + c) = float4_t{v[0], v[1], v[2], v[3]};
     *reinterpret_cast<float4_t*>(stash + c + 4) = float4_t{v[4], v[5], v[6], v[7]};
     *reinterpret_cast<half8_t*>(hstash + c) = q.wv[g];
     *reinterpret_cast<half8_t*>(hstash + c + NT * 4) = q.bv[g];
-    *reinterpret_cast<half8_t*>(hstash + c + NT * 8) = q.pv[g];
+    *reinterpret_cast<half8_t*>(hstash + c + NT * 8) = q.pv[m][g];
     *reinterpret_cast<half8_t*>(hstash + c + NT * 12) = q.mv[g];
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -555,8 +563,8 @@ __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8>& q, const LnP
         xo[e] = f2h(ve);
       }
       if (store) {
-        *reinterpret_cast<half8_t*>(ln.ln_out + c) = yv;
-        if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + c) = xo;
+        *reinterpret_cast<half8_t*>(ln.ln_out + row + c) = yv;
+        if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + row + c) = xo;
       }
     }
     *reinterpret_cast<half8_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
@@ -569,11 +577,11 @@ __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8>& q, const LnP
 // launch, while a prologue before them leaves HBM idle for its 1.5 us.  So the wavefronts share the work: some
 // compute the prologue and request their weights afterwards, the others request theirs at once and meet the first
 // at the barrier (7.2B shape, int8: 1.79 -> 1.72 ms per step against the prologue in every wavefront first).
-template <int FMT, int NT, bool LN>
+template <int FMT, int NT, bool LN, int M>
 __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const LinearProblem& prob, int blk, half_t* xs,
                                                float* red) {
   using T = FmtTraits<FMT>;
-  constexpr int KCAP = LN ? NT * 4 : NT * 8;  // values of x the block stages: one slice per thread
+  constexpr int KCAP = LN ? NT * 4 : NT * 8;  // values of x the block stages per row: one slice per thread
   using Cfg = Row1Cfg<FMT, KCAP>;
   constexpr int R = Cfg::kRows;
   constexpr int S = Cfg::kSteps;
@@ -595,25 +603,35 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   constexpr int NTL = NT / (FMT == RWKV_FMT_W4 ? 4 : 2);  // threads that compute the prologue
   constexpr int V8 = NT * 4 / (NTL * 8);  // groups of eight values per computing thread
   const bool ln_wave = LN && wave < NTL / 64;
-  uint4_t xq = {0u, 0u, 0u, 0u};
+  uint4_t xq[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) xq[m] = uint4_t{0u, 0u, 0u, 0u};
   if constexpr (LN) {
     // (below, after the row scales)
   } else if (prob.x_f32 != nullptr) {
     // x = f16(x_f32 * gate): the products are formed here, one rounding each
     if (static_cast<int>(threadIdx.x) * 8 < K) {
-      const float4_t f0 = *reinterpret_cast<const float4_t*>(prob.x_f32 + threadIdx.x * 8);
-      const float4_t f1 = *reinterpret_cast<const float4_t*>(prob.x_f32 + threadIdx.x * 8 + 4);
-      const half8_t gq = *reinterpret_cast<const half8_t*>(prob.x_gate + threadIdx.x * 8);
-      half8_t xh;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        xh[e] = f2h(f0[e] * h2f(gq[e]));
-        xh[4 + e] = f2h(f1[e] * h2f(gq[4 + e]));
+      for (int m = 0; m < M; ++m) {
+        const float* xf = prob.x_f32 + static_cast<int64_t>(m) * K + threadIdx.x * 8;
+        const float4_t f0 = *reinterpret_cast<const float4_t*>(xf);
+        const float4_t f1 = *reinterpret_cast<const float4_t*>(xf + 4);
+        const half8_t gq = *reinterpret_cast<const half8_t*>(prob.x_gate + static_cast<int64_t>(m) * K + threadIdx.x * 8);
+        half8_t xh;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          xh[e] = f2h(f0[e] * h2f(gq[e]));
+          xh[4 + e] = f2h(f1[e] * h2f(gq[4 + e]));
+        }
+        xq[m] = __builtin_bit_cast(uint4_t, xh);
       }
-      xq = __builtin_bit_cast(uint4_t, xh);
     }
   } else {
-    if (static_cast<int>(threadIdx.x) * 8 < K) xq = *reinterpret_cast<const uint4_t*>(prob.x + threadIdx.x * 8);
+    if (static_cast<int>(threadIdx.x) * 8 < K) {
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        xq[m] = *reinterpret_cast<const uint4_t*>(prob.x + static_cast<int64_t>(m) * K + threadIdx.x * 8);
+    }
   }
   // the int8 rows' output scales too: read at the end they would cost every wavefront one more trip to memory
   half_t row_scale[R];
@@ -643,26 +661,34 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
       }
     }
   };
-  // x in LDS: one slice per thread, zeros beyond K
+  // x in LDS: one slice per thread and row (rows KCAP values apart), zeros beyond K
   if constexpr (LN) {
     // two code paths, so that the prologue's operands and the weight vectors never hold registers together; the
-    // second path passes the two barriers of the first one's block sums
+    // second path passes the two barriers of the first one's block sums, once per row
     if (ln_wave) {
-      const LnRow1xV<V8> lnq = ln_row1_request8<V8, NTL>(args.ln, prob.mu, K);
+      const LnRow1xV<V8, M> lnq = ln_row1_request8<V8, NTL, M>(args.ln, prob.mu, K);
       __builtin_amdgcn_sched_barrier(0);
-      ln_row1_finish8<NT, V8, NTL>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0, wave);
-      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        ln_row1_finish8<NT, V8, NTL, M>(lnq, args.ln, K, m, xs + m * KCAP, reinterpret_cast<float*>(xs + M * KCAP), red,
+                                        blockIdx.x == 0, wave);
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int st = 0; st < S; ++st) request(st);
     } else {
 #pragma unroll
       for (int st = 0; st < S; ++st) request(st);
       __builtin_amdgcn_sched_barrier(0);
-      __syncthreads();
-      __syncthreads();
+#pragma unroll 1
+      for (int m = 0; m < M; ++m) {
+        __syncthreads();
+        __syncthreads();
+      }
     }
   } else {
-    *reinterpret_cast<uint4_t*>(xs + threadIdx.x * 8) = xq;
+#pragma unroll
+    for (int m = 0; m < M; ++m) *reinterpret_cast<uint4_t*>(xs + m * KCAP + threadIdx.x * 8) = xq[m];
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int st = 0; st < S; ++st) request(st);
@@ -671,62 +697,78 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   __syncthreads();
   if (!active) return;
 
-  float acc[R];
+  // per (row of W, row of x): steps in order, the lane's pairs in order - the order of one-row launches, same bits
+  float acc[R][M];
 #pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
 #pragma unroll
   for (int st = 0; st < S; ++st) {
     const int k0 = st * T::kStep + lane * T::kElems;
     if (st * T::kStep < K && k0 + T::kElems <= KCAP) {  // (the second test only where a step is wider than KCAP)
       constexpr int XV = T::kElems / 2;
-      half2_t xv[XV];
 #pragma unroll
-      for (int q = 0; q < XV / 4; ++q) {
-        const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + k0 + q * 8);
+      for (int m = 0; m < M; ++m) {
+        half2_t xv[XV];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
-      }
-      if constexpr (FMT == RWKV_FMT_W4) {
-        half2_t xp[XV];
-        WeightVec<FMT>::pair_x(xv, xp);
+        for (int q = 0; q < XV / 4; ++q) {
+          const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KCAP + k0 + q * 8);
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const half_t zf = static_cast<half_t>(1024.0f + static_cast<float>(zp[st][r]));
-          const half2_t zb = {zf, zf};
-          const float part = WeightVec<FMT>::dot(w[st][r], xp, zb, 0.0f);
-          acc[r] = fmaf(part, h2f(sc[st][r]), acc[r]);
+          for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
         }
-      } else {
+        if constexpr (FMT == RWKV_FMT_W4) {
+          half2_t xp[XV];
+          WeightVec<FMT>::pair_x(xv, xp);
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[r] = WeightVec<FMT>::dot(w[st][r], xv, acc[r]);
+          for (int r = 0; r < R; ++r) {
+            const half_t zf = static_cast<half_t>(1024.0f + static_cast<float>(zp[st][r]));
+            const half2_t zb = {zf, zf};
+            const float part = WeightVec<FMT>::dot(w[st][r], xp, zb, 0.0f);
+            acc[r][m] = fmaf(part, h2f(sc[st][r]), acc[r][m]);
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(w[st][r], xv, acc[r][m]);
+        }
       }
     }
   }
 #pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[r][m] = wave_sum(acc[r][m]);
   if (lane == 0) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int n = row0 + r;
-      float v = round_h(acc[r] * h2f(row_scale[r]));
-      if (args.epilogue == RWKV_EPI_RELU_SQUARE) {
-        v = fmaxf(v, 0.0f);
-        v = round_h(v * v);
-      }
-      if (args.out_f32) {
-        static_cast<float*>(prob.y)[n] = v;
-      } else {
-        static_cast<half_t*>(prob.y)[n] = f2h(v);
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float v = round_h(acc[r][m] * h2f(row_scale[r]));
+        if (args.epilogue == RWKV_EPI_RELU_SQUARE) {
+          v = fmaxf(v, 0.0f);
+          v = round_h(v * v);
+        }
+        const int64_t o = static_cast<int64_t>(m) * N + n;
+        if (args.out_f32) {
+          static_cast<float*>(prob.y)[o] = v;
+        } else {
+          static_cast<half_t*>(prob.y)[o] = f2h(v);
+        }
       }
     }
   }
 }
 
-// grid = blocks over all problems; a block of NT threads covers NT/64 * (1 or 2) rows; dynamic LDS = x (NT * 4 fp16
-// values with the prologue, NT * 8 without).  DF is the format of the launch's quantised problems; fp16 problems
-// (the LoRA rank-ins) may ride along.
-template <int NT, bool LN, int DF>
-__global__ __launch_bounds__(NT) void linear_gemv_row1_kernel(LinearArgs args) {
+// grid = blocks over all problems; a block of NT threads covers NT/64 * (1 or 2) rows of W for all M rows of x; dynamic
+// LDS = M rows of x (NT * 4 fp16 values each with the prologue, NT * 8 without) + the prologue's stash.  DF is the
+// format of the launch's quantised problems; fp16 problems (the LoRA rank-ins) may ride along.
+// With the prologue and 1024 threads two blocks must share a CU (every block of the launch resident at once): 8
+// wavefronts per SIMD, i.e. at most 64 registers - asked for here, and checked from the compiler's resource report at
+// build time.  (Two rows of int4 codes do not fit that budget and run one block per CU.)
+template <int NT, bool LN, int DF, int M>
+__global__ __launch_bounds__(NT, (LN && NT == 1024 && (M == 1 || DF != RWKV_FMT_W4)) ? 8 : 1)
+void linear_gemv_row1_kernel(LinearArgs args) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   __shared__ float red[2 * (NT / 64)];
   half_t* xs = reinterpret_cast<half_t*>(lds_raw);
@@ -745,9 +787,9 @@ __global__ __launch_bounds__(NT) void linear_gemv_row1_kernel(LinearArgs args) {
   const LinearProblem prob = args.p[pi];
   const int blk = blockIdx.x - first;
   if (DF != RWKV_FMT_F16 && prob.fmt == DF) {  // uniform per block
-    gemv_row1_block<DF, NT, LN>(args, prob, blk, xs, red);
+    gemv_row1_block<DF, NT, LN, M>(args, prob, blk, xs, red);
   } else {
-    gemv_row1_block<RWKV_FMT_F16, NT, LN>(args, prob, blk, xs, red);
+    gemv_row1_block<RWKV_FMT_F16, NT, LN, M>(args, prob, blk, xs, red);
   }
 }
 
@@ -765,7 +807,13 @@ static int row1_format(const LinearArgs& args) {
   return df;
 }
 
-template <int NT, bool LN, int DF>
+// Rows of x the whole-rows-in-flight kernel takes: up to 4 (each more row costs every weight vector another eight
+// v_dot2 and two LDS reads; beyond 4 the matrix core is the better tool), up to 2 with the LayerNorm prologue (each
+// row's prologue runs before the computing wavefronts request their weights, and the stash shares the LDS).
+constexpr int kRow1MaxRows = 4;
+constexpr int kRow1MaxRowsLn = 2;
+
+template <int NT, bool LN, int DF, int M>
 static int launch_row1(hipStream_t st, LinearArgs& args) {
   int total = 0;
   for (int i = 0; i < args.n_problems; ++i) {
@@ -774,34 +822,47 @@ static int launch_row1(hipStream_t st, LinearArgs& args) {
     args.block_end[i] = total;
   }
   args.KT = LN ? NT * 4 : NT * 8;
-  // x; with the prologue also its stash: the fp32 row sum and four fp16 vectors
-  const size_t lds = static_cast<size_t>(args.KT) * (LN ? 2 + 4 + 4 * 2 : 2);
-  hipLaunchKernelGGL((linear_gemv_row1_kernel<NT, LN, DF>), dim3(total), dim3(NT), lds, st, args);
+  // x rows; with the prologue also its stash: the fp32 row sum and four fp16 vectors
+  const size_t lds = static_cast<size_t>(args.KT) * (2 * M + (LN ? 4 + 4 * 2 : 0));
+  if (lds > 48 * 1024) {  // beyond the default limit of dynamic LDS: raised once per instantiation
+    static bool raised = false;
+    if (!raised) {
+      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_gemv_row1_kernel<NT, LN, DF, M>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL((linear_gemv_row1_kernel<NT, LN, DF, M>), dim3(total), dim3(NT), lds, st, args);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
-template <int NT, bool LN>
+template <int NT, bool LN, int M>
 static int launch_row1_fmt(hipStream_t st, LinearArgs& args, int df) {
   switch (df) {
-    case RWKV_FMT_W8: return launch_row1<NT, LN, RWKV_FMT_W8>(st, args);
-    case RWKV_FMT_W4: return launch_row1<NT, LN, RWKV_FMT_W4>(st, args);
-    default: return launch_row1<NT, LN, RWKV_FMT_F16>(st, args);
+    case RWKV_FMT_W8: return launch_row1<NT, LN, RWKV_FMT_W8, M>(st, args);
+    case RWKV_FMT_W4: return launch_row1<NT, LN, RWKV_FMT_W4, M>(st, args);
+    default: return launch_row1<NT, LN, RWKV_FMT_F16, M>(st, args);
   }
 }
 
 // Block size by row length: one slice of x per thread (4 values with the prologue, 8 without).
+template <int M>
 static int launch_row1_any(hipStream_t st, LinearArgs& args, int df) {
   const int K = args.K;
-  if (args.ln.mode != 0) {
-    if (K <= 1024) return launch_row1_fmt<256, true>(st, args, df);
-    if (K <= 2048) return launch_row1_fmt<512, true>(st, args, df);
-    return launch_row1_fmt<1024, true>(st, args, df);
+  if constexpr (M <= kRow1MaxRowsLn) {
+    if (args.ln.mode != 0) {
+      if (K <= 1024) return launch_row1_fmt<256, true, M>(st, args, df);
+      if (K <= 2048) return launch_row1_fmt<512, true, M>(st, args, df);
+      return launch_row1_fmt<1024, true, M>(st, args, df);
+    }
   }
-  if (K <= 2048) return launch_row1_fmt<256, false>(st, args, df);
-  return launch_row1_fmt<512, false>(st, args, df);
+  if (K <= 2048) return launch_row1_fmt<256, false, M>(st, args, df);
+  return launch_row1_fmt<512, false, M>(st, args, df);
 }
 
+
+int linear_ln_prologue_max_rows(int K) { return K <= 4096 && K % 8 == 0 ? kRow1MaxRowsLn : 0; }
 
 // Batched small-M linear: n_problems problems sharing M (<= 8), K, epilogue and output type.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
@@ -852,11 +913,19 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
     gated = true;
     RWKV_REQUIRE(problems[i].x_gate != nullptr && K % 8 == 0, "linear: a gated x needs its gate and K %% 8 == 0");
   }
-  if (M == 1) {
+  if (M <= (args.ln.mode != 0 ? kRow1MaxRowsLn : kRow1MaxRows)) {
     const int df = row1_format(args);
-    if (df >= 0 && !(gated && args.ln.mode != 0)) return launch_row1_any(st, args, df);
+    if (df >= 0 && !(gated && args.ln.mode != 0)) {
+      switch (M) {
+        case 1: return launch_row1_any<1>(st, args, df);
+        case 2: return launch_row1_any<2>(st, args, df);
+        case 3: return launch_row1_any<3>(st, args, df);
+        default: return launch_row1_any<4>(st, args, df);
+      }
+    }
   }
-  RWKV_REQUIRE(!gated, "linear: x = x_f32 * gate is formed by one-row launches only (M = %d, K = %d)", M, K);
+  RWKV_REQUIRE(!gated, "linear: x = x_f32 * gate is formed by launches of up to %d rows of at most 4096 values (M = %d, K = %d)",
+               kRow1MaxRows, M, K);
   switch (M) {
     case 1: return launch_one<1, 2, 1>(st, args);
     case 2: return launch_one<2, 2, 1>(st, args);

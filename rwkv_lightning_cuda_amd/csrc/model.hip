@@ -72,13 +72,15 @@ struct GraphEntry {
 };
 
 constexpr size_t kMaxGraphs = 8;
-// Calls with at least this many rows stream the packed copy through MFMA; below, the weight-streaming GEMV.  The
-// crossover moves with the width (decode ms per step, GEMV / streaming GEMM: C = 4096, int8: 2 rows 2.62 / -, 3 rows
-// 3.08 / 2.79, 8 rows 5.52 / 2.83 - the GEMV pays one v_dot2 per row and weight pair; C = 2048, int8: 3 rows 1.27 /
-// 1.38, 4 rows 1.38 / 1.38, 5 rows 1.74 / 1.39; C = 768, fp16: 3 rows 0.46 / 0.62, 4 rows 0.50 / 0.62, 5 rows 0.63 /
-// 0.63): the narrower the matrices, the more of a GEMM launch is fixed cost.
-constexpr int kPackedMinRows = 3;  // the smallest crossover: what gets a packed copy at all
-inline int packed_min_rows(int C) { return C >= 4096 ? 3 : (C >= 2048 ? 4 : 5); }
+// Calls with at least this many rows stream the packed copy through MFMA; below, the weight-streaming GEMV that keeps
+// whole weight rows in flight for up to 4 rows of x (decode ms per step, GEMV / streaming GEMM: 7.2B shape, int8: 3 rows
+// 2.39 / 2.79, 4 rows 2.56 / 2.82; 1.5B shape: 3 rows 1.20 / 1.45, 4 rows 1.31 / 1.51, 5 rows 1.55 / 1.31; 0.1B shape,
+// fp16: 3 rows 0.51 / 0.63, 4 rows 0.57 / 0.67).  RWKV_PACKED_MIN_ROWS (tuning hook) overrides the crossover.
+constexpr int kPackedMinRows = 3;  // what gets a packed copy at all: rows too long for the GEMV (ffn.value) use it from here
+inline int packed_min_rows(int /*C*/) {
+  static const int forced = getenv("RWKV_PACKED_MIN_ROWS") ? atoi(getenv("RWKV_PACKED_MIN_ROWS")) : 0;
+  return forced >= kPackedMinRows ? forced : 5;
+}
 // most blocks of a single-launch time-mix core beyond 8 rows (one round on the chip's compute units; us per layer at the 7.2B shape,
 // this launch / the row-tiled kernels: 16 rows 14 / 17, 32 rows 25 / 24)
 inline int tmix_step_max_blocks() { return device_cu_count(); }
@@ -130,7 +132,8 @@ struct rwkv_hip_session {
   size_t gemm_ws_bytes = 0;
   void* sparse_ws = nullptr;  // partial rows of the row-skipping ffn.value product
   size_t sparse_ws_bytes = 0;
-  int sparse_ffn_rows = 2;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
+  int sparse_ffn_rows = 4;    // decode steps of up to this many rows read only the ffn.value rows with a non-zero activation
+                              // (2..4 rows share one walk over the rows that are non-zero for any of them)
   bool wkv_fp16 = false;      // the WKV state tensor is fp16 [L,B,H,64,64] (the reference's use_wkv32 == false)
   int tmix_rows = -1;         // decode steps' single-launch time-mix core: rows per block 1/2/4, 0 never, < 0 by batch
   int fused_ln = -1;          // decode steps fold LayerNorm + token shift into the linear launches: 1 always, 0 never,
@@ -287,7 +290,8 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
 int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int K, const half_t* x, int epilogue,
                  int out_f32, void* y, DeferredReduce* defer = nullptr, const RowCopy* copy = nullptr) {
   if (defer) *defer = DeferredReduce{};
-  if (M >= packed_min_rows(s->model->C) && mat.packed) {
+  // (rows longer than the few-row GEMV keeps in registers go to the packed product from its smallest row count on)
+  if (mat.packed && (M >= packed_min_rows(s->model->C) || (M >= kPackedMinRows && K > 4096))) {
     return linear_packed(s->stream, mat.fmt, M, N, K, x, mat.packed, mat.scale, mat.zp, epilogue, out_f32, y, s->gemm_ws,
                          s->gemm_ws_bytes, defer, copy);
   }
@@ -374,10 +378,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   // Decode steps on the GEMV path can fold both LayerNorm + token-shift kernels of a layer into the prologue of the
   // linear launch that consumes them (r/k/v + LoRA rank-ins; ffn.key): by default for one row of up to 4096
   // channels.  The residual-stream tap needs the stand-alone kernels.
-  const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows == 1 && C <= 4096);
+  const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows <= linear_ln_prologue_max_rows(C));
   // (the shift row that the prologue leaves for later is stored by the single-launch time-mix core)
   const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace && fused_tmix &&
-                            static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152;
+                            (rows <= linear_ln_prologue_max_rows(C) ||
+                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152);
   // One row: the gate rank-out of the time-mix core (more than half of its bytes) runs in blocks of its own and the
   // output projection's launch applies the gate while it stages x.
   const bool gate_split = fused_tmix && rows == 1 && C <= 4096 && !s->trace;
@@ -681,7 +686,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       cp.src = b.ln2; cp.dst = shift1; cp.n = rows * C;
       if (sparse_value && mv.sparse_t) {
         TRY_AUX(ffn_sparse_launch(st, mv.fmt, rows, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
-                                  &cp));
+                                  &cp, true));
       } else {
         LinearProblem pv = {mv.data, mv.scale, mv.zp, b.act, b.cm, C, mv.fmt, nullptr};
         TRY_PROF(linear_small_m(st, rows, F, 1, &pv, RWKV_EPI_NONE, 0, nullptr, &cp));
@@ -693,7 +698,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       const Matrix& mv = w.m[RWKV_M_FFN_VALUE];
       if (sparse_value && mv.sparse_t) {
         TRY_AUX(ffn_sparse_launch(st, mv.fmt, rows, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
-                                  nullptr));
+                                  nullptr, true));
       } else {
         TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm, defer_ok ? &cm_partial : nullptr));
       }

@@ -54,6 +54,8 @@ struct RowCopy {
 // share M and K (each with its own weight format, x and y) in one launch.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
                    int out_f32, const LnPrologue* ln = nullptr, const RowCopy* copy = nullptr);
+// Rows of a decode step that linear_small_m takes with the LayerNorm prologue at this row length (0: none).
+int linear_ln_prologue_max_rows(int K);
 // Any M: MFMA tiles for M >= 16 where supported, else row tiles through the GEMV kernel.
 int linear_any_m(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* w, const half_t* scale,
                  const uint8_t* zp, int epilogue, int out_f32, void* y);
@@ -206,8 +208,12 @@ size_t ffn_sparse_workspace_bytes(int rows, int C, int F);
 int ffn_sparse_pack_launch(hipStream_t st, int fmt, int C, int F, const void* w, void* wt);
 // `in` [rows,F], `out` [rows,C].  activated != 0: `in` holds f16(relu(preact)^2) already; else the kernel applies it.
 // `copy` (optional) rides on the second launch.  scale: per output channel for int8 codes, unused for fp16.
+// one_walk: 2 .. kSparseUnionMaxRows tokens share one walk over the rows that are non-zero for any of them (each such
+// row is read once); otherwise every token walks its own rows.
+constexpr int kSparseUnionMaxRows = 4;
 int ffn_sparse_launch(hipStream_t st, int fmt, int rows, int C, int F, int activated, const half_t* in, const void* wt,
-                      const half_t* scale, void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy);
+                      const half_t* scale, void* workspace, size_t workspace_bytes, half_t* out, const RowCopy* copy,
+                      bool one_walk);
 
 // ---- sampler.hip --------------------------------------------------------------------------------
 int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out);

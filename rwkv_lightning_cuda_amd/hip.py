@@ -40,6 +40,7 @@ EXPORTS = [
     "rwkv_hip_cmix_sparse_pack", "rwkv_hip_cmix_sparse_pack_w4", "rwkv_hip_cmix_sparse_packed_bytes",
     "rwkv_hip_cmix_sparse_workspace", "rwkv_hip_cmix_sparse_down_relu_one",
     "rwkv_hip_cmix_sparse_down_relu_rows", "rwkv_hip_cmix_sparse_down_relu_rows_static",
+    "rwkv_hip_cmix_sparse_down_relu_rows_shared",
     "rwkv_hip_session_set_sparse_ffn", "rwkv_hip_session_set_fused_ln", "rwkv_hip_session_set_tmix_rows", "rwkv_hip_session_set_wkv_fp16",
     "rwkv_hip_layer_norm", "rwkv_hip_add_layer_norm", "rwkv_hip_add_last_layer_norm", "rwkv_hip_token_shift_mix",
     "rwkv_hip_add_layer_norm_cmix_mix", "rwkv_hip_add_layer_norm_tmix_mix6", "rwkv_hip_kk_a_gate",
@@ -290,6 +291,13 @@ def cmix_sparse_down_relu_one(fmt, C, F, preact, wt, scale, workspace, out, stre
 def cmix_sparse_down_relu_rows(fmt, rows, C, F, preact, wt, scale, workspace, out, stream=None):
     check(load().rwkv_hip_cmix_sparse_down_relu_rows(_p(stream), _i(fmt), _i(rows), _i(C), _i(F), _p(preact), _p(wt),
                                                      _p(scale), _p(workspace), ctypes.c_size_t(workspace.nbytes), _p(out)))
+
+
+def cmix_sparse_down_relu_rows_shared(fmt, rows, C, F, preact, wt, scale, workspace, out, stream=None):
+    """2..4 tokens in one walk over the rows that are non-zero for any of them."""
+    check(load().rwkv_hip_cmix_sparse_down_relu_rows_shared(_p(stream), _i(fmt), _i(rows), _i(C), _i(F), _p(preact),
+                                                            _p(wt), _p(scale), _p(workspace),
+                                                            ctypes.c_size_t(workspace.nbytes), _p(out)))
 
 
 def measure_launch_chain(links, blocks=1, threads=64, use_graph=True, reps=20):

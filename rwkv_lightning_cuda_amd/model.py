@@ -267,8 +267,8 @@ class Session:
         return out
 
     def set_fused_ln(self, on):
-        """Decode steps fold LayerNorm + token shift into the linear launches (bitwise the same): True always, False
-        never, None (the default of a new session) for one row of at most 4096 channels."""
+        """Decode steps fold LayerNorm + token shift into the linear launches: True always, False never, None (the
+        default of a new session) for one or two rows of at most 4096 channels."""
         hip.check(hip.load().rwkv_hip_session_set_fused_ln(self.handle, ctypes.c_int(-1 if on is None else 1 if on else 0)))
 
     def set_tmix_rows(self, rows):
@@ -283,7 +283,7 @@ class Session:
 
     def set_sparse_ffn(self, max_rows):
         """Decode steps of up to max_rows rows (0..12; True = 1, False = 0) read only the ffn.value rows with a
-        non-zero activation (default 2)."""
+        non-zero activation (default 4; two to four rows share one walk over the rows any of them needs)."""
         hip.check(hip.load().rwkv_hip_session_set_sparse_ffn(self.handle, ctypes.c_int(int(max_rows))))
 
     def set_profile(self, mode):

@@ -699,6 +699,61 @@ def test_cmix_sparse_down_rows_matches_the_one_row_product(gpu, orc, fmt_name):
         hip.cmix_sparse_down_relu_rows(fmt, rows, C, F, dev(hip, pre), wt, sd, ws1, out)  # workspace of one row
 
 
+@pytest.mark.parametrize("fmt_name", ["w8", "f16", "w4"])
+@pytest.mark.parametrize("C,F,rows", [(768, 3072, 2), (2048, 8192, 3), (4096, 16384, 4)])
+def test_cmix_sparse_down_shared_walk_matches_oracle_and_per_token_walks(gpu, orc, fmt_name, C, F, rows):
+    """2..4 tokens in one walk over the union of their non-zero rows, at the three benchmark widths: against the
+    oracle's dense product (the bar of the fp16 paths) and against one walk per token (equal up to the last bits of
+    the fp32 sums: within an fp16 ulp of the output's scale after rounding, mostly identical); a token without any active row comes
+    out as zeros; two calls give the same bits."""
+    hip = gpu
+    rng = np.random.default_rng(C + rows)
+    w = (rng.standard_normal((C, F)) * 0.02).astype(np.float16)
+    z = None
+    if fmt_name == "w4":
+        fmt = hip.FMT_W4
+        q, s, z, wt = _sparse_w4_pack(hip, orc, w)
+        sd = None
+    elif fmt_name == "w8":
+        fmt = hip.FMT_W8
+        q, s = orc.quantize_w8(w)
+        sd = dev(hip, s)
+        wt = hip.DeviceArray((F, C), np.uint8)
+    else:
+        fmt = hip.FMT_F16
+        q, s, sd = w, None, None
+        wt = hip.DeviceArray((F, C), np.float16)
+    if fmt_name != "w4":
+        hip.cmix_sparse_pack(fmt, C, F, dev(hip, q), wt)
+    pre = rng.standard_normal((rows, F)).astype(np.float16)
+    pre[1, : F // 2] = -np.abs(pre[1, : F // 2])   # the tokens' masks differ in whole wavefront ranges too
+    if rows >= 3:
+        pre[2] = -np.abs(pre[2])                   # a token with no active row at all
+    ws = hip.DeviceArray.zeros((hip.cmix_sparse_workspace(C, F, rows),), np.uint8)
+    out = hip.DeviceArray((rows, C), np.float16)
+    hip.cmix_sparse_down_relu_rows_shared(fmt, rows, C, F, dev(hip, pre), wt, sd, ws, out)
+    hip.device_sync()
+    got = out.numpy()
+    want = orc.gemv(fmt, orc.relu_square(pre), q, s, z)
+    assert rel_err(got.astype(np.float32), want.astype(np.float32)) <= F16_TOL
+    if rows >= 3:
+        assert not got[2].any()
+    per_token = hip.DeviceArray((rows, C), np.float16)
+    hip.cmix_sparse_down_relu_rows(fmt, rows, C, F, dev(hip, pre), wt, sd, ws, per_token)
+    hip.device_sync()
+    ref = per_token.numpy()
+    same = float(np.mean(ref.view(np.uint16) == got.view(np.uint16)))
+    assert same >= 0.9, same
+    # (a sum that cancels to almost nothing can move by more than its own ulp: the bar is an ulp of the row's scale)
+    assert rel_err(got.astype(np.float32), ref.astype(np.float32)) <= 2.0 ** -10
+    again = hip.DeviceArray((rows, C), np.float16)
+    hip.cmix_sparse_down_relu_rows_shared(fmt, rows, C, F, dev(hip, pre), wt, sd, ws, again)
+    hip.device_sync()
+    assert np.array_equal(again.numpy().view(np.uint16), got.view(np.uint16))
+    with pytest.raises(hip.RwkvHipError):
+        hip.cmix_sparse_down_relu_rows_shared(fmt, 5, C, F, dev(hip, pre), wt, sd, ws, out)   # more tokens than one walk takes
+
+
 def test_cmix_sparse_rejects_bad_arguments(gpu):
     hip = gpu
     with pytest.raises(hip.RwkvHipError):
