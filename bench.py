@@ -337,6 +337,37 @@ def secondary_measurements(hip, model, dims, rng):
     return res
 
 
+def engine_boundary_rates(preset, fmt_name):
+    """tok/s through the drop-in boundary: the C++ host API (InferenceEngine::batch_generate_stream over ModelBackend,
+    one fresh GenerationState and logits buffer per request, device sampler + picked ids back to the host every step)
+    as its own GenerationStats report them - the reference server's decode_speed / prefill_speed counters.  Runs the
+    tool tests/cpp/bin/engine_rate_bench as a child process (its own model of the same shape and format)."""
+    import subprocess
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "engine_rate_bench")
+    if not os.path.exists(exe):
+        return {"error": "tests/cpp/bin/engine_rate_bench is not built"}
+    out = {}
+    for name, batch, tokens, sampled in (("greedy_bs1", 1, 128, 0), ("sampled_bs1", 1, 128, 1), ("greedy_bs16", 16, 64, 0),
+                                         ("sampled_bs16", 16, 64, 1)):
+        cmd = [exe, ROOT, "synthetic:%s:%s" % (preset, fmt_name), str(batch), str(tokens), "3", str(sampled), "1"]
+        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        if proc.returncode != 0:
+            out[name] = {"error": proc.stderr.strip()[-300:]}
+            continue
+        reqs = [json.loads(line) for line in proc.stdout.splitlines() if line.startswith("{")]
+        out[name] = {
+            "first_request_decode_tok_s": reqs[0]["decode_tok_s"],
+            "steady_decode_tok_s": reqs[-1]["decode_tok_s"],
+            "steady_decode_ms_per_step": reqs[-1]["decode_ms_per_step"],
+            "steady_prefill_tok_s": reqs[-1]["prefill_tok_s"],
+            "prompt_tokens": reqs[-1]["prompt_tokens"], "generated_tokens": reqs[-1]["generated_tokens"],
+            "graph_captures_per_request": [r["graph_captures"] for r in reqs],
+        }
+    out["what"] = ("InferenceEngine::batch_generate_stream over ModelBackend(synthetic:%s:%s, fp32 WKV state), 3 requests "
+                   "of identical prompts each; rates from GenerationStats" % (preset, fmt_name))
+    return out
+
+
 def other_configs(hip, rng):
     """Benchmark configurations 1 and 2 on the same GPU: the 0.1B shape with fp16 weights (512-token prompt in chunks
     of 128, then 128 greedy steps at batch 1) and the 1.5B shape W8A16 (256-token prefill per sequence, then decode at
@@ -610,6 +641,7 @@ def main():
         # what a launch that waits for its predecessor costs on this box: a captured graph of 260 near-empty launches
         also["launch_chain_us_per_link_graph"] = hip.measure_launch_chain(260, 256, 256, True, 20)
         also["launch_chain_us_per_link_direct"] = hip.measure_launch_chain(260, 256, 256, False, 20)
+        also["engine_boundary"] = engine_boundary_rates(args.preset, args.fmt)
     if not args.no_parity and args.preset == "7.2B":
         out["parity"], more = parity_legs(hip, args.fmt, not args.no_also)
         also.update(more)

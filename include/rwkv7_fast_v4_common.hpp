@@ -33,12 +33,12 @@ struct DeviceBuffer {
   DeviceBuffer() = default;
   DeviceBuffer(const DeviceBuffer&) = delete;
   DeviceBuffer& operator=(const DeviceBuffer&) = delete;
-  DeviceBuffer(DeviceBuffer&& o) noexcept : p(o.p), n(o.n) { o.p = nullptr; o.n = 0; }
+  DeviceBuffer(DeviceBuffer&& o) noexcept : p(o.p), n(o.n), recycled(o.recycled) { o.p = nullptr; o.n = 0; o.recycled = false; }
   DeviceBuffer& operator=(DeviceBuffer&& o) noexcept {
     if (this != &o) {
       release();
-      p = o.p; n = o.n;
-      o.p = nullptr; o.n = 0;
+      p = o.p; n = o.n; recycled = o.recycled;
+      o.p = nullptr; o.n = 0; o.recycled = false;
     }
     return *this;
   }
@@ -53,16 +53,33 @@ struct DeviceBuffer {
     n = count;
   }
 
+  // The same from the recycled blocks (rwkv_hip_malloc_recycled): freed buffers of this size come back at their old
+  // addresses.  For buffers that a serving loop allocates per request (generation state, logits).
+  void resize_recycled(std::size_t count, const char* what) {
+    if (count <= n) return;
+    release();
+    void* q = nullptr;
+    check_hip(rwkv_hip_malloc_recycled(&q, count * sizeof(T)), what);
+    p = static_cast<T*>(q);
+    n = count;
+    recycled = true;
+  }
+
   void zero(const char* what) {
     if (p && n) check_hip(rwkv_hip_memset(p, 0, n * sizeof(T)), what);
   }
 
  private:
   void release() {
-    if (p) rwkv_hip_free(p);
+    if (p) {
+      if (recycled) rwkv_hip_free_recycled(p, n * sizeof(T));
+      else rwkv_hip_free(p);
+    }
     p = nullptr;
     n = 0;
+    recycled = false;
   }
+  bool recycled = false;
 };
 
 struct ModelDims {

@@ -48,6 +48,16 @@ int rwkv_hip_device_count(int* count);
 int rwkv_hip_device_name(char* buf, size_t buf_len);
 int rwkv_hip_malloc(void** ptr, size_t bytes);
 int rwkv_hip_free(void* ptr);
+/* Blocks that come back: rwkv_hip_free_recycled keeps the block (after waiting for the device, as hipFree does) and
+ * the next rwkv_hip_malloc_recycled of the same byte size on the same device returns it - last in, first out, not
+ * cleared.  The generation state and logits of consecutive requests of one shape then sit at the same addresses,
+ * which is what a session's captured decode graphs are keyed by.  At most 24 GiB are held (oldest freed first);
+ * an allocation that fails for lack of memory frees them all and tries again; rwkv_hip_mem_info counts them as
+ * free; rwkv_hip_recycle_trim frees them.  No counterpart in the reference (cudaMalloc / cudaFree per
+ * DeviceBuffer, include/rwkv7_fast_v4_common.hpp:64-110). */
+int rwkv_hip_malloc_recycled(void** ptr, size_t bytes);
+int rwkv_hip_free_recycled(void* ptr, size_t bytes);
+int rwkv_hip_recycle_trim(void);
 int rwkv_hip_host_alloc(void** ptr_host, size_t bytes); /* pinned */
 int rwkv_hip_host_free(void* ptr_host);
 int rwkv_hip_memcpy_h2d(void* dst, const void* src_host, size_t bytes);
@@ -323,6 +333,9 @@ int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host
  * duration does not depend on the data, and this gives the kernels' launch-to-launch time without event
  * overhead between them; state and logits hold garbage afterwards.  read_profile waits for the stream
  * and returns the number of linear launches and the summed bracketed time since the last read. */
+/* Decode graphs captured so far in this process, over all sessions: a serving loop in its steady state captures
+ * none (a step whose batch width, state and logits addresses have been seen replays the graph captured then). */
+int rwkv_hip_graph_capture_count(int64_t* count);
 int rwkv_hip_session_set_profile(rwkv_hip_session* s, int mode);
 int rwkv_hip_session_read_profile(rwkv_hip_session* s, int64_t* launches, double* total_ms);
 /* Decode steps of up to max_rows rows (0..12) use the row-skipping ffn.value product (CmixMode::NoFcOne / NoFcRows2

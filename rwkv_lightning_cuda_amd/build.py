@@ -5,7 +5,7 @@
   csrc/*.hip -> librwkv_hip.so    gfx950 kernels behind the C ABI of include/rwkv_hip.h (hipcc; it
                                   cross-compiles without a GPU present).  No Python or torch dependency.
   host/*.cpp -> librwkv_host.so   the C++ host API of include/*.hpp (g++), linked against librwkv_hip.so.
-  tests/cpp/*_test.cpp -> tests/cpp/bin/*   test executables of the host API.
+  tests/cpp/*_test.cpp, *_bench.cpp -> tests/cpp/bin/*   test executables and measurement tools of the host API.
 """
 import concurrent.futures
 import os
@@ -121,12 +121,17 @@ def host_test_names():
     return sorted(f[:-4] for f in os.listdir(TEST_SRC) if f.endswith("_test.cpp"))
 
 
+def host_tool_names():
+    """Measurement tools over the host API (run by bench.py), built like the tests."""
+    return sorted(f[:-4] for f in os.listdir(TEST_SRC) if f.endswith("_bench.cpp"))
+
+
 def build_host_tests(verbose=True):
     """Compiles every tests/cpp/*_test.cpp into tests/cpp/bin/ (needs both libraries)."""
     os.makedirs(TEST_BIN, exist_ok=True)
     rpath = "-Wl,-rpath," + PKG_DIR + ":$ORIGIN/../../../rwkv_lightning_cuda_amd"
     outs = []
-    for name in host_test_names():
+    for name in host_test_names() + host_tool_names():
         out = os.path.join(TEST_BIN, name)
         cmd = ([CXX] + CXX_FLAGS + ["-I" + TEST_SRC, os.path.join(TEST_SRC, name + ".cpp"), "-o", out,
                                    "-L" + PKG_DIR, "-lrwkv_host", "-lrwkv_hip", "-pthread", rpath])

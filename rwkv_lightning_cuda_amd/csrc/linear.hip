@@ -571,6 +571,125 @@ __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8, M>& q, const 
   }
 }
 
+// The prologue of a one-row launch, kept as its own set of functions beside the several-row ones above (same
+// arithmetic): written through the several-row form with M = 1, the int4 kernel came out four registers heavier -
+// past the 64 that let two 1024-thread blocks share a CU - and spilled.
+template <int V8>
+struct LnRowOne {  // V8 groups of eight values
+  half8_t xv[V8], rv[V8], wv[V8], bv[V8], pv[V8], mv[V8];
+};
+
+// thread t of the computing wavefronts owns the groups t, t + NTL, ... (NTL computing threads)
+template <int V8, int NTL>
+__device__ __forceinline__ LnRowOne<V8> ln_one_request8(const LnPrologue& ln, const half_t* __restrict__ mu, int K) {
+  const int64_t xsrc = ln.mode == 2 ? ln.tokens[0] * static_cast<int64_t>(K) : 0;
+  LnRowOne<V8> q;
+#pragma unroll
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
+    const int cc = c < K ? c : 0;
+    q.xv[g] = *reinterpret_cast<const half8_t*>(ln.x + xsrc + cc);
+    q.rv[g] = *reinterpret_cast<const half8_t*>(ln.mode == 1 ? ln.res + cc : ln.x + xsrc + cc);
+    q.wv[g] = *reinterpret_cast<const half8_t*>(ln.w + cc);
+    q.bv[g] = *reinterpret_cast<const half8_t*>(ln.b + cc);
+    q.pv[g] = *reinterpret_cast<const half8_t*>(ln.shift + cc);
+    q.mv[g] = *reinterpret_cast<const half8_t*>(mu + cc);
+  }
+  return q;
+}
+
+// sum over the first NWL wavefronts of the block (the callers); the other wavefronts pass the barrier too
+template <int NWL>
+__device__ __forceinline__ float front_waves_sum_one(float v, int wave, float* scratch) {
+  v = wave_sum_uniform(v);
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NWL; ++i) t += scratch[i];
+  return t;
+}
+
+template <int NT, int V8, int NTL>
+__device__ __forceinline__ void ln_one_finish8(const LnRowOne<V8>& q, const LnPrologue& ln, int K, half_t* xs,
+                                                float* stash, float* red, bool store, int wave) {
+  constexpr int NWL = NTL / 64;  // wavefronts that compute
+  half_t* hstash = reinterpret_cast<half_t*>(stash + NT * 4);
+  float sum = 0.0f;
+#pragma unroll
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
+    float v[8];
+    if (ln.mode == 1) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[g][e]) + h2f(q.rv[g][e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = h2f(q.xv[g][e]);
+    }
+    if (c < K) sum += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    *reinterpret_cast<float4_t*>(stash + c) = float4_t{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<float4_t*>(stash + c + 4) = float4_t{v[4], v[5], v[6], v[7]};
+    *reinterpret_cast<half8_t*>(hstash + c) = q.wv[g];
+    *reinterpret_cast<half8_t*>(hstash + c + NT * 4) = q.bv[g];
+    *reinterpret_cast<half8_t*>(hstash + c + NT * 8) = q.pv[g];
+    *reinterpret_cast<half8_t*>(hstash + c + NT * 12) = q.mv[g];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  sum = front_waves_sum_one<NWL>(sum, wave, red);
+  const float mean = sum / static_cast<float>(K);
+  float sv = 0.0f;
+#pragma unroll
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
+    if (c < K) {
+      const float4_t v0 = *reinterpret_cast<const float4_t*>(stash + c);
+      const float4_t v1 = *reinterpret_cast<const float4_t*>(stash + c + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float d = v0[e] - mean;
+        sv = fmaf(d, d, sv);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float d = v1[e] - mean;
+        sv = fmaf(d, d, sv);
+      }
+    }
+  }
+  sv = front_waves_sum_one<NWL>(sv, wave, red + NT / 64);
+  const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
+#pragma unroll
+  for (int g = 0; g < V8; ++g) {
+    const int c = (threadIdx.x + g * NTL) * 8;
+    half8_t ov;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ov[e] = static_cast<half_t>(0.0f);
+    if (c < K) {
+      const float4_t v0 = *reinterpret_cast<const float4_t*>(stash + c);
+      const float4_t v1 = *reinterpret_cast<const float4_t*>(stash + c + 4);
+      const half8_t wv = *reinterpret_cast<const half8_t*>(hstash + c);
+      const half8_t bv = *reinterpret_cast<const half8_t*>(hstash + c + NT * 4);
+      const half8_t pv = *reinterpret_cast<const half8_t*>(hstash + c + NT * 8);
+      const half8_t mv = *reinterpret_cast<const half8_t*>(hstash + c + NT * 12);
+      half8_t yv, xo;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float ve = e < 4 ? v0[e & 3] : v1[e & 3];
+        yv[e] = f2h(fmaf((ve - mean) * rstd, h2f(wv[e]), h2f(bv[e])));
+        const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
+        ov[e] = f2h(fmaf(h2f(pv[e]) - yf, h2f(mv[e]), yf));
+        xo[e] = f2h(ve);
+      }
+      if (store) {
+        *reinterpret_cast<half8_t*>(ln.ln_out + c) = yv;
+        if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + c) = xo;
+      }
+    }
+    *reinterpret_cast<half8_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
+  }
+}
+
 // One block.  A wavefront cannot do both at once: it stalls on its weight requests until the memory pipeline has
 // room for them - late in a 67 MB launch that takes microseconds (timestamps: the last wavefronts get their
 // requests out 11 us after the launch began) - and a prologue behind the requests would end up at the tail of the
@@ -666,6 +785,12 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
     // two code paths, so that the prologue's operands and the weight vectors never hold registers together; the
     // second path passes the two barriers of the first one's block sums, once per row
     if (ln_wave) {
+      if constexpr (M == 1) {
+        const LnRowOne<V8> lnq = ln_one_request8<V8, NTL>(args.ln, prob.mu, K);
+        __builtin_amdgcn_sched_barrier(0);
+        ln_one_finish8<NT, V8, NTL>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0, wave);
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
       const LnRow1xV<V8, M> lnq = ln_row1_request8<V8, NTL, M>(args.ln, prob.mu, K);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -673,6 +798,7 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
         ln_row1_finish8<NT, V8, NTL, M>(lnq, args.ln, K, m, xs + m * KCAP, reinterpret_cast<float*>(xs + M * KCAP), red,
                                         blockIdx.x == 0, wave);
         __builtin_amdgcn_sched_barrier(0);
+      }
       }
 #pragma unroll
       for (int st = 0; st < S; ++st) request(st);

@@ -10,6 +10,7 @@
 //   * T == 1 steps are captured once into a HIP graph per (batch, state, logits) tuple and replayed;
 //   * LN1 + the six token-shift lerps are fused for every batch size (the reference does it for B == 1).
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -759,6 +760,8 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   return RWKV_OK;
 }
 
+std::atomic<int64_t> g_graph_captures{0};  // decode graphs captured in this process (all sessions)
+
 GraphEntry* find_graph(rwkv_hip_session* s, int B, void* shift, void* wkv, void* elapsed, void* logits) {
   for (auto& g : s->graphs) {
     if (g.B == B && g.shift == shift && g.wkv == wkv && g.elapsed == elapsed && g.logits == logits) return &g;
@@ -795,6 +798,7 @@ int run_step(rwkv_hip_session* s, int B, half_t* shift, void* wkv, int* elapsed,
     }
     e.graph = graph;
     RWKV_HIP_TRY(hipGraphInstantiate(&e.exec, graph, nullptr, nullptr, 0));
+    g_graph_captures.fetch_add(1, std::memory_order_relaxed);
     s->graphs.push_back(e);
     g = &s->graphs.back();
   }
@@ -1046,6 +1050,12 @@ static int drop_graphs(rwkv_hip_session* s) {
     if (g.graph) (void)hipGraphDestroy(g.graph);
   }
   s->graphs.clear();
+  return RWKV_OK;
+}
+
+int rwkv_hip_graph_capture_count(int64_t* count) {
+  RWKV_REQUIRE(count != nullptr, "count is NULL");
+  *count = g_graph_captures.load(std::memory_order_relaxed);
   return RWKV_OK;
 }
 

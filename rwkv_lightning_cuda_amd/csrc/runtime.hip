@@ -1,6 +1,9 @@
 // Runtime plumbing behind the C ABI: memory, copies, streams, events, error text.
 #include <cstdarg>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
 
 #include "common.h"
 
@@ -150,6 +153,100 @@ int rwkv_hip_free(void* ptr) {
   return RWKV_OK;
 }
 
+// ---- recycled blocks: generation states and logits of a serving loop ----------------------------------------------
+// A block given back through rwkv_hip_free_recycled is kept (per device and byte size, last in first out) and
+// handed to the next rwkv_hip_malloc_recycled of that size, so the buffers of one request come back at the same
+// addresses for the next one of the same shape - which is what a session's captured decode graphs are keyed by.
+namespace {
+struct RecycleBin {
+  std::mutex lock;
+  std::map<std::pair<int, size_t>, std::vector<void*>> blocks;  // (device, bytes) -> free blocks
+  std::vector<std::pair<std::pair<int, size_t>, void*>> order;  // oldest first, for trimming
+  size_t held = 0;
+};
+RecycleBin& recycle_bin() {
+  static RecycleBin* bin = new RecycleBin();  // never destroyed: the runtime may be gone at exit
+  return *bin;
+}
+constexpr size_t kRecycleMaxHeld = static_cast<size_t>(24) << 30;
+
+// frees the oldest blocks until at most `keep` bytes are held (lock taken by the caller)
+void recycle_trim_locked(RecycleBin& bin, size_t keep) {
+  while (bin.held > keep && !bin.order.empty()) {
+    const auto entry = bin.order.front();
+    bin.order.erase(bin.order.begin());
+    auto& list = bin.blocks[entry.first];
+    for (size_t i = 0; i < list.size(); ++i) {
+      if (list[i] == entry.second) {
+        list.erase(list.begin() + static_cast<long>(i));
+        break;
+      }
+    }
+    (void)hipFree(entry.second);
+    bin.held -= entry.first.second;
+  }
+}
+}  // namespace
+
+int rwkv_hip_malloc_recycled(void** ptr, size_t bytes) {
+  RWKV_REQUIRE(ptr != nullptr, "ptr is NULL");
+  *ptr = nullptr;
+  if (bytes == 0) return RWKV_OK;
+  int dev = 0;
+  RWKV_HIP_TRY(hipGetDevice(&dev));
+  RecycleBin& bin = recycle_bin();
+  {
+    std::lock_guard<std::mutex> guard(bin.lock);
+    auto it = bin.blocks.find(std::make_pair(dev, bytes));
+    if (it != bin.blocks.end() && !it->second.empty()) {
+      void* p = it->second.back();
+      it->second.pop_back();
+      for (size_t i = bin.order.size(); i-- > 0;) {
+        if (bin.order[i].second == p) {
+          bin.order.erase(bin.order.begin() + static_cast<long>(i));
+          break;
+        }
+      }
+      bin.held -= bytes;
+      *ptr = p;
+      return RWKV_OK;
+    }
+  }
+  hipError_t err = hipMalloc(ptr, bytes);
+  if (err == hipErrorOutOfMemory) {  // give the held blocks back and try once more
+    (void)hipGetLastError();
+    std::lock_guard<std::mutex> guard(bin.lock);
+    recycle_trim_locked(bin, 0);
+    err = hipMalloc(ptr, bytes);
+  }
+  RWKV_HIP_TRY(err);
+  return RWKV_OK;
+}
+
+int rwkv_hip_free_recycled(void* ptr, size_t bytes) {
+  if (!ptr) return RWKV_OK;
+  if (bytes == 0 || bytes > kRecycleMaxHeld) return rwkv_hip_free(ptr);
+  // like hipFree, returns only when the device no longer uses the block
+  RWKV_HIP_TRY(hipDeviceSynchronize());
+  int dev = 0;
+  RWKV_HIP_TRY(hipGetDevice(&dev));
+  RecycleBin& bin = recycle_bin();
+  std::lock_guard<std::mutex> guard(bin.lock);
+  recycle_trim_locked(bin, kRecycleMaxHeld - bytes);
+  const auto key = std::make_pair(dev, bytes);
+  bin.blocks[key].push_back(ptr);
+  bin.order.push_back(std::make_pair(key, ptr));
+  bin.held += bytes;
+  return RWKV_OK;
+}
+
+int rwkv_hip_recycle_trim(void) {
+  RecycleBin& bin = recycle_bin();
+  std::lock_guard<std::mutex> guard(bin.lock);
+  recycle_trim_locked(bin, 0);
+  return RWKV_OK;
+}
+
 int rwkv_hip_host_alloc(void** ptr_host, size_t bytes) {
   RWKV_REQUIRE(ptr_host != nullptr, "ptr is NULL");
   *ptr_host = nullptr;
@@ -194,6 +291,11 @@ int rwkv_hip_memset(void* ptr, int value, size_t bytes) {
 int rwkv_hip_mem_info(size_t* free_bytes, size_t* total_bytes) {
   RWKV_REQUIRE(free_bytes && total_bytes, "NULL output");
   RWKV_HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));
+  {  // blocks held for recycling are free memory to the caller (an allocation that needs them gets them)
+    RecycleBin& bin = recycle_bin();
+    std::lock_guard<std::mutex> guard(bin.lock);
+    *free_bytes += bin.held;
+  }
   return RWKV_OK;
 }
 

@@ -28,6 +28,7 @@ M_ATT_R, M_ATT_K, M_ATT_V, M_ATT_O, M_FFN_KEY, M_FFN_VALUE, M_HEAD = range(7)
 # every symbol include/rwkv_hip.h declares; checked at load time and by the CPU test-suite
 EXPORTS = [
     "rwkv_hip_last_error", "rwkv_hip_device_count", "rwkv_hip_device_name", "rwkv_hip_malloc", "rwkv_hip_free",
+    "rwkv_hip_malloc_recycled", "rwkv_hip_free_recycled", "rwkv_hip_recycle_trim", "rwkv_hip_graph_capture_count",
     "rwkv_hip_host_alloc", "rwkv_hip_host_free", "rwkv_hip_memcpy_h2d", "rwkv_hip_memcpy_d2h", "rwkv_hip_memcpy_d2d",
     "rwkv_hip_memcpy_h2d_async", "rwkv_hip_memcpy_d2h_async", "rwkv_hip_memcpy_d2d_async", "rwkv_hip_memset",
     "rwkv_hip_mem_info", "rwkv_hip_stream_create", "rwkv_hip_stream_destroy", "rwkv_hip_stream_sync",

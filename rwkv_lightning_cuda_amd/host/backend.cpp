@@ -583,7 +583,7 @@ struct ModelBackend::Impl {
 
   void forward(const std::vector<int64_t>& flat, int B, int T, GenerationState& state, DeviceLogits& out) const {
     const int V = spec.dims.vocab;
-    out.values.resize(static_cast<std::size_t>(B) * V, "alloc backend logits f32");
+    out.values.resize_recycled(static_cast<std::size_t>(B) * V, "alloc backend logits f32");
     rwkv_hip_session* s = acquire();
     int rc = rwkv_hip_session_set_wkv_fp16(s, use_wkv32 ? 0 : 1);
     if (rc == RWKV_OK) {
@@ -620,14 +620,14 @@ GenerationState ModelBackend::create_state(int batch_size) const {
   GenerationState state;
   state.batch_size = batch_size;
   state.wkv32 = impl_->use_wkv32;   // src/rwkv7_fast_v4.cu:1379-1396: one of the two state tensors, by mode
-  state.shift.resize(static_cast<std::size_t>(d.layers) * 2 * batch_size * d.channels, "alloc backend shift state");
+  state.shift.resize_recycled(static_cast<std::size_t>(d.layers) * 2 * batch_size * d.channels, "alloc backend shift state");
   const std::size_t state_elems = static_cast<std::size_t>(d.layers) * batch_size * d.heads * d.head_size * d.head_size;
   if (impl_->use_wkv32) {
-    state.wkv_state32.resize(state_elems, "alloc backend wkv32 state");
+    state.wkv_state32.resize_recycled(state_elems, "alloc backend wkv32 state");
   } else {
-    state.wkv_state.resize(state_elems, "alloc backend wkv state");
+    state.wkv_state.resize_recycled(state_elems, "alloc backend wkv state");
   }
-  state.elapsed.resize(batch_size, "alloc backend elapsed");
+  state.elapsed.resize_recycled(batch_size, "alloc backend elapsed");
   state.shift.zero("zero backend shift");
   if (impl_->use_wkv32) {
     state.wkv_state32.zero("zero backend wkv32");

@@ -348,6 +348,94 @@ HOST_TEST(checkpoint_written_by_torch_save) {
   }
 }
 
+// Damaged pickles out of a real checkpoint: the committed file's own data.pkl cut short at every length, with single
+// bytes replaced, and with a dimension blown up.  Whatever the bytes, the reader answers with a Status - no
+// exception leaves it, nothing is allocated from an unchecked count, no read leaves a buffer (this case is also
+// built with the address and undefined-behaviour sanitizers, tests/test_host_api.py).  The reference's checks of
+// the same kind: src/pth_archive.cpp:511,578.
+HOST_TEST(hostile_pickles) {
+  const std::string pth = host_test::repo_root() + "/tests/golden/rwkv7_tiny.pth";
+  auto ar = PthArchive::open(pth);
+  if (!ar.ok()) FAIL_HERE(ar.status().message());
+  std::vector<Member> members;
+  std::size_t pkl = 0;
+  for (const PthEntry& e : ar.value().entries()) {
+    auto bytes = ar.value().read_stored_entry(e);
+    CHECK(bytes.ok());
+    if (e.name.size() >= 8 && e.name.compare(e.name.size() - 8, 8, "data.pkl") == 0) pkl = members.size();
+    members.push_back(Member{e.name, bytes.value()});
+  }
+  const std::vector<std::uint8_t> good = members[pkl].data;
+  CHECK(good.size() > 64);
+
+  // every tensor of a parsed directory is loaded: any outcome but a crash is fine for a damaged file
+  auto exercise = [&](const std::vector<std::uint8_t>& pickle, bool must_fail) {
+    members[pkl].data = pickle;
+    const std::string path = write_temp("hostile", zip_bytes(members, false));
+    for (bool lazy : {false, true}) {
+      auto opened = PthArchive::open(path, lazy);
+      CHECK(opened.ok());
+      auto recs = parse_pth_tensor_records(opened.value());
+      if (must_fail) CHECK(!recs.ok());
+      if (!recs.ok()) continue;
+      for (const TensorRecord& rec : recs.value()) {
+        auto data = load_bf16_tensor_select(opened.value(), rec, true, true, false);
+        if (data.ok()) CHECK_EQ(data.value().values_bf16.size(), data.value().values_f16.size());
+        (void)compute_tensor_stats(opened.value(), rec);
+      }
+    }
+    std::remove(path.c_str());
+  };
+
+  exercise(good, false);
+  // cut short: every prefix in the first 300 bytes, then every 37th length
+  for (std::size_t n = 0; n < good.size(); n += (n < 300 ? 1 : 37)) {
+    exercise(std::vector<std::uint8_t>(good.begin(), good.begin() + static_cast<long>(n)), true);
+  }
+  // one byte replaced (a fixed pseudo-random walk over positions and values)
+  std::uint32_t rng = 12345u;
+  for (int i = 0; i < 600; ++i) {
+    rng = rng * 1664525u + 1013904223u;
+    std::vector<std::uint8_t> bad = good;
+    bad[(rng >> 8) % bad.size()] = static_cast<std::uint8_t>(rng >> 24);
+    exercise(bad, false);
+  }
+  // a dimension blown up: every BININT (opcode J, four bytes) and BININT2 (opcode M, two bytes) operand in turn set
+  // to its largest value - shapes of 2^31 - 1 and 65535 rows against storages of a few kilobytes
+  int patched = 0;
+  for (std::size_t i = 0; i + 5 <= good.size() && patched < 200; ++i) {
+    if (good[i] != 'J' && good[i] != 'M') continue;
+    std::vector<std::uint8_t> bad = good;
+    if (good[i] == 'J') {
+      bad[i + 1] = 0xff; bad[i + 2] = 0xff; bad[i + 3] = 0xff; bad[i + 4] = 0x7f;
+    } else {
+      bad[i + 1] = 0xff; bad[i + 2] = 0xff;
+    }
+    exercise(bad, false);
+    ++patched;
+  }
+  CHECK(patched > 10);
+  // hand-made records that no pickle would give: the loaders check them against the storage before reserving
+  members[pkl].data = good;
+  const std::string path = write_temp("hostile_rec", zip_bytes(members, false));
+  auto opened = PthArchive::open(path);
+  CHECK(opened.ok());
+  auto recs = parse_pth_tensor_records(opened.value());
+  CHECK(recs.ok() && !recs.value().empty());
+  TensorRecord huge = recs.value().front();
+  huge.shape = {std::int64_t(1) << 40, std::int64_t(1) << 40};   // the product overflows 64 bits
+  huge.stride = {std::int64_t(1) << 40, 1};
+  CHECK(!load_bf16_tensor_select(opened.value(), huge, true, true, true).ok());
+  huge.shape = {std::int64_t(1) << 33};
+  huge.stride = {0};                                              // every element at the same place: 2^33 of them
+  CHECK(!load_bf16_tensor_select(opened.value(), huge, true, false, false).ok());
+  huge.shape = {-4};
+  huge.stride = {1};
+  auto negative = load_bf16_tensor_select(opened.value(), huge, true, false, false);
+  CHECK(!negative.ok() || negative.value().values_bf16.empty());
+  std::remove(path.c_str());
+}
+
 int main(int argc, char** argv) {
   if (argc > 3) {
     g_pth = argv[2];

@@ -89,8 +89,43 @@ def test_checkpoint_reader_cpu():
     committed checkpoint written by torch.save against its manifest - whole-file and on-demand reading."""
     out = _run("pth_cpu_test")
     for case in ("stored_zip_whole_and_on_demand_agree", "zip64_records", "damaged_and_unsupported_archives",
-                 "scalar_conversions_over_every_bf16_pattern", "checkpoint_written_by_torch_save"):
+                 "scalar_conversions_over_every_bf16_pattern", "checkpoint_written_by_torch_save", "hostile_pickles"):
         assert "ok   " + case in out
+
+
+def test_untrusted_input_code_under_sanitizers(tmp_path):
+    """The code that reads bytes it did not write - the checkpoint's ZIP directory and pickle, the vocabulary file, prompt
+    text - built with g++ -fsanitize=address,undefined (host code only: the sources are compiled into the test
+    executables instead of coming from librwkv_host.so) and run over the same cases, among them the damaged pickles
+    of pth_cpu_test (cut short, bytes replaced, dimensions blown up).  A read or write outside a buffer, a signed
+    overflow or a misaligned access ends the run with a report."""
+    from rwkv_lightning_cuda_amd import build
+    _exe("host_cpu_test")
+    cxx = os.environ.get("CXX", "g++")
+    probe = subprocess.run([cxx, "-fsanitize=address,undefined", "-x", "c++", "-", "-o", str(tmp_path / "probe")],
+                           input="int main(){return 0;}", capture_output=True, text=True)
+    if probe.returncode != 0:
+        pytest.skip("this compiler has no sanitizer runtimes: " + probe.stderr[-200:])
+    host = os.path.join(REPO, "rwkv_lightning_cuda_amd", "host")
+    flags = ["-std=c++17", "-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined",
+             "-fno-sanitize-recover=all", "-I" + os.path.join(REPO, "include"), "-I" + os.path.join(REPO, "tests", "cpp")]
+    link = ["-L" + build.PKG_DIR, "-lrwkv_hip", "-ldl", "-pthread", "-Wl,-rpath," + build.PKG_DIR]
+    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0:abort_on_error=0",
+               UBSAN_OPTIONS="print_stacktrace=1")
+    for name, sources in (("pth_cpu_test", ["pth_archive.cpp", "pth_tensor.cpp"]),
+                          ("host_cpu_test", sorted(f for f in os.listdir(host) if f.endswith(".cpp")))):
+        exe = str(tmp_path / (name + "_san"))
+        cmd = [cxx] + flags + [os.path.join(REPO, "tests", "cpp", name + ".cpp")] + [os.path.join(host, f) for f in sources] + \
+              ["-o", exe] + link
+        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-3000:]
+        run = subprocess.run([exe, REPO], capture_output=True, text=True, timeout=600, env=env)
+        report = run.stdout[-3000:] + run.stderr[-3000:]
+        assert run.returncode == 0, "%s under sanitizers exited with %d:\n%s" % (name, run.returncode, report)
+        assert " 0 failed" in run.stdout, report
+        assert "runtime error" not in run.stderr and "AddressSanitizer" not in run.stderr, report
+        if name == "pth_cpu_test":
+            assert "ok   hostile_pickles" in run.stdout
 
 
 @pytest.mark.parametrize("variant", ["ordered_with_metadata", "plain_dict", "many_small_tensors"])
