@@ -4,6 +4,7 @@
 #include <cstring>
 #include <thread>
 
+#include "rwkv_hip.h"
 #include "rwkv_inference_engine.hpp"
 #include "rwkv_prefill_admission.hpp"
 #include "test_common.hpp"
@@ -378,6 +379,55 @@ HOST_TEST(alternating_states_on_one_session_keep_apart) {
   const auto hc = host_test::to_host<float>(lc.values), hc2 = host_test::to_host<float>(lc2.values);
   CHECK(std::memcmp(ha.data(), ha2.data(), ha.size() * sizeof(float)) == 0);
   CHECK(std::memcmp(hc.data(), hc2.data(), hc.size() * sizeof(float)) == 0);
+}
+
+// Recycled blocks: the state and logits of a request come back at the addresses the last request of that shape had,
+// so its decode steps replay the graph captured then (none is captured again); a recycled state is cleared like a
+// new one; the blocks held count as free memory and can be given back.
+HOST_TEST(consecutive_requests_reuse_buffers_and_the_captured_graph) {
+  auto b = tiny();
+  std::vector<float> first;
+  const void* shift_at = nullptr;
+  const void* logits_at = nullptr;
+  int64_t after_first = 0;
+  for (int request = 0; request < 3; ++request) {
+    GenerationState st = b->create_state(3);
+    for (uint16_t h : host_test::to_host<uint16_t>(st.shift)) CHECK_EQ(h, uint16_t(0));
+    for (float f : host_test::to_host<float>(st.wkv_state32)) CHECK_EQ(f, 0.0f);
+    CHECK(host_test::to_host<int>(st.elapsed) == (std::vector<int>{0, 0, 0}));
+    DeviceLogits lg;
+    b->forward_prefill({ramp(6, 1), ramp(6, 2), ramp(6, 3)}, st, lg);
+    int64_t before = 0, after = 0;
+    CHECK_EQ(rwkv_hip_graph_capture_count(&before), RWKV_OK);
+    for (int i = 0; i < 5; ++i) b->forward_decode({int64_t(10 + i), int64_t(20 + i), int64_t(30 + i)}, st, lg);
+    CHECK_EQ(rwkv_hip_graph_capture_count(&after), RWKV_OK);
+    const auto host = host_test::to_host<float>(lg.values);
+    if (request == 0) {
+      first = host;
+      shift_at = st.shift.p;
+      logits_at = lg.values.p;
+      after_first = after;
+    } else {
+      CHECK(st.shift.p == shift_at && lg.values.p == logits_at);      // the same blocks again
+      CHECK_EQ(after, before);                                        // and no new capture
+      CHECK_EQ(after, after_first);
+      CHECK(std::memcmp(host.data(), first.data(), host.size() * sizeof(float)) == 0);
+    }
+  }
+  // the blocks just given back are held: they count as free, and trimming returns them to the device
+  std::size_t free0 = 0, free1 = 0, total = 0;
+  CHECK_EQ(rwkv_hip_mem_info(&free0, &total), RWKV_OK);
+  CHECK_EQ(rwkv_hip_recycle_trim(), RWKV_OK);
+  CHECK_EQ(rwkv_hip_mem_info(&free1, &total), RWKV_OK);
+  CHECK(free1 + (std::size_t(64) << 20) >= free0);   // nothing was double counted (other processes aside)
+  void* p = nullptr;
+  void* q = nullptr;
+  CHECK_EQ(rwkv_hip_malloc_recycled(&p, 4096), RWKV_OK);
+  CHECK_EQ(rwkv_hip_free_recycled(p, 4096), RWKV_OK);
+  CHECK_EQ(rwkv_hip_malloc_recycled(&q, 4096), RWKV_OK);
+  CHECK(p == q);
+  CHECK_EQ(rwkv_hip_free_recycled(q, 4096), RWKV_OK);
+  CHECK_EQ(rwkv_hip_recycle_trim(), RWKV_OK);
 }
 
 int main(int argc, char** argv) { return host_test::run_all(argc, argv, true); }
