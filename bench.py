@@ -37,10 +37,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak, published
 # figure is stale and `traffic` is reported as null until the counters are collected again.
 MEASURED_TRAFFIC = {
     ("7.2B", "w8", 1): {
-        "bytes_per_launch": 49933517,
+        "bytes_per_launch": 49938432,
         "profile": "profiles/linear_gemv_row1_decode_7p2b_w8_bs1_pmc_traffic.md",
         "kernel_source": "rwkv_lightning_cuda_amd/csrc/linear.hip",
-        "kernel_source_sha256": "66443a40d73900f94cbbab57c99dc72619713fe1c6913218840cc3b31ff6328c",
+        "kernel_source_sha256": "3d86f203333b1f8bc32836715fb113630898ddffb9f39c7ba7f4a7c0448d302c",
     },
 }
 
@@ -73,6 +73,8 @@ def parse_args():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="only run a device-to-device copy of BYTES (twice) and exit: the known-size kernel that "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--wkv7-op-only", action="store_true", help="only run the WKV7 op at the long-context configuration "
+                    "(B 16, T 16384, 64 heads; two calls) and exit: the target of rocprofv3 counter runs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--fused-ln", type=int, default=-1, help="tuning hook: 1 / 0 force LayerNorm inside / outside the linear "
@@ -221,6 +223,57 @@ def sampled_decode(hip, sess, dims, state, logits, B, first, steps=64):
     return {"decode_sampled_bs%d_tok_s" % B: steps * B / dt, "decode_sampled_bs%d_ms_per_step" % B: dt * 1e3 / steps}
 
 
+def wkv7_op_long_context(hip, H, reps=3):
+    """The WKV7 op alone at the long-context configuration: fp16 r,w,k,v,a,b [16,16384,64 H], fp32 state, raw-logit
+    decay, one call.  Rows are 4096-token windows of one host-generated sequence (r,k,v ~ N(0,1); decay =
+    exp(-exp(U(-6,-0.5))) given as its raw logit; kk = k/|k| per head, a = -kk, b = kk * sigmoid(U(-3,3)))."""
+    res = {}
+    Bw, Tw, seg = 16, 16384, 4096
+    C = H * 64
+    n = Bw * Tw * C
+    n_win = Bw * (Tw // seg)
+    base_T = seg + 64 * (n_win - 1)
+    g = np.random.default_rng(11)
+    kf = g.standard_normal((base_T, H, 64)).astype(np.float32)
+    kk = kf / np.linalg.norm(kf, axis=-1, keepdims=True)
+    sg = np.exp(g.uniform(-6.0, -0.5, (base_T, C)).astype(np.float32) + np.float32(0.5))
+    host = [g.standard_normal((base_T, C)).astype(np.float16), np.log(sg / (1.0 - sg)).astype(np.float16),
+            kf.reshape(base_T, C).astype(np.float16), g.standard_normal((base_T, C)).astype(np.float16),
+            (-kk).reshape(base_T, C).astype(np.float16),
+            (kk.reshape(base_T, C) / (1.0 + np.exp(-g.uniform(-3.0, 3.0, (base_T, C)).astype(np.float32)))).astype(np.float16)]
+    del kf, kk, sg
+    bufs = []
+    for h in host:
+        src = hip.DeviceArray.from_numpy(h)
+        d = hip.DeviceArray((Bw, Tw, C), np.float16)
+        for w_i in range(n_win):
+            d.view(w_i * seg * C, (seg, C)).copy_from(src.view(64 * w_i * C, (seg, C)))
+        src.free()
+        bufs.append(d)
+    del host
+    bufs.append(hip.DeviceArray((Bw, Tw, C), np.float16))
+    wstate = hip.DeviceArray.zeros((Bw, H, 64, 64), np.float32)
+    r, w, k, v, a, b, y = bufs
+    hip.wkv7(Bw, Tw, C, H, hip.W_RAW_LOGIT, hip.IO_F16, wstate, r, w, k, v, a, b, y)
+    hip.device_sync()
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record()
+    for _ in range(reps):
+        hip.wkv7(Bw, Tw, C, H, hip.W_RAW_LOGIT, hip.IO_F16, wstate, r, w, k, v, a, b, y)
+    e1.record()
+    hip.device_sync()
+    ms = e0.elapsed_ms(e1) / reps
+    res["wkv7_op"] = {"workload": "B=%d T=%d H=%d N=64, fp16 io, fp32 state, one call (average of %d)" % (Bw, Tw, H, reps),
+                      "tok_s": Bw * Tw / (ms * 1e-3), "ms": ms,
+                      "fp32_tflops": Bw * Tw * H * 10.0 * 64 * 64 / (ms * 1e-3) / 1e12,
+                      "io_gb_s": n * 7 * 2 / (ms * 1e-3) / 1e9, "us_per_token_step": ms * 1e3 / Tw,
+                      "outputs_finite": bool(np.isfinite(y.view(0, (Tw, C)).numpy().astype(np.float32)).all())}
+    for d in bufs:
+        d.free()
+
+    return res["wkv7_op"]
+
+
 def secondary_measurements(hip, model, dims, rng):
     """Batch-1, -2, -4, -8, -16 and -64 decode of the same model (128-token prefill per row, 64 timed steps) and the WKV7
     op alone."""
@@ -269,51 +322,8 @@ def secondary_measurements(hip, model, dims, rng):
         sess.close()
         del state, logits
 
-    # WKV7 op alone at the long-context configuration: fp16 r,w,k,v,a,b [16,16384,4096], fp32 state, raw-logit
-    # decay, one call.  Rows are 4096-token windows of one host-generated sequence (r,k,v ~ N(0,1); decay =
-    # exp(-exp(U(-6,-0.5))) given as its raw logit; kk = k/|k| per head, a = -kk, b = kk * sigmoid(U(-3,3))).
-    Bw, Tw, H, seg = 16, 16384, dims.H, 4096
-    C = H * 64
-    n = Bw * Tw * C
-    n_win = Bw * (Tw // seg)
-    base_T = seg + 64 * (n_win - 1)
-    g = np.random.default_rng(11)
-    kf = g.standard_normal((base_T, H, 64)).astype(np.float32)
-    kk = kf / np.linalg.norm(kf, axis=-1, keepdims=True)
-    sg = np.exp(g.uniform(-6.0, -0.5, (base_T, C)).astype(np.float32) + np.float32(0.5))
-    host = [g.standard_normal((base_T, C)).astype(np.float16), np.log(sg / (1.0 - sg)).astype(np.float16),
-            kf.reshape(base_T, C).astype(np.float16), g.standard_normal((base_T, C)).astype(np.float16),
-            (-kk).reshape(base_T, C).astype(np.float16),
-            (kk.reshape(base_T, C) / (1.0 + np.exp(-g.uniform(-3.0, 3.0, (base_T, C)).astype(np.float32)))).astype(np.float16)]
-    del kf, kk, sg
-    bufs = []
-    for h in host:
-        src = hip.DeviceArray.from_numpy(h)
-        d = hip.DeviceArray((Bw, Tw, C), np.float16)
-        for w_i in range(n_win):
-            d.view(w_i * seg * C, (seg, C)).copy_from(src.view(64 * w_i * C, (seg, C)))
-        src.free()
-        bufs.append(d)
-    del host
-    bufs.append(hip.DeviceArray((Bw, Tw, C), np.float16))
-    wstate = hip.DeviceArray.zeros((Bw, H, 64, 64), np.float32)
-    r, w, k, v, a, b, y = bufs
-    hip.wkv7(Bw, Tw, C, H, hip.W_RAW_LOGIT, hip.IO_F16, wstate, r, w, k, v, a, b, y)
-    hip.device_sync()
+    res["wkv7_op"] = wkv7_op_long_context(hip, dims.H)
     e0, e1 = hip.Event(), hip.Event()
-    e0.record()
-    for _ in range(3):
-        hip.wkv7(Bw, Tw, C, H, hip.W_RAW_LOGIT, hip.IO_F16, wstate, r, w, k, v, a, b, y)
-    e1.record()
-    hip.device_sync()
-    ms = e0.elapsed_ms(e1) / 3
-    res["wkv7_op"] = {"workload": "B=%d T=%d H=%d N=64, fp16 io, fp32 state, one call (average of 3)" % (Bw, Tw, H),
-                      "tok_s": Bw * Tw / (ms * 1e-3), "ms": ms,
-                      "fp32_tflops": Bw * Tw * H * 10.0 * 64 * 64 / (ms * 1e-3) / 1e12,
-                      "io_gb_s": n * 7 * 2 / (ms * 1e-3) / 1e9, "us_per_token_step": ms * 1e3 / Tw,
-                      "outputs_finite": bool(np.isfinite(y.view(0, (Tw, C)).numpy().astype(np.float32)).all())}
-    for d in bufs:
-        d.free()
 
     # the reference's own small operator case: B = 1, T = 64, H = 12, fp32 io (average over 20 calls)
     B0, T0, H0 = 1, 64, 12
@@ -448,6 +458,9 @@ def main():
             dst.copy_from(src)
         hip.device_sync()
         print(json.dumps({"copy_calibration_bytes": args.copy_calibration}))
+        return
+    if args.wkv7_op_only:
+        print(json.dumps({"wkv7_op": wkv7_op_long_context(hip, 64, reps=1)}))
         return
     dims = PRESETS[args.preset]
     fmt = {"f16": hip.FMT_F16, "w8": hip.FMT_W8, "w4": hip.FMT_W4}[args.fmt]
