@@ -36,10 +36,12 @@ HIP_FLAGS = [
 # the compiler's resource report is checked at build time, so that a change that costs a few registers fails the
 # build instead of silently halving the occupancy.  The one-row GEMV with the LayerNorm prologue needs two
 # 1024-thread blocks per CU (all blocks of a launch resident at once), i.e. at most 64 registers.
-# (template arguments: threads, prologue, format of the quantised problems 0 fp16 / 1 int8 / 2 int4, rows of x; two
-# rows of int4 codes need more registers and run one block per CU)
-REQUIRED_OCCUPANCY = {"linear_gemv_row1_kernelILi1024ELb1ELi0ELi1E": 8, "linear_gemv_row1_kernelILi1024ELb1ELi1ELi1E": 8,
-                      "linear_gemv_row1_kernelILi1024ELb1ELi2ELi1E": 8, "linear_gemv_row1_kernelILi1024ELb1ELi1ELi2E": 8}
+# (template arguments: threads, prologue, format of the quantised problems 0 fp16 / 1 int8 / 2 int4, rows of x, row
+# multiplier; two rows of int4 codes need more registers and run one block per CU; with the row multiplier 2 - int4
+# launches with more blocks than CUs - a launch has one 1024-thread block per CU and needs 4 wavefronts per SIMD)
+REQUIRED_OCCUPANCY = {"linear_gemv_row1_kernelILi1024ELb1ELi0ELi1ELi1E": 8, "linear_gemv_row1_kernelILi1024ELb1ELi1ELi1ELi1E": 8,
+                      "linear_gemv_row1_kernelILi1024ELb1ELi2ELi1ELi1E": 8, "linear_gemv_row1_kernelILi1024ELb1ELi1ELi2ELi1E": 8,
+                      "linear_gemv_row1_kernelILi1024ELb1ELi2ELi1ELi2E": 4, "linear_gemv_row1_kernelILi1024ELb1ELi2ELi2ELi2E": 4}
 
 
 def _check_occupancy(src, stderr_text):

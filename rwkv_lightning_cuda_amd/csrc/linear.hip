@@ -208,6 +208,51 @@ struct WeightVec<RWKV_FMT_W4> {
   }
 };
 
+// ---- int4 codes in the whole-rows-in-flight kernel ------------------------------------------------------------------
+// A block whose weights are int4 codes keeps x in LDS in the order the nibble pairs want it - every 8 values
+// (x0..x7) as (x0,x4)(x1,x5)(x2,x6)(x3,x7) - and, beside it, the fp32 sum of every 32 values (one lane's slice, inside
+// one 128-group).  A nibble pair (n_j, n_{j+4}) of a dword is shifted into the top four mantissa bits of two fp16
+// numbers with the exponent of 16: 0x4c00 | n << 6 is 16 + n, exactly.  Then
+//   sum_k (q_k - zp) x_k = sum_k (16 + q_k) x_k - (16 + zp) sum_k x_k:
+// the zero point and the offset leave in one multiply-add per slice instead of one packed subtract per pair, and
+// x needs no pairing per wavefront (per 16-byte vector of 32 codes: 28 shift / mask instructions and 16 v_dot2
+// where the pairing, the subtracts and the masks were 72).  Products (16 + q) x are exact in fp32; the offset is
+// small against the terms (at most 31 |x| each), so nothing is lost to cancellation.
+__device__ __forceinline__ uint4_t w4_pair_order(uint4_t v) {
+  uint4_t o;
+  o[0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+  o[1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+  o[2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+  o[3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+  return o;
+}
+
+// fp32 sum of the 32 values that four neighbouring lanes hold eight each (in every one of the four lanes)
+__device__ __forceinline__ float w4_slice_sum(uint4_t v) {
+  const half2_t a = as_half2(v[0]), b = as_half2(v[1]), c = as_half2(v[2]), d = as_half2(v[3]);
+  float s = ((h2f(a[0]) + h2f(a[1])) + (h2f(b[0]) + h2f(b[1]))) + ((h2f(c[0]) + h2f(c[1])) + (h2f(d[0]) + h2f(d[1])));
+  s = dpp_add<0xB1>(s);  // quad_perm [1,0,3,2]
+  s = dpp_add<0x4E>(s);  // quad_perm [2,3,0,1]
+  return s;
+}
+
+// sum_k (16 + code_k) x_k over a lane's 32 codes; xp[4i + j] holds (x_{8i+j}, x_{8i+j+4})
+__device__ __forceinline__ float w4_dot_offset16(const uint4_t& wv, const half2_t* xp, float acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t d = wv[i];
+    const uint32_t p0 = ((d << 6) & 0x03c003c0u) | 0x4c004c00u;
+    const uint32_t p1 = ((d << 2) & 0x03c003c0u) | 0x4c004c00u;
+    const uint32_t p2 = ((d >> 2) & 0x03c003c0u) | 0x4c004c00u;
+    const uint32_t p3 = ((d >> 6) & 0x03c003c0u) | 0x4c004c00u;
+    acc = dot2(as_half2(p0), xp[4 * i + 0], acc);
+    acc = dot2(as_half2(p1), xp[4 * i + 1], acc);
+    acc = dot2(as_half2(p2), xp[4 * i + 2], acc);
+    acc = dot2(as_half2(p3), xp[4 * i + 3], acc);
+  }
+  return acc;
+}
+
 template <int FMT>
 struct FmtTraits {
   static constexpr int kElems = WeightVec<FMT>::kElems;
@@ -490,9 +535,10 @@ __device__ __forceinline__ float front_waves_sum(float v, int wave, float* scrat
   return t;
 }
 
-template <int NT, int V8, int NTL, int M>
+// (W4: xs in nibble-pair order, the slice sums to xsum - see w4_pair_order)
+template <int NT, int V8, int NTL, int M, bool W4>
 __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8, M>& q, const LnPrologue& ln, int K, int m, half_t* xs,
-                                                float* stash, float* red, bool store, int wave) {
+                                                float* xsum, float* stash, float* red, bool store, int wave) {
   const int64_t row = static_cast<int64_t>(m) * K;
   constexpr int NWL = NTL / 64;  // wavefronts that compute
   half_t* hstash = reinterpret_cast<half_t*>(stash + NT * 4);
@@ -567,7 +613,15 @@ __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8, M>& q, const 
         if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + row + c) = xo;
       }
     }
-    *reinterpret_cast<half8_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
+    // zeros beyond K: the lanes past the end of a row multiply by them
+    if constexpr (W4) {
+      const uint4_t raw = __builtin_bit_cast(uint4_t, ov);
+      const float s32 = w4_slice_sum(raw);
+      *reinterpret_cast<uint4_t*>(xs + c) = w4_pair_order(raw);
+      if ((threadIdx.x & 3) == 0) xsum[c >> 5] = s32;
+    } else {
+      *reinterpret_cast<half8_t*>(xs + c) = ov;
+    }
   }
 }
 
@@ -598,21 +652,52 @@ __device__ __forceinline__ LnRowOne<V8> ln_one_request8(const LnPrologue& ln, co
   return q;
 }
 
-// sum over the first NWL wavefronts of the block (the callers); the other wavefronts pass the barrier too
-template <int NWL>
-__device__ __forceinline__ float front_waves_sum_one(float v, int wave, float* scratch) {
+#ifndef RWKV_LN_FLAGS
+#define RWKV_LN_FLAGS 1
+#endif
+
+// Counters in LDS by which the wavefronts of a one-row prologue block meet without s_barrier: a barrier counts every
+// wavefront of the block, and the ones that are not computing the prologue reach it only when the memory pipeline
+// has taken all their weight requests - microseconds into a large launch.  [0], [1]: the computing wavefronts that
+// have delivered their partial row sum / sum of squares; [2]: those whose part of x is in LDS.  Zeroed by the
+// block's first threads before the one barrier every wavefront passes on entry.
+struct LnFlags {
+  unsigned count[3];
+};
+
+// waits (bounded: no wavefront may spin for ever whatever happens to the others) until `n` wavefronts have arrived
+__device__ __forceinline__ void ln_flag_wait(unsigned* count, unsigned n) {
+  int spins = 0;
+  while (__hip_atomic_load(count, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < n && ++spins < (1 << 22))
+    __builtin_amdgcn_s_sleep(1);
+}
+
+__device__ __forceinline__ void ln_flag_arrive(unsigned* count) {
+  if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// sum over the first NWL wavefronts of the block (the callers).  With FLAGS they meet at the counter; without, at a
+// barrier that the other wavefronts pass too.
+template <int NWL, bool FLAGS>
+__device__ __forceinline__ float front_waves_sum_one(float v, int wave, float* scratch, unsigned* count) {
   v = wave_sum_uniform(v);
   if ((threadIdx.x & 63) == 0) scratch[wave] = v;
-  __syncthreads();
+  if constexpr (FLAGS) {
+    ln_flag_arrive(count);
+    ln_flag_wait(count, NWL);
+  } else {
+    __syncthreads();
+  }
   float t = 0.0f;
 #pragma unroll
   for (int i = 0; i < NWL; ++i) t += scratch[i];
   return t;
 }
 
-template <int NT, int V8, int NTL>
+template <int NT, int V8, int NTL, bool W4, bool FLAGS>
 __device__ __forceinline__ void ln_one_finish8(const LnRowOne<V8>& q, const LnPrologue& ln, int K, half_t* xs,
-                                                float* stash, float* red, bool store, int wave) {
+                                                float* xsum, float* stash, float* red, LnFlags* flags, bool store,
+                                                int wave) {
   constexpr int NWL = NTL / 64;  // wavefronts that compute
   half_t* hstash = reinterpret_cast<half_t*>(stash + NT * 4);
   float sum = 0.0f;
@@ -636,7 +721,7 @@ __device__ __forceinline__ void ln_one_finish8(const LnRowOne<V8>& q, const LnPr
     *reinterpret_cast<half8_t*>(hstash + c + NT * 12) = q.mv[g];
   }
   __builtin_amdgcn_sched_barrier(0);
-  sum = front_waves_sum_one<NWL>(sum, wave, red);
+  sum = front_waves_sum_one<NWL, FLAGS>(sum, wave, red, &flags->count[0]);
   const float mean = sum / static_cast<float>(K);
   float sv = 0.0f;
 #pragma unroll
@@ -657,7 +742,7 @@ __device__ __forceinline__ void ln_one_finish8(const LnRowOne<V8>& q, const LnPr
       }
     }
   }
-  sv = front_waves_sum_one<NWL>(sv, wave, red + NT / 64);
+  sv = front_waves_sum_one<NWL, FLAGS>(sv, wave, red + NT / 64, &flags->count[1]);
   const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
 #pragma unroll
   for (int g = 0; g < V8; ++g) {
@@ -686,7 +771,15 @@ __device__ __forceinline__ void ln_one_finish8(const LnRowOne<V8>& q, const LnPr
         if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + c) = xo;
       }
     }
-    *reinterpret_cast<half8_t*>(xs + c) = ov;  // zeros beyond K: the lanes past the end of a row multiply by them
+    // zeros beyond K: the lanes past the end of a row multiply by them
+    if constexpr (W4) {
+      const uint4_t raw = __builtin_bit_cast(uint4_t, ov);
+      const float s32 = w4_slice_sum(raw);
+      *reinterpret_cast<uint4_t*>(xs + c) = w4_pair_order(raw);
+      if ((threadIdx.x & 3) == 0) xsum[c >> 5] = s32;
+    } else {
+      *reinterpret_cast<half8_t*>(xs + c) = ov;
+    }
   }
 }
 
@@ -696,13 +789,13 @@ __device__ __forceinline__ void ln_one_finish8(const LnRowOne<V8>& q, const LnPr
 // launch, while a prologue before them leaves HBM idle for its 1.5 us.  So the wavefronts share the work: some
 // compute the prologue and request their weights afterwards, the others request theirs at once and meet the first
 // at the barrier (7.2B shape, int8: 1.79 -> 1.72 ms per step against the prologue in every wavefront first).
-template <int FMT, int NT, bool LN, int M>
+template <int FMT, int NT, bool LN, int M, int RX>
 __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const LinearProblem& prob, int blk, half_t* xs,
-                                               float* red) {
+                                               float* red, LnFlags* flags) {
   using T = FmtTraits<FMT>;
   constexpr int KCAP = LN ? NT * 4 : NT * 8;  // values of x the block stages per row: one slice per thread
   using Cfg = Row1Cfg<FMT, KCAP>;
-  constexpr int R = Cfg::kRows;
+  constexpr int R = Cfg::kRows * RX;
   constexpr int S = Cfg::kSteps;
   constexpr int NW = NT / 64;
   const int K = args.K;
@@ -719,6 +812,10 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   // weights afterwards; the second half requests its weights at once, so that HBM streams while the prologue runs.
   // (half of them for int8 and fp16 weights; a quarter for int4, whose wavefronts have three requests per vector
   // to get out: 7.2B shape, ms per step with a half / a quarter: int8 1.72 / 1.75, int4 1.70 / 1.64)
+  constexpr bool kW4 = FMT == RWKV_FMT_W4;
+  // LDS: M rows of x, then (used by int4 blocks) the sums of every 32 values of each row, then the prologue's stash
+  float* xsum = reinterpret_cast<float*>(xs + M * KCAP);
+  float* stash = xsum + M * (KCAP / 32);
   constexpr int NTL = NT / (FMT == RWKV_FMT_W4 ? 4 : 2);  // threads that compute the prologue
   constexpr int V8 = NT * 4 / (NTL * 8);  // groups of eight values per computing thread
   const bool ln_wave = LN && wave < NTL / 64;
@@ -752,14 +849,10 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
         xq[m] = *reinterpret_cast<const uint4_t*>(prob.x + static_cast<int64_t>(m) * K + threadIdx.x * 8);
     }
   }
-  // the int8 rows' output scales too: read at the end they would cost every wavefront one more trip to memory
   half_t row_scale[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    row_scale[r] = static_cast<half_t>(1.0f);
-    if constexpr (FMT == RWKV_FMT_W8) row_scale[r] = prob.scale[active ? row0 + r : r];
-  }
-  // the compiler must not move these reads behind the weight reads below (loads complete in issue order)
+  for (int r = 0; r < R; ++r) row_scale[r] = static_cast<half_t>(1.0f);
+  // the compiler must not move the reads of x behind the weight reads below (loads complete in issue order)
   __builtin_amdgcn_sched_barrier(0);
 
   // No load sits under a branch: a lane past the end of the row re-reads the row's last vector (and multiplies it
@@ -771,12 +864,100 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
     const int k0 = st * T::kStep + lane * T::kElems;
     const int kc = k0 < K ? k0 : K - T::kElems;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
+    for (int r = 0; r < R; ++r)
       w[st][r] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wbase + r * row_bytes + T::byte_off(kc)));
-      if constexpr (FMT == RWKV_FMT_W4) {
-        const int64_t gi = static_cast<int64_t>(active ? row0 + r : r) * (K >> 7) + (kc >> 7);
-        sc[st][r] = prob.scale[gi];
-        zp[st][r] = prob.zp[gi];
+  };
+  // int4: every group's scale and zero point, requested before any codes.  Loads return in issue order: were these
+  // issued among the codes (where the compiler would put them), the first product would wait for the last codes,
+  // and the whole dot phase - a few microseconds of VALU work on a launch of this size - would start only when the
+  // stream from HBM has ended, instead of running under it.
+  auto request_all = [&]() {
+    // the int8 rows' output scales too, ahead of the codes: read at the end they would cost every wavefront one
+    // more trip to memory (and before the prologue, its wavefronts would sit out that trip before their own reads)
+    if constexpr (FMT == RWKV_FMT_W8) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) row_scale[r] = prob.scale[active ? row0 + r : r];
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (FMT == RWKV_FMT_W4) {
+#pragma unroll
+      for (int st = 0; st < S; ++st) {
+        const int k0 = st * T::kStep + lane * T::kElems;
+        const int kc = k0 < K ? k0 : K - T::kElems;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int64_t gi = static_cast<int64_t>(active ? row0 + r : r) * (K >> 7) + (kc >> 7);
+          sc[st][r] = prob.scale[gi];
+          zp[st][r] = prob.zp[gi];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int st = 0; st < S; ++st) request(st);
+  };
+  // The products, once x is in LDS.  per (row of W, row of x): steps in order, the lane's pairs in order - the order
+  // of one-row launches, same bits
+  auto dots = [&]() {
+    float acc[R][M];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
+#pragma unroll
+    for (int st = 0; st < S; ++st) {
+      const int k0 = st * T::kStep + lane * T::kElems;
+      if (st * T::kStep < K && k0 + T::kElems <= KCAP) {  // (the second test only where a step is wider than KCAP)
+        constexpr int XV = T::kElems / 2;
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          half2_t xv[XV];
+#pragma unroll
+          for (int q = 0; q < XV / 4; ++q) {
+            const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KCAP + k0 + q * 8);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
+          }
+          if constexpr (kW4) {
+            // xv is in nibble-pair order already; the slice's sum takes out the offset of 16 and the zero point
+            const float xs32 = xsum[m * (KCAP / 32) + (k0 >> 5)];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const float part = w4_dot_offset16(w[st][r], xv, 0.0f);
+              const float off = -(16.0f + static_cast<float>(zp[st][r]));
+              acc[r][m] = fmaf(fmaf(off, xs32, part), h2f(sc[st][r]), acc[r][m]);
+              // one vector's arithmetic stays together, in the order the vectors were requested
+              __builtin_amdgcn_sched_barrier(0);
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(w[st][r], xv, acc[r][m]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < M; ++m) acc[r][m] = wave_sum(acc[r][m]);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = row0 + r;
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          float v = round_h(acc[r][m] * h2f(row_scale[r]));
+          if (args.epilogue == RWKV_EPI_RELU_SQUARE) {
+            v = fmaxf(v, 0.0f);
+            v = round_h(v * v);
+          }
+          const int64_t o = static_cast<int64_t>(m) * N + n;
+          if (args.out_f32) {
+            static_cast<float*>(prob.y)[o] = v;
+          } else {
+            static_cast<half_t*>(prob.y)[o] = f2h(v);
+          }
+        }
       }
     }
   };
@@ -784,106 +965,80 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   if constexpr (LN) {
     // two code paths, so that the prologue's operands and the weight vectors never hold registers together; the
     // second path passes the two barriers of the first one's block sums, once per row
+    constexpr bool kFlags = RWKV_LN_FLAGS != 0 && M == 1;
+    constexpr unsigned NWL = NTL / 64;
     if (ln_wave) {
       if constexpr (M == 1) {
         const LnRowOne<V8> lnq = ln_one_request8<V8, NTL>(args.ln, prob.mu, K);
         __builtin_amdgcn_sched_barrier(0);
-        ln_one_finish8<NT, V8, NTL>(lnq, args.ln, K, xs, reinterpret_cast<float*>(xs + NT * 4), red, blockIdx.x == 0, wave);
+        if constexpr (kFlags) {
+          // the prologue's operands are in the memory pipeline ahead of any weights of this block
+          if (threadIdx.x < 3) flags->count[threadIdx.x] = 0u;
+          __syncthreads();
+          // (nothing that waits for the operands may move above the barrier: the other wavefronts wait there)
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        ln_one_finish8<NT, V8, NTL, kW4, kFlags>(lnq, args.ln, K, xs, xsum, stash, red, flags, blockIdx.x == 0, wave);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (kFlags) ln_flag_arrive(&flags->count[2]);
       } else {
       const LnRow1xV<V8, M> lnq = ln_row1_request8<V8, NTL, M>(args.ln, prob.mu, K);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        ln_row1_finish8<NT, V8, NTL, M>(lnq, args.ln, K, m, xs + m * KCAP, reinterpret_cast<float*>(xs + M * KCAP), red,
-                                        blockIdx.x == 0, wave);
+        ln_row1_finish8<NT, V8, NTL, M, kW4>(lnq, args.ln, K, m, xs + m * KCAP, xsum + m * (KCAP / 32), stash, red,
+                                             blockIdx.x == 0, wave);
         __builtin_amdgcn_sched_barrier(0);
       }
       }
-#pragma unroll
-      for (int st = 0; st < S; ++st) request(st);
-    } else {
-#pragma unroll
-      for (int st = 0; st < S; ++st) request(st);
+      request_all();
+      // Each path has its own copy of the products.  Where the two paths met before them, the compiler's wait for
+      // the first vector became a wait for one of the last (it merges the two paths' lists of loads in flight
+      // conservatively), and the arithmetic - microseconds of it per launch - ran after the stream, not under it.
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll 1
-      for (int m = 0; m < M; ++m) {
-        __syncthreads();
+      if constexpr (kFlags) {
+        ln_flag_wait(&flags->count[2], NWL);
+      } else {
         __syncthreads();
       }
+      if (active) dots();
+      return;
+    } else {
+      if constexpr (kFlags) __syncthreads();
+      request_all();
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kFlags) {
+        ln_flag_wait(&flags->count[2], NWL);
+      } else {
+#pragma unroll 1
+        for (int m = 0; m < M; ++m) {
+          __syncthreads();
+          __syncthreads();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+      }
+      if (active) dots();
+      return;
     }
   } else {
 #pragma unroll
-    for (int m = 0; m < M; ++m) *reinterpret_cast<uint4_t*>(xs + m * KCAP + threadIdx.x * 8) = xq[m];
+    for (int m = 0; m < M; ++m) {
+      if constexpr (kW4) {
+        const float s32 = w4_slice_sum(xq[m]);
+        *reinterpret_cast<uint4_t*>(xs + m * KCAP + threadIdx.x * 8) = w4_pair_order(xq[m]);
+        if ((threadIdx.x & 3) == 0) xsum[m * (KCAP / 32) + (threadIdx.x >> 2)] = s32;
+      } else {
+        *reinterpret_cast<uint4_t*>(xs + m * KCAP + threadIdx.x * 8) = xq[m];
+      }
+    }
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int st = 0; st < S; ++st) request(st);
+    request_all();
   }
   __builtin_amdgcn_sched_barrier(0);
   __syncthreads();
   if (!active) return;
-
-  // per (row of W, row of x): steps in order, the lane's pairs in order - the order of one-row launches, same bits
-  float acc[R][M];
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
-#pragma unroll
-  for (int st = 0; st < S; ++st) {
-    const int k0 = st * T::kStep + lane * T::kElems;
-    if (st * T::kStep < K && k0 + T::kElems <= KCAP) {  // (the second test only where a step is wider than KCAP)
-      constexpr int XV = T::kElems / 2;
-#pragma unroll
-      for (int m = 0; m < M; ++m) {
-        half2_t xv[XV];
-#pragma unroll
-        for (int q = 0; q < XV / 4; ++q) {
-          const uint4_t t = *reinterpret_cast<const uint4_t*>(xs + m * KCAP + k0 + q * 8);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) xv[q * 4 + e] = as_half2(t[e]);
-        }
-        if constexpr (FMT == RWKV_FMT_W4) {
-          half2_t xp[XV];
-          WeightVec<FMT>::pair_x(xv, xp);
-#pragma unroll
-          for (int r = 0; r < R; ++r) {
-            const half_t zf = static_cast<half_t>(1024.0f + static_cast<float>(zp[st][r]));
-            const half2_t zb = {zf, zf};
-            const float part = WeightVec<FMT>::dot(w[st][r], xp, zb, 0.0f);
-            acc[r][m] = fmaf(part, h2f(sc[st][r]), acc[r][m]);
-          }
-        } else {
-#pragma unroll
-          for (int r = 0; r < R; ++r) acc[r][m] = WeightVec<FMT>::dot(w[st][r], xv, acc[r][m]);
-        }
-      }
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int m = 0; m < M; ++m) acc[r][m] = wave_sum(acc[r][m]);
-  if (lane == 0) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int n = row0 + r;
-#pragma unroll
-      for (int m = 0; m < M; ++m) {
-        float v = round_h(acc[r][m] * h2f(row_scale[r]));
-        if (args.epilogue == RWKV_EPI_RELU_SQUARE) {
-          v = fmaxf(v, 0.0f);
-          v = round_h(v * v);
-        }
-        const int64_t o = static_cast<int64_t>(m) * N + n;
-        if (args.out_f32) {
-          static_cast<float*>(prob.y)[o] = v;
-        } else {
-          static_cast<half_t*>(prob.y)[o] = f2h(v);
-        }
-      }
-    }
-  }
+  dots();
 }
 
 // grid = blocks over all problems; a block of NT threads covers NT/64 * (1 or 2) rows of W for all M rows of x; dynamic
@@ -892,11 +1047,12 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
 // With the prologue and 1024 threads two blocks must share a CU (every block of the launch resident at once): 8
 // wavefronts per SIMD, i.e. at most 64 registers - asked for here, and checked from the compiler's resource report at
 // build time.  (Two rows of int4 codes do not fit that budget and run one block per CU.)
-template <int NT, bool LN, int DF, int M>
-__global__ __launch_bounds__(NT, (LN && NT == 1024 && (M == 1 || DF != RWKV_FMT_W4)) ? 8 : 1)
+template <int NT, bool LN, int DF, int M, int RX>
+__global__ __launch_bounds__(NT, (LN && NT == 1024 && (M == 1 || DF != RWKV_FMT_W4)) ? 8 / RX : (LN && NT == 1024 ? 4 : 1))
 void linear_gemv_row1_kernel(LinearArgs args) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   __shared__ float red[2 * (NT / 64)];
+  __shared__ LnFlags flags;
   half_t* xs = reinterpret_cast<half_t*>(lds_raw);
   if (blockIdx.x == 0 && args.copy.n > 0) {
     for (int i = threadIdx.x * 8; i < args.copy.n; i += NT * 8)
@@ -913,9 +1069,9 @@ void linear_gemv_row1_kernel(LinearArgs args) {
   const LinearProblem prob = args.p[pi];
   const int blk = blockIdx.x - first;
   if (DF != RWKV_FMT_F16 && prob.fmt == DF) {  // uniform per block
-    gemv_row1_block<DF, NT, LN, M>(args, prob, blk, xs, red);
+    gemv_row1_block<DF, NT, LN, M, RX>(args, prob, blk, xs, red, &flags);
   } else {
-    gemv_row1_block<RWKV_FMT_F16, NT, LN, M>(args, prob, blk, xs, red);
+    gemv_row1_block<RWKV_FMT_F16, NT, LN, M, RX>(args, prob, blk, xs, red, &flags);
   }
 }
 
@@ -939,26 +1095,33 @@ static int row1_format(const LinearArgs& args) {
 constexpr int kRow1MaxRows = 4;
 constexpr int kRow1MaxRowsLn = 2;
 
-template <int NT, bool LN, int DF, int M>
+template <int NT, bool LN, int DF, int M, int RX = 1>
 static int launch_row1(hipStream_t st, LinearArgs& args) {
   int total = 0;
   for (int i = 0; i < args.n_problems; ++i) {
-    const int rows_per_block = (NT / 64) * (args.p[i].fmt == RWKV_FMT_F16 ? 1 : 2);
+    const int rows_per_block = (NT / 64) * (args.p[i].fmt == RWKV_FMT_F16 ? 1 : 2) * RX;
     total += ceil_div(args.p[i].N, rows_per_block);
     args.block_end[i] = total;
   }
+  // int4 codes, rows of 4096: a launch with more blocks than CUs doubles the rows per wavefront, so that one block
+  // per CU covers it (one prologue per CU instead of two, whose second one has its operands queued behind the first
+  // block's weights; the short int4 stream cannot hide that: 7.2B shape, 1.56 -> 1.48 ms per step).  The int8
+  // stream is long enough to hide it and runs a little better with two blocks per CU (1.70 against 1.73 ms).
+  if constexpr (RX == 1 && LN && NT == 1024 && DF == RWKV_FMT_W4) {
+    if (total > device_cu_count()) return launch_row1<NT, LN, DF, M, 2>(st, args);
+  }
   args.KT = LN ? NT * 4 : NT * 8;
-  // x rows; with the prologue also its stash: the fp32 row sum and four fp16 vectors
-  const size_t lds = static_cast<size_t>(args.KT) * (2 * M + (LN ? 4 + 4 * 2 : 0));
+  // x rows, the slice sums of int4 blocks (4 bytes per 32 values and row), with the prologue also its stash
+  const size_t lds = static_cast<size_t>(args.KT) * (2 * M + (LN ? 4 + 4 * 2 : 0)) + static_cast<size_t>(M) * (args.KT / 32) * 4;
   if (lds > 48 * 1024) {  // beyond the default limit of dynamic LDS: raised once per instantiation
     static bool raised = false;
     if (!raised) {
-      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_gemv_row1_kernel<NT, LN, DF, M>),
+      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_gemv_row1_kernel<NT, LN, DF, M, RX>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
       raised = true;
     }
   }
-  hipLaunchKernelGGL((linear_gemv_row1_kernel<NT, LN, DF, M>), dim3(total), dim3(NT), lds, st, args);
+  hipLaunchKernelGGL((linear_gemv_row1_kernel<NT, LN, DF, M, RX>), dim3(total), dim3(NT), lds, st, args);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
