@@ -523,12 +523,43 @@ __device__ __forceinline__ LnRow1xV<V8, M> ln_row1_request8(const LnPrologue& ln
   return q;
 }
 
-// sum over the first NWL wavefronts of the block (the callers); the other wavefronts pass the barrier too
-template <int NWL>
-__device__ __forceinline__ float front_waves_sum(float v, int wave, float* scratch) {
+#ifndef RWKV_LN_FLAGS
+#define RWKV_LN_FLAGS 1
+#endif
+
+// Counters in LDS by which the wavefronts of a prologue block meet without s_barrier: a barrier counts every
+// wavefront of the block, and the ones that are not computing the prologue reach it only when the memory pipeline
+// has taken all their weight requests - microseconds into a large launch.  [2m], [2m + 1]: the computing wavefronts
+// that have delivered their partial sum / sum of squares of row m; [kLnFlagX]: those whose part of x is in LDS.
+// Zeroed by the block's first threads before the one barrier every wavefront passes on entry.
+constexpr int kLnFlagX = 4;  // (up to two rows with the prologue)
+struct LnFlags {
+  unsigned count[kLnFlagX + 1];
+};
+
+// waits (bounded: no wavefront may spin for ever whatever happens to the others) until `n` wavefronts have arrived
+__device__ __forceinline__ void ln_flag_wait(unsigned* count, unsigned n) {
+  int spins = 0;
+  while (__hip_atomic_load(count, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < n && ++spins < (1 << 22))
+    __builtin_amdgcn_s_sleep(1);
+}
+
+__device__ __forceinline__ void ln_flag_arrive(unsigned* count) {
+  if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// sum over the first NWL wavefronts of the block (the callers).  With FLAGS they meet at the counter; without, at a
+// barrier that the other wavefronts pass too.
+template <int NWL, bool FLAGS>
+__device__ __forceinline__ float front_waves_sum(float v, int wave, float* scratch, unsigned* count) {
   v = wave_sum_uniform(v);
   if ((threadIdx.x & 63) == 0) scratch[wave] = v;
-  __syncthreads();
+  if constexpr (FLAGS) {
+    ln_flag_arrive(count);
+    ln_flag_wait(count, NWL);
+  } else {
+    __syncthreads();
+  }
   float t = 0.0f;
 #pragma unroll
   for (int i = 0; i < NWL; ++i) t += scratch[i];
@@ -536,9 +567,10 @@ __device__ __forceinline__ float front_waves_sum(float v, int wave, float* scrat
 }
 
 // (W4: xs in nibble-pair order, the slice sums to xsum - see w4_pair_order)
-template <int NT, int V8, int NTL, int M, bool W4>
+template <int NT, int V8, int NTL, int M, bool W4, bool FLAGS>
 __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8, M>& q, const LnPrologue& ln, int K, int m, half_t* xs,
-                                                float* xsum, float* stash, float* red, bool store, int wave) {
+                                                float* xsum, float* stash, float* red, LnFlags* flags, bool store,
+                                                int wave) {
   const int64_t row = static_cast<int64_t>(m) * K;
   constexpr int NWL = NTL / 64;  // wavefronts that compute
   half_t* hstash = reinterpret_cast<half_t*>(stash + NT * 4);
@@ -563,7 +595,7 @@ __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8, M>& q, const 
     *reinterpret_cast<half8_t*>(hstash + c + NT * 12) = q.mv[g];
   }
   __builtin_amdgcn_sched_barrier(0);
-  sum = front_waves_sum<NWL>(sum, wave, red);
+  sum = front_waves_sum<NWL, FLAGS>(sum, wave, red, &flags->count[2 * m]);
   const float mean = sum / static_cast<float>(K);
   float sv = 0.0f;
 #pragma unroll
@@ -584,7 +616,7 @@ __device__ __forceinline__ void ln_row1_finish8(const LnRow1xV<V8, M>& q, const 
       }
     }
   }
-  sv = front_waves_sum<NWL>(sv, wave, red + NT / 64);
+  sv = front_waves_sum<NWL, FLAGS>(sv, wave, red + NT / 64, &flags->count[2 * m + 1]);
   const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
 #pragma unroll
   for (int g = 0; g < V8; ++g) {
@@ -650,30 +682,6 @@ __device__ __forceinline__ LnRowOne<V8> ln_one_request8(const LnPrologue& ln, co
     q.mv[g] = *reinterpret_cast<const half8_t*>(mu + cc);
   }
   return q;
-}
-
-#ifndef RWKV_LN_FLAGS
-#define RWKV_LN_FLAGS 1
-#endif
-
-// Counters in LDS by which the wavefronts of a one-row prologue block meet without s_barrier: a barrier counts every
-// wavefront of the block, and the ones that are not computing the prologue reach it only when the memory pipeline
-// has taken all their weight requests - microseconds into a large launch.  [0], [1]: the computing wavefronts that
-// have delivered their partial row sum / sum of squares; [2]: those whose part of x is in LDS.  Zeroed by the
-// block's first threads before the one barrier every wavefront passes on entry.
-struct LnFlags {
-  unsigned count[3];
-};
-
-// waits (bounded: no wavefront may spin for ever whatever happens to the others) until `n` wavefronts have arrived
-__device__ __forceinline__ void ln_flag_wait(unsigned* count, unsigned n) {
-  int spins = 0;
-  while (__hip_atomic_load(count, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < n && ++spins < (1 << 22))
-    __builtin_amdgcn_s_sleep(1);
-}
-
-__device__ __forceinline__ void ln_flag_arrive(unsigned* count) {
-  if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
 // sum over the first NWL wavefronts of the block (the callers).  With FLAGS they meet at the counter; without, at a
@@ -965,7 +973,7 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
   if constexpr (LN) {
     // two code paths, so that the prologue's operands and the weight vectors never hold registers together; the
     // second path passes the two barriers of the first one's block sums, once per row
-    constexpr bool kFlags = RWKV_LN_FLAGS != 0 && M == 1;
+    constexpr bool kFlags = RWKV_LN_FLAGS != 0;
     constexpr unsigned NWL = NTL / 64;
     if (ln_wave) {
       if constexpr (M == 1) {
@@ -973,31 +981,38 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (kFlags) {
           // the prologue's operands are in the memory pipeline ahead of any weights of this block
-          if (threadIdx.x < 3) flags->count[threadIdx.x] = 0u;
+          if (threadIdx.x <= kLnFlagX) flags->count[threadIdx.x] = 0u;
           __syncthreads();
           // (nothing that waits for the operands may move above the barrier: the other wavefronts wait there)
           __builtin_amdgcn_sched_barrier(0);
         }
         ln_one_finish8<NT, V8, NTL, kW4, kFlags>(lnq, args.ln, K, xs, xsum, stash, red, flags, blockIdx.x == 0, wave);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (kFlags) ln_flag_arrive(&flags->count[2]);
       } else {
-      const LnRow1xV<V8, M> lnq = ln_row1_request8<V8, NTL, M>(args.ln, prob.mu, K);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int m = 0; m < M; ++m) {
-        ln_row1_finish8<NT, V8, NTL, M, kW4>(lnq, args.ln, K, m, xs + m * KCAP, xsum + m * (KCAP / 32), stash, red,
-                                             blockIdx.x == 0, wave);
+        const LnRow1xV<V8, M> lnq = ln_row1_request8<V8, NTL, M>(args.ln, prob.mu, K);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (kFlags) {
+          if (threadIdx.x <= kLnFlagX) flags->count[threadIdx.x] = 0u;
+          __syncthreads();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          // (the stash of row m is rewritten by row m + 1 only after every wavefront has passed row m's second
+          // meeting, i.e. has read what it needs of it: each thread reads only what it wrote)
+          ln_row1_finish8<NT, V8, NTL, M, kW4, kFlags>(lnq, args.ln, K, m, xs + m * KCAP, xsum + m * (KCAP / 32), stash,
+                                                       red, flags, blockIdx.x == 0, wave);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
-      }
+      if constexpr (kFlags) ln_flag_arrive(&flags->count[kLnFlagX]);
       request_all();
       // Each path has its own copy of the products.  Where the two paths met before them, the compiler's wait for
       // the first vector became a wait for one of the last (it merges the two paths' lists of loads in flight
       // conservatively), and the arithmetic - microseconds of it per launch - ran after the stream, not under it.
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (kFlags) {
-        ln_flag_wait(&flags->count[2], NWL);
+        ln_flag_wait(&flags->count[kLnFlagX], NWL);
       } else {
         __syncthreads();
       }
@@ -1008,7 +1023,7 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
       request_all();
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (kFlags) {
-        ln_flag_wait(&flags->count[2], NWL);
+        ln_flag_wait(&flags->count[kLnFlagX], NWL);
       } else {
 #pragma unroll 1
         for (int m = 0; m < M; ++m) {
@@ -1094,6 +1109,7 @@ static int row1_format(const LinearArgs& args) {
 // row's prologue runs before the computing wavefronts request their weights, and the stash shares the LDS).
 constexpr int kRow1MaxRows = 4;
 constexpr int kRow1MaxRowsLn = 2;
+static_assert(2 * kRow1MaxRowsLn <= kLnFlagX, "two counters per prologue row");
 
 template <int NT, bool LN, int DF, int M, int RX = 1>
 static int launch_row1(hipStream_t st, LinearArgs& args) {
