@@ -1167,12 +1167,280 @@ static int launch_row1_any(hipStream_t st, LinearArgs& args, int df) {
 }
 
 
+// ---- 5..16 rows: the same stream of whole rows, the products on the matrix core --------------------------------------
+// From five rows on, the GEMV's per-row VALU work (one v_dot2 per row and pair of weights) costs more than the stream
+// it runs under.  Here v_mfma_f32_16x16x32_f16 takes the rows of x as the sixteen columns of its B operand: a
+// wavefront owns sixteen rows of W and a part of K - lane (r, q) = (lane % 16, lane / 16) requests, per step, the
+// 16 bytes of row r that follow the 16 bytes of lane (r, q - 1), so a step covers 64 bytes of each of the sixteen
+// rows - and has up to 16 vectors in flight at once (K = 4096 int8 codes in 4 parts: all of them), as the GEMV's
+// wavefronts have theirs.  A block of 16 wavefronts is G groups of sixteen rows x 16 / G parts of K (G = 4 where
+// that still gives every CU a block, else 1); the parts' 16 x 16 partial products meet in LDS and are added in part
+// order.  x (M rows, fp16) is staged in LDS once per block, rows K + 8 values apart (the sixteen lanes of a b128
+// read then hit different banks); lanes whose column is no row of x read row 0 and their products are dropped.
+// int8 codes become fp16 (exact) on the way, the row scale multiplies the sum.
+//
+// Up to 8 rows of x the wavefronts share the start of the launch like those of the GEMV with the LayerNorm prologue:
+// the first half brings x into LDS (and requests its weights afterwards), the second half requests its weights at
+// once; they meet at a counter in LDS, not at a barrier - a barrier counts every wavefront, and a wavefront reaches
+// it only when the memory pipeline has taken all its requests.  With 9..16 rows (twice the registers for x) every
+// wavefront stages its share of x first and requests its weights after the barrier.
+constexpr int kRowsMfmaMax = 16;
+constexpr int kRowsMfmaMin = 5;
+constexpr int kRowsMfmaThreads = 1024;
+constexpr int kRowsMfmaXVecs = 8;  // 16-byte vectors of x per staging thread
+
+// Groups of sixteen rows in a block of fp16 weights, by those of the launch's int8 blocks: half as many where that
+// is possible, so that every block of a launch streams the same number of bytes and a wavefront's vectors of either
+// format fit one batch (7.2B shape, r/k/v with the fp16 rank-ins riding along).
+constexpr int rows_mfma_groups_f16(int g) { return g >= 2 ? g / 2 : g; }
+
+template <int FMT, int NB, int G, bool SPLIT>
+__device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const LinearProblem& prob, int blk, int M,
+                                                half_t* xs, int xstride, float* part, unsigned* flag) {
+  constexpr int EB = FMT == RWKV_FMT_F16 ? 2 : 1;    // bytes per weight
+  constexpr int KV = 16 / EB;                         // weights per 16-byte vector
+  constexpr int P = 16 / G;                           // parts of K
+  const int K = args.K;
+  const int N = prob.N;
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int lane = threadIdx.x & 63;
+  const int g = wave / P, kp = wave % P;
+  const int r = lane & 15, kq = lane >> 4;
+  const int KP = K / P;                               // this wavefront's part of K
+  const int steps = KP / (4 * KV);                    // vectors per lane: a step is 4 * KV values of a row
+  const int n0 = (blk * G + g) * 16;
+  const bool active = n0 < N;
+  const unsigned char* wrow = static_cast<const unsigned char*>(prob.w) +
+                              (static_cast<int64_t>(active ? n0 + r : r) * K + static_cast<int64_t>(kp) * KP + kq * KV) * EB;
+  const half_t* xrow = xs + (r < M ? r : 0) * xstride + kp * KP + kq * KV;
+  float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  uint4_t w[NB];
+  auto request = [&](int s0) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i)
+      w[i] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wrow + static_cast<int64_t>(s0 + i) * 64));
+  };
+  auto products = [&](int s0) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const half_t* xp = xrow + (s0 + i) * 4 * KV;
+      if constexpr (FMT == RWKV_FMT_F16) {
+        const half8_t b = *reinterpret_cast<const half8_t*>(xp);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, w[i]), b, acc, 0, 0, 0);
+      } else {
+        half2_t c[8];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) cvt_i8x4(w[i][d], c[2 * d], c[2 * d + 1]);
+        const half8_t a0 = {c[0][0], c[0][1], c[1][0], c[1][1], c[2][0], c[2][1], c[3][0], c[3][1]};
+        const half8_t a1 = {c[4][0], c[4][1], c[5][0], c[5][1], c[6][0], c[6][1], c[7][0], c[7][1]};
+        const half8_t b0 = *reinterpret_cast<const half8_t*>(xp);
+        const half8_t b1 = *reinterpret_cast<const half8_t*>(xp + 8);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc, 0, 0, 0);
+      }
+    }
+  };
+  // x of this problem: M rows of K / 8 vectors, contiguous
+  const int kv = K >> 3;
+  constexpr int NTS = SPLIT ? kRowsMfmaThreads / 2 : kRowsMfmaThreads;  // staging threads
+  auto stage_x = [&]() {
+    uint4_t xv[kRowsMfmaXVecs];
+#pragma unroll
+    for (int j = 0; j < kRowsMfmaXVecs; ++j) {
+      const int i = threadIdx.x + j * NTS;
+      xv[j] = uint4_t{0u, 0u, 0u, 0u};
+      if (i < M * kv) xv[j] = *reinterpret_cast<const uint4_t*>(prob.x + static_cast<int64_t>(i) * 8);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (SPLIT) {
+      // x is in the memory pipeline ahead of any weights of this block
+      if (threadIdx.x == 0) *flag = 0u;
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int j = 0; j < kRowsMfmaXVecs; ++j) {
+      const int i = threadIdx.x + j * NTS;
+      if (i < M * kv) {
+        const int m = i / kv, c = (i - m * kv) * 8;
+        *reinterpret_cast<uint4_t*>(xs + m * xstride + c) = xv[j];
+      }
+    }
+  };
+  if constexpr (SPLIT) {
+    constexpr unsigned NWS = NTS / 64;
+    if (wave < static_cast<int>(NWS)) {
+      stage_x();
+      __builtin_amdgcn_sched_barrier(0);
+      ln_flag_arrive(flag);
+      request(0);
+      __builtin_amdgcn_sched_barrier(0);
+      ln_flag_wait(flag, NWS);
+    } else {
+      __syncthreads();
+      request(0);
+      __builtin_amdgcn_sched_barrier(0);
+      ln_flag_wait(flag, NWS);
+    }
+  } else {
+    stage_x();
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    request(0);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  products(0);
+#pragma unroll 1
+  for (int s0 = NB; s0 < steps; s0 += NB) {
+    request(s0);
+    products(s0);
+  }
+  // lane (j, i4) = (lane % 16, lane / 16) holds the products of rows n0 + 4 * i4 + v (v = 0..3) of W with row j of x
+#pragma unroll
+  for (int v = 0; v < 4; ++v) part[wave * 256 + v * 64 + lane] = acc[v];
+  __syncthreads();
+  // G * 256 sums: thread t adds the parts of one (row of W, row of x), in part order
+  {
+    const int t = threadIdx.x;
+    const int og = t >> 8, v = (t >> 6) & 3, l = t & 63;
+    const int n = (blk * G + og) * 16 + 4 * (l >> 4) + v;
+    const int m = l & 15;
+    if (og < G && m < M && n < N) {
+      const float* ps = part + og * P * 256 + v * 64 + l;
+      float sum = ps[0];
+#pragma unroll
+      for (int q = 1; q < P; ++q) sum += ps[q * 256];
+      if constexpr (FMT == RWKV_FMT_W8) sum *= h2f(prob.scale[n]);
+      sum = round_h(sum);
+      if (args.epilogue == RWKV_EPI_RELU_SQUARE) {
+        sum = fmaxf(sum, 0.0f);
+        sum = round_h(sum * sum);
+      }
+      const int64_t o = static_cast<int64_t>(m) * N + n;
+      if (args.out_f32) {
+        static_cast<float*>(prob.y)[o] = sum;
+      } else {
+        static_cast<half_t*>(prob.y)[o] = f2h(sum);
+      }
+    }
+  }
+}
+
+// grid = blocks of 16 * G rows of W over all problems, which share x (M <= 16 rows) only in shape: each problem has
+// its own x.  Dynamic LDS: M rows of K + 8 fp16 values, then 16 x 256 floats of partial products.  One block per CU
+// (1024 threads, up to 128 registers).  DF: format of the quantised problems (int8); fp16 problems may ride along
+// (twice the steps, in batches of the same size).
+template <int DF, int NB, int G, bool SPLIT>
+__global__ __launch_bounds__(kRowsMfmaThreads)
+void linear_rows_mfma_kernel(LinearArgs args, int M) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  __shared__ unsigned flag;
+  half_t* xs = reinterpret_cast<half_t*>(lds_raw);
+  const int xstride = args.K + 8;
+  float* part = reinterpret_cast<float*>(lds_raw + static_cast<size_t>(M) * xstride * sizeof(half_t));
+  if (blockIdx.x == 0 && args.copy.n > 0) {
+    for (int i = threadIdx.x * 8; i < args.copy.n; i += kRowsMfmaThreads * 8)
+      *reinterpret_cast<uint4_t*>(args.copy.dst + i) = *reinterpret_cast<const uint4_t*>(args.copy.src + i);
+  }
+  int pi = 0;
+  int first = 0;
+  for (int i = 0; i < args.n_problems - 1; ++i) {
+    if (static_cast<int>(blockIdx.x) >= args.block_end[i]) {
+      pi = i + 1;
+      first = args.block_end[i];
+    }
+  }
+  const LinearProblem prob = args.p[pi];
+  const int blk = blockIdx.x - first;
+  if (DF != RWKV_FMT_F16 && prob.fmt == DF) {  // uniform per block
+    rows_mfma_block<DF, NB, G, SPLIT>(args, prob, blk, M, xs, xstride, part, &flag);
+  } else {
+    rows_mfma_block<RWKV_FMT_F16, NB, rows_mfma_groups_f16(G), SPLIT>(args, prob, blk, M, xs, xstride, part, &flag);
+  }
+}
+
+// Formats and shapes of the few-row matrix-core launch: int8 or fp16 weights, K a multiple of 512 up to 4096 (a
+// sixteenth of K in whole steps of both formats, x in LDS), N a multiple of 16.
+static bool rows_mfma_shape_ok(int M, int K, int n_problems, const LinearProblem* problems) {
+  if (M < 1 || M > kRowsMfmaMax || K < 1024 || K > 4096 || K % 1024 != 0) return false;
+  for (int i = 0; i < n_problems; ++i) {
+    const LinearProblem& p = problems[i];
+    if (p.fmt != RWKV_FMT_W8 && p.fmt != RWKV_FMT_F16) return false;
+    if (p.N % 16 != 0 || p.x == nullptr || p.x_f32 != nullptr) return false;
+  }
+  return true;
+}
+
+bool linear_rows_mfma_supported(int fmt, int N, int K) {
+  LinearProblem p;
+  p.fmt = fmt;
+  p.N = N;
+  p.x = reinterpret_cast<const half_t*>(&p);  // (only tested against NULL)
+  return rows_mfma_shape_ok(kRowsMfmaMin, K, 1, &p);
+}
+
+template <int DF, int NB, int G, bool SPLIT>
+static int launch_rows_mfma(hipStream_t st, LinearArgs& args, int M) {
+  int total = 0;
+  for (int i = 0; i < args.n_problems; ++i) {
+    total += ceil_div(args.p[i].N, 16 * (args.p[i].fmt == RWKV_FMT_F16 ? rows_mfma_groups_f16(G) : G));
+    args.block_end[i] = total;
+  }
+  const size_t lds = static_cast<size_t>(M) * (args.K + 8) * sizeof(half_t) + 16 * 256 * sizeof(float);
+  if (lds > 48 * 1024) {  // beyond the default limit of dynamic LDS: raised once per instantiation (to the largest M)
+    static bool raised = false;
+    if (!raised) {
+      const size_t most = static_cast<size_t>(kRowsMfmaMax) * (4096 + 8) * sizeof(half_t) + 16 * 256 * sizeof(float);
+      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_rows_mfma_kernel<DF, NB, G, SPLIT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(most)));
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL((linear_rows_mfma_kernel<DF, NB, G, SPLIT>), dim3(total), dim3(kRowsMfmaThreads), lds, st, args, M);
+  RWKV_LAUNCH_CHECK();
+  return RWKV_OK;
+}
+
+// Vectors per batch (NB) by shape: a wavefront has K * G / 1024 vectors of int8 codes to request (as many of fp16
+// weights with half the groups per block, twice as many with one group) and takes them in batches of up to 16.
+template <int DF, int G, bool SPLIT>
+static int launch_rows_mfma_g(hipStream_t st, LinearArgs& args, int M) {
+  const int steps = args.K * G / 1024;
+  if constexpr (G == 4) {
+    if (steps % 16 == 0) return launch_rows_mfma<DF, 16, G, SPLIT>(st, args, M);
+    if (steps % 8 == 0) return launch_rows_mfma<DF, 8, G, SPLIT>(st, args, M);
+  }
+  if (steps % 4 == 0) return launch_rows_mfma<DF, 4, G, SPLIT>(st, args, M);
+  if (steps % 2 == 0) return launch_rows_mfma<DF, 2, G, SPLIT>(st, args, M);
+  return launch_rows_mfma<DF, 1, G, SPLIT>(st, args, M);
+}
+
+template <int DF>
+static int launch_rows_mfma_fmt(hipStream_t st, LinearArgs& args, int M) {
+  // four groups of rows per block where that leaves no more than a quarter of the CUs without one
+  int blocks4 = 0;
+  for (int i = 0; i < args.n_problems; ++i)
+    blocks4 += ceil_div(args.p[i].N, 16 * (args.p[i].fmt == RWKV_FMT_F16 ? rows_mfma_groups_f16(4) : 4));
+  const bool g4 = blocks4 * 4 >= device_cu_count() * 3;
+  // the first half of the wavefronts stages x if eight vectors per thread cover it
+  const bool split = M * (args.K / 8) <= kRowsMfmaXVecs * (kRowsMfmaThreads / 2);
+  if (g4) {
+    return split ? launch_rows_mfma_g<DF, 4, true>(st, args, M) : launch_rows_mfma_g<DF, 4, false>(st, args, M);
+  }
+  return split ? launch_rows_mfma_g<DF, 1, true>(st, args, M) : launch_rows_mfma_g<DF, 1, false>(st, args, M);
+}
+
+static int launch_rows_mfma_any(hipStream_t st, LinearArgs& args, int M, int df) {
+  if (df == RWKV_FMT_W8) return launch_rows_mfma_fmt<RWKV_FMT_W8>(st, args, M);
+  return launch_rows_mfma_fmt<RWKV_FMT_F16>(st, args, M);
+}
+
 int linear_ln_prologue_max_rows(int K) { return K <= 4096 && K % 8 == 0 ? kRow1MaxRowsLn : 0; }
 
 // Batched small-M linear: n_problems problems sharing M (<= 8), K, epilogue and output type.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
                    int out_f32, const LnPrologue* ln, const RowCopy* copy) {
-  RWKV_REQUIRE(M >= 1 && M <= 8, "linear_small_m: M %d out of range", M);
+  RWKV_REQUIRE(M >= 1 && M <= kRowsMfmaMax, "linear_small_m: M %d out of range", M);
   RWKV_REQUIRE(n_problems >= 1 && n_problems <= kMaxProblems, "linear_small_m: %d problems", n_problems);
   LinearArgs args = {};
   int max_elems = 8;
@@ -1218,6 +1486,16 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
     gated = true;
     RWKV_REQUIRE(problems[i].x_gate != nullptr && K % 8 == 0, "linear: a gated x needs its gate and K %% 8 == 0");
   }
+  static const int rows_mfma_min = [] {
+    const char* e = getenv("RWKV_ROWS_MFMA_MIN");  // tuning hook: rows from which the matrix-core launch is used
+    return e ? atoi(e) : kRowsMfmaMin;
+  }();
+  if (M >= rows_mfma_min && args.ln.mode == 0 && rows_mfma_shape_ok(M, K, n_problems, problems)) {
+    int df = RWKV_FMT_F16;
+    for (int i = 0; i < n_problems; ++i) df = problems[i].fmt == RWKV_FMT_W8 ? RWKV_FMT_W8 : df;
+    return launch_rows_mfma_any(st, args, M, df);
+  }
+  RWKV_REQUIRE(M <= 8, "linear: %d rows of this shape or format (K = %d) have no few-row launch", M, K);
   if (M <= (args.ln.mode != 0 ? kRow1MaxRowsLn : kRow1MaxRows)) {
     const int df = row1_format(args);
     if (df >= 0 && !(gated && args.ln.mode != 0)) {
@@ -1247,11 +1525,13 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
 int linear_any_m(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* w, const half_t* scale,
                  const uint8_t* zp, int epilogue, int out_f32, void* y) {
   RWKV_REQUIRE(M > 0, "linear: M must be positive");
-  if (M >= 16 && linear_mfma_supported(fmt, M, N, K)) {
+  const bool few = linear_rows_mfma_supported(fmt, N, K);
+  if (M >= 16 && !(few && M <= kRowsMfmaMax) && linear_mfma_supported(fmt, M, N, K)) {
     return linear_mfma(st, fmt, M, N, K, x, w, scale, zp, epilogue, out_f32, y);
   }
-  for (int m0 = 0; m0 < M; m0 += 8) {
-    const int mt = std::min(8, M - m0);
+  const int tile = few ? kRowsMfmaMax : 8;
+  for (int m0 = 0; m0 < M; m0 += tile) {
+    const int mt = std::min(tile, M - m0);
     LinearProblem p;
     p.w = w;
     p.scale = scale;

@@ -73,14 +73,30 @@ struct GraphEntry {
 };
 
 constexpr size_t kMaxGraphs = 8;
-// Calls with at least this many rows stream the packed copy through MFMA; below, the weight-streaming GEMV that keeps
+// Calls with at least this many rows stream the packed copy through MFMA.  Below: the weight-streaming GEMV that keeps
 // whole weight rows in flight for up to 4 rows of x (decode ms per step, GEMV / streaming GEMM: 7.2B shape, int8: 3 rows
 // 2.39 / 2.79, 4 rows 2.56 / 2.82; 1.5B shape: 3 rows 1.20 / 1.45, 4 rows 1.31 / 1.51, 5 rows 1.55 / 1.31; 0.1B shape,
-// fp16: 3 rows 0.51 / 0.63, 4 rows 0.57 / 0.67).  RWKV_PACKED_MIN_ROWS (tuning hook) overrides the crossover.
+// fp16: 3 rows 0.51 / 0.63, 4 rows 0.57 / 0.67), and from 5 to 16 rows - for int8 and fp16 weights in rows of 1024,
+// 2048, 3072 or 4096 values - the same stream with the products on the matrix core (7.2B shape, int8, this / streaming
+// GEMM: 5 rows 2.84 / 3.01, 8 rows 2.69 / 2.87, 16 rows 2.99 / 3.06).  RWKV_PACKED_MIN_ROWS (tuning hook) overrides
+// the crossover.
 constexpr int kPackedMinRows = 3;  // what gets a packed copy at all: rows too long for the GEMV (ffn.value) use it from here
-inline int packed_min_rows(int /*C*/) {
+constexpr int kFewRowsMax = 16;    // most rows of the few-row matrix-core launch
+inline bool few_rows_on_matrix_core(const rwkv_hip_model* m) {
+  if (m->layers.empty()) return false;
+  const Layer& l0 = m->layers[0];
+  const int mids[5] = {RWKV_M_ATT_R, RWKV_M_ATT_K, RWKV_M_ATT_V, RWKV_M_ATT_O, RWKV_M_FFN_KEY};
+  for (int id : mids)
+    if (!linear_rows_mfma_supported(l0.m[id].fmt, id == RWKV_M_FFN_KEY ? m->F : m->C, m->C)) return false;
+  const int ranks[4] = {m->Rw, m->Ra, m->Rg, m->Rv};
+  for (int r : ranks)
+    if (!linear_rows_mfma_supported(RWKV_FMT_F16, r, m->C)) return false;
+  return true;
+}
+inline int packed_min_rows(const rwkv_hip_model* m) {
   static const int forced = getenv("RWKV_PACKED_MIN_ROWS") ? atoi(getenv("RWKV_PACKED_MIN_ROWS")) : 0;
-  return forced >= kPackedMinRows ? forced : 5;
+  if (forced >= kPackedMinRows) return forced;
+  return few_rows_on_matrix_core(m) ? kFewRowsMax + 1 : 5;
 }
 // most blocks of a single-launch time-mix core beyond 8 rows (one round on the chip's compute units; us per layer at the 7.2B shape,
 // this launch / the row-tiled kernels: 16 rows 14 / 17, 32 rows 25 / 24)
@@ -234,7 +250,9 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
     s->arena_B = B;
     s->arena_T = T;
   }
-  if (rows >= static_cast<size_t>(packed_min_rows(m->C))) {
+  // (from the smallest row count that any matrix takes through its packed copy: ffn.value's rows are too long for
+  // the few-row launches)
+  if (rows >= static_cast<size_t>(kPackedMinRows)) {
     const int R = static_cast<int>(rows);
     const int qkv_ns[7] = {m->C, m->C, m->C, m->Rw, m->Ra, m->Rg, m->Rv};
     size_t ws = std::max(linear_packed_multi_workspace_bytes(R, m->C, 7, qkv_ns),
@@ -292,7 +310,7 @@ int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int
                  int out_f32, void* y, DeferredReduce* defer = nullptr, const RowCopy* copy = nullptr) {
   if (defer) *defer = DeferredReduce{};
   // (rows longer than the few-row GEMV keeps in registers go to the packed product from its smallest row count on)
-  if (mat.packed && (M >= packed_min_rows(s->model->C) || (M >= kPackedMinRows && K > 4096))) {
+  if (mat.packed && (M >= packed_min_rows(s->model) || (M >= kPackedMinRows && K > 4096))) {
     return linear_packed(s->stream, mat.fmt, M, N, K, x, mat.packed, mat.scale, mat.zp, epilogue, out_f32, y, s->gemm_ws,
                          s->gemm_ws_bytes, defer, copy);
   }
@@ -356,7 +374,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   bool packable = true;
   for (const Matrix& mat : m->layers[0].m) packable = packable && mat.packed != nullptr;
   for (int i = 0; i < 3; ++i) packable = packable && m->layers[0].lora_in_packed[i] != nullptr;
-  const bool small = rows < packed_min_rows(C) || (rows <= 8 && !packable);
+  const bool small = rows < packed_min_rows(m) || (rows <= 8 && !packable);
   hipEvent_t pass_begin = nullptr;
   if (s->profile == 2) {
     RWKV_HIP_TRY(hipEventCreate(&pass_begin));
@@ -399,7 +417,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   // launch it saves (prefill of a 4096-token prompt in chunks of 128: 22.6 -> 23.2 k tok/s at batch 1, 54.2 ->
   // 53.4 k at batch 16).  RWKV_SEQ_LN=0 (tuning hook) switches it off.
   static const bool seq_ln_on = !(getenv("RWKV_SEQ_LN") && atoi(getenv("RWKV_SEQ_LN")) == 0);
-  const bool seq_fused = seq_ln_on && !step && !s->trace && C <= 4096 && rows >= packed_min_rows(C) && rows <= 256;
+  const bool seq_fused = seq_ln_on && !step && !s->trace && C <= 4096 && rows >= packed_min_rows(m) && rows <= 256;
   RowCopy pending;  // shift rows waiting to be moved
   auto flush_pending = [&]() -> int {
     if (pending.n > 0) {
@@ -502,7 +520,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
           TRY_PROF(linear_small_m(st, rows, C, 3 + n_lora, p, RWKV_EPI_NONE, 0));
         }
       } else {
-        bool all_packed = rows >= packed_min_rows(C);
+        bool all_packed = rows >= packed_min_rows(m);
         for (int i = 0; i < 3; ++i) all_packed = all_packed && w.m[mids[i]].packed != nullptr;
         for (int i = 0; i < n_lora; ++i) all_packed = all_packed && w.lora_in_packed[i] != nullptr;
         if (all_packed) {

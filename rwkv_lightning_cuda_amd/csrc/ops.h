@@ -50,10 +50,13 @@ struct RowCopy {
   int n = 0;
 };
 
-// Batched small-M (<= 8) linear through the weight-streaming GEMV kernel: up to kMaxProblems problems that
-// share M and K (each with its own weight format, x and y) in one launch.
+// Batched small-M linear through the weight-streaming kernels (the GEMV up to 8 rows; the few-row matrix-core
+// launch from 5 to 16 rows where linear_rows_mfma_supported): up to kMaxProblems problems that share M and K (each
+// with its own weight format, x and y) in one launch.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
                    int out_f32, const LnPrologue* ln = nullptr, const RowCopy* copy = nullptr);
+// Whether 5..16 rows of this format and shape run on the few-row matrix-core launch (weights in their plain order).
+bool linear_rows_mfma_supported(int fmt, int N, int K);
 // Rows of a decode step that linear_small_m takes with the LayerNorm prologue at this row length (0: none).
 int linear_ln_prologue_max_rows(int K);
 // Any M: MFMA tiles for M >= 16 where supported, else row tiles through the GEMV kernel.

@@ -335,6 +335,38 @@ def test_linear_small_m(gpu, orc, fmt_name, M):
     assert err <= F16_TOL
 
 
+@pytest.mark.parametrize("fmt_name", ["w8", "f16"])
+@pytest.mark.parametrize("M,N,K", [(5, 272, 4096), (8, 64, 2048), (11, 1040, 4096), (16, 16384, 4096), (13, 96, 1024),
+                                   (7, 12304, 3072), (6, 4096, 4096), (37, 128, 1024), (8, 16400, 2048)])
+def test_linear_few_rows_on_the_matrix_core(gpu, orc, fmt_name, M, N, K):
+    """5..16 rows of int8 or fp16 weights whose K is a multiple of 1024 (<= 4096): the whole-rows-in-flight launch
+    with the products on the matrix core (more rows: tiles of 16 of the same launch).  fp16 output, the relu^2
+    epilogue and the fp32 output against the oracle; both block shapes (16 and 64 rows of W), both ways of staging
+    x (up to 8 rows / more), N that is no multiple of the block's rows."""
+    hip = gpu
+    rng = np.random.default_rng(M * 131 + N + K)
+    w = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    fmt = {"f16": hip.FMT_F16, "w8": hip.FMT_W8}[fmt_name]
+    parts = (w, None, None) if fmt == hip.FMT_F16 else orc.quantize_w8(w) + (None,)
+    hid = orc.gemv(fmt, x, parts[0], parts[1], parts[2])
+    dparts = [dev(hip, p) if p is not None else None for p in parts]
+    dx = dev(hip, x)
+    y = hip.DeviceArray((M, N), np.float16)
+    hip.linear(fmt, M, N, K, dx, dparts[0], dparts[1], dparts[2], y)
+    act = hip.DeviceArray((M, N), np.float16)
+    hip.linear(fmt, M, N, K, dx, dparts[0], dparts[1], dparts[2], act, epilogue=hip.EPI_RELU_SQUARE)
+    y32 = hip.DeviceArray((M, N), np.float32)
+    hip.linear(fmt, M, N, K, dx, dparts[0], dparts[1], dparts[2], y32, out_f32=1)
+    hip.device_sync()
+    assert rel_err(y.numpy().astype(np.float32), hid.astype(np.float32)) <= F16_TOL
+    assert rel_err(act.numpy().astype(np.float32), orc.relu_square(hid).astype(np.float32)) <= 2 * F16_TOL
+    got32 = y32.numpy()
+    assert rel_err(got32, hid.astype(np.float32)) <= F16_TOL
+    same = np.array_equal(got32, got32.astype(np.float16).astype(np.float32))
+    assert same
+
+
 @pytest.mark.parametrize("K", [1024, 2560, 4096, 16384])
 def test_linear_w8_relu_square_and_f32_out(gpu, orc, K):
     hip = gpu
