@@ -1189,14 +1189,142 @@ constexpr int kRowsMfmaMin = 5;
 constexpr int kRowsMfmaThreads = 1024;
 constexpr int kRowsMfmaXVecs = 8;  // 16-byte vectors of x per staging thread
 
+// LayerNorm(x + res) (or of a gathered table row) + token-shift lerp of up to 8 rows straight into the block's LDS
+// copy of x, by the staging wavefronts of a few-row matrix-core block: wavefront m owns row m (lane l the 8-value
+// slices l, l + 64, ...), so a row's statistics need no other wavefront.  Same formulas and rounding points as
+// ln_fused_kernel (fused_ops.hip), whose thread j * 64 + l holds this lane's slice j (one wavefront sum per j, added
+// in j order); the sums inside a slice and a wavefront associate differently, so the last bits may differ from that
+// kernel's.  LN weight, bias and this problem's lerp coefficients, which every row
+// needs whole, are fetched once per block (thread t its slice t) and passed through LDS (hst: 3 x K values);
+// block 0 of the launch also stores the residual sum and the LN output.
+constexpr int kRowsMfmaLnRows = 8;
+constexpr int kRowsMfmaLnSlices = 8;  // K <= 4096 = 8 x 64 lanes x 8 values
+
+__device__ __forceinline__ void rows_mfma_ln_prologue(const LnPrologue& ln, const half_t* __restrict__ mu, int K, int M,
+                                                      half_t* xs, int xstride, half_t* hst, LnFlags* flags, bool store) {
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int lane = threadIdx.x & 63;
+  const int nj = K >> 9;             // slices per lane
+  const bool row = wave < M;         // (wavefront-uniform)
+  const int64_t roff = static_cast<int64_t>(wave) * K;
+  // In the order of use, which is the order of arrival: the previous token's LN output (parked in the row's place in
+  // xs until the lerp), the shared vectors (to hst), then x and the residual, which stay in registers.
+  half8_t xv[kRowsMfmaLnSlices], rv[kRowsMfmaLnSlices];
+  {
+    half8_t pv[kRowsMfmaLnSlices];
+    if (row) {
+      const half_t* ps = ln.shift + roff + lane * 8;
+#pragma unroll
+      for (int j = 0; j < kRowsMfmaLnSlices; ++j)
+        if (j < nj) pv[j] = *reinterpret_cast<const half8_t*>(ps + j * 512);
+    }
+    const int ct = static_cast<int>(threadIdx.x) * 8;  // (staging threads: 0 .. 511)
+    const int cc = ct < K ? ct : 0;
+    const half8_t wv = *reinterpret_cast<const half8_t*>(ln.w + cc);
+    const half8_t bv = *reinterpret_cast<const half8_t*>(ln.b + cc);
+    const half8_t mv = *reinterpret_cast<const half8_t*>(mu + cc);
+    __builtin_amdgcn_sched_barrier(0);
+    if (row) {
+      const int64_t xsrc = ln.mode == 2 ? ln.tokens[wave] * static_cast<int64_t>(K) : roff;
+      const half_t* px = ln.x + xsrc + lane * 8;
+      const half_t* pr = ln.mode == 1 ? ln.res + roff + lane * 8 : px;
+#pragma unroll
+      for (int j = 0; j < kRowsMfmaLnSlices; ++j) {
+        if (j < nj) {
+          xv[j] = *reinterpret_cast<const half8_t*>(px + j * 512);
+          rv[j] = *reinterpret_cast<const half8_t*>(pr + j * 512);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // everything the prologue reads is in the memory pipeline ahead of any weights of this block
+    if (threadIdx.x <= kLnFlagX) flags->count[threadIdx.x] = 0u;
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    if (row) {
+#pragma unroll
+      for (int j = 0; j < kRowsMfmaLnSlices; ++j)
+        if (j < nj) *reinterpret_cast<half8_t*>(xs + wave * xstride + (j * 64 + lane) * 8) = pv[j];
+    }
+    if (ct < K) {
+      *reinterpret_cast<half8_t*>(hst + ct) = wv;
+      *reinterpret_cast<half8_t*>(hst + K + ct) = bv;
+      *reinterpret_cast<half8_t*>(hst + 2 * K + ct) = mv;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  ln_flag_arrive(&flags->count[0]);
+  if (row) {
+    // the row as fp32 sums from here on (as many registers as x and the residual took)
+    float v[kRowsMfmaLnSlices][8];
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kRowsMfmaLnSlices; ++j) {
+      if (j < nj) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[j][e] = ln.mode == 1 ? h2f(xv[j][e]) + h2f(rv[j][e]) : h2f(xv[j][e]);
+        sum += wave_sum_uniform(((v[j][0] + v[j][1]) + (v[j][2] + v[j][3])) + ((v[j][4] + v[j][5]) + (v[j][6] + v[j][7])));
+        // (slice by slice: converted all at once, the fp32 sums and their fp16 sources would not fit the registers)
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    const float mean = sum / static_cast<float>(K);
+    float sv = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kRowsMfmaLnSlices; ++j) {
+      if (j < nj) {
+        float q = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = v[j][e] - mean;
+          q = fmaf(d, d, q);
+        }
+        sv += wave_sum_uniform(q);
+      }
+    }
+    const float rstd = rsqrtf(sv / static_cast<float>(K) + ln.eps);
+    // (the differences from the mean are formed again below: kept from the pass above - which the compiler would do,
+    // seeing the same subtraction - they would be 64 registers more than there are)
+    float mean_again = mean;
+    asm volatile("" : "+v"(mean_again));
+    ln_flag_wait(&flags->count[0], kRowsMfmaThreads / 128);  // LN weight, bias and coefficients are in LDS
+#pragma unroll
+    for (int j = 0; j < kRowsMfmaLnSlices; ++j) {
+      if (j < nj) {
+        const int c = (j * 64 + lane) * 8;
+        const half8_t w8 = *reinterpret_cast<const half8_t*>(hst + c);
+        const half8_t b8 = *reinterpret_cast<const half8_t*>(hst + K + c);
+        const half8_t m8 = *reinterpret_cast<const half8_t*>(hst + 2 * K + c);
+        const half8_t p8 = *reinterpret_cast<const half8_t*>(xs + wave * xstride + c);  // (parked above by this lane)
+        half8_t yv, ov, xo;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float ve = v[j][e];
+          yv[e] = f2h(fmaf((ve - mean_again) * rstd, h2f(w8[e]), h2f(b8[e])));
+          const float yf = h2f(yv[e]);  // the lerp reads the fp16-rounded LN output
+          ov[e] = f2h(fmaf(h2f(p8[e]) - yf, h2f(m8[e]), yf));
+          xo[e] = f2h(ve);
+        }
+        *reinterpret_cast<half8_t*>(xs + wave * xstride + c) = ov;
+        if (store) {
+          *reinterpret_cast<half8_t*>(ln.ln_out + roff + c) = yv;
+          if (ln.x_out) *reinterpret_cast<half8_t*>(ln.x_out + roff + c) = xo;
+        }
+      }
+    }
+  }
+}
+
 // Groups of sixteen rows in a block of fp16 weights, by those of the launch's int8 blocks: half as many where that
 // is possible, so that every block of a launch streams the same number of bytes and a wavefront's vectors of either
 // format fit one batch (7.2B shape, r/k/v with the fp16 rank-ins riding along).
 constexpr int rows_mfma_groups_f16(int g) { return g >= 2 ? g / 2 : g; }
 
-template <int FMT, int NB, int G, bool SPLIT>
+template <int FMT, int NB, int G, bool SPLIT, bool LN>
 __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const LinearProblem& prob, int blk, int M,
-                                                half_t* xs, int xstride, float* part, unsigned* flag) {
+                                                half_t* xs, int xstride, float* part, LnFlags* flags) {
+  static_assert(SPLIT || !LN, "the prologue belongs to the staging half of the wavefronts");
+  unsigned* flag = &flags->count[kLnFlagX];
   constexpr int EB = FMT == RWKV_FMT_F16 ? 2 : 1;    // bytes per weight
   constexpr int KV = 16 / EB;                         // weights per 16-byte vector
   constexpr int P = 16 / G;                           // parts of K
@@ -1210,8 +1338,9 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
   const int steps = KP / (4 * KV);                    // vectors per lane: a step is 4 * KV values of a row
   const int n0 = (blk * G + g) * 16;
   const bool active = n0 < N;
+  const int64_t ldw = prob.ldw ? prob.ldw : K;
   const unsigned char* wrow = static_cast<const unsigned char*>(prob.w) +
-                              (static_cast<int64_t>(active ? n0 + r : r) * K + static_cast<int64_t>(kp) * KP + kq * KV) * EB;
+                              (static_cast<int64_t>(active ? n0 + r : r) * ldw + static_cast<int64_t>(kp) * KP + kq * KV) * EB;
   const half_t* xrow = xs + (r < M ? r : 0) * xstride + kp * KP + kq * KV;
   float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
   uint4_t w[NB];
@@ -1240,8 +1369,9 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
       }
     }
   };
-  // x of this problem: M rows of K / 8 vectors, contiguous
+  // x of this problem: M rows of K / 8 vectors (the rows ldx values apart)
   const int kv = K >> 3;
+  const int64_t ldx = prob.ldx ? prob.ldx : K;
   constexpr int NTS = SPLIT ? kRowsMfmaThreads / 2 : kRowsMfmaThreads;  // staging threads
   auto stage_x = [&]() {
     uint4_t xv[kRowsMfmaXVecs];
@@ -1249,12 +1379,15 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
     for (int j = 0; j < kRowsMfmaXVecs; ++j) {
       const int i = threadIdx.x + j * NTS;
       xv[j] = uint4_t{0u, 0u, 0u, 0u};
-      if (i < M * kv) xv[j] = *reinterpret_cast<const uint4_t*>(prob.x + static_cast<int64_t>(i) * 8);
+      if (i < M * kv) {
+        const int m = i / kv, c = (i - m * kv) * 8;
+        xv[j] = *reinterpret_cast<const uint4_t*>(prob.x + m * ldx + c);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (SPLIT) {
       // x is in the memory pipeline ahead of any weights of this block
-      if (threadIdx.x == 0) *flag = 0u;
+      if (threadIdx.x <= kLnFlagX) flags->count[threadIdx.x] = 0u;
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1270,7 +1403,12 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
   if constexpr (SPLIT) {
     constexpr unsigned NWS = NTS / 64;
     if (wave < static_cast<int>(NWS)) {
-      stage_x();
+      if constexpr (LN) {
+        half_t* hst = reinterpret_cast<half_t*>(part + 16 * 256);
+        rows_mfma_ln_prologue(args.ln, prob.mu, K, M, xs, xstride, hst, flags, blockIdx.x == 0);
+      } else {
+        stage_x();
+      }
       __builtin_amdgcn_sched_barrier(0);
       ln_flag_arrive(flag);
       request(0);
@@ -1310,13 +1448,17 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
       float sum = ps[0];
 #pragma unroll
       for (int q = 1; q < P; ++q) sum += ps[q * 256];
+      const int64_t o = static_cast<int64_t>(m) * N + n;
+      if (prob.raw_f32) {  // (uniform per block)
+        static_cast<float*>(prob.y)[o] = sum;
+        return;
+      }
       if constexpr (FMT == RWKV_FMT_W8) sum *= h2f(prob.scale[n]);
       sum = round_h(sum);
       if (args.epilogue == RWKV_EPI_RELU_SQUARE) {
         sum = fmaxf(sum, 0.0f);
         sum = round_h(sum * sum);
       }
-      const int64_t o = static_cast<int64_t>(m) * N + n;
       if (args.out_f32) {
         static_cast<float*>(prob.y)[o] = sum;
       } else {
@@ -1327,14 +1469,15 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
 }
 
 // grid = blocks of 16 * G rows of W over all problems, which share x (M <= 16 rows) only in shape: each problem has
-// its own x.  Dynamic LDS: M rows of K + 8 fp16 values, then 16 x 256 floats of partial products.  One block per CU
+// its own x.  Dynamic LDS: M rows of K + 8 fp16 values, then 16 x 256 floats of partial products, with the
+// LayerNorm prologue also 3 x K fp16 values (LN weight, bias, lerp coefficients).  One block per CU
 // (1024 threads, up to 128 registers).  DF: format of the quantised problems (int8); fp16 problems may ride along
 // (twice the steps, in batches of the same size).
-template <int DF, int NB, int G, bool SPLIT>
+template <int DF, int NB, int G, bool SPLIT, bool LN>
 __global__ __launch_bounds__(kRowsMfmaThreads)
 void linear_rows_mfma_kernel(LinearArgs args, int M) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  __shared__ unsigned flag;
+  __shared__ LnFlags flags;
   half_t* xs = reinterpret_cast<half_t*>(lds_raw);
   const int xstride = args.K + 8;
   float* part = reinterpret_cast<float*>(lds_raw + static_cast<size_t>(M) * xstride * sizeof(half_t));
@@ -1353,9 +1496,9 @@ void linear_rows_mfma_kernel(LinearArgs args, int M) {
   const LinearProblem prob = args.p[pi];
   const int blk = blockIdx.x - first;
   if (DF != RWKV_FMT_F16 && prob.fmt == DF) {  // uniform per block
-    rows_mfma_block<DF, NB, G, SPLIT>(args, prob, blk, M, xs, xstride, part, &flag);
+    rows_mfma_block<DF, NB, G, SPLIT, LN>(args, prob, blk, M, xs, xstride, part, &flags);
   } else {
-    rows_mfma_block<RWKV_FMT_F16, NB, rows_mfma_groups_f16(G), SPLIT>(args, prob, blk, M, xs, xstride, part, &flag);
+    rows_mfma_block<RWKV_FMT_F16, NB, rows_mfma_groups_f16(G), SPLIT, LN>(args, prob, blk, M, xs, xstride, part, &flags);
   }
 }
 
@@ -1366,53 +1509,60 @@ static bool rows_mfma_shape_ok(int M, int K, int n_problems, const LinearProblem
   for (int i = 0; i < n_problems; ++i) {
     const LinearProblem& p = problems[i];
     if (p.fmt != RWKV_FMT_W8 && p.fmt != RWKV_FMT_F16) return false;
-    if (p.N % 16 != 0 || p.x == nullptr || p.x_f32 != nullptr) return false;
+    if (p.N % 16 != 0 || p.x_f32 != nullptr) return false;
   }
   return true;
+}
+
+// With the LayerNorm prologue: up to 8 rows (a staging wavefront each) of 1024 .. 4096 values, staged by half of the
+// wavefronts.
+static bool rows_mfma_ln_ok(int M, int K) {
+  return M <= kRowsMfmaLnRows && K % 512 == 0 && M * (K / 8) <= kRowsMfmaXVecs * (kRowsMfmaThreads / 2);
 }
 
 bool linear_rows_mfma_supported(int fmt, int N, int K) {
   LinearProblem p;
   p.fmt = fmt;
   p.N = N;
-  p.x = reinterpret_cast<const half_t*>(&p);  // (only tested against NULL)
   return rows_mfma_shape_ok(kRowsMfmaMin, K, 1, &p);
 }
 
-template <int DF, int NB, int G, bool SPLIT>
+template <int DF, int NB, int G, bool SPLIT, bool LN>
 static int launch_rows_mfma(hipStream_t st, LinearArgs& args, int M) {
   int total = 0;
   for (int i = 0; i < args.n_problems; ++i) {
     total += ceil_div(args.p[i].N, 16 * (args.p[i].fmt == RWKV_FMT_F16 ? rows_mfma_groups_f16(G) : G));
     args.block_end[i] = total;
   }
-  const size_t lds = static_cast<size_t>(M) * (args.K + 8) * sizeof(half_t) + 16 * 256 * sizeof(float);
+  const size_t lds = static_cast<size_t>(M) * (args.K + 8) * sizeof(half_t) + 16 * 256 * sizeof(float) +
+                     (LN ? static_cast<size_t>(3) * args.K * sizeof(half_t) : 0);
   if (lds > 48 * 1024) {  // beyond the default limit of dynamic LDS: raised once per instantiation (to the largest M)
     static bool raised = false;
     if (!raised) {
-      const size_t most = static_cast<size_t>(kRowsMfmaMax) * (4096 + 8) * sizeof(half_t) + 16 * 256 * sizeof(float);
-      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_rows_mfma_kernel<DF, NB, G, SPLIT>),
+      const size_t most = static_cast<size_t>(LN ? kRowsMfmaLnRows : kRowsMfmaMax) * (4096 + 8) * sizeof(half_t) +
+                          16 * 256 * sizeof(float) + (LN ? static_cast<size_t>(3) * 4096 * sizeof(half_t) : 0);
+      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_rows_mfma_kernel<DF, NB, G, SPLIT, LN>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(most)));
       raised = true;
     }
   }
-  hipLaunchKernelGGL((linear_rows_mfma_kernel<DF, NB, G, SPLIT>), dim3(total), dim3(kRowsMfmaThreads), lds, st, args, M);
+  hipLaunchKernelGGL((linear_rows_mfma_kernel<DF, NB, G, SPLIT, LN>), dim3(total), dim3(kRowsMfmaThreads), lds, st, args, M);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
 // Vectors per batch (NB) by shape: a wavefront has K * G / 1024 vectors of int8 codes to request (as many of fp16
 // weights with half the groups per block, twice as many with one group) and takes them in batches of up to 16.
-template <int DF, int G, bool SPLIT>
+template <int DF, int G, bool SPLIT, bool LN>
 static int launch_rows_mfma_g(hipStream_t st, LinearArgs& args, int M) {
   const int steps = args.K * G / 1024;
   if constexpr (G == 4) {
-    if (steps % 16 == 0) return launch_rows_mfma<DF, 16, G, SPLIT>(st, args, M);
-    if (steps % 8 == 0) return launch_rows_mfma<DF, 8, G, SPLIT>(st, args, M);
+    if (steps % 16 == 0) return launch_rows_mfma<DF, 16, G, SPLIT, LN>(st, args, M);
+    if (steps % 8 == 0) return launch_rows_mfma<DF, 8, G, SPLIT, LN>(st, args, M);
   }
-  if (steps % 4 == 0) return launch_rows_mfma<DF, 4, G, SPLIT>(st, args, M);
-  if (steps % 2 == 0) return launch_rows_mfma<DF, 2, G, SPLIT>(st, args, M);
-  return launch_rows_mfma<DF, 1, G, SPLIT>(st, args, M);
+  if (steps % 4 == 0) return launch_rows_mfma<DF, 4, G, SPLIT, LN>(st, args, M);
+  if (steps % 2 == 0) return launch_rows_mfma<DF, 2, G, SPLIT, LN>(st, args, M);
+  return launch_rows_mfma<DF, 1, G, SPLIT, LN>(st, args, M);
 }
 
 template <int DF>
@@ -1422,12 +1572,15 @@ static int launch_rows_mfma_fmt(hipStream_t st, LinearArgs& args, int M) {
   for (int i = 0; i < args.n_problems; ++i)
     blocks4 += ceil_div(args.p[i].N, 16 * (args.p[i].fmt == RWKV_FMT_F16 ? rows_mfma_groups_f16(4) : 4));
   const bool g4 = blocks4 * 4 >= device_cu_count() * 3;
+  if (args.ln.mode != 0) {
+    return g4 ? launch_rows_mfma_g<DF, 4, true, true>(st, args, M) : launch_rows_mfma_g<DF, 1, true, true>(st, args, M);
+  }
   // the first half of the wavefronts stages x if eight vectors per thread cover it
   const bool split = M * (args.K / 8) <= kRowsMfmaXVecs * (kRowsMfmaThreads / 2);
   if (g4) {
-    return split ? launch_rows_mfma_g<DF, 4, true>(st, args, M) : launch_rows_mfma_g<DF, 4, false>(st, args, M);
+    return split ? launch_rows_mfma_g<DF, 4, true, false>(st, args, M) : launch_rows_mfma_g<DF, 4, false, false>(st, args, M);
   }
-  return split ? launch_rows_mfma_g<DF, 1, true>(st, args, M) : launch_rows_mfma_g<DF, 1, false>(st, args, M);
+  return split ? launch_rows_mfma_g<DF, 1, true, false>(st, args, M) : launch_rows_mfma_g<DF, 1, false, false>(st, args, M);
 }
 
 static int launch_rows_mfma_any(hipStream_t st, LinearArgs& args, int M, int df) {
@@ -1435,7 +1588,43 @@ static int launch_rows_mfma_any(hipStream_t st, LinearArgs& args, int M, int df)
   return launch_rows_mfma_fmt<RWKV_FMT_F16>(st, args, M);
 }
 
+int linear_rows_mfma_sliced(hipStream_t st, int fmt, int M, int N, int K, int slice, const half_t* x, const void* w,
+                            float* partial, const RowCopy* copy) {
+  RWKV_REQUIRE(slice > 0 && K % slice == 0 && K / slice >= 1 && K / slice <= kMaxProblems,
+               "linear: %d columns in slices of %d", K, slice);
+  RWKV_REQUIRE(M >= 1 && M <= kRowsMfmaMax && linear_rows_mfma_supported(fmt, N, slice),
+               "linear: no few-row launch for %d rows of this format and shape (N = %d, K = %d)", M, N, slice);
+  RWKV_REQUIRE(x && w && partial, "linear: NULL tensor");
+  LinearArgs args = {};
+  args.n_problems = K / slice;
+  args.K = slice;
+  args.epilogue = RWKV_EPI_NONE;
+  args.out_f32 = 1;
+  const int eb = fmt == RWKV_FMT_F16 ? 2 : 1;
+  for (int i = 0; i < args.n_problems; ++i) {
+    LinearProblem& p = args.p[i];
+    p.w = static_cast<const unsigned char*>(w) + static_cast<int64_t>(i) * slice * eb;
+    p.x = x + static_cast<int64_t>(i) * slice;
+    p.y = partial + static_cast<int64_t>(i) * M * N;
+    p.N = N;
+    p.fmt = fmt;
+    p.ldw = K;
+    p.ldx = K;
+    p.raw_f32 = 1;
+  }
+  if (copy && copy->n > 0) {
+    RWKV_REQUIRE(copy->src && copy->dst && copy->n % 8 == 0, "linear: bad row copy");
+    args.copy = *copy;
+  }
+  return launch_rows_mfma_any(st, args, M, fmt);
+}
+
 int linear_ln_prologue_max_rows(int K) { return K <= 4096 && K % 8 == 0 ? kRow1MaxRowsLn : 0; }
+
+bool linear_ln_prologue_rows_ok(int fmt, int M, int N, int K) {
+  if (M >= 1 && M <= linear_ln_prologue_max_rows(K)) return true;
+  return M >= kRowsMfmaMin && linear_rows_mfma_supported(fmt, N, K) && rows_mfma_ln_ok(M, K);
+}
 
 // Batched small-M linear: n_problems problems sharing M (<= 8), K, epilogue and output type.
 int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearProblem* problems, int epilogue,
@@ -1468,9 +1657,17 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
   int kt = (65536 / (2 * M)) / step * step;
   if (kt < step) kt = step;
   args.KT = std::min(kt, k_round);
-  if (ln && ln->mode != 0) {
+  static const int rows_mfma_min = [] {
+    const char* e = getenv("RWKV_ROWS_MFMA_MIN");  // tuning hook: rows from which the matrix-core launch is used
+    return e ? atoi(e) : kRowsMfmaMin;
+  }();
+  const bool with_ln = ln && ln->mode != 0;
+  const bool few_rows = M >= rows_mfma_min && rows_mfma_shape_ok(M, K, n_problems, problems) &&
+                        (!with_ln || rows_mfma_ln_ok(M, K));
+  if (with_ln) {
     RWKV_REQUIRE(ln->mode == 1 || ln->mode == 2, "linear: bad LayerNorm prologue mode %d", ln->mode);
-    RWKV_REQUIRE(args.KT >= K && K % 8 == 0 && static_cast<size_t>(M) * args.KT * 2 + static_cast<size_t>(K) * 4 <= 65536,
+    RWKV_REQUIRE(few_rows || (args.KT >= K && K % 8 == 0 &&
+                              static_cast<size_t>(M) * args.KT * 2 + static_cast<size_t>(K) * 4 <= 65536),
                  "linear: LayerNorm prologue needs the whole row in LDS (M = %d, K = %d)", M, K);
     RWKV_REQUIRE(ln->x && ln->w && ln->b && ln->shift && ln->ln_out && (ln->mode == 2 ? ln->tokens != nullptr : ln->res != nullptr),
                  "linear: LayerNorm prologue has a NULL tensor");
@@ -1486,11 +1683,9 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
     gated = true;
     RWKV_REQUIRE(problems[i].x_gate != nullptr && K % 8 == 0, "linear: a gated x needs its gate and K %% 8 == 0");
   }
-  static const int rows_mfma_min = [] {
-    const char* e = getenv("RWKV_ROWS_MFMA_MIN");  // tuning hook: rows from which the matrix-core launch is used
-    return e ? atoi(e) : kRowsMfmaMin;
-  }();
-  if (M >= rows_mfma_min && args.ln.mode == 0 && rows_mfma_shape_ok(M, K, n_problems, problems)) {
+  if (few_rows) {
+    for (int i = 0; i < n_problems; ++i)
+      RWKV_REQUIRE(with_ln ? problems[i].mu != nullptr : problems[i].x != nullptr, "linear: NULL tensor");
     int df = RWKV_FMT_F16;
     for (int i = 0; i < n_problems; ++i) df = problems[i].fmt == RWKV_FMT_W8 ? RWKV_FMT_W8 : df;
     return launch_rows_mfma_any(st, args, M, df);

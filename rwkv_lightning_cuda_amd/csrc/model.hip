@@ -265,6 +265,8 @@ int ensure_arena(rwkv_hip_session* s, int B, int T) {
     ws = std::max(ws, linear_packed_workspace_bytes(R, m->F, m->C));
     ws = std::max(ws, linear_packed_workspace_bytes(R, m->C, m->F));
     ws = std::max(ws, linear_packed_workspace_bytes(B, m->V, m->C));
+    // (the column slices of ffn.value on the few-row launch: F / C planes of fp32 partial sums)
+    if (R <= kFewRowsMax && m->F % m->C == 0) ws = std::max(ws, static_cast<size_t>(m->F / m->C) * R * m->C * sizeof(float));
     if (ws > s->gemm_ws_bytes) {
       for (auto& g : s->graphs) {
         if (g.exec) (void)hipGraphExecDestroy(g.exec);
@@ -318,6 +320,29 @@ int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int
     RWKV_HIP_TRY(hipMemcpyAsync(copy->dst, copy->src, sizeof(half_t) * copy->n, hipMemcpyDeviceToDevice, s->stream));
   }
   return linear_any_m(s->stream, mat.fmt, M, N, K, x, mat.data, mat.scale, mat.zp, epilogue, out_f32, y);
+}
+
+// ffn.value of 5 to 16 rows on the few-row launch: F / C column slices of C values each, whose partial sums the
+// LayerNorm kernel that consumes the result adds up and scales (7.2B shape, 8 rows: 19.4 us for the packed product).
+bool sliced_value_ok(const rwkv_hip_session* s, const Matrix& mv, int rows) {
+  const rwkv_hip_model* m = s->model;
+  static const bool off = getenv("RWKV_SLICED_VALUE") && atoi(getenv("RWKV_SLICED_VALUE")) == 0;  // tuning hook
+  return !off && rows >= 5 && rows <= kFewRowsMax && m->F % m->C == 0 && m->F / m->C <= kMaxProblems &&
+         (mv.fmt == RWKV_FMT_W8 || mv.fmt == RWKV_FMT_F16) && linear_rows_mfma_supported(mv.fmt, m->C, m->C) &&
+         s->gemm_ws_bytes >= static_cast<size_t>(m->F / m->C) * rows * m->C * sizeof(float);
+}
+
+int sliced_value(const rwkv_hip_session* s, const Matrix& mv, int rows, const half_t* act, DeferredReduce* defer,
+                 const RowCopy* copy = nullptr) {
+  const rwkv_hip_model* m = s->model;
+  float* ws = static_cast<float*>(s->gemm_ws);
+  const int rc = linear_rows_mfma_sliced(s->stream, mv.fmt, rows, m->C, m->F, m->C, act, mv.data, ws, copy);
+  if (rc != RWKV_OK) return rc;
+  defer->partial = ws;
+  defer->scale = mv.fmt == RWKV_FMT_W8 ? mv.scale : nullptr;
+  defer->plane = static_cast<int64_t>(rows) * m->C;
+  defer->splits = m->F / m->C;
+  return RWKV_OK;
 }
 
 void take_deferred(LnArgs& a, const DeferredReduce& d) {
@@ -402,6 +427,12 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace && fused_tmix &&
                             (rows <= linear_ln_prologue_max_rows(C) ||
                              static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152);
+  // 5 to 8 rows on the few-row matrix-core launch: LN2 (+ its token shift) folds into the ffn.key launch.  LN1 stays a
+  // launch of its own there: it sums the split-K partials of the packed ffn.value product, which would otherwise
+  // cost the reduce launch that the folded LayerNorm saves.
+  const bool ln2_in_linear =
+      ln_in_linear || (s->fused_ln != 0 && step && small && !s->trace && rows >= 5 &&
+                       linear_ln_prologue_rows_ok(m->layers[0].m[RWKV_M_FFN_KEY].fmt, rows, F, C));
   // One row: the gate rank-out of the time-mix core (more than half of its bytes) runs in blocks of its own and the
   // output projection's launch applies the gate while it stages x.
   const bool gate_split = fused_tmix && rows == 1 && C <= 4096 && !s->trace;
@@ -662,7 +693,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
     }
 
     // residual add + LN2 + channel-mix token shift
-    if (ln_in_linear) {
+    if (ln2_in_linear) {
       // folded into the ffn.key launch below
     } else if (step) {
       LnArgs a = {};
@@ -692,7 +723,7 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
 
     // channel mix
     DeferredReduce cm_partial;
-    if (ln_in_linear) {
+    if (ln2_in_linear) {
       const Matrix& mk = w.m[RWKV_M_FFN_KEY];
       LinearProblem pk = {mk.data, mk.scale, mk.zp, nullptr, b.act, F, mk.fmt, w.t[RWKV_T_FFN_X_K]};
       LnPrologue ln;
@@ -706,6 +737,11 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       if (sparse_value && mv.sparse_t) {
         TRY_AUX(ffn_sparse_launch(st, mv.fmt, rows, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
                                   &cp, true));
+      } else if (defer_ok && sliced_value_ok(s, mv, rows)) {
+        TRY_PROF(sliced_value(s, mv, rows, b.act, &cm_partial, &cp));
+      } else if (rows > 8 || (mv.packed && rows >= kPackedMinRows)) {
+        // (rows too long for the few-row launches: the packed product, whose first block moves the row too)
+        TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm, defer_ok ? &cm_partial : nullptr, &cp));
       } else {
         LinearProblem pv = {mv.data, mv.scale, mv.zp, b.act, b.cm, C, mv.fmt, nullptr};
         TRY_PROF(linear_small_m(st, rows, F, 1, &pv, RWKV_EPI_NONE, 0, nullptr, &cp));
@@ -718,6 +754,8 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
       if (sparse_value && mv.sparse_t) {
         TRY_AUX(ffn_sparse_launch(st, mv.fmt, rows, C, F, 1, b.act, mv.sparse_t, mv.scale, s->sparse_ws, s->sparse_ws_bytes, b.cm,
                                   nullptr, true));
+      } else if (defer_ok && step && sliced_value_ok(s, mv, rows)) {
+        TRY_PROF(sliced_value(s, mv, rows, b.act, &cm_partial));
       } else {
         TRY_PROF(apply_matrix(s, mv, rows, C, F, b.act, RWKV_EPI_NONE, 0, b.cm, defer_ok ? &cm_partial : nullptr));
       }

@@ -21,6 +21,12 @@ struct LinearProblem {
   // (the gate of the time-mix output, whose rank-out runs beside the heads' blocks instead of inside them).
   const float* x_f32 = nullptr;
   const half_t* x_gate = nullptr;
+  // The few-row matrix-core launch only: a problem may be a slice of K columns of longer rows - values between the
+  // starts of consecutive rows of W (ldw) and of x (ldx), 0 = K - and may leave its unscaled fp32 sums in y
+  // (raw_f32: one of several slices' partial products, for a consumer that adds them up and scales).
+  int ldw = 0;
+  int ldx = 0;
+  int raw_f32 = 0;
 };
 
 // LayerNorm + token-shift prologue of a small-M linear launch (decode steps): every block recomputes, for each
@@ -57,8 +63,15 @@ int linear_small_m(hipStream_t st, int M, int K, int n_problems, const LinearPro
                    int out_f32, const LnPrologue* ln = nullptr, const RowCopy* copy = nullptr);
 // Whether 5..16 rows of this format and shape run on the few-row matrix-core launch (weights in their plain order).
 bool linear_rows_mfma_supported(int fmt, int N, int K);
-// Rows of a decode step that linear_small_m takes with the LayerNorm prologue at this row length (0: none).
+// y = x W^T for rows of W longer than that launch takes (K a multiple of `slice`, a supported row length): one launch
+// over K / slice column slices, whose fp32 partial sums [K / slice][M][N] go to `partial` for the consumer to add
+// and scale (DeferredReduce).  M in 5..16.
+int linear_rows_mfma_sliced(hipStream_t st, int fmt, int M, int N, int K, int slice, const half_t* x, const void* w,
+                            float* partial, const RowCopy* copy = nullptr);
+// Rows of a decode step that linear_small_m takes with the LayerNorm prologue at this row length (0: none): through
+// the GEMV; and whether M rows of a format and shape go with it at all (the few-row matrix-core launch takes 5..8).
 int linear_ln_prologue_max_rows(int K);
+bool linear_ln_prologue_rows_ok(int fmt, int M, int N, int K);
 // Any M: MFMA tiles for M >= 16 where supported, else row tiles through the GEMV kernel.
 int linear_any_m(hipStream_t st, int fmt, int M, int N, int K, const half_t* x, const void* w, const half_t* scale,
                  const uint8_t* zp, int epilogue, int out_f32, void* y);

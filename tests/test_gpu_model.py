@@ -798,6 +798,45 @@ def test_decode_step_with_layernorm_folded_into_linear_matches_the_unfused_step(
     sess.close()
 
 
+@pytest.mark.parametrize("B,C", [(5, 1024), (8, 1024), (7, 2048), (8, 4096)])
+def test_decode_step_of_five_to_eight_rows_folds_layernorm_into_the_few_row_launch(gpu, B, C):
+    """Decode steps of 5 to 8 rows run their int8 and fp16 products with rows of 1024 .. 4096 values on the few-row
+    matrix-core launch, and by default fold LN2 + its token shift into the ffn.key launch: a staging wavefront per row
+    computes LayerNorm with the stand-alone kernel's formulas and rounding points (sums associated differently), so
+    the step agrees with the one through the stand-alone kernels to fp16 rounding (logits and shift rows within 2e-3
+    of their scale, WKV state within 1e-3).  The same bars with LN1 folded as well (forced: the r/k/v launch, with
+    layer 0 gathering its embedding rows itself; the ffn.value product is then reduced by a launch of its own
+    instead of by the LayerNorm kernel)."""
+    from rwkv_lightning_cuda_amd.model import HipModel, ModelDims, Session, State, synth_weights
+    hip = gpu
+    dims = ModelDims(L=2, C=C, H=C // 64, F=4 * C, V=512, Rw=32, Ra=32, Rg=64, Rv=32)
+    gmodel = HipModel.from_host_weights(dims, synth_weights(dims, 19), hip.FMT_W8)
+    rng = np.random.default_rng(B)
+    prompt = rng.integers(0, dims.V, (B, 3))
+    sess = Session(gmodel)
+    sess.set_graph(False)
+    states = [State(dims, B) for _ in range(3)]
+    logits = [hip.DeviceArray((B, dims.V), np.float32) for _ in range(3)]
+    for st, lg in zip(states, logits):
+        sess.forward(prompt, st, lg)
+    for step in range(3):
+        tok = rng.integers(0, dims.V, (B, 1))
+        for mode, st, lg in zip((None, False, True), states, logits):
+            sess.set_fused_ln(mode)
+            sess.forward(tok, st, lg)
+        for name, i in (("LN2 folded", 0), ("both folded", 2)):
+            if i == 2 and B * C * 2 + C * 4 > 49152:  # (rows that the session folds LN1 for when asked to)
+                continue
+            err = rel_err(logits[i].numpy(), logits[1].numpy())
+            assert err <= 2e-3, "%s: logits at step %d" % (name, step)
+            err = rel_err(states[i].shift.numpy().astype(np.float32), states[1].shift.numpy().astype(np.float32))
+            assert err <= 2e-3, "%s: shift state at step %d" % (name, step)
+            err = rel_err(states[i].wkv.numpy(), states[1].wkv.numpy())
+            assert err <= 1e-3, "%s: wkv state at step %d" % (name, step)
+    assert states[0].elapsed.numpy().tolist() == [6] * B
+    sess.close()
+
+
 @pytest.mark.parametrize("B", [4, 8, 16, 12])
 def test_decode_time_mix_core_with_several_batch_rows_per_block(gpu, B):
     """The single-launch time-mix core of a decode step serves 1, 2 or 4 batch rows of a head per block (the head's
