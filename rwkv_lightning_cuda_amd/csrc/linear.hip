@@ -236,15 +236,23 @@ __device__ __forceinline__ float w4_slice_sum(uint4_t v) {
   return s;
 }
 
+// (v & 0x03c003c0) | 0x4c004c00 as one v_bfi_b32 - the mask picks v's bits, the rest comes from the constant; the
+// compiler emits the and and the or apart (v_and_or_b32 takes no two literals on this target)
+__device__ __forceinline__ uint32_t w4_mask_or(uint32_t v) {
+  uint32_t d;
+  asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "s"(0x03c003c0u), "v"(v), "v"(0x4c004c00u));
+  return d;
+}
+
 // sum_k (16 + code_k) x_k over a lane's 32 codes; xp[4i + j] holds (x_{8i+j}, x_{8i+j+4})
 __device__ __forceinline__ float w4_dot_offset16(const uint4_t& wv, const half2_t* xp, float acc) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const uint32_t d = wv[i];
-    const uint32_t p0 = ((d << 6) & 0x03c003c0u) | 0x4c004c00u;
-    const uint32_t p1 = ((d << 2) & 0x03c003c0u) | 0x4c004c00u;
-    const uint32_t p2 = ((d >> 2) & 0x03c003c0u) | 0x4c004c00u;
-    const uint32_t p3 = ((d >> 6) & 0x03c003c0u) | 0x4c004c00u;
+    const uint32_t p0 = w4_mask_or(d << 6);
+    const uint32_t p1 = w4_mask_or(d << 2);
+    const uint32_t p2 = w4_mask_or(d >> 2);
+    const uint32_t p3 = w4_mask_or(d >> 6);
     acc = dot2(as_half2(p0), xp[4 * i + 0], acc);
     acc = dot2(as_half2(p1), xp[4 * i + 1], acc);
     acc = dot2(as_half2(p2), xp[4 * i + 2], acc);

@@ -327,7 +327,8 @@ int apply_matrix(const rwkv_hip_session* s, const Matrix& mat, int M, int N, int
 bool sliced_value_ok(const rwkv_hip_session* s, const Matrix& mv, int rows) {
   const rwkv_hip_model* m = s->model;
   static const bool off = getenv("RWKV_SLICED_VALUE") && atoi(getenv("RWKV_SLICED_VALUE")) == 0;  // tuning hook
-  return !off && rows >= 5 && rows <= kFewRowsMax && m->F % m->C == 0 && m->F / m->C <= kMaxProblems &&
+  static const int min_rows = getenv("RWKV_ROWS_MFMA_MIN") ? atoi(getenv("RWKV_ROWS_MFMA_MIN")) : 5;  // tuning hook
+  return !off && rows >= min_rows && rows <= kFewRowsMax && m->F % m->C == 0 && m->F / m->C <= kMaxProblems &&
          (mv.fmt == RWKV_FMT_W8 || mv.fmt == RWKV_FMT_F16) && linear_rows_mfma_supported(mv.fmt, m->C, m->C) &&
          s->gemm_ws_bytes >= static_cast<size_t>(m->F / m->C) * rows * m->C * sizeof(float);
 }
