@@ -1187,15 +1187,15 @@ static int launch_row1_any(hipStream_t st, LinearArgs& args, int df) {
 // read then hit different banks); lanes whose column is no row of x read row 0 and their products are dropped.
 // int8 codes become fp16 (exact) on the way, the row scale multiplies the sum.
 //
-// Up to 8 rows of x the wavefronts share the start of the launch like those of the GEMV with the LayerNorm prologue:
-// the first half brings x into LDS (and requests its weights afterwards), the second half requests its weights at
-// once; they meet at a counter in LDS, not at a barrier - a barrier counts every wavefront, and a wavefront reaches
-// it only when the memory pipeline has taken all its requests.  With 9..16 rows (twice the registers for x) every
-// wavefront stages its share of x first and requests its weights after the barrier.
+// The wavefronts share the start of the launch like those of the GEMV with the LayerNorm prologue: the first half
+// brings x into LDS (8 or, for 9..16 rows of 4096 values, 16 vectors per thread) and requests its weights
+// afterwards, the second half requests its weights at once; they meet at a counter in LDS, not at a barrier - a
+// barrier counts every wavefront, and a wavefront reaches it only when the memory pipeline has taken all its
+// requests.
 constexpr int kRowsMfmaMax = 16;
 constexpr int kRowsMfmaMin = 5;
 constexpr int kRowsMfmaThreads = 1024;
-constexpr int kRowsMfmaXVecs = 8;  // 16-byte vectors of x per staging thread
+constexpr int kRowsMfmaXVecs = 8;  // 16-byte vectors of x per staging thread (twice as many for 9..16 rows of 4096)
 
 // LayerNorm(x + res) (or of a gathered table row) + token-shift lerp of up to 8 rows straight into the block's LDS
 // copy of x, by the staging wavefronts of a few-row matrix-core block: wavefront m owns row m (lane l the 8-value
@@ -1328,10 +1328,9 @@ __device__ __forceinline__ void rows_mfma_ln_prologue(const LnPrologue& ln, cons
 // format fit one batch (7.2B shape, r/k/v with the fp16 rank-ins riding along).
 constexpr int rows_mfma_groups_f16(int g) { return g >= 2 ? g / 2 : g; }
 
-template <int FMT, int NB, int G, bool SPLIT, bool LN>
+template <int FMT, int NB, int G, bool LN, int XV>
 __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const LinearProblem& prob, int blk, int M,
                                                 half_t* xs, int xstride, float* part, LnFlags* flags) {
-  static_assert(SPLIT || !LN, "the prologue belongs to the staging half of the wavefronts");
   unsigned* flag = &flags->count[kLnFlagX];
   constexpr int EB = FMT == RWKV_FMT_F16 ? 2 : 1;    // bytes per weight
   constexpr int KV = 16 / EB;                         // weights per 16-byte vector
@@ -1380,11 +1379,11 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
   // x of this problem: M rows of K / 8 vectors (the rows ldx values apart)
   const int kv = K >> 3;
   const int64_t ldx = prob.ldx ? prob.ldx : K;
-  constexpr int NTS = SPLIT ? kRowsMfmaThreads / 2 : kRowsMfmaThreads;  // staging threads
+  constexpr int NTS = kRowsMfmaThreads / 2;  // staging threads: the first half of the wavefronts
   auto stage_x = [&]() {
-    uint4_t xv[kRowsMfmaXVecs];
+    uint4_t xv[XV];
 #pragma unroll
-    for (int j = 0; j < kRowsMfmaXVecs; ++j) {
+    for (int j = 0; j < XV; ++j) {
       const int i = threadIdx.x + j * NTS;
       xv[j] = uint4_t{0u, 0u, 0u, 0u};
       if (i < M * kv) {
@@ -1393,14 +1392,12 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (SPLIT) {
-      // x is in the memory pipeline ahead of any weights of this block
-      if (threadIdx.x <= kLnFlagX) flags->count[threadIdx.x] = 0u;
-      __syncthreads();
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    // x is in the memory pipeline ahead of any weights of this block
+    if (threadIdx.x <= kLnFlagX) flags->count[threadIdx.x] = 0u;
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < kRowsMfmaXVecs; ++j) {
+    for (int j = 0; j < XV; ++j) {
       const int i = threadIdx.x + j * NTS;
       if (i < M * kv) {
         const int m = i / kv, c = (i - m * kv) * 8;
@@ -1408,31 +1405,24 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
       }
     }
   };
-  if constexpr (SPLIT) {
-    constexpr unsigned NWS = NTS / 64;
-    if (wave < static_cast<int>(NWS)) {
-      if constexpr (LN) {
-        half_t* hst = reinterpret_cast<half_t*>(part + 16 * 256);
-        rows_mfma_ln_prologue(args.ln, prob.mu, K, M, xs, xstride, hst, flags, blockIdx.x == 0);
-      } else {
-        stage_x();
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      ln_flag_arrive(flag);
-      request(0);
-      __builtin_amdgcn_sched_barrier(0);
-      ln_flag_wait(flag, NWS);
+  constexpr unsigned NWS = NTS / 64;
+  if (wave < static_cast<int>(NWS)) {
+    if constexpr (LN) {
+      half_t* hst = reinterpret_cast<half_t*>(part + 16 * 256);
+      rows_mfma_ln_prologue(args.ln, prob.mu, K, M, xs, xstride, hst, flags, blockIdx.x == 0);
     } else {
-      __syncthreads();
-      request(0);
-      __builtin_amdgcn_sched_barrier(0);
-      ln_flag_wait(flag, NWS);
+      stage_x();
     }
-  } else {
-    stage_x();
-    __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
+    ln_flag_arrive(flag);
     request(0);
+    __builtin_amdgcn_sched_barrier(0);
+    ln_flag_wait(flag, NWS);
+  } else {
+    __syncthreads();
+    request(0);
+    __builtin_amdgcn_sched_barrier(0);
+    ln_flag_wait(flag, NWS);
   }
   __builtin_amdgcn_sched_barrier(0);
   products(0);
@@ -1481,7 +1471,7 @@ __device__ __forceinline__ void rows_mfma_block(const LinearArgs& args, const Li
 // LayerNorm prologue also 3 x K fp16 values (LN weight, bias, lerp coefficients).  One block per CU
 // (1024 threads, up to 128 registers).  DF: format of the quantised problems (int8); fp16 problems may ride along
 // (twice the steps, in batches of the same size).
-template <int DF, int NB, int G, bool SPLIT, bool LN>
+template <int DF, int NB, int G, bool LN, int XV>
 __global__ __launch_bounds__(kRowsMfmaThreads)
 void linear_rows_mfma_kernel(LinearArgs args, int M) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -1504,9 +1494,9 @@ void linear_rows_mfma_kernel(LinearArgs args, int M) {
   const LinearProblem prob = args.p[pi];
   const int blk = blockIdx.x - first;
   if (DF != RWKV_FMT_F16 && prob.fmt == DF) {  // uniform per block
-    rows_mfma_block<DF, NB, G, SPLIT, LN>(args, prob, blk, M, xs, xstride, part, &flags);
+    rows_mfma_block<DF, NB, G, LN, XV>(args, prob, blk, M, xs, xstride, part, &flags);
   } else {
-    rows_mfma_block<RWKV_FMT_F16, NB, rows_mfma_groups_f16(G), SPLIT, LN>(args, prob, blk, M, xs, xstride, part, &flags);
+    rows_mfma_block<RWKV_FMT_F16, NB, rows_mfma_groups_f16(G), LN, XV>(args, prob, blk, M, xs, xstride, part, &flags);
   }
 }
 
@@ -1535,7 +1525,7 @@ bool linear_rows_mfma_supported(int fmt, int N, int K) {
   return rows_mfma_shape_ok(kRowsMfmaMin, K, 1, &p);
 }
 
-template <int DF, int NB, int G, bool SPLIT, bool LN>
+template <int DF, int NB, int G, bool LN, int XV>
 static int launch_rows_mfma(hipStream_t st, LinearArgs& args, int M) {
   int total = 0;
   for (int i = 0; i < args.n_problems; ++i) {
@@ -1549,28 +1539,28 @@ static int launch_rows_mfma(hipStream_t st, LinearArgs& args, int M) {
     if (!raised) {
       const size_t most = static_cast<size_t>(LN ? kRowsMfmaLnRows : kRowsMfmaMax) * (4096 + 8) * sizeof(half_t) +
                           16 * 256 * sizeof(float) + (LN ? static_cast<size_t>(3) * 4096 * sizeof(half_t) : 0);
-      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_rows_mfma_kernel<DF, NB, G, SPLIT, LN>),
+      RWKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_rows_mfma_kernel<DF, NB, G, LN, XV>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(most)));
       raised = true;
     }
   }
-  hipLaunchKernelGGL((linear_rows_mfma_kernel<DF, NB, G, SPLIT, LN>), dim3(total), dim3(kRowsMfmaThreads), lds, st, args, M);
+  hipLaunchKernelGGL((linear_rows_mfma_kernel<DF, NB, G, LN, XV>), dim3(total), dim3(kRowsMfmaThreads), lds, st, args, M);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
 
 // Vectors per batch (NB) by shape: a wavefront has K * G / 1024 vectors of int8 codes to request (as many of fp16
 // weights with half the groups per block, twice as many with one group) and takes them in batches of up to 16.
-template <int DF, int G, bool SPLIT, bool LN>
+template <int DF, int G, bool LN, int XV>
 static int launch_rows_mfma_g(hipStream_t st, LinearArgs& args, int M) {
   const int steps = args.K * G / 1024;
   if constexpr (G == 4) {
-    if (steps % 16 == 0) return launch_rows_mfma<DF, 16, G, SPLIT, LN>(st, args, M);
-    if (steps % 8 == 0) return launch_rows_mfma<DF, 8, G, SPLIT, LN>(st, args, M);
+    if (steps % 16 == 0) return launch_rows_mfma<DF, 16, G, LN, XV>(st, args, M);
+    if (steps % 8 == 0) return launch_rows_mfma<DF, 8, G, LN, XV>(st, args, M);
   }
-  if (steps % 4 == 0) return launch_rows_mfma<DF, 4, G, SPLIT, LN>(st, args, M);
-  if (steps % 2 == 0) return launch_rows_mfma<DF, 2, G, SPLIT, LN>(st, args, M);
-  return launch_rows_mfma<DF, 1, G, SPLIT, LN>(st, args, M);
+  if (steps % 4 == 0) return launch_rows_mfma<DF, 4, G, LN, XV>(st, args, M);
+  if (steps % 2 == 0) return launch_rows_mfma<DF, 2, G, LN, XV>(st, args, M);
+  return launch_rows_mfma<DF, 1, G, LN, XV>(st, args, M);
 }
 
 template <int DF>
@@ -1580,15 +1570,16 @@ static int launch_rows_mfma_fmt(hipStream_t st, LinearArgs& args, int M) {
   for (int i = 0; i < args.n_problems; ++i)
     blocks4 += ceil_div(args.p[i].N, 16 * (args.p[i].fmt == RWKV_FMT_F16 ? rows_mfma_groups_f16(4) : 4));
   const bool g4 = blocks4 * 4 >= device_cu_count() * 3;
+  constexpr int XV = kRowsMfmaXVecs;
   if (args.ln.mode != 0) {
-    return g4 ? launch_rows_mfma_g<DF, 4, true, true>(st, args, M) : launch_rows_mfma_g<DF, 1, true, true>(st, args, M);
+    return g4 ? launch_rows_mfma_g<DF, 4, true, XV>(st, args, M) : launch_rows_mfma_g<DF, 1, true, XV>(st, args, M);
   }
-  // the first half of the wavefronts stages x if eight vectors per thread cover it
-  const bool split = M * (args.K / 8) <= kRowsMfmaXVecs * (kRowsMfmaThreads / 2);
-  if (g4) {
-    return split ? launch_rows_mfma_g<DF, 4, true, false>(st, args, M) : launch_rows_mfma_g<DF, 4, false, false>(st, args, M);
+  // the first half of the wavefronts stages x: eight vectors per thread cover 8 rows of 4096 values, sixteen all 16
+  // (16 rows, 7.2B shape: 3.05 -> 2.85 ms per step against every wavefront staging its share before any request)
+  if (M * (args.K / 8) <= XV * (kRowsMfmaThreads / 2)) {
+    return g4 ? launch_rows_mfma_g<DF, 4, false, XV>(st, args, M) : launch_rows_mfma_g<DF, 1, false, XV>(st, args, M);
   }
-  return split ? launch_rows_mfma_g<DF, 1, true, false>(st, args, M) : launch_rows_mfma_g<DF, 1, false, false>(st, args, M);
+  return g4 ? launch_rows_mfma_g<DF, 4, false, 2 * XV>(st, args, M) : launch_rows_mfma_g<DF, 1, false, 2 * XV>(st, args, M);
 }
 
 static int launch_rows_mfma_any(hipStream_t st, LinearArgs& args, int M, int df) {
