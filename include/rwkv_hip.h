@@ -139,8 +139,10 @@ int rwkv_hip_fill_normal_f16(rwkv_stream_t s, int64_t n, uint64_t seed, float me
 /* ---- linear layers, y[M,N] = x[M,K] . W[N,K]^T, fp32 accumulate.
  * Replaces rwkv7_v3a_linear_orig_rows_exact_f16_launch / _orig_rows_f16_launch / _f16_orig_launch /
  * _f16_orig_lt_cfg_launch (cuda/rwkv7_fast_v4_kernels.cuh:155-177) and the dispatch in
- * linear_orig_layout_launch (src/rwkv7_fast_v4.cu:709-959).  Any M: small M streams the weights
- * once through a GEMV kernel, M >= 16 uses MFMA tiles.
+ * linear_orig_layout_launch (src/rwkv7_fast_v4.cu:709-959).  Any M: up to 4 rows stream the weights
+ * once through a GEMV kernel that keeps whole weight rows in flight; 5 to 16 rows of int8 / fp16
+ * weights with K a multiple of 1024 up to 4096 stream them the same way with the products on the
+ * matrix core; otherwise up to 8 rows per pass of a GEMV with K tiles, and from 16 rows MFMA tiles.
  * out_f32 == 0: y is f16 [M,N].  out_f32 == 1: y is f32 [M,N] holding the f16-rounded value
  * (the lm_head path, src/rwkv7_fast_v4.cu:1325-1341 + rwkv7_v4_f16_to_f32_launch).
  * epilogue RWKV_EPI_RELU_SQUARE applies relu(.)^2 to the f16-rounded result and rounds again
