@@ -354,13 +354,14 @@ int rwkv_hip_session_set_sparse_ffn(rwkv_hip_session* s, int max_rows);
  * longer ones round w12 + w0 to fp16 first).  Default off: fp32 state.  A state belongs to one mode. */
 int rwkv_hip_session_set_wkv_fp16(rwkv_hip_session* s, int on);
 /* Decode steps on the GEMV path can fold the two LayerNorm + token-shift kernels of a layer into the prologue of
- * the linear launches that consume them.  on > 0: always (where the rows fit), 0: never, < 0 (the default): for one
- * or two rows of at most 4096 channels.  Those go through a kernel that requests whole weight rows up front and
- * normalises while they are in flight (two launches fewer per layer: 7.2B shape, one row 2.04 -> 1.92 ms per step,
- * 0.1B shape 0.413 -> 0.373; same formulas and rounding points as the stand-alone kernels, sums associated
- * differently); more rows, when forced, through a prologue that is bitwise the stand-alone kernels but slower than
- * them from 2048 channels on.  No counterpart in the reference (its fused decode kernels are
- * cuda/rwkv7_v3a_ops.cu:1637-1798). */
+ * the linear launches that consume them.  on > 0: always (where a launch with a prologue takes the rows), 0: never,
+ * < 0 (the default): both LayerNorms for one or two rows of at most 4096 channels, LN2 for 5 to 8 rows of int8 / fp16
+ * weights with 1024 .. 4096 channels (the few-row matrix-core launch).  One and two rows go through a kernel that
+ * requests whole weight rows up front and normalises while they are in flight (two launches fewer per layer: 7.2B
+ * shape, one row 2.04 -> 1.92 ms per step, 0.1B shape 0.413 -> 0.373; same formulas and rounding points as the
+ * stand-alone kernels, sums associated differently); 3 to 8 rows of other shapes, when forced, through a prologue
+ * that is bitwise the stand-alone kernels but slower than them from 2048 channels on.  No counterpart in the
+ * reference (its fused decode kernels are cuda/rwkv7_v3a_ops.cu:1637-1798). */
 int rwkv_hip_session_set_fused_ln(rwkv_hip_session* s, int on);
 /* Decode steps run everything between the r/k/v projections and the output projection as one launch per layer, one
  * block per head and 1, 2 or 4 batch rows (the head's LoRA rows are loaded once per block), up to 8 rows and while

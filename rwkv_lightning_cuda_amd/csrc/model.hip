@@ -425,9 +425,13 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
   // channels.  The residual-stream tap needs the stand-alone kernels.
   const bool want_ln_in_linear = s->fused_ln > 0 || (s->fused_ln < 0 && rows <= linear_ln_prologue_max_rows(C));
   // (the shift row that the prologue leaves for later is stored by the single-launch time-mix core)
+  // (forced on, it also takes the rows that a launch with a prologue exists for: 5 to 8 on the few-row matrix-core
+  // launch, up to 8 through the tiled GEMV while the rows fit its LDS)
   const bool ln_in_linear = want_ln_in_linear && step && small && !s->trace && fused_tmix &&
                             (rows <= linear_ln_prologue_max_rows(C) ||
-                             static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152);
+                             (linear_ln_prologue_rows_ok(m->layers[0].m[RWKV_M_ATT_R].fmt, rows, C, C) &&
+                              linear_ln_prologue_rows_ok(m->layers[0].m[RWKV_M_FFN_KEY].fmt, rows, F, C)) ||
+                             (rows <= 8 && static_cast<size_t>(rows) * C * 2 + static_cast<size_t>(C) * 4 <= 49152));
   // 5 to 8 rows on the few-row matrix-core launch: LN2 (+ its token shift) folds into the ffn.key launch.  LN1 stays a
   // launch of its own there: it sums the split-K partials of the packed ffn.value product, which would otherwise
   // cost the reduce launch that the folded LayerNorm saves.
