@@ -177,11 +177,11 @@ def parity_legs(hip, fmt_name, with_others):
         d = PRESETS[preset]
         return ModelDims(L=layers, C=d.C, H=d.H, F=d.F, V=d.V, Rw=d.Rw, Ra=d.Ra, Rg=d.Rg, Rv=d.Rv)
 
-    def leg(dims, weights, fmt_key, prompt_len, steps, what):
-        prompt = np.random.default_rng(89).integers(0, dims.V, (1, prompt_len))
+    def leg(dims, weights, fmt_key, prompt_len, steps, what, rows=1):
+        prompt = np.random.default_rng(89).integers(0, dims.V, (rows, prompt_len))
         res = greedy_parity(hip, oracle, dims, weights, fmts[fmt_key], prompt, steps, control=True)
-        res["workload"] = "%s, %s weights: %d-token prompt, then %d greedy steps at batch 1, all %d logits of every step " \
-                          "against the CPU oracle" % (what, fmt_key, prompt_len, steps, dims.V)
+        res["workload"] = "%s, %s weights: %d-token prompt, then %d greedy steps at batch %d, all %d logits of every step " \
+                          "and row against the CPU oracle" % (what, fmt_key, prompt_len, steps, rows, dims.V)
         return res
 
     d8 = sliced("7.2B", 8)
@@ -192,6 +192,14 @@ def parity_legs(hip, fmt_name, with_others):
     if with_others:
         if fmt_name == "w8":
             others["w4_parity"] = leg(d8, w8, "w4", 8, 16, what)
+            # the few-row launches of 5 to 16 rows (products on the matrix core, LN2 folded into ffn.key, ffn.value in
+            # column slices) and of 2 to 4 rows (the GEMV with several rows of x, one walk of ffn.value)
+            d2l = sliced("7.2B", 2)
+            w2l = synth_weights(d2l, 90)
+            two = "7.2B shape, 2 of 32 layers (C 4096, full 65536-row head)"
+            others["bs8_parity"] = leg(d2l, w2l, "w8", 4, 6, two, rows=8)
+            others["bs3_parity"] = leg(d2l, w2l, "w8", 4, 6, two, rows=3)
+            del w2l
         del w8
         d1 = PRESETS["0.1B"]
         others["cfg1_0p1b_f16_parity"] = leg(d1, synth_weights(d1, 12), "f16", 128, 32, "0.1B shape, all 12 layers")
