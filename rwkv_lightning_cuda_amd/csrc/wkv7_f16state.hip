@@ -25,98 +25,262 @@ namespace rwkv {
 namespace {
 
 constexpr int kPairs = kPairs16;
-constexpr int kAhead = 4;  // tokens whose operands are in flight
+constexpr int kAhead = 4;  // tokens whose operands are in flight from memory
+constexpr int kRing = 4;   // tokens whose operands have a place in LDS
 
 struct TokenOps {  // one token's per-column operands in LDS
   half_t a[kHead], b[kHead], k[kHead], wd[kHead], r[kHead];
   half_t v[kHead];  // per state row, not per column: parked here between its arrival and its step
 };
 
-__global__ __launch_bounds__(kWave) void wkv7_f16state_kernel(int T, int C, int H, half_t* __restrict__ state,
-                                                              const half_t* __restrict__ r, const half_t* __restrict__ w,
-                                                              const half_t* __restrict__ w0, const half_t* __restrict__ k,
-                                                              const half_t* __restrict__ v, const half_t* __restrict__ a,
-                                                              const half_t* __restrict__ b, half_t* __restrict__ y,
-                                                              const int* __restrict__ elapsed) {
-  __shared__ __align__(16) TokenOps ops[2];
+// The block's two wavefronts meet once per token.  LDS only: what either has in flight to or from memory (the
+// feeder's loads of later tokens, the other's stores of y) does not have to land first.
+__device__ __forceinline__ void token_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Lanes in groups of LPR (2 or 4): every lane takes the value of its left neighbour in the group (the first keeps
+// its own) / of the group's last lane.  DPP quad_perm, two bits per lane of a quad.
+template <int LPR>
+__device__ __forceinline__ half2_t group_from_left(half2_t x) {
+  constexpr int kCtrl = LPR == 4 ? (0 | 0 << 2 | 1 << 4 | 2 << 6) : (0 | 0 << 2 | 2 << 4 | 2 << 6);
+  const int xi = __builtin_bit_cast(int, x);  // (also as the value of disabled lanes - there are none - so that none is made up)
+  return __builtin_bit_cast(half2_t, __builtin_amdgcn_update_dpp(xi, xi, kCtrl, 0xf, 0xf, false));
+}
+template <int LPR>
+__device__ __forceinline__ half2_t group_from_last(half2_t x) {
+  constexpr int kCtrl = LPR == 4 ? (3 | 3 << 2 | 3 << 4 | 3 << 6) : (1 | 1 << 2 | 3 << 4 | 3 << 6);
+  const int xi = __builtin_bit_cast(int, x);
+  return __builtin_bit_cast(half2_t, __builtin_amdgcn_update_dpp(xi, xi, kCtrl, 0xf, 0xf, false));
+}
+
+// LPR + 1 wavefronts per (batch row, head); LPR = lanes per state row, 1, 2 or 4.
+//
+// A wavefront that is alone on its SIMD issues one instruction every four cycles whatever the instruction is, so
+// everything that is not the recurrence itself is taken off the wavefronts that own the state: the last wavefront
+// (the feeder) fetches the operands of token t + 2 + kAhead, converts the decay logit of token t + 2 and drops that
+// token's operands into a ring of kRing LDS buffers while the others run token t from the ring.
+//
+// LPR = 1: one wavefront owns the head, lane = state row (32 pairs): 160 packed FMAs, 40 16-byte LDS broadcasts and
+// one store per token.  LPR = 4 (while the grid leaves SIMDs idle): four wavefronts own sixteen rows each, and four
+// neighbouring lanes share a row, sixteen columns each.  The two chains still run over the pairs in order - all
+// lanes run every quarter of a chain on their own columns, the running value moves one lane to the right between
+// the quarters (DPP), and only what has come through lanes 0, 1, 2, 3 in turn is used, so every sum sees the same
+// operations in the same order - but the update, the LDS reads and the registers per lane are a quarter: a token
+// costs a wavefront 64 + 24 packed FMAs instead of 160.  LPR = 2 likewise with halves (64 + 48).  (The four
+// wavefronts together issue twice the instructions of the one: where every SIMD has a head of its own, LPR = 1 is
+// the faster one.)
+template <int LPR>
+__global__ __launch_bounds__((LPR + 1) * kWave) void wkv7_f16state_kernel(int T, int C, int H, half_t* __restrict__ state,
+                                                                          const half_t* __restrict__ r, const half_t* __restrict__ w,
+                                                                          const half_t* __restrict__ w0, const half_t* __restrict__ k,
+                                                                          const half_t* __restrict__ v, const half_t* __restrict__ a,
+                                                                          const half_t* __restrict__ b, half_t* __restrict__ y,
+                                                                          const int* __restrict__ elapsed) {
+  static_assert(LPR == 1 || LPR == 2 || LPR == 4, "lanes per state row: 1, 2 or 4");
+  constexpr int NP = kPairs / LPR;  // pairs of a row per lane
+  __shared__ __align__(16) TokenOps ops[kRing];
   const int bh = blockIdx.x;
   const int bi = bh / H;
   const int h = bh - bi * H;
-  const int lane = threadIdx.x;
-  const int c = h * kHead + lane;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  // Element c of token t of this head sits (t * C + c) * 2 bytes behind a base that is the same for the whole
+  // block: one 32-bit offset per token serves all six loads or the store (the launcher checks that it fits).
+  const int64_t head0 = static_cast<int64_t>(bi) * T * C + h * kHead;
+  const unsigned row_bytes = static_cast<unsigned>(C) * 2u;
 
-  // state row `lane`: 128 bytes
-  half_t* srow = state + (static_cast<int64_t>(bh) * kHead + lane) * kHead;
-  half2_t S[kPairs];
+  if (wave == LPR) {  // the feeder: lane = column (and row, for v)
+    const unsigned lane2 = static_cast<unsigned>(lane) * 2u;
+    const int c = h * kHead + lane;
+    const half_t* pr = r + head0;
+    const half_t* pw = w + head0;
+    const half_t* pk = k + head0;
+    const half_t* pv = v + head0;
+    const half_t* pa = a + head0;
+    const half_t* pb = b + head0;
+    const int phase0 = elapsed[bi] + c;
+    // w0 once, not under a branch inside every step (adding 0.0f changes no decay)
+    const float w0f = w0 ? h2f(w0[c]) : 0.0f;
+    auto at = [](const half_t* base, unsigned byte_off) {
+      return *reinterpret_cast<const half_t*>(reinterpret_cast<const char*>(base) + byte_off);
+    };
+    // The elements of kAhead tokens wait in registers (slot = token mod kAhead): requested one token ahead only,
+    // every step would last a whole trip to memory.  Tokens past the end re-read the last one (no load under a
+    // branch) and land in ring places nobody reads any more.
+    half_t qa[kAhead], qb[kAhead], qk[kAhead], qr[kAhead], qw[kAhead], qv[kAhead];
+    auto request = [&](int slot, int t) {
+      const unsigned off = lane2 + static_cast<unsigned>(t < T ? t : T - 1) * row_bytes;
+      qa[slot] = at(pa, off);
+      qb[slot] = at(pb, off);
+      qk[slot] = at(pk, off);
+      qr[slot] = at(pr, off);
+      qw[slot] = at(pw, off);
+      qv[slot] = at(pv, off);
+    };
+    auto place = [&](int slot, int t) {  // token t from its slot into its place in the ring
+      TokenOps& o = ops[t & (kRing - 1)];
+      o.a[lane] = qa[slot];
+      o.b[lane] = qb[slot];
+      o.k[lane] = qk[slot];
+      o.r[lane] = qr[slot];
+      o.wd[lane] = decay_delta16_of(h2f(qw[slot]) + w0f, phase0 + t);
+      o.v[lane] = qv[slot];
+    };
+    request(0, 0);
+    request(1, 1);
+    place(0, 0);
+    place(1, 1);
 #pragma unroll
-  for (int q = 0; q < kPairs / 4; ++q) {
-    const uint4_t t = *reinterpret_cast<const uint4_t*>(srow + 8 * q);
+    for (int u = 0; u < kAhead; ++u) request((2 + u) % kAhead, 2 + u);
+    token_barrier();
+    // step t: token t + 2 into the ring (its place was token t - 2's, which the others left two meetings ago), its
+    // slot requested again for token t + 2 + kAhead
+    auto step = [&](int t, int slot) {
+      place(slot, t + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      request(slot, t + 2 + kAhead);
+      token_barrier();
+    };
+    // whole rounds of kAhead tokens as straight-line code (a loop with an exit between the steps would wait for
+    // every outstanding request at its head), then the rest
+    int t = 0;
+    for (; t + kAhead <= T; t += kAhead) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) S[4 * q + e] = as_half2(t[e]);
+      for (int u = 0; u < kAhead; ++u) step(t + u, (2 + u) % kAhead);
+    }
+#pragma unroll
+    for (int u = 0; u < kAhead - 1; ++u) {
+      if (t + u < T) step(t + u, (2 + u) % kAhead);
+    }
+    return;
   }
 
-  const int phase0 = elapsed[bi] + c;
-  // w0 once, not under a branch inside every step (adding 0.0f changes no decay)
-  const float w0f = w0 ? h2f(w0[c]) : 0.0f;
-  const int64_t tok0 = static_cast<int64_t>(bi) * T * C + c;  // this lane's element of token 0
-  // token 0's operands
-  {
-    ops[0].a[lane] = a[tok0];
-    ops[0].b[lane] = b[tok0];
-    ops[0].k[lane] = k[tok0];
-    ops[0].r[lane] = r[tok0];
-    ops[0].wd[lane] = decay_delta16_of(h2f(w[tok0]) + w0f, phase0);
-  }
-  ops[0].v[lane] = v[tok0];
-  // The elements of tokens t + 1 .. t + kAhead wait in registers (slot = token mod kAhead): requested one token
-  // ahead only, every step would last a whole trip to memory.  Tokens past the end re-read the last one (no load
-  // under a branch).
-  half_t qa[kAhead], qb[kAhead], qk[kAhead], qr[kAhead], qw[kAhead], qv[kAhead];
-  auto request = [&](int slot, int t) {
-    const int64_t i = tok0 + static_cast<int64_t>(t < T ? t : T - 1) * C;
-    qa[slot] = a[i];
-    qb[slot] = b[i];
-    qk[slot] = k[i];
-    qr[slot] = r[i];
-    qw[slot] = w[i];
-    qv[slot] = v[i];
-  };
+  // ---- the wavefronts that own the state: this lane's NP pairs of its row
+  const int row = wave * (kWave / LPR) + lane / LPR;
+  const int col0 = (lane % LPR) * (2 * NP);
+  half_t* srow = state + (static_cast<int64_t>(bh) * kHead + row) * kHead + col0;
+  half_t* py = y + head0;
+  const unsigned row2 = static_cast<unsigned>(row) * 2u;
+  auto read_part = [&](const half_t* vec, half2_t(&dst)[NP]) {  // this lane's columns of a per-column vector
 #pragma unroll
-  for (int u = 1; u <= kAhead; ++u) request(u % kAhead, u);
-  __syncthreads();
-
-  // One token: token t + 1's elements leave their slot for the other buffer first (nobody reads it during this
-  // step), then the slot is requested again for token t + 1 + kAhead - in that order, so that the new request can
-  // take the registers of the old values - and then the state step with the operands in ops[t & 1].
-  auto step = [&](int t, int slot) {
-    const TokenOps& cur = ops[t & 1];
-    TokenOps& nxt = ops[(t + 1) & 1];
-    nxt.a[lane] = qa[slot];
-    nxt.b[lane] = qb[slot];
-    nxt.k[lane] = qk[slot];
-    nxt.r[lane] = qr[slot];
-    nxt.wd[lane] = decay_delta16_of(h2f(qw[slot]) + w0f, phase0 + t + 1);
-    nxt.v[lane] = qv[slot];
-    __builtin_amdgcn_sched_barrier(0);
-    request(slot, t + 1 + kAhead);
-    __builtin_amdgcn_sched_barrier(0);
-    y[tok0 + static_cast<int64_t>(t) * C] = wkv16_row_step(S, cur.a, cur.b, cur.k, cur.wd, cur.r, cur.v[lane]);
-    __syncthreads();
+    for (int q = 0; q < NP / 4; ++q) {
+      const uint4_t t = *reinterpret_cast<const uint4_t*>(vec + col0 + 8 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[4 * q + e] = as_half2(t[e]);
+    }
   };
-  // whole rounds of kAhead tokens as straight-line code (a loop with an exit between the steps would wait for every
-  // outstanding request at its head), then the rest
+  half2_t S[NP];
+  read_part(srow - col0, S);
+  token_barrier();
+
+  // One token, in an order that leaves no packed FMA right behind the one it depends on (the hardware wants an idle
+  // issue slot there, which costs a wavefront as much as an instruction):
+  //   - the chain over a of this token runs interleaved with the chain over r of the token BEFORE (both read the
+  //     state between the two tokens; r of that token stays in registers), whose y is stored one step late;
+  //   - the update runs over eight pairs at a time, one of its three FMAs for all eight before the next.
+  // Every value sees the same operations in the same order as in wkv16_row_step.
+  // Where the LDS reads sit: the first half of b / k / decay delta of token t is requested ahead of the two chains
+  // of step t, the second half, r of token t and a of token t + 1 right after them (r and a into the registers the
+  // chains have just finished with; LPR = 1: a half way through the update, so that the step fits the 256
+  // registers): each is there by the time it is used.
+  half2_t r_prev[NP], a_cur[NP];
+#pragma unroll
+  for (int j = 0; j < NP; ++j) r_prev[j] = half2_t{static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+  read_part(ops[0].a, a_cur);
+  auto step = [&](int t) {
+    const TokenOps& cur = ops[t & (kRing - 1)];
+    const TokenOps& nxt = ops[(t + 1) & (kRing - 1)];
+    const half_t v_cur = cur.v[row];
+    half2_t bv[NP], kv[NP], wv[NP];
+    auto read_bkw = [&](int q) {  // pairs 4q .. 4q + 3 of this lane's b, k and decay delta
+      const uint4_t tb = *reinterpret_cast<const uint4_t*>(cur.b + col0 + 8 * q);
+      const uint4_t tk = *reinterpret_cast<const uint4_t*>(cur.k + col0 + 8 * q);
+      const uint4_t tw = *reinterpret_cast<const uint4_t*>(cur.wd + col0 + 8 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        bv[4 * q + e] = as_half2(tb[e]);
+        kv[4 * q + e] = as_half2(tk[e]);
+        wv[4 * q + e] = as_half2(tw[e]);
+      }
+    };
+#pragma unroll
+    for (int q = 0; q < NP / 8; ++q) read_bkw(q);
+    __builtin_amdgcn_sched_barrier(0);
+    half2_t sa2 = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+    half2_t y2 = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+#pragma unroll
+    for (int part = 0; part < LPR; ++part) {
+      if (part > 0) {  // what the lane to the left has summed over its columns goes on over this lane's
+        sa2 = group_from_left<LPR>(sa2);
+        y2 = group_from_left<LPR>(y2);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int j = 0; j < NP; ++j) {
+        sa2 = pk_fma16(a_cur[j], S[j], sa2);
+        y2 = pk_fma16(S[j], r_prev[j], y2);
+        __builtin_amdgcn_sched_barrier(0);  // (left alone, the compiler may run one chain after the other)
+      }
+    }
+    if constexpr (LPR > 1) {  // the sums over all 64 columns are in the last lane of the four
+      sa2 = group_from_last<LPR>(sa2);
+      y2 = group_from_last<LPR>(y2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = NP / 8; q < NP / 4; ++q) read_bkw(q);
+    read_part(cur.r, r_prev);
+    if constexpr (LPR > 1) read_part(nxt.a, a_cur);
+    // y of token t - 1 (at t = 0: a zero into y of token 0, which the next step overwrites); the lanes that share
+    // a row store the same value
+    *reinterpret_cast<half_t*>(reinterpret_cast<char*>(py) + (row2 + static_cast<unsigned>(t > 0 ? t - 1 : 0) * row_bytes)) =
+        y2[0] + y2[1];
+    const half_t sa = sa2[0] + sa2[1];
+    const half2_t sa_b = {sa, sa};
+    const half2_t vv = {v_cur, v_cur};
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int g = 0; g < NP / 8; ++g) {
+      half2_t u[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) u[e] = pk_fma16(sa_b, bv[8 * g + e], S[8 * g + e]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) u[e] = pk_fma16(kv[8 * g + e], vv, u[e]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) S[8 * g + e] = pk_fma16(S[8 * g + e], wv[8 * g + e], u[e]);
+      if (LPR == 1 && g == 1) read_part(nxt.a, a_cur);  // (registers: half of b / k / decay delta are done with)
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    token_barrier();
+  };
   int t = 0;
   for (; t + kAhead <= T; t += kAhead) {
 #pragma unroll
-    for (int u = 0; u < kAhead; ++u) step(t + u, (u + 1) % kAhead);
+    for (int u = 0; u < kAhead; ++u) step(t + u);
   }
 #pragma unroll
   for (int u = 0; u < kAhead - 1; ++u) {
-    if (t + u < T) step(t + u, (u + 1) % kAhead);
+    if (t + u < T) step(t + u);
+  }
+  {  // y of the last token
+    half2_t y2 = {static_cast<half_t>(0.0f), static_cast<half_t>(0.0f)};
+#pragma unroll
+    for (int part = 0; part < LPR; ++part) {
+      if (part > 0) y2 = group_from_left<LPR>(y2);
+#pragma unroll
+      for (int j = 0; j < NP; ++j) y2 = pk_fma16(S[j], r_prev[j], y2);
+    }
+    if constexpr (LPR > 1) y2 = group_from_last<LPR>(y2);
+    *reinterpret_cast<half_t*>(reinterpret_cast<char*>(py) + (row2 + static_cast<unsigned>(T - 1) * row_bytes)) = y2[0] + y2[1];
   }
 
 #pragma unroll
-  for (int q = 0; q < kPairs / 4; ++q) {
+  for (int q = 0; q < NP / 4; ++q) {
     uint4_t t;
 #pragma unroll
     for (int e = 0; e < 4; ++e) t[e] = __builtin_bit_cast(uint32_t, S[4 * q + e]);
@@ -229,7 +393,18 @@ int wkv7_f16state_launch(hipStream_t st, int B, int T, int C, int H, half_t* sta
   RWKV_REQUIRE(B > 0 && T > 0 && H > 0, "wkv7_f16state: B, T, H must be positive");
   RWKV_REQUIRE(C == H * kHead, "wkv7_f16state: C (%d) must equal H*64 (H=%d)", C, H);
   RWKV_REQUIRE(state && r && w && k && v && a && b && y && elapsed, "wkv7_f16state: NULL tensor");
-  hipLaunchKernelGGL(wkv7_f16state_kernel, dim3(B * H), dim3(kWave), 0, st, T, C, H, state, r, w, w0, k, v, a, b, y, elapsed);
+  RWKV_REQUIRE(static_cast<int64_t>(T) * C < (int64_t{1} << 31), "wkv7_f16state: T * C = %lld does not fit the kernel's 32-bit byte offsets",
+               static_cast<long long>(static_cast<int64_t>(T) * C));
+  // four (two) lanes per state row while that leaves no SIMD with more than one state-owning wavefront
+  const int64_t heads = static_cast<int64_t>(B) * H;
+  const int cus = device_cu_count();
+  if (heads <= cus) {
+    hipLaunchKernelGGL(wkv7_f16state_kernel<4>, dim3(B * H), dim3(5 * kWave), 0, st, T, C, H, state, r, w, w0, k, v, a, b, y, elapsed);
+  } else if (heads <= 2 * cus) {
+    hipLaunchKernelGGL(wkv7_f16state_kernel<2>, dim3(B * H), dim3(3 * kWave), 0, st, T, C, H, state, r, w, w0, k, v, a, b, y, elapsed);
+  } else {
+    hipLaunchKernelGGL(wkv7_f16state_kernel<1>, dim3(B * H), dim3(2 * kWave), 0, st, T, C, H, state, r, w, w0, k, v, a, b, y, elapsed);
+  }
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }

@@ -74,7 +74,9 @@ def test_wkv7_drift_over_16384_tokens_against_the_fp32_oracle(gpu, orc):
     assert y_all <= F16_TOL
 
 
-@pytest.mark.parametrize("B,T,H,with_w0", [(1, 64, 12, False), (2, 7, 3, True), (3, 1, 2, True), (5, 33, 2, False)])
+# (the last two: more than one and more than two heads per CU of a 256-CU chip, i.e. two and one lanes per state row)
+@pytest.mark.parametrize("B,T,H,with_w0", [(1, 64, 12, False), (2, 7, 3, True), (3, 1, 2, True), (5, 33, 2, False),
+                                          (5, 9, 64, True), (9, 6, 64, False)])
 def test_wkv7_f16state_matches_oracle(gpu, orc, B, T, H, with_w0):
     """The fp16-state recurrence (the reference server's default mode) against the oracle's restatement of
     cuda/rwkv7_wkv_fp16_v2.cu: same fp16 fused multiply-adds in the same order, so outputs and state agree
@@ -105,6 +107,37 @@ def test_wkv7_f16state_matches_oracle(gpu, orc, B, T, H, with_w0):
     same = float(np.mean(got_s.view(np.uint16) == s_ref.view(np.uint16)))
     assert same >= 0.9, same
     assert d_elapsed.numpy().tolist() == elapsed.tolist()   # the kernel only reads elapsed
+
+
+def test_wkv7_f16state_lanes_per_row_variants_are_bitwise(gpu):
+    """The kernel gives a state row to one, two or four lanes by how many heads the call has (four while every head
+    can have a CU to itself).  The sums run over the columns in the same order in all three, so a batch row gives
+    the same bits whether it is computed alone, among five or among nine."""
+    hip = gpu
+    B, T, H = 9, 6, 64
+    C = H * 64
+    inp = wkv_inputs(B, T, H, seed=77, dtype=np.float16)
+    names = ["r", "w_raw", "k", "v", "a", "b"]
+    rng = np.random.default_rng(5)
+    w0 = dev(hip, (rng.standard_normal(C) * 0.3).astype(np.float16))
+    elapsed = rng.integers(0, 900, B).astype(np.int32)
+    s0 = (rng.standard_normal((B, H, 64, 64)) * 0.2).astype(np.float16)
+
+    def run(rows):
+        n = len(rows)
+        state = dev(hip, np.ascontiguousarray(s0[rows]))
+        y = hip.DeviceArray((n, T, C), np.float16)
+        d = [dev(hip, np.ascontiguousarray(inp[name][rows])) for name in names]
+        hip.wkv7_f16state(n, T, C, H, state, *d, y, dev(hip, np.ascontiguousarray(elapsed[rows])), w0=w0)
+        hip.device_sync()
+        return y.numpy().view(np.uint16), state.numpy().view(np.uint16)
+
+    y9, s9 = run(list(range(9)))        # 576 heads: one lane per row
+    y5, s5 = run(list(range(5)))        # 320 heads: two lanes per row
+    assert np.array_equal(y5, y9[:5]) and np.array_equal(s5, s9[:5])
+    for b in (0, 8):                    # 64 heads: four lanes per row
+        y1, s1 = run([b])
+        assert np.array_equal(y1[0], y9[b]) and np.array_equal(s1[0], s9[b])
 
 
 def test_wkv7_f16state_call_split_is_bitwise(gpu):
