@@ -129,6 +129,38 @@ __device__ __forceinline__ float row16_sum(float x) {
   x = dpp_add<0x140>(x);  // row_mirror: quads (0,1) <-> (3,2)
   return x;
 }
+// wave_sum without the trips through LDS (`__shfl_xor` is a ds_bpermute, a hundred cycles and more each, six in a
+// row): the same six levels - lane i adds what lane i ^ 32, then i ^ 16, 8, 4, 2, 1 holds - so the same bits in every
+// lane, with gfx950's row swaps for the two levels that cross DPP rows and DPP moves for the others.  For sums at the
+// end of a wavefront's work, where nothing is left to hide that latency behind.
+template <bool ROWS32>
+__device__ __forceinline__ float add_swapped_rows(float x) {
+  // v_permlane32_swap: lanes 32-63 of the first operand change places with lanes 0-31 of the second (permlane16:
+  // rows 1 and 3 of the first with rows 0 and 2 of the second); both start as x, so their sum is x[i] + x[i ^ 32]
+  // (x[i ^ 16]) in every lane.  Two idle slots between a register's write and the swap that reads it.  (The
+  // compiler's builtin for these returns the first operand twice.)
+  float d = x, s = x;
+  if constexpr (ROWS32) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(d), "+v"(s));
+  } else {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(d), "+v"(s));
+  }
+  return d + s;
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v = add_swapped_rows<true>(v);
+  v = add_swapped_rows<false>(v);
+  v = dpp_add<0x128>(v);  // row_ror:8 - lane i ^ 8 of the row
+  {                       // lane i ^ 4: the mirror image within eight lanes (i ^ 7), then within the quad (^ 3)
+    const int m = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false);
+    const int q = __builtin_amdgcn_update_dpp(0, m, 0x1B, 0xf, 0xf, false);
+    v += __builtin_bit_cast(float, q);
+  }
+  v = dpp_add<0x4E>(v);  // quad_perm [2,3,0,1]
+  v = dpp_add<0xB1>(v);  // quad_perm [1,0,3,2]
+  return v;
+}
+
 // Sum over the 64 lanes of a wave without index registers (DPP inside the four rows, then the four row sums through
 // scalar registers); the result is wave-uniform.  For kernels that are short of vector registers.
 __device__ __forceinline__ float wave_sum_uniform(float v) {
@@ -156,7 +188,7 @@ __device__ __forceinline__ float block_sum_uniform(float v, float* scratch) {
 // Block-wide sum for blocks of NW waves; `scratch` holds NW floats of LDS.  All threads get the sum.
 template <int NW>
 __device__ __forceinline__ float block_sum(float v, float* scratch) {
-  v = wave_sum(v);
+  v = wave_sum_dpp(v);
   if constexpr (NW == 1) return v;
   const int wave = threadIdx.x >> 6;
   __syncthreads();  // scratch may still be read from a previous call

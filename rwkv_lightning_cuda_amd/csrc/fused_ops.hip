@@ -182,8 +182,8 @@ __global__ __launch_bounds__(NT) void ln_fused_kernel(LnArgs a) {
 // the caller moves it over afterwards.
 template <int NT>
 __device__ __forceinline__ void block_sum2(float& a, float& b, float* scratch) {  // block_sum's order, two values
-  a = wave_sum(a);
-  b = wave_sum(b);
+  a = wave_sum_dpp(a);
+  b = wave_sum_dpp(b);
   if constexpr (NT / 64 == 1) return;
   const int wave = threadIdx.x >> 6;
   __syncthreads();

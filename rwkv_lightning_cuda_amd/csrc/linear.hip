@@ -43,7 +43,7 @@ struct LinearArgs {
 // weight-streaming loop its occupancy.  256 threads; red holds 16 floats.
 __device__ __forceinline__ float ln_block_sum4(float (&x)[4], float* red) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) x[j] = wave_sum(x[j]);
+  for (int j = 0; j < 4; ++j) x[j] = wave_sum_dpp(x[j]);
   __syncthreads();  // red may still be read from a previous call
   if ((threadIdx.x & 63) == 0) {
 #pragma unroll
@@ -401,7 +401,7 @@ __device__ __forceinline__ void gemv_block(const LinearArgs& args, const LinearP
 #pragma unroll
   for (int r = 0; r < R; ++r)
 #pragma unroll
-    for (int m = 0; m < M; ++m) acc[r][m] = wave_sum(acc[r][m]);
+    for (int m = 0; m < M; ++m) acc[r][m] = wave_sum_dpp(acc[r][m]);
 
   if (lane == 0) {
 #pragma unroll
@@ -955,7 +955,7 @@ __device__ __forceinline__ void gemv_row1_block(const LinearArgs& args, const Li
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int m = 0; m < M; ++m) acc[r][m] = wave_sum(acc[r][m]);
+      for (int m = 0; m < M; ++m) acc[r][m] = wave_sum_dpp(acc[r][m]);
     if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
