@@ -37,10 +37,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak, published
 # figure is stale and `traffic` is reported as null until the counters are collected again.
 MEASURED_TRAFFIC = {
     ("7.2B", "w8", 1): {
-        "bytes_per_launch": 49974285,
+        "bytes_per_launch": 49977226,
         "profile": "profiles/linear_gemv_row1_decode_7p2b_w8_bs1_pmc_traffic.md",
         "kernel_source": "rwkv_lightning_cuda_amd/csrc/linear.hip",
-        "kernel_source_sha256": "58912a6a991e6bb8f3d55d5442a8ab0ae60ee48df8bfb6c46edab5664d018dd1",
+        "kernel_source_sha256": "80f6b9afc28f817c5b9ae5e25654c011378935dd2cceed2a2299f90b05f38d9e",
     },
 }
 
