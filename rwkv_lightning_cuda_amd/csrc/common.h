@@ -161,6 +161,42 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
   return v;
 }
 
+// The same butterfly for any operation on 32-bit values: lane_xor_dpp<D>(x) is what `__shfl_xor(x, D, 64)` returns.
+template <int D>
+__device__ __forceinline__ int lane_xor_dpp(int x) {
+  static_assert(D == 32 || D == 16 || D == 8 || D == 4 || D == 2 || D == 1, "a single bit of the lane index");
+  if constexpr (D == 32 || D == 16) {
+    // after the swap the first operand holds x of the rows [0, 1, 0, 1] ([0, 0, 2, 2]), the second [2, 3, 2, 3] ([1, 1, 3, 3])
+    int d = x, s = x;
+    if constexpr (D == 32) {
+      asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(d), "+v"(s));
+    } else {
+      asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(d), "+v"(s));
+    }
+    return (threadIdx.x & D) ? d : s;
+  } else if constexpr (D == 8) {
+    return __builtin_amdgcn_update_dpp(0, x, 0x128, 0xf, 0xf, false);
+  } else if constexpr (D == 4) {
+    return __builtin_amdgcn_update_dpp(0, __builtin_amdgcn_update_dpp(0, x, 0x141, 0xf, 0xf, false), 0x1B, 0xf, 0xf, false);
+  } else if constexpr (D == 2) {
+    return __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xf, 0xf, false);
+  } else {
+    return __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xf, 0xf, false);
+  }
+}
+// v = op(v, value of lane i ^ 32), then ^ 16, 8, 4, 2, 1: every lane ends with the reduction over the wavefront
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_reduce_dpp(T v, Op op) {
+  static_assert(sizeof(T) == 4, "32-bit values");
+  v = op(v, __builtin_bit_cast(T, lane_xor_dpp<32>(__builtin_bit_cast(int, v))));
+  v = op(v, __builtin_bit_cast(T, lane_xor_dpp<16>(__builtin_bit_cast(int, v))));
+  v = op(v, __builtin_bit_cast(T, lane_xor_dpp<8>(__builtin_bit_cast(int, v))));
+  v = op(v, __builtin_bit_cast(T, lane_xor_dpp<4>(__builtin_bit_cast(int, v))));
+  v = op(v, __builtin_bit_cast(T, lane_xor_dpp<2>(__builtin_bit_cast(int, v))));
+  v = op(v, __builtin_bit_cast(T, lane_xor_dpp<1>(__builtin_bit_cast(int, v))));
+  return v;
+}
+
 // Sum over the 64 lanes of a wave without index registers (DPP inside the four rows, then the four row sums through
 // scalar registers); the result is wave-uniform.  For kernels that are short of vector registers.
 __device__ __forceinline__ float wave_sum_uniform(float v) {

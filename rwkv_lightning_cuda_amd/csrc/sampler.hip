@@ -10,7 +10,8 @@
 // for rows of up to 65536 entries the float4 t, t + 1024, ..., loaded once (coalesced) and kept in registers
 // through the softmax, the bisection and the draw; for larger rows a contiguous slice that stays in `probs` -
 // so the draw is a single inverse-CDF walk with one uniform number over a fixed order of the row; block
-// reductions are wave64 shuffles + one LDS exchange; top_k == 1 (greedy, what top_p == 0 normalises to) skips the
+// reductions are wave64 butterflies (DPP and row swaps, no LDS) + one LDS exchange; a bisection step skips the
+// slots whose largest entry lies below its threshold; top_k == 1 (greedy, what top_p == 0 normalises to) skips the
 // bisection.  Randomness is counter-based Philox4x32-10 keyed by (seed; row, step) instead of a
 // per-row cuRAND state seeded from the wall clock (src/rwkv_sampler.cpp:14-19), so a run is reproducible.
 #include <cfloat>
@@ -34,8 +35,7 @@ struct BlockRed {
 
 template <typename Op>
 __device__ __forceinline__ float block_reduce_f(float v, Op op, float* buf) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, 64));
+  v = wave_reduce_dpp(v, op);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) buf[threadIdx.x >> 6] = v;
   __syncthreads();
@@ -46,8 +46,7 @@ __device__ __forceinline__ float block_reduce_f(float v, Op op, float* buf) {
 }
 
 __device__ __forceinline__ unsigned block_sum_u(unsigned v, unsigned* buf) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  v = wave_reduce_dpp(v, [](unsigned x, unsigned y) { return x + y; });
   __syncthreads();
   if ((threadIdx.x & 63) == 0) buf[threadIdx.x >> 6] = v;
   __syncthreads();
@@ -115,11 +114,8 @@ struct SampleArgs {
 // count and mass of one bisection step through one LDS exchange (the same sums, in the same order, as
 // block_sum_u and block_reduce_f one after the other)
 __device__ __forceinline__ void block_count_mass(unsigned& c, float& m, BlockRed& red) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    c += __shfl_xor(c, off, 64);
-    m += __shfl_xor(m, off, 64);
-  }
+  c = wave_reduce_dpp(c, [](unsigned x, unsigned y) { return x + y; });
+  m = wave_reduce_dpp(m, [](float x, float y) { return x + y; });
   __syncthreads();
   if ((threadIdx.x & 63) == 0) {
     red.u[threadIdx.x >> 6] = c;
@@ -213,8 +209,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
   if (a.top_k == 1) {
     // greedy: lowest index among the maxima (the reference draws uniformly among exact ties)
     unsigned cand = (maxu == gmax) ? static_cast<unsigned>(maxi) : 0x7fffffffu;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) cand = min(cand, static_cast<unsigned>(__shfl_xor(static_cast<int>(cand), off, 64)));
+    cand = wave_reduce_dpp(cand, [](unsigned x, unsigned y) { return min(x, y); });
     __syncthreads();
     if ((t & 63) == 0) red.u[t >> 6] = cand;
     __syncthreads();
@@ -243,6 +238,23 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
       }
       put(q, i, l);
     });
+    // REG: the largest probability among the 256 entries that this wavefront holds in slot q (bit pattern; the same
+    // in every lane).  A bisection step whose threshold lies above it has nothing to count there.
+    unsigned slot_max[REG ? kSampleRegVecs : 1];
+    const bool bisect = a.top_k < V || a.top_p < 1.0f;  // (else the loop below does not run: no threshold to find)
+    if constexpr (REG) {
+#pragma unroll
+      for (int q = 0; q < kSampleRegVecs; ++q) slot_max[q] = 0xffffffffu;
+    }
+    if (REG && bisect) {
+#pragma unroll
+      for (int q = 0; q < kSampleRegVecs; ++q) {
+        float mx = 0.0f;
+        if (q < n) mx = fmaxf(fmaxf(vals[q][0], vals[q][1]), fmaxf(vals[q][2], vals[q][3]));
+        mx = wave_reduce_dpp(mx, fmax_op);
+        slot_max[q] = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, mx)));
+      }
+    }
     pmax = block_reduce_f(pmax, fmax_op, red.f);
     pmin = block_reduce_f(pmin, fmin_op, red.f);
 
@@ -255,15 +267,34 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
       const float thr = __uint_as_float(mid);
       unsigned c = 0;
       float m = 0.0f;
-      for_each([&](int q, int i) {
-        const float4_t l = get(q, i);
+      if constexpr (REG) {
+        // (probabilities are not negative: their order is the order of their bit patterns, which the bisection
+        // itself relies on; the comparison of two wavefront-wide values is a scalar one)
+        const unsigned mid_u = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(mid)));
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (l[j] >= thr) {
-            ++c;
-            m += l[j];
+        for (int q = 0; q < kSampleRegVecs; ++q) {
+          if (slot_max[q] >= mid_u) {
+            if (q < n) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                if (vals[q][j] >= thr) {
+                  ++c;
+                  m += vals[q][j];
+                }
+            }
           }
-      });
+        }
+      } else {
+        for_each([&](int q, int i) {
+          const float4_t l = get(q, i);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (l[j] >= thr) {
+              ++c;
+              m += l[j];
+            }
+        });
+      }
       block_count_mass(c, m, red);
       if (c < static_cast<unsigned>(a.top_k) && m < a.top_p) {
         right = mid;
