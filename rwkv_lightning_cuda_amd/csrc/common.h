@@ -132,7 +132,9 @@ __device__ __forceinline__ float row16_sum(float x) {
 // wave_sum without the trips through LDS (`__shfl_xor` is a ds_bpermute, a hundred cycles and more each, six in a
 // row): the same six levels - lane i adds what lane i ^ 32, then i ^ 16, 8, 4, 2, 1 holds - so the same bits in every
 // lane, with gfx950's row swaps for the two levels that cross DPP rows and DPP moves for the others.  For sums at the
-// end of a wavefront's work, where nothing is left to hide that latency behind.
+// end of a wavefront's work, where nothing is left to hide that latency behind.  Every lane of the wavefront has to
+// be active (a lane that is switched off would neither give nor take its value): call them from code that whole
+// wavefronts run, as all their callers do.
 template <bool ROWS32>
 __device__ __forceinline__ float add_swapped_rows(float x) {
   // v_permlane32_swap: lanes 32-63 of the first operand change places with lanes 0-31 of the second (permlane16:
