@@ -231,6 +231,30 @@ def sampled_decode(hip, sess, dims, state, logits, B, first, steps=64):
     return {"decode_sampled_bs%d_tok_s" % B: steps * B / dt, "decode_sampled_bs%d_ms_per_step" % B: dt * 1e3 / steps}
 
 
+def sampler_call_us(hip, V, calls=200):
+    """Microseconds per call of the device sampler alone (one launch; rows of V logits ~ N(0, 9), penalties on): without
+    filters, with top-k 50 + top-p 0.6, and with top-p 0.9 alone, at 1 and 64 rows."""
+    res = {}
+    for B in (1, 64):
+        g = np.random.default_rng(B)
+        logits = hip.DeviceArray.from_numpy((g.standard_normal((B, V)) * 3).astype(np.float32))
+        pen = hip.DeviceArray.zeros((B, V), np.float32)
+        probs = hip.DeviceArray((B, V), np.float32)
+        picked = hip.DeviceArray((B,), np.int32)
+        for name, kw in (("plain", dict(top_k=0, top_p=1.0)), ("top_k50_top_p0.6", dict(top_k=50, top_p=0.6)),
+                         ("top_p0.9", dict(top_k=0, top_p=0.9))):
+            for phase in (5, calls):
+                hip.device_sync()
+                t0 = time.perf_counter()
+                for i in range(phase):
+                    hip.sample(B, V, logits, pen, probs, picked, presence=0.5, frequency=0.1, decay=0.99, temperature=1.0,
+                               seed=3, step=i, **kw)
+                hip.device_sync()
+                dt = time.perf_counter() - t0
+            res["bs%d_%s" % (B, name)] = dt * 1e6 / calls
+    return res
+
+
 def wkv7_op_long_context(hip, H, reps=3):
     """The WKV7 op alone at the long-context configuration: fp16 r,w,k,v,a,b [16,16384,64 H], fp32 state, raw-logit
     decay, one call.  Rows are 4096-token windows of one host-generated sequence (r,k,v ~ N(0,1); decay =
@@ -663,6 +687,7 @@ def main():
         also["launch_chain_us_per_link_graph"] = hip.measure_launch_chain(260, 256, 256, True, 20)
         also["launch_chain_us_per_link_direct"] = hip.measure_launch_chain(260, 256, 256, False, 20)
         also["engine_boundary"] = engine_boundary_rates(args.preset, args.fmt)
+        also["sampler_us_per_call"] = sampler_call_us(hip, dims.V)
     if not args.no_parity and args.preset == "7.2B":
         out["parity"], more = parity_legs(hip, args.fmt, not args.no_also)
         also.update(more)
