@@ -877,15 +877,6 @@ int check_forward_args(const rwkv_hip_session* s, int B, int T, const void* shif
   return model_ready(s->model);
 }
 
-__global__ void feed_tokens_kernel(int B, const int* __restrict__ picked, int64_t* __restrict__ tokens,
-                                   int* __restrict__ history) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < B) {
-    tokens[i] = picked[i];
-    history[i] = picked[i];
-  }
-}
-
 }  // namespace
 
 extern "C" {
@@ -1246,10 +1237,9 @@ int rwkv_hip_decode_greedy(rwkv_hip_session* s, const int64_t* first_tokens_host
   RWKV_HIP_TRY(hipMemcpyAsync(s->tokens_dev, s->tokens_pinned, sizeof(int64_t) * B, hipMemcpyHostToDevice, s->stream));
   for (int i = 0; i < steps; ++i) {
     TRY(run_step(s, B, static_cast<half_t*>(shift), wkv, static_cast<int*>(elapsed), static_cast<float*>(logits)));
-    TRY(argmax_launch(s->stream, B, s->model->V, static_cast<float*>(logits), s->argmax_dev));
-    hipLaunchKernelGGL(feed_tokens_kernel, dim3(ceil_div(B, 64)), dim3(64), 0, s->stream, B, s->argmax_dev,
-                       s->tokens_dev, s->history_dev + static_cast<size_t>(i) * B);
-    RWKV_LAUNCH_CHECK();
+    // the picked ids are the next step's input tokens and step i of the list that goes back to the host
+    TRY(argmax_launch(s->stream, B, s->model->V, static_cast<float*>(logits), s->argmax_dev, s->tokens_dev,
+                      s->history_dev + static_cast<size_t>(i) * B));
   }
   RWKV_HIP_TRY(hipMemcpyAsync(out_tokens_host, s->history_dev, sizeof(int) * hist, hipMemcpyDeviceToHost, s->stream));
   RWKV_HIP_TRY(hipStreamSynchronize(s->stream));

@@ -232,7 +232,8 @@ int ffn_sparse_launch(hipStream_t st, int fmt, int rows, int C, int F, int activ
                       bool one_walk);
 
 // ---- sampler.hip --------------------------------------------------------------------------------
-int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out);
+// out[b] = index of the largest logit of row b (the lowest one among equals); next / history (may be null) get the same id
+int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out, int64_t* next = nullptr, int* history = nullptr);
 
 // ---- wkv7.hip -----------------------------------------------------------------------------------
 // T tokens of the recurrence from fp32 operands (decay applied); v, y fp16.  op_bs / io_bs: elements

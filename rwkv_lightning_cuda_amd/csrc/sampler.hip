@@ -394,7 +394,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleArgs a) {
 // the kernel is pure load latency).  Lowest index among equal maxima.
 constexpr int kArgmaxThreads = 1024;
 
-__global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(int V, const float* __restrict__ logits, int* __restrict__ out) {
+// next / history (may be null): the picked id also becomes the row's next input token and an entry of the caller's
+// list of generated tokens - what a greedy decode loop would otherwise launch a second kernel for.
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(int V, const float* __restrict__ logits, int* __restrict__ out,
+                                                               int64_t* __restrict__ next, int* __restrict__ history) {
   __shared__ float bv[kArgmaxThreads / 64];
   __shared__ int bi[kArgmaxThreads / 64];
   const float* row = logits + static_cast<int64_t>(blockIdx.x) * V;
@@ -449,12 +452,15 @@ __global__ __launch_bounds__(kArgmaxThreads) void argmax_kernel(int V, const flo
         best = bv[i];
         idx = bi[i];
       }
-    out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    const int pick = idx == 0x7fffffff ? 0 : idx;
+    out[blockIdx.x] = pick;
+    if (next) next[blockIdx.x] = pick;
+    if (history) history[blockIdx.x] = pick;
   }
 }
 
-int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out) {
-  hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(kArgmaxThreads), 0, st, V, logits, out);
+int argmax_launch(hipStream_t st, int B, int V, const float* logits, int* out, int64_t* next, int* history) {
+  hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(kArgmaxThreads), 0, st, V, logits, out, next, history);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;
 }
