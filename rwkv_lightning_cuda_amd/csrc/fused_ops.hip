@@ -440,10 +440,12 @@ __global__ __launch_bounds__(256) void kk_a_gate_kernel(KkArgs p) {
     p.d32[idx] = exp2f(-0.8750387749145276f / (1.0f + exp2f(-1.4426950408889634f * wraw)));
     p.r32[idx] = h2f(p.r[idx]);
   }
+  if (p.w_sum16) p.w_sum16[idx] = f2h(h2f(p.w12[idx]) + h2f(p.w0[c]));
 }
 
 int kk_a_gate_launch(hipStream_t st, const KkArgs& p) {
   RWKV_REQUIRE(p.rows_heads > 0 && p.H > 0, "kk_a_gate: bad shape");
+  RWKV_REQUIRE(p.w_sum16 == nullptr || (p.w12 && p.w0), "kk_a_gate: the rounded decay logit needs w12 and w0");
   hipLaunchKernelGGL(kk_a_gate_kernel, dim3(ceil_div(p.rows_heads, 4)), dim3(256), 0, st, p);
   RWKV_LAUNCH_CHECK();
   return RWKV_OK;

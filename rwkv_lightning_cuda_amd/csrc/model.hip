@@ -648,14 +648,14 @@ int enqueue_forward(rwkv_hip_session* s, int B, int T, half_t* shift, void* wkv_
         p.k = b.k; p.k_k = w.t[RWKV_T_K_K]; p.a0 = w.t[RWKV_T_A0]; p.a12 = b.a12; p.k_a = w.t[RWKV_T_K_A];
         p.new_k = b.k2; p.neg_kk = b.nkk; p.kka = b.kka;
         p.rows_heads = static_cast<int64_t>(rows) * H; p.H = H;
-        TRY_AUX(kk_a_gate_launch(st, p));
         const half_t* w_in = b.w12;
         const half_t* w0 = w.t[RWKV_T_W0];
-        if (T > 16) {
-          TRY_AUX(add_vec_launch(st, rows, C, b.w12, w.t[RWKV_T_W0], b.scratch));
+        if (T > 16) {  // w12 + w0 rounded to fp16 first: the same pass writes it
+          p.w12 = b.w12; p.w0 = w.t[RWKV_T_W0]; p.w_sum16 = b.scratch;
           w_in = b.scratch;
           w0 = nullptr;
         }
+        TRY_AUX(kk_a_gate_launch(st, p));
         TRY_AUX(wkv7_f16state_launch(st, B, T, C, H, S16, b.r, w_in, w0, b.k2, v_cur, b.nkk, b.kka, b.y, elapsed));
         TRY_AUX(lnx_launch(st, static_cast<int64_t>(rows) * H, H, b.y, b.r, b.k2, v_cur, w.t[RWKV_T_R_K], w.t[RWKV_T_LNX_W],
                            w.t[RWKV_T_LNX_B], b.g, b.y2));

@@ -180,6 +180,9 @@ struct KkArgs {
   float* b32;
   float* d32;
   float* r32;
+  // optional (needs w12 and w0): f16(w12 + w0), the decay logit as the fp16-state recurrence takes it for calls of
+  // more than 16 tokens (src/rwkv7_fast_v4.cu:1266-1271) - what add_vec_launch would write in a launch of its own
+  half_t* w_sum16;
   int64_t rows_heads;
   int H;
 };
