@@ -13,11 +13,12 @@
 // sums do not associate), so it is kept: the kernel is bit-identical to a scalar restatement of the reference except
 // where v_exp_f32 and the host's exp2f differ in the last bit before the decay delta is rounded to fp16.
 //
-// gfx950 layout: one wavefront per (batch row, head), lane = state row, the row's 64 values in 32 registers as half2
-// pairs (v_pk_fma_f16 does both columns of a pair).  The five per-column vectors of a token (a, b, k, decay delta,
-// r) are the same for every lane: lane c fetches element c of each for the NEXT token while the current one is
-// computed, converts its decay logit, and drops them into LDS, from where every lane reads them back as 16-byte
-// broadcasts.  The state is read and written once per call, 16 bytes per lane and instruction.
+// gfx950 layout of the sequence kernel: a block per (batch row, head); one, two or four lanes share a state row and
+// hold its 64 values as half2 pairs in registers for the whole call (v_pk_fma_f16 does both columns of a pair).  The
+// five per-column vectors of a token (a, b, k, decay delta, r) are the same for every row: a wavefront of its own
+// fetches them some tokens ahead, lane c element c of each, converts the decay logit and drops them into LDS, from
+// where the wavefronts that own the state read them back as 16-byte pieces.  The state is read and written once
+// per call, 16 bytes per lane and instruction.  Details at the kernel.
 #include "wkv7_f16state.h"
 
 namespace rwkv {
@@ -33,8 +34,8 @@ struct TokenOps {  // one token's per-column operands in LDS
   half_t v[kHead];  // per state row, not per column: parked here between its arrival and its step
 };
 
-// The block's two wavefronts meet once per token.  LDS only: what either has in flight to or from memory (the
-// feeder's loads of later tokens, the other's stores of y) does not have to land first.
+// The block's wavefronts meet once per token.  LDS only: what they have in flight to or from memory (the feeder's
+// loads of later tokens, the others' stores of y) does not have to land first.
 __device__ __forceinline__ void token_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
