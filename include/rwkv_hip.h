@@ -108,7 +108,8 @@ int rwkv_hip_wkv7(rwkv_stream_t s, int B, int T, int C, int H, int w_mode, int i
  * elapsed i32 [B] = tokens each row has seen before this call (read only: it phases the dither that the
  * reference adds to the decay before rounding it to fp16, cuda/rwkv7_wkv_fp16_v2.cu:41-52).  Every operation is an
  * fp16 fused multiply-add in the reference's order.  T1+T2 tokens in one call or in two (elapsed advanced by T1
- * in between) give bitwise the same result. */
+ * in between) give bitwise the same result, and so does any batch size (the kernel gives a state row to four, two
+ * or one lanes by the number of heads in the call; the sums keep their order).  T * C must stay below 2^31. */
 int rwkv_hip_wkv7_f16state(rwkv_stream_t s, int B, int T, int C, int H, void* state, const void* r, const void* w,
                            const void* w0, const void* k, const void* v, const void* a, const void* b, void* y,
                            const void* elapsed);
