@@ -163,6 +163,11 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
   return v;
 }
 
+// wave_sum(a * b) as the compiler builds it where the product is formed right in front of the shuffles: the first
+// level is a fused multiply-add, fma(a, b, the other lane's rounded product) - one rounding fewer than product +
+// product, and so other bits.  Code that has to give the bits of such a kernel without its shuffles says it
+// explicitly (wave_sum_dpp_of_product, below).
+
 // The same butterfly for any operation on 32-bit values: lane_xor_dpp<D>(x) is what `__shfl_xor(x, D, 64)` returns.
 template <int D>
 __device__ __forceinline__ int lane_xor_dpp(int x) {
@@ -196,6 +201,21 @@ __device__ __forceinline__ T wave_reduce_dpp(T v, Op op) {
   v = op(v, __builtin_bit_cast(T, lane_xor_dpp<4>(__builtin_bit_cast(int, v))));
   v = op(v, __builtin_bit_cast(T, lane_xor_dpp<2>(__builtin_bit_cast(int, v))));
   v = op(v, __builtin_bit_cast(T, lane_xor_dpp<1>(__builtin_bit_cast(int, v))));
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum_dpp_of_product(float a, float b) {
+  float p;
+  {
+#pragma clang fp contract(off)
+    p = a * b;
+  }
+  float v = fmaf(a, b, __builtin_bit_cast(float, lane_xor_dpp<32>(__builtin_bit_cast(int, p))));
+  v = add_swapped_rows<false>(v);
+  v = dpp_add<0x128>(v);
+  v += __builtin_bit_cast(float, lane_xor_dpp<4>(__builtin_bit_cast(int, v)));
+  v = dpp_add<0x4E>(v);
+  v = dpp_add<0xB1>(v);
   return v;
 }
 

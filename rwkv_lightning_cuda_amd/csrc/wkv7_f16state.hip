@@ -330,7 +330,9 @@ __global__ __launch_bounds__(256) void tmix16_rows_kernel(Tmix16RowsArgs p) {
   // ---- kk normalise, a-gate, decay delta (kk_a_gate_kernel; decay_delta16 with w0 added unrounded)
   const float kv = h2f(k_h);
   const float u = kv * h2f(kk_h);
-  const float total = wave_sum(u * u);
+  // (this wavefront has its SIMD nearly to itself at the batch sizes this kernel serves: sums without LDS round
+  // trips, in the stand-alone kernels' order and with their fused first level)
+  const float total = wave_sum_dpp_of_product(u, u);
   const float inv = 1.0f / fmaxf(sqrtf(total), kKkEps);
   const float kk = u * inv;
   const float av = sigmoid_f(h2f(a0_h) + h2f(a12_h));
@@ -367,11 +369,16 @@ __global__ __launch_bounds__(256) void tmix16_rows_kernel(Tmix16RowsArgs p) {
 
   // ---- GroupNorm over the head, bonus, gate (lnx_rkvres_xg_kernel)
   const float yv = h2f(y16);
-  const float mean = wave_sum(yv) * (1.0f / 64.0f);
+  const float mean = wave_sum_dpp(yv) * (1.0f / 64.0f);
   const float d = yv - mean;
-  const float var = wave_sum(d * d) * (1.0f / 64.0f);
+  const float var = wave_sum_dpp_of_product(d, d) * (1.0f / 64.0f);
   const float rstd = rsqrtf(var + kLnxEps);
-  const float rkv = wave_sum(h2f(r_h) * h2f(nk) * h2f(rk_h));
+  float rk2;
+  {
+#pragma clang fp contract(off)
+    rk2 = h2f(r_h) * h2f(nk);
+  }
+  const float rkv = wave_sum_dpp_of_product(rk2, h2f(rk_h));
   const float o = (d * rstd * h2f(lnw_h) + h2f(lnb_h) + rkv * h2f(v_h)) * h2f(g_h);
   p.y2[idx] = f2h(o);
 }
